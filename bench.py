@@ -1,0 +1,365 @@
+#!/usr/bin/env python3
+"""Benchmark of the mi355x hot path on ONE MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only NAME]
+
+Prints one JSON line.  The headline workload is BASELINE config 2, the
+memory-bound residual-add + LayerNorm fusion in bf16 on [8192, 4096]; a "step"
+is one launch of the fused op over one batch of seeded synthetic input that is
+already resident in HBM.  `value` is algorithmic bytes moved per second through
+the product path (torch.ops.xpu_ops -> C ABI -> HIP kernel).  `roofline` is the
+same kernel launched back-to-back straight through the C ABI, timed with HIP
+events on the launch stream.  `cpu_baseline` is the same eager function on the
+host cores (through this package's default, non-vendor compile path when it is
+available).  `configs` carries the same three figures for the other benchmark
+configurations.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
+BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 MFMA, published
+FP8_PEAK_TFLOPS = 5000.0
+N_SETS = 6  # rotating buffer sets so that timed launches stream from HBM, not from the 256 MB last-level cache
+
+
+def _p(t):
+    return ctypes.c_void_p(t.data_ptr())
+
+
+def _events_time(torch, fn, n_sets, steps, warmup):
+    """Average seconds per call of fn(i) over `steps` back-to-back calls, by HIP events on the current stream."""
+    for i in range(warmup):
+        fn(i % n_sets)
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for i in range(steps):
+        fn(i % n_sets)
+    stop.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) * 1e-3 / steps
+
+
+def _wall_time(torch, fn, n_sets, steps, warmup):
+    for i in range(warmup):
+        fn(i % n_sets)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        fn(i % n_sets)
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps
+
+
+def _cpu_time(fn, min_iters=3, budget_s=12.0, max_iters=30):
+    fn()  # warm-up (also compiles the default path)
+    fn()
+    times = []
+    t_end = time.perf_counter() + budget_s
+    while len(times) < min_iters or (time.perf_counter() < t_end and len(times) < max_iters):
+        t0 = time.perf_counter()
+        fn()
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    return times[len(times) // 2], len(times)
+
+
+def _default_path_compile(fn):
+    """The reference's non-vendor path: XpuGraph(XpuGraphConfig(is_training=False)) on CPU tensors."""
+    import torch
+
+    try:
+        from xpu_graph_amd import XpuGraph, XpuGraphConfig
+
+        return torch.compile(fn, backend=XpuGraph(XpuGraphConfig(is_training=False)), dynamic=False), "XpuGraph default path (target=none, level1)"
+    except ImportError:
+        return fn, "eager"
+
+
+class Workload:
+    name = ""
+    bound = "hbm"
+    dtype = ""
+    unit = "GB/s"
+
+    def setup(self, torch, dev):
+        raise NotImplementedError
+
+    def op_call(self, i):  # product path
+        raise NotImplementedError
+
+    def abi_call(self, i):  # straight C ABI
+        raise NotImplementedError
+
+    def check(self, torch):
+        raise NotImplementedError
+
+    def cpu_fn(self, torch):
+        raise NotImplementedError
+
+    work = 0  # algorithmic bytes (hbm) or flops (mfma) per launch
+
+
+class AddLayerNormC2(Workload):
+    name = "C2 residual-add + LayerNorm bf16 [8192,4096] -> (y, h)"
+    dtype = "bf16"
+    kernel = "norm_rows_kernel<bf16,bf16,LAYER>"
+    work = 4 * 8192 * 4096 * 2 + 2 * 4096 * 2
+
+    def setup(self, torch, dev):
+        from oracle import inputs
+
+        self.torch = torch
+        self.sets = [inputs.c2_add_layernorm(device=dev, seed=i) for i in range(N_SETS)]
+        self.y = [torch.empty_like(s[0]) for s in self.sets]
+        self.h = [torch.empty_like(s[0]) for s in self.sets]
+        from xpu_graph_amd import _lib
+
+        self.lib = _lib.lib()
+        self.st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def op_call(self, i):
+        x, r, g, b = self.sets[i]
+        return self.torch.ops.xpu_ops.add_layer_norm(x, r, g, b, 1e-5)
+
+    def abi_call(self, i):
+        x, r, g, b = self.sets[i]
+        self.lib.xg_add_layer_norm(_p(x), _p(r), _p(g), _p(b), _p(self.y[i]), _p(self.h[i]), 8192, 4096, 4096, 4096, 1e-5, 2, 2, self.st)
+
+    def check(self, torch):
+        from oracle import eager
+
+        x, r, g, b = self.sets[0]
+        y, h = self.op_call(0)
+        y_ref, h_ref = eager.add_layernorm_eager(x, r, g, b, 1e-5)
+        assert torch.equal(h, h_ref)
+        torch.testing.assert_close(y, y_ref, rtol=1.6e-2, atol=1e-5)
+
+    def cpu_fn(self, torch):
+        from oracle import eager, inputs
+
+        x, r, g, b = inputs.c2_add_layernorm(device="cpu", seed=0)
+        fn, how = _default_path_compile(lambda x, r, g, b: eager.add_layernorm_eager(x, r, g, b, 1e-5))
+        return (lambda: fn(x, r, g, b)), how
+
+
+class RmsNormC1(Workload):
+    name = "C1 RMSNorm fp32 [2048,4096]"
+    dtype = "f32"
+    kernel = "norm_rows_kernel<f32,f32,RMS>"
+    work = 2 * 2048 * 4096 * 4 + 4096 * 4
+
+    def setup(self, torch, dev):
+        from oracle import inputs
+        from xpu_graph_amd import _lib
+
+        self.torch = torch
+        self.sets = [inputs.c1_rmsnorm(device=dev, seed=i) for i in range(N_SETS)]
+        self.y = [torch.empty_like(s[0]) for s in self.sets]
+        self.lib = _lib.lib()
+        self.st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def op_call(self, i):
+        x, w = self.sets[i]
+        return self.torch.ops.xpu_ops.rms_norm(x, w, 1e-6)
+
+    def abi_call(self, i):
+        x, w = self.sets[i]
+        self.lib.xg_rms_norm(_p(x), _p(w), _p(self.y[i]), 2048, 4096, 4096, 1e-6, 0, 0, self.st)
+
+    def check(self, torch):
+        from oracle import eager
+
+        x, w = self.sets[0]
+        torch.testing.assert_close(self.op_call(0), eager.rmsnorm_eager(x, w, 1e-6), rtol=1e-5, atol=1e-5)
+
+    def cpu_fn(self, torch):
+        from oracle import eager, inputs
+
+        x, w = inputs.c1_rmsnorm(device="cpu", seed=0)
+        fn, how = _default_path_compile(lambda x, w: eager.rmsnorm_eager(x, w, 1e-6))
+        return (lambda: fn(x, w)), how
+
+
+class SliceCatC3a(Workload):
+    name = "C3a slice/cat fp32 [4096,8192] -> 64x32 -> [4096,2048]"
+    dtype = "b32"
+    kernel = "slice_cat_kernel<16>"
+    work = 2 * 4096 * 2048 * 4 + 64 * 8
+
+    def setup(self, torch, dev):
+        from oracle import inputs
+        from xpu_graph_amd import _lib, ops
+
+        self.torch = torch
+        self.srcs = []
+        for i in range(N_SETS):
+            src, self.slices = inputs.c3_slice_cat(device=dev, seed=i)
+            self.srcs.append(src)
+        table, self.chunk, self.out_cols = ops.build_slice_table([self.slices], 8192, 4, 8192)
+        self.table = table.to(dev)
+        self.outs = [torch.empty(4096, 2048, device=dev) for _ in range(N_SETS)]
+        self.lib = _lib.lib()
+        self.st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        self.ptrs = [(ctypes.c_void_p * 1)(o.data_ptr()) for o in self.outs]
+        self.rbs = (ctypes.c_int64 * 1)(2048 * 4)
+
+    def op_call(self, i):
+        return self.torch.ops.xpu_ops.slice_cat(self.srcs[i], self.table, self.chunk, self.out_cols[0])
+
+    def abi_call(self, i):
+        self.lib.xg_slice_cat(_p(self.srcs[i]), 8192 * 4, 4096, self.ptrs[i], self.rbs, 1, _p(self.table), self.table.shape[0], self.chunk, self.st)
+
+    def check(self, torch):
+        from oracle import eager
+
+        assert torch.equal(self.op_call(0), eager.slice_cat_eager(self.srcs[0], self.slices))
+
+    def cpu_fn(self, torch):
+        from oracle import eager, inputs
+
+        src, slices = inputs.c3_slice_cat(device="cpu", seed=0)
+        fn, how = _default_path_compile(lambda s: eager.slice_cat_eager(s, slices))
+        return (lambda: fn(src)), how
+
+
+class AddNC3b(Workload):
+    name = "C3b sum of 32 x [4096,256] fp32"
+    dtype = "f32"
+    kernel = "addn_kernel<f32>"
+    work = 33 * 4096 * 256 * 4
+
+    def setup(self, torch, dev):
+        from oracle import inputs
+        from xpu_graph_amd import _lib
+
+        self.torch = torch
+        self.sets = [inputs.c3_addn(device=dev, seed=i) for i in range(N_SETS)]
+        self.outs = [torch.empty(4096, 256, device=dev) for _ in range(N_SETS)]
+        self.arrs = [(ctypes.c_void_p * 32)(*[t.data_ptr() for t in s]) for s in self.sets]
+        self.lib = _lib.lib()
+        self.st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def op_call(self, i):
+        return self.torch.ops.xpu_ops.addn(self.sets[i])
+
+    def abi_call(self, i):
+        self.lib.xg_addn(self.arrs[i], 32, _p(self.outs[i]), 4096 * 256, 0, self.st)
+
+    def check(self, torch):
+        from oracle import eager
+
+        assert torch.equal(self.op_call(0), eager.addn_eager(self.sets[0]))
+
+    def cpu_fn(self, torch):
+        from oracle import eager, inputs
+
+        ts = inputs.c3_addn(device="cpu", seed=0)
+        fn, how = _default_path_compile(lambda *t: eager.addn_eager(list(t)))
+        return (lambda: fn(*ts)), how
+
+
+HEADLINE = AddLayerNormC2
+OTHERS = [RmsNormC1, SliceCatC3a, AddNC3b]
+
+
+def run_workload(torch, dev, wl, steps, warmup, with_cpu=True):
+    wl.setup(torch, dev)
+    wl.check(torch)
+    peak = HBM_PEAK_GBPS if wl.bound == "hbm" else (FP8_PEAK_TFLOPS if wl.dtype == "fp8" else BF16_PEAK_TFLOPS)
+    scale = 1e9 if wl.bound == "hbm" else 1e12
+    t_op = _wall_time(torch, wl.op_call, N_SETS, steps, warmup)
+    t_k = _events_time(torch, wl.abi_call, N_SETS, max(steps, 100), max(warmup, 20))
+    res = {
+        "workload": wl.name,
+        "dtype": wl.dtype,
+        "value": wl.work / t_op / scale,
+        "unit": "GB/s" if wl.bound == "hbm" else "TFLOP/s",
+        "ms_per_step": t_op * 1e3,
+        "roofline": {
+            "bound": wl.bound,
+            "kernel": wl.kernel,
+            "achieved": wl.work / t_k / scale,
+            "peak": peak,
+            "unit": "GB/s" if wl.bound == "hbm" else "TFLOP/s",
+            "frac": wl.work / t_k / scale / peak,
+            "kernel_us": t_k * 1e6,
+            "traffic": getattr(wl, "traffic", None),
+        },
+    }
+    if with_cpu:
+        fn, how = wl.cpu_fn(torch)
+        t_cpu, n = _cpu_time(fn)
+        res["cpu_baseline"] = {
+            "value": wl.work / t_cpu / scale,
+            "unit": res["unit"],
+            "cores": torch.get_num_threads(),
+            "kind": "port",
+            "sample": f"{n} timed runs of the full-size workload through {how}, median {t_cpu * 1e3:.2f} ms",
+        }
+    return res
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--only", default=None, help="headline only, or a substring of another workload's name")
+    ap.add_argument("--no-cpu", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py measures one GPU: the hot path has no cross-GPU part; run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (the mi355x path has no CPU fallback)", file=sys.stderr)
+        sys.exit(1)
+    import xpu_graph_amd.ops  # noqa: F401
+
+    torch.set_num_threads(min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16"))))
+    dev = torch.device("cuda:0")
+    head = run_workload(torch, dev, HEADLINE(), args.steps, args.warmup, with_cpu=not args.no_cpu)
+    out = {
+        "metric": "fused-op GB/s (residual-add + LayerNorm, % of HBM peak in roofline.frac)",
+        "value": head["value"],
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": head["ms_per_step"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": head["dtype"],
+        "data": "synthetic",
+        "config": {"workload": head["workload"], "buffer_sets": N_SETS},
+        "roofline": head["roofline"],
+    }
+    if "cpu_baseline" in head:
+        out["cpu_baseline"] = head["cpu_baseline"]
+    others = []
+    if args.only != "headline":
+        for cls in OTHERS:
+            wl = cls()
+            if args.only and args.only.lower() not in wl.name.lower():
+                continue
+            others.append(run_workload(torch, dev, wl, args.steps, args.warmup, with_cpu=not args.no_cpu))
+            del wl
+            torch.cuda.empty_cache()
+    out["configs"] = others
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

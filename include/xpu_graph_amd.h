@@ -1,0 +1,193 @@
+/*
+ * xpu_graph_amd.h -- C ABI of the MI355X (gfx950) kernel library behind the
+ * `mi355x` target of the xpu_graph FX/Aten compiler.
+ *
+ * Every entry point
+ *   - takes plain device pointers, sizes, strides (in ELEMENTS unless the name
+ *     says bytes) and a HIP stream (`void*` == hipStream_t, NULL = default);
+ *   - only enqueues work on that stream: it never allocates, never frees and
+ *     never synchronises, so it can be recorded into a HIP graph;
+ *   - validates its arguments on the host and returns XG_OK (0) or a negative
+ *     xg_status code without launching anything when they do not fit what the
+ *     kernel assumes;  xg_status_string() names the code.
+ *
+ * The reference (XPU-Forces/xpu_graph, 100 % Python) has no FFI of its own: its
+ * target packages call vendor operator libraries.  Each declaration below cites
+ * the reference call site whose arithmetic it replaces.
+ */
+#ifndef XPU_GRAPH_AMD_H
+#define XPU_GRAPH_AMD_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* xg_stream_t; /* hipStream_t */
+
+typedef enum {
+  XG_OK = 0,
+  XG_ERR_BAD_DTYPE = -1,   /* dtype / dtype combination has no kernel            */
+  XG_ERR_BAD_SHAPE = -2,   /* negative or inconsistent sizes / strides           */
+  XG_ERR_BAD_ALIGN = -3,   /* pointer or stride alignment the kernel cannot take */
+  XG_ERR_NULL_PTR = -4,    /* a required pointer is NULL                         */
+  XG_ERR_TOO_LARGE = -5,   /* size beyond what the entry point supports          */
+  XG_ERR_LAUNCH = -6,      /* hipLaunchKernel reported an error                  */
+  XG_ERR_BAD_ARG = -7      /* other invalid argument (enum value, flag)          */
+} xg_status;
+
+typedef enum { XG_F32 = 0, XG_F16 = 1, XG_BF16 = 2, XG_FP8_E4M3 = 3 } xg_dtype;
+
+typedef enum { XG_ACT_NONE = 0, XG_ACT_RELU = 1, XG_ACT_GELU = 2, XG_ACT_SILU = 3, XG_ACT_SIGMOID = 4 } xg_act;
+
+/* Library version (major*10000 + minor*100 + patch) and status text. */
+int xg_version(void);
+const char* xg_status_string(int status);
+
+/* ---------------------------------------------------------------------------
+ * Row normalisation.  x, y, h, res are [rows, cols] with unit column stride;
+ * x_stride / res_stride are row strides in elements, outputs are contiguous.
+ * w and b are [cols] of dtype `wb_dtype`, which must equal `dtype` or XG_F32.
+ * Statistics and the affine transform are computed in fp32 and rounded once
+ * to `dtype`.
+ *
+ * xg_rms_norm:   y = x * rsqrt(mean(x^2) + eps) * w            (w may be NULL)
+ *   replaces DefaultRMSNorm.forward
+ *   (src/xpu_graph/passes/patterns/utils/default_replacements.py:19-25) and the
+ *   vendor calls torch_mlu_ops.fused_rms_norm
+ *   (passes/patterns/targets/mlu/structure_replacements/norm_modules.py:4-10),
+ *   torch_npu.npu_rms_norm
+ *   (passes/patterns/targets/npu/structure_replacements/rms_norm_module.py:6-10).
+ *
+ * xg_layer_norm: y = (x - mean) * rsqrt(var + eps) * w + b     (w, b may be NULL)
+ *   replaces DefaultLayerNorm.forward (default_replacements.py:28-36) and
+ *   torch_mlu_ops.fused_layer_norm (norm_modules.py:13-21).
+ *
+ * xg_add_rms_norm / xg_add_layer_norm: h = round_to_dtype(x + res), then the
+ *   norm of h (statistics taken of the ROUNDED h, as the unfused graph does).
+ *   h_out may be NULL (store_output_before_norm == False).
+ *   replace FusedNormReplacement.forward
+ *   (passes/patterns/targets/mlu/fuse_add_norm.py:21-83) and the op
+ *   torch_npu_triton::fused_add_rmsnorm
+ *   (passes/patterns/targets/npu/triton_kernel/fused_add_rmsnorm.py:8-72).
+ * ------------------------------------------------------------------------- */
+int xg_rms_norm(const void* x, const void* w, void* y, int64_t rows, int64_t cols, int64_t x_stride, float eps,
+                int dtype, int wb_dtype, xg_stream_t stream);
+int xg_layer_norm(const void* x, const void* w, const void* b, void* y, int64_t rows, int64_t cols,
+                  int64_t x_stride, float eps, int dtype, int wb_dtype, xg_stream_t stream);
+int xg_add_rms_norm(const void* x, const void* res, const void* w, void* y, void* h_out, int64_t rows,
+                    int64_t cols, int64_t x_stride, int64_t res_stride, float eps, int dtype, int wb_dtype,
+                    xg_stream_t stream);
+int xg_add_layer_norm(const void* x, const void* res, const void* w, const void* b, void* y, void* h_out,
+                      int64_t rows, int64_t cols, int64_t x_stride, int64_t res_stride, float eps, int dtype,
+                      int wb_dtype, xg_stream_t stream);
+
+/* ---------------------------------------------------------------------------
+ * Column slice + concatenate (bit-exact byte mover, dtype-agnostic).
+ *
+ * For every row r < rows and every chunk i < n_chunks, copies `chunk_bytes`
+ * bytes from   src + r*src_row_bytes + table[i].src_off
+ *        to    outs[table[i].out_id] + r*out_row_bytes[out_id] + table[i].dst_off.
+ * `table` lives in DEVICE memory (built once by the caller for a static slice
+ * list); chunk_bytes is one of 1,2,4,8,16.  src, src_row_bytes, every src_off,
+ * every out pointer / out_row_bytes / dst_off must be multiples of
+ * min(chunk_bytes, 4) for the source side and of chunk_bytes for the output
+ * side.  n_outs <= XG_SLICE_CAT_MAX_OUTS.
+ *
+ * replaces torch_mlu_triton::fused_slice_cat
+ *   (passes/patterns/targets/mlu/triton_kernel/fused_slice_cat.py:10-73; one
+ *   output) and torch_mlu_triton::fused_slice_low_v2
+ *   (.../triton_kernel/fused_slice_v2.py:9-114; several outputs in one launch).
+ * ------------------------------------------------------------------------- */
+#define XG_SLICE_CAT_MAX_OUTS 32
+typedef struct {
+  int32_t src_off; /* byte offset inside a source row */
+  int32_t dst_off; /* byte offset inside a row of the chosen output */
+  int32_t out_id;  /* which output */
+  int32_t pad;
+} xg_chunk;
+int xg_slice_cat(const void* src, int64_t src_row_bytes, int64_t rows, void* const* outs,
+                 const int64_t* out_row_bytes, int n_outs, const xg_chunk* table_dev, int64_t n_chunks,
+                 int chunk_bytes, xg_stream_t stream);
+
+/* ---------------------------------------------------------------------------
+ * add-N: out = ((t0 + t1) + t2) + ... strictly left to right, fp32 accumulate,
+ * one rounding to `dtype` at the end.  `inputs` is a HOST array of n device
+ * pointers to contiguous tensors of `numel` elements.  n >= 1.
+ * replaces the stack + sum(dim 0) that FusedAddN emits
+ *   (passes/patterns/common/fuse_addn.py:27-76).
+ * ------------------------------------------------------------------------- */
+int xg_addn(const void* const* inputs, int n, void* out, int64_t numel, int dtype, xg_stream_t stream);
+
+/* ---------------------------------------------------------------------------
+ * combo-sum: n_jobs independent reductions in one launch.  Job j reduces a
+ * contiguous [s0, s1, s2] tensor over dim 1 (-> [s0, s2]) or dim 2 (-> [s0, s1]),
+ * fp32 accumulate in index order, one rounding.  All arrays are HOST arrays of
+ * length n_jobs; n_jobs <= XG_COMBO_SUM_MAX_JOBS.
+ * replaces torch_mlu_triton::fused_sum_3d_input
+ *   (passes/patterns/targets/mlu/triton_kernel/fused_sum_3d.py:84-205).
+ * ------------------------------------------------------------------------- */
+#define XG_COMBO_SUM_MAX_JOBS 64
+int xg_combo_sum(const void* const* inputs, void* const* outputs, const int64_t* s0, const int64_t* s1,
+                 const int64_t* s2, int n_jobs, int dim, int dtype, xg_stream_t stream);
+
+/* ---------------------------------------------------------------------------
+ * SwiGLU gate: y[r, c] = silu(x[r, c]) * x[r, d + c], x is [rows, 2d] with row
+ * stride x_stride, y is contiguous [rows, d]; fp32 math.
+ * replaces torch_npu_triton::fused_silu_mul
+ *   (passes/patterns/targets/npu/triton_kernel/fused_silu_mul.py:8-60).
+ * xg_silu_mul2 takes gate and up as two separate [rows, d] tensors.
+ * ------------------------------------------------------------------------- */
+int xg_silu_mul(const void* x, void* y, int64_t rows, int64_t d, int64_t x_stride, int dtype,
+                xg_stream_t stream);
+int xg_silu_mul2(const void* gate, const void* up, void* y, int64_t rows, int64_t d, int64_t gate_stride,
+                 int64_t up_stride, int dtype, xg_stream_t stream);
+
+/* ---------------------------------------------------------------------------
+ * Dense layer: out[M,N] = act(a[M,K] @ B + bias (+ residual)), fp32 accumulate.
+ *   a: row-major, row stride lda.  B is [K,N] row-major with row stride ldb when
+ *   b_trans == 0, or the transpose of a row-major [N,K] (row stride ldb) when
+ *   b_trans == 1 (the nn.Linear weight layout).
+ *   bias: NULL or [N] (dtype `dtype` or XG_F32 via bias_dtype).
+ *   residual: NULL or [M,N] row stride ldr, added before the activation.
+ *   dtype: XG_BF16 or XG_F16 (inputs and output).
+ * replaces torch_mlu_ops.matmul as called by DenseLayerModule.forward
+ *   (passes/patterns/targets/mlu/structure_replacements/dense_layer_modules.py:4-56).
+ *
+ * xg_dense_fp8: a_q [M,K] and b_q ([K,N] or [N,K], as above) are OCP e4m3fn
+ *   bytes; out = act((a_q @ b_q) * a_scale * b_scale[n] + bias) in `out_dtype`
+ *   (XG_BF16 / XG_F16 / XG_F32).  b_scale is f32[N], bias f32-or-out_dtype.
+ *   No counterpart in the reference (it has no fp8 path).
+ * ------------------------------------------------------------------------- */
+int xg_dense(const void* a, const void* b, const void* bias, const void* residual, void* out, int64_t M,
+             int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldr, int b_trans, int act, int dtype,
+             int bias_dtype, xg_stream_t stream);
+int xg_dense_fp8(const void* a_q, const void* b_q, const float* a_scale_dev, const float* b_scale_dev,
+                 const void* bias, void* out, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
+                 int b_trans, int act, int out_dtype, int bias_dtype, xg_stream_t stream);
+
+/* ---------------------------------------------------------------------------
+ * Scaled dot-product attention, optional causal mask, no dropout.
+ *   q [B,H,Sq,D], k/v [B,Hkv,Skv,D], out [B,H,Sq,D]; strides in elements for
+ *   batch, head and sequence; the D axis has unit stride; D in {64, 128}.
+ *   softmax in fp32 with running max; causal aligns the LAST query with the
+ *   last key (top-left aligned when Sq == Skv).
+ * replaces aten.scaled_dot_product_attention as emitted by FusedSDPA
+ *   (passes/patterns/common/fuse_scaled_dot_product_attention.py:184-234).
+ * ------------------------------------------------------------------------- */
+int xg_sdpa(const void* q, const void* k, const void* v, void* out, int64_t B, int64_t H, int64_t Hkv,
+            int64_t Sq, int64_t Skv, int64_t D, const int64_t q_strides[3], const int64_t k_strides[3],
+            const int64_t v_strides[3], const int64_t o_strides[3], float scale, int causal, int dtype,
+            xg_stream_t stream);
+
+/* ---------------------------------------------------------------------------
+ * Plain device copy of `bytes` bytes (16-byte aligned), used as the known-size
+ * yardstick that scales the FETCH_SIZE / WRITE_SIZE profiler counters.
+ * ------------------------------------------------------------------------- */
+int xg_copy_bytes(const void* src, void* dst, int64_t bytes, xg_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* XPU_GRAPH_AMD_H */

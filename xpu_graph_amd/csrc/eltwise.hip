@@ -1,0 +1,134 @@
+// Elementwise kernels for gfx950: the SwiGLU gate silu(a) * b, and the plain
+// copy used as the known-size yardstick for the memory-traffic counters.
+#include "xg_common.hpp"
+
+namespace xg {
+namespace {
+
+__device__ __forceinline__ float silu_f32(float v) { return v / (1.0f + __expf(-v)); }
+
+// gate/up are [rows, d] views with row strides in elements; nvec = d / VW.
+template <typename T, int VW>
+__global__ __launch_bounds__(256) void silu_mul_kernel(const T* __restrict__ gate, const T* __restrict__ up,
+                                                       T* __restrict__ y, int64_t rows, int64_t nvec,
+                                                       int64_t gate_stride, int64_t up_stride) {
+  typedef T VT __attribute__((ext_vector_type(VW)));
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= rows * nvec) return;
+  const int64_t r = i / nvec, c = i % nvec;
+  const VT g = __builtin_nontemporal_load(reinterpret_cast<const VT*>(gate + r * gate_stride) + c);
+  const VT u = __builtin_nontemporal_load(reinterpret_cast<const VT*>(up + r * up_stride) + c);
+  VT o;
+#pragma unroll
+  for (int j = 0; j < VW; ++j) o[j] = from_f32<T>(silu_f32(to_f32(g[j])) * to_f32(u[j]));
+  __builtin_nontemporal_store(o, reinterpret_cast<VT*>(y) + i);
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void silu_mul_scalar_kernel(const T* __restrict__ gate, const T* __restrict__ up,
+                                                              T* __restrict__ y, int64_t rows, int64_t d,
+                                                              int64_t gate_stride, int64_t up_stride) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= rows * d) return;
+  const int64_t r = i / d, c = i % d;
+  y[i] = from_f32<T>(silu_f32(to_f32(gate[r * gate_stride + c])) * to_f32(up[r * up_stride + c]));
+}
+
+template <typename T>
+int silu_mul_typed(const void* gate, const void* up, void* y, int64_t rows, int64_t d, int64_t gs, int64_t us,
+                   hipStream_t stream) {
+  constexpr int VN = VecOf<T>::N;
+  const bool vec_ok = d % VN == 0 && gs % VN == 0 && us % VN == 0 && aligned_to(gate, 16) && aligned_to(up, 16) &&
+                      aligned_to(y, 16);
+  const int64_t work = vec_ok ? rows * (d / VN) : rows * d;
+  const int64_t blocks = (work + 255) / 256;
+  if (blocks > 0x7fffffffLL) return XG_ERR_TOO_LARGE;
+  if (vec_ok)
+    hipLaunchKernelGGL((silu_mul_kernel<T, VN>), dim3((unsigned)blocks), dim3(256), 0, stream, (const T*)gate,
+                       (const T*)up, (T*)y, rows, d / VN, gs, us);
+  else
+    hipLaunchKernelGGL((silu_mul_scalar_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, stream, (const T*)gate,
+                       (const T*)up, (T*)y, rows, d, gs, us);
+  return status_from_hip(hipGetLastError());
+}
+
+int silu_mul_dispatch(const void* gate, const void* up, void* y, int64_t rows, int64_t d, int64_t gs, int64_t us,
+                      int dtype, hipStream_t stream) {
+  if (gate == nullptr || up == nullptr || y == nullptr) return XG_ERR_NULL_PTR;
+  if (rows < 0 || d < 0 || gs < d || us < d) return XG_ERR_BAD_SHAPE;
+  if (rows == 0 || d == 0) return XG_OK;
+  switch (dtype) {
+    case XG_F32:
+      return silu_mul_typed<float>(gate, up, y, rows, d, gs, us, stream);
+    case XG_BF16:
+      return silu_mul_typed<bf16_t>(gate, up, y, rows, d, gs, us, stream);
+    case XG_F16:
+      return silu_mul_typed<f16_t>(gate, up, y, rows, d, gs, us, stream);
+    default:
+      return XG_ERR_BAD_DTYPE;
+  }
+}
+
+__global__ __launch_bounds__(256) void copy_kernel(const u32x4* __restrict__ src, u32x4* __restrict__ dst, int64_t n) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
+}
+
+}  // namespace
+}  // namespace xg
+
+extern "C" {
+
+int xg_silu_mul(const void* x, void* y, int64_t rows, int64_t d, int64_t x_stride, int dtype, xg_stream_t stream) {
+  if (x == nullptr) return XG_ERR_NULL_PTR;
+  if (d < 0 || x_stride < 2 * d) return XG_ERR_BAD_SHAPE;
+  const size_t esz = dtype == XG_F32 ? 4 : 2;
+  const char* up = (const char*)x + (size_t)d * esz;
+  return xg::silu_mul_dispatch(x, up, y, rows, d, x_stride, x_stride, dtype, (hipStream_t)stream);
+}
+
+int xg_silu_mul2(const void* gate, const void* up, void* y, int64_t rows, int64_t d, int64_t gate_stride,
+                 int64_t up_stride, int dtype, xg_stream_t stream) {
+  return xg::silu_mul_dispatch(gate, up, y, rows, d, gate_stride, up_stride, dtype, (hipStream_t)stream);
+}
+
+int xg_copy_bytes(const void* src, void* dst, int64_t bytes, xg_stream_t stream) {
+  using namespace xg;
+  if (src == nullptr || dst == nullptr) return XG_ERR_NULL_PTR;
+  if (bytes < 0 || bytes % 16 != 0) return XG_ERR_BAD_SHAPE;
+  if (!aligned_to(src, 16) || !aligned_to(dst, 16)) return XG_ERR_BAD_ALIGN;
+  if (bytes == 0) return XG_OK;
+  const int64_t n = bytes / 16;
+  const int64_t blocks = (n + 255) / 256;
+  if (blocks > 0x7fffffffLL) return XG_ERR_TOO_LARGE;
+  hipLaunchKernelGGL(copy_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (const u32x4*)src,
+                     (u32x4*)dst, n);
+  return status_from_hip(hipGetLastError());
+}
+
+int xg_version(void) { return 100; }
+
+const char* xg_status_string(int status) {
+  switch (status) {
+    case XG_OK:
+      return "ok";
+    case XG_ERR_BAD_DTYPE:
+      return "unsupported dtype combination";
+    case XG_ERR_BAD_SHAPE:
+      return "inconsistent sizes or strides";
+    case XG_ERR_BAD_ALIGN:
+      return "pointer or stride alignment not supported";
+    case XG_ERR_NULL_PTR:
+      return "required pointer is NULL";
+    case XG_ERR_TOO_LARGE:
+      return "size beyond what the entry point supports";
+    case XG_ERR_LAUNCH:
+      return "kernel launch failed";
+    case XG_ERR_BAD_ARG:
+      return "invalid argument";
+    default:
+      return "unknown status";
+  }
+}
+
+}  // extern "C"

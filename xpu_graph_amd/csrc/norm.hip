@@ -1,0 +1,316 @@
+// Row normalisation kernels for gfx950: RMSNorm / LayerNorm with optional
+// fused residual add and optional second output (the pre-norm sum).
+//
+// Layout: a row of `cols` elements is split into 16-byte vectors.  TPR threads
+// share one row and each keeps VPT vectors of it in registers in the storage
+// dtype, so HBM is read exactly once and written exactly once per element.
+// Statistics are two-pass over the registers (mean, then centred second
+// moment) in fp32; lanes combine with wavefront shuffles and, when a row spans
+// several wavefronts, a few floats of LDS.
+#include "xg_common.hpp"
+
+#include <stdlib.h>
+
+namespace xg {
+namespace {
+
+template <typename T, int N>
+struct Pack {
+  typedef typename VecOf<T>::type V;
+  static constexpr int NV = N / VecOf<T>::N;  // 16-byte vectors in a pack of N elements
+  V v[NV > 0 ? NV : 1];
+};
+
+// Load N consecutive elements of WT (N a multiple of the 16-byte vector width of WT) as fp32.
+template <typename WT, int N>
+__device__ __forceinline__ void load_row_params(const WT* p, float (&out)[N]) {
+  typedef typename VecOf<WT>::type V;
+  constexpr int VN = VecOf<WT>::N;
+  static_assert(N % VN == 0, "vector width mismatch");
+#pragma unroll
+  for (int i = 0; i < N / VN; ++i) {
+    V t = *reinterpret_cast<const V*>(p + i * VN);
+#pragma unroll
+    for (int j = 0; j < VN; ++j) out[i * VN + j] = to_f32(t[j]);
+  }
+}
+
+template <typename T, typename WT, int TPR, int VPT, bool LAYER>
+__global__ __launch_bounds__((TPR > 256 ? TPR : 256)) void norm_rows_kernel(
+    const T* __restrict__ x, const T* __restrict__ res, const WT* __restrict__ w, const WT* __restrict__ b,
+    T* __restrict__ y, T* __restrict__ h_out, int64_t rows, int nvec, int64_t x_stride, int64_t res_stride,
+    float eps, float inv_cols) {
+  typedef typename VecOf<T>::type V;
+  constexpr int VN = VecOf<T>::N;
+  constexpr int BLOCK = TPR > 256 ? TPR : 256;
+  constexpr int RPB = BLOCK / TPR;  // rows per block
+  constexpr int NW = TPR > kWave ? TPR / kWave : 1;
+  __shared__ float red_all[RPB * NW];
+
+  const int group = threadIdx.x / TPR;
+  const int lir = threadIdx.x % TPR;  // lane in row
+  float* red = red_all + group * NW;
+  int64_t row = (int64_t)blockIdx.x * RPB + group;
+  const bool row_ok = row < rows;
+  if (!row_ok) row = rows - 1;  // keep every lane alive for the barriers; stores are masked below
+
+  const V* xr = reinterpret_cast<const V*>(x + row * x_stride);
+  V hv[VPT];
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) {
+    const int c = lir + i * TPR;
+    if (c < nvec) hv[i] = load_vec_nt(xr + c);
+  }
+  if (res != nullptr) {
+    const V* rr = reinterpret_cast<const V*>(res + row * res_stride);
+    V rv[VPT];
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+      const int c = lir + i * TPR;
+      if (c < nvec) rv[i] = load_vec_nt(rr + c);
+    }
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+      const int c = lir + i * TPR;
+      if (c < nvec) {
+#pragma unroll
+        for (int j = 0; j < VN; ++j) hv[i][j] = from_f32<T>(to_f32(hv[i][j]) + to_f32(rv[i][j]));
+      }
+    }
+    if (h_out != nullptr && row_ok) {
+      V* hr = reinterpret_cast<V*>(h_out + row * (int64_t)nvec * VN);
+#pragma unroll
+      for (int i = 0; i < VPT; ++i) {
+        const int c = lir + i * TPR;
+        if (c < nvec) store_vec_nt(hr + c, hv[i]);
+      }
+    }
+  }
+
+  float mean = 0.f;
+  if constexpr (LAYER) {
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+      if (lir + i * TPR < nvec) {
+#pragma unroll
+        for (int j = 0; j < VN; ++j) s += to_f32(hv[i][j]);
+      }
+    }
+    mean = group_sum<TPR>(s, red, lir) * inv_cols;
+  }
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) {
+    if (lir + i * TPR < nvec) {
+#pragma unroll
+      for (int j = 0; j < VN; ++j) {
+        const float d = to_f32(hv[i][j]) - mean;
+        ss += d * d;
+      }
+    }
+  }
+  const float rstd = rsqrtf(group_sum<TPR>(ss, red, lir) * inv_cols + eps);
+
+  if (!row_ok) return;
+  V* yr = reinterpret_cast<V*>(y + row * (int64_t)nvec * VN);
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) {
+    const int c = lir + i * TPR;
+    if (c < nvec) {
+      float wv[VN], bv[VN];
+      if (w != nullptr) {
+        load_row_params<WT, VN>(w + (int64_t)c * VN, wv);
+      } else {
+#pragma unroll
+        for (int j = 0; j < VN; ++j) wv[j] = 1.f;
+      }
+      if (LAYER && b != nullptr) {
+        load_row_params<WT, VN>(b + (int64_t)c * VN, bv);
+      } else {
+#pragma unroll
+        for (int j = 0; j < VN; ++j) bv[j] = 0.f;
+      }
+      V o;
+#pragma unroll
+      for (int j = 0; j < VN; ++j) o[j] = from_f32<T>((to_f32(hv[i][j]) - mean) * rstd * wv[j] + bv[j]);
+      store_vec_nt(yr + c, o);
+    }
+  }
+}
+
+// Any shape / alignment: one 256-thread block per row, three strided passes over
+// the row (the re-reads come from cache).  Correctness net for odd column
+// counts and unaligned views; the vector kernel above is the fast path.
+template <typename T, typename WT, bool LAYER>
+__global__ __launch_bounds__(256) void norm_rows_generic_kernel(const T* __restrict__ x, const T* __restrict__ res,
+                                                                 const WT* __restrict__ w, const WT* __restrict__ b,
+                                                                 T* __restrict__ y, T* __restrict__ h_out,
+                                                                 int64_t cols, int64_t x_stride, int64_t res_stride,
+                                                                 float eps, float inv_cols) {
+  __shared__ float red[4];
+  const int64_t row = blockIdx.x;
+  const T* xr = x + row * x_stride;
+  const T* rr = res ? res + row * res_stride : nullptr;
+  auto elem = [&](int64_t c) -> float {
+    if (rr) return to_f32(from_f32<T>(to_f32(xr[c]) + to_f32(rr[c])));
+    return to_f32(xr[c]);
+  };
+  float mean = 0.f;
+  if constexpr (LAYER) {
+    float s = 0.f;
+    for (int64_t c = threadIdx.x; c < cols; c += 256) s += elem(c);
+    mean = group_sum<256>(s, red, threadIdx.x) * inv_cols;
+  }
+  float ss = 0.f;
+  for (int64_t c = threadIdx.x; c < cols; c += 256) {
+    const float d = elem(c) - mean;
+    ss += d * d;
+  }
+  const float rstd = rsqrtf(group_sum<256>(ss, red, threadIdx.x) * inv_cols + eps);
+  for (int64_t c = threadIdx.x; c < cols; c += 256) {
+    const float hval = elem(c);
+    if (rr && h_out) h_out[row * cols + c] = from_f32<T>(hval);
+    const float wv = w ? to_f32(w[c]) : 1.f;
+    const float bv = (LAYER && b) ? to_f32(b[c]) : 0.f;
+    y[row * cols + c] = from_f32<T>((hval - mean) * rstd * wv + bv);
+  }
+}
+
+struct NormArgs {
+  const void* x;
+  const void* res;
+  const void* w;
+  const void* b;
+  void* y;
+  void* h_out;
+  int64_t rows, cols, x_stride, res_stride;
+  float eps;
+  hipStream_t stream;
+};
+
+int tuned_tpr() {
+  static int v = [] {
+    const char* s = getenv("XG_NORM_TPR");
+    return s ? atoi(s) : 0;
+  }();
+  return v;
+}
+
+template <typename T, typename WT, int TPR, int VPT, bool LAYER>
+int launch_vec(const NormArgs& a, int nvec) {
+  constexpr int BLOCK = TPR > 256 ? TPR : 256;
+  constexpr int RPB = BLOCK / TPR;
+  const int64_t blocks = (a.rows + RPB - 1) / RPB;
+  if (blocks > 0x7fffffffLL) return XG_ERR_TOO_LARGE;
+  hipLaunchKernelGGL((norm_rows_kernel<T, WT, TPR, VPT, LAYER>), dim3((unsigned)blocks), dim3(BLOCK), 0, a.stream,
+                     (const T*)a.x, (const T*)a.res, (const WT*)a.w, (const WT*)a.b, (T*)a.y, (T*)a.h_out, a.rows, nvec,
+                     a.x_stride, a.res_stride, a.eps, 1.0f / (float)a.cols);
+  return status_from_hip(hipGetLastError());
+}
+
+template <typename T, typename WT, int TPR, bool LAYER>
+int launch_tpr(const NormArgs& a, int nvec) {
+  const int per = (nvec + TPR - 1) / TPR;
+  if (per <= 1) return launch_vec<T, WT, TPR, 1, LAYER>(a, nvec);
+  if (per <= 2) return launch_vec<T, WT, TPR, 2, LAYER>(a, nvec);
+  if (per <= 4) return launch_vec<T, WT, TPR, 4, LAYER>(a, nvec);
+  if (per <= 8) return launch_vec<T, WT, TPR, 8, LAYER>(a, nvec);
+  return XG_ERR_TOO_LARGE;
+}
+
+template <typename T, typename WT, bool LAYER>
+int launch_typed(const NormArgs& a) {
+  constexpr int VN = VecOf<T>::N;
+  const bool vec_ok = a.cols % VN == 0 && a.x_stride % VN == 0 && aligned_to(a.x, 16) && aligned_to(a.y, 16) &&
+                      (a.res == nullptr || (a.res_stride % VN == 0 && aligned_to(a.res, 16))) &&
+                      (a.h_out == nullptr || aligned_to(a.h_out, 16)) && (a.w == nullptr || aligned_to(a.w, 16)) &&
+                      (a.b == nullptr || aligned_to(a.b, 16)) && a.cols / VN <= 1024 * 8;
+  if (vec_ok) {
+    const int nvec = (int)(a.cols / VN);
+    int tpr = tuned_tpr();
+    if (tpr == 0) {
+      // Heuristic: the fewest threads per row that keep <= 8 vectors per thread,
+      // preferring whole-wavefront rows (no LDS, no barrier) up to 512 vectors.
+      if (nvec <= 16 * 2)
+        tpr = 16;
+      else if (nvec <= 64 * 8)
+        tpr = 64;
+      else if (nvec <= 256 * 8)
+        tpr = 256;
+      else
+        tpr = 1024;
+    }
+    if (tpr * 8 < nvec) tpr = nvec <= 64 * 8 ? 64 : (nvec <= 256 * 8 ? 256 : 1024);
+    switch (tpr) {
+      case 16:
+        return launch_tpr<T, WT, 16, LAYER>(a, nvec);
+      case 64:
+        return launch_tpr<T, WT, 64, LAYER>(a, nvec);
+      case 128:
+        return launch_tpr<T, WT, 128, LAYER>(a, nvec);
+      case 256:
+        return launch_tpr<T, WT, 256, LAYER>(a, nvec);
+      case 1024:
+        return launch_tpr<T, WT, 1024, LAYER>(a, nvec);
+      default:
+        return XG_ERR_BAD_ARG;
+    }
+  }
+  if (a.rows > 0x7fffffffLL) return XG_ERR_TOO_LARGE;
+  hipLaunchKernelGGL((norm_rows_generic_kernel<T, WT, LAYER>), dim3((unsigned)a.rows), dim3(256), 0, a.stream,
+                     (const T*)a.x, (const T*)a.res, (const WT*)a.w, (const WT*)a.b, (T*)a.y, (T*)a.h_out, a.cols,
+                     a.x_stride, a.res_stride, a.eps, 1.0f / (float)a.cols);
+  return status_from_hip(hipGetLastError());
+}
+
+template <bool LAYER>
+int dispatch(const NormArgs& a, int dtype, int wb_dtype) {
+  if (a.x == nullptr || a.y == nullptr) return XG_ERR_NULL_PTR;
+  if (a.rows < 0 || a.cols <= 0 || a.x_stride < a.cols || (a.res != nullptr && a.res_stride < a.cols))
+    return XG_ERR_BAD_SHAPE;
+  if (a.rows == 0) return XG_OK;
+  const size_t esz = dtype == XG_F32 ? 4 : 2;
+  if (!aligned_to(a.x, esz) || !aligned_to(a.y, esz)) return XG_ERR_BAD_ALIGN;
+  if (dtype == XG_F32 && wb_dtype == XG_F32) return launch_typed<float, float, LAYER>(a);
+  if (dtype == XG_BF16 && wb_dtype == XG_BF16) return launch_typed<bf16_t, bf16_t, LAYER>(a);
+  if (dtype == XG_BF16 && wb_dtype == XG_F32) return launch_typed<bf16_t, float, LAYER>(a);
+  if (dtype == XG_F16 && wb_dtype == XG_F16) return launch_typed<f16_t, f16_t, LAYER>(a);
+  if (dtype == XG_F16 && wb_dtype == XG_F32) return launch_typed<f16_t, float, LAYER>(a);
+  return XG_ERR_BAD_DTYPE;
+}
+
+}  // namespace
+}  // namespace xg
+
+extern "C" {
+
+int xg_rms_norm(const void* x, const void* w, void* y, int64_t rows, int64_t cols, int64_t x_stride, float eps,
+                int dtype, int wb_dtype, xg_stream_t stream) {
+  xg::NormArgs a{x, nullptr, w, nullptr, y, nullptr, rows, cols, x_stride, 0, eps, (hipStream_t)stream};
+  return xg::dispatch<false>(a, dtype, wb_dtype);
+}
+
+int xg_layer_norm(const void* x, const void* w, const void* b, void* y, int64_t rows, int64_t cols,
+                  int64_t x_stride, float eps, int dtype, int wb_dtype, xg_stream_t stream) {
+  xg::NormArgs a{x, nullptr, w, b, y, nullptr, rows, cols, x_stride, 0, eps, (hipStream_t)stream};
+  return xg::dispatch<true>(a, dtype, wb_dtype);
+}
+
+int xg_add_rms_norm(const void* x, const void* res, const void* w, void* y, void* h_out, int64_t rows,
+                    int64_t cols, int64_t x_stride, int64_t res_stride, float eps, int dtype, int wb_dtype,
+                    xg_stream_t stream) {
+  if (res == nullptr) return XG_ERR_NULL_PTR;
+  xg::NormArgs a{x, res, w, nullptr, y, h_out, rows, cols, x_stride, res_stride, eps, (hipStream_t)stream};
+  return xg::dispatch<false>(a, dtype, wb_dtype);
+}
+
+int xg_add_layer_norm(const void* x, const void* res, const void* w, const void* b, void* y, void* h_out,
+                      int64_t rows, int64_t cols, int64_t x_stride, int64_t res_stride, float eps, int dtype,
+                      int wb_dtype, xg_stream_t stream) {
+  if (res == nullptr) return XG_ERR_NULL_PTR;
+  xg::NormArgs a{x, res, w, b, y, h_out, rows, cols, x_stride, res_stride, eps, (hipStream_t)stream};
+  return xg::dispatch<true>(a, dtype, wb_dtype);
+}
+
+}  // extern "C"

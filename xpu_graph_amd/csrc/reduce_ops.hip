@@ -1,0 +1,253 @@
+// Multi-tensor sums for gfx950.
+//  * add-N: one launch reads n tensors through a pointer table held in the
+//    kernel arguments and adds them strictly left to right in fp32, so an fp32
+//    result is bit-identical to the eager chain ((t0+t1)+t2)+...
+//  * combo-sum: many independent [s0,s1,s2] -> 2-D reductions behind one launch,
+//    driven by a job table in the kernel arguments.
+#include "xg_common.hpp"
+
+#include <stdlib.h>
+
+namespace xg {
+namespace {
+
+constexpr int kAddnMax = 64;  // pointers per launch; longer chains continue from the partial result
+
+struct AddnTable {
+  const void* p[kAddnMax];
+};
+
+// VW = elements per lane access: the 16-byte vector width, or 1 for the
+// unaligned / tail-safe scalar form.
+template <typename T, int VW, int U>
+__global__ __launch_bounds__(256) void addn_kernel(AddnTable tbl, int n, T* __restrict__ out, int64_t nvec) {
+  typedef T VT __attribute__((ext_vector_type(VW)));
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= nvec) return;
+  float acc[VW];
+  {
+    VT v = __builtin_nontemporal_load(reinterpret_cast<const VT*>(tbl.p[0]) + i);
+#pragma unroll
+    for (int j = 0; j < VW; ++j) acc[j] = to_f32(v[j]);
+  }
+  int t = 1;
+  // U loads are kept in flight per lane
+  for (; t + U <= n; t += U) {
+    VT v[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) v[u] = __builtin_nontemporal_load(reinterpret_cast<const VT*>(tbl.p[t + u]) + i);
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+#pragma unroll
+      for (int j = 0; j < VW; ++j) acc[j] += to_f32(v[u][j]);
+    }
+  }
+  for (; t < n; ++t) {
+    VT v = __builtin_nontemporal_load(reinterpret_cast<const VT*>(tbl.p[t]) + i);
+#pragma unroll
+    for (int j = 0; j < VW; ++j) acc[j] += to_f32(v[j]);
+  }
+  VT o;
+#pragma unroll
+  for (int j = 0; j < VW; ++j) o[j] = from_f32<T>(acc[j]);
+  __builtin_nontemporal_store(o, reinterpret_cast<VT*>(out) + i);
+}
+
+// Scalar specialisation helper: ext_vector_type(1) is awkward, so VW == 1 goes through this kernel.
+template <typename T>
+__global__ __launch_bounds__(256) void addn_scalar_kernel(AddnTable tbl, int n, T* __restrict__ out, int64_t base,
+                                                          int64_t numel) {
+  const int64_t i = base + (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= numel) return;
+  float acc = to_f32(reinterpret_cast<const T*>(tbl.p[0])[i]);
+  for (int t = 1; t < n; ++t) acc += to_f32(reinterpret_cast<const T*>(tbl.p[t])[i]);
+  out[i] = from_f32<T>(acc);
+}
+
+template <typename T>
+int addn_launch(const AddnTable& tbl, int n, T* out, int64_t numel, hipStream_t stream) {
+  constexpr int VN = VecOf<T>::N;
+  bool vec_ok = aligned_to(out, 16);
+  for (int i = 0; i < n; ++i) vec_ok = vec_ok && aligned_to(tbl.p[i], 16);
+  int64_t done = 0;
+  if (vec_ok && numel >= VN) {
+    const int64_t nvec = numel / VN;
+    const int64_t blocks = (nvec + 255) / 256;
+    if (blocks > 0x7fffffffLL) return XG_ERR_TOO_LARGE;
+    static int u = [] { const char* e = getenv("XG_ADDN_U"); return e ? atoi(e) : 8; }();
+    if (u == 4) hipLaunchKernelGGL((addn_kernel<T, VN, 4>), dim3((unsigned)blocks), dim3(256), 0, stream, tbl, n, out, nvec);
+    else if (u == 16) hipLaunchKernelGGL((addn_kernel<T, VN, 16>), dim3((unsigned)blocks), dim3(256), 0, stream, tbl, n, out, nvec);
+    else if (u == 31) hipLaunchKernelGGL((addn_kernel<T, VN, 31>), dim3((unsigned)blocks), dim3(256), 0, stream, tbl, n, out, nvec);
+    else hipLaunchKernelGGL((addn_kernel<T, VN, 8>), dim3((unsigned)blocks), dim3(256), 0, stream, tbl, n, out, nvec);
+    done = nvec * VN;
+  }
+  if (done < numel) {
+    const int64_t blocks = (numel - done + 255) / 256;
+    if (blocks > 0x7fffffffLL) return XG_ERR_TOO_LARGE;
+    hipLaunchKernelGGL((addn_scalar_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, stream, tbl, n, out, done, numel);
+  }
+  return status_from_hip(hipGetLastError());
+}
+
+template <typename T>
+int addn_typed(const void* const* inputs, int n, void* out, int64_t numel, hipStream_t stream) {
+  // Chains longer than the table continue with the partial result as operand 0,
+  // which keeps the left-to-right order.  The partial result is rounded to T
+  // between launches; for fp32 that is exact.
+  int pos = 0;
+  bool first = true;
+  while (pos < n || first) {
+    AddnTable tbl;
+    int k = 0;
+    if (!first) tbl.p[k++] = out;
+    while (k < kAddnMax && pos < n) tbl.p[k++] = inputs[pos++];
+    for (int i = k; i < kAddnMax; ++i) tbl.p[i] = nullptr;
+    int st = addn_launch<T>(tbl, k, (T*)out, numel, stream);
+    if (st != XG_OK) return st;
+    first = false;
+  }
+  return XG_OK;
+}
+
+// ------------------------------------------------------------------ combo-sum
+struct ComboJob {
+  const void* in;
+  void* out;
+  int32_t s0, s1, s2;
+  int32_t block_begin;  // first block of this job
+};
+struct ComboTable {
+  ComboJob job[XG_COMBO_SUM_MAX_JOBS];
+};
+
+// dim == 1: out[a, c] = sum_b in[a, b, c].  One lane per output element; lanes
+// run along c (unit stride), so each step over b is a coalesced row read.
+// dim == 2: out[a, b] = sum_c in[a, b, c].  A group of G lanes (G = power of two
+// <= 64) owns one output element and strides over c, then reduces by shuffle.
+template <typename T, int DIM>
+__global__ __launch_bounds__(256) void combo_sum_kernel(ComboTable tbl, int n_jobs, int group_log2) {
+  // Locate the job of this block (uniform binary search over block_begin).
+  int lo = 0, hi = n_jobs - 1;
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if ((int)blockIdx.x >= tbl.job[mid].block_begin)
+      lo = mid;
+    else
+      hi = mid - 1;
+  }
+  const ComboJob jb = tbl.job[lo];
+  const int64_t local_block = (int64_t)blockIdx.x - jb.block_begin;
+  const T* in = reinterpret_cast<const T*>(jb.in);
+  T* out = reinterpret_cast<T*>(jb.out);
+  if constexpr (DIM == 1) {
+    const int64_t o = local_block * 256 + threadIdx.x;
+    const int64_t n_out = (int64_t)jb.s0 * jb.s2;
+    if (o >= n_out) return;
+    const int64_t a = o / jb.s2, c = o % jb.s2;
+    const T* p = in + a * (int64_t)jb.s1 * jb.s2 + c;
+    float acc = 0.f;
+    for (int b = 0; b < jb.s1; ++b) acc += to_f32(p[(int64_t)b * jb.s2]);
+    out[o] = from_f32<T>(acc);
+  } else {
+    const int G = 1 << group_log2;
+    const int per_block = 256 >> group_log2;
+    const int64_t o = local_block * per_block + (threadIdx.x >> group_log2);
+    const int64_t n_out = (int64_t)jb.s0 * jb.s1;
+    const int lane = threadIdx.x & (G - 1);
+    float acc = 0.f;
+    if (o < n_out) {
+      const T* p = in + o * (int64_t)jb.s2;
+      for (int c = lane; c < jb.s2; c += G) acc += to_f32(p[c]);
+    }
+    for (int off = G >> 1; off > 0; off >>= 1) acc += __shfl_xor(acc, off, kWave);
+    if (o < n_out && lane == 0) out[o] = from_f32<T>(acc);
+  }
+}
+
+template <typename T>
+int combo_typed(const void* const* inputs, void* const* outputs, const int64_t* s0, const int64_t* s1,
+                const int64_t* s2, int n_jobs, int dim, hipStream_t stream) {
+  ComboTable tbl;
+  int64_t blocks = 0;
+  int group_log2 = 0;
+  if (dim == 2) {
+    int64_t max_s2 = 1;
+    for (int j = 0; j < n_jobs; ++j) max_s2 = s2[j] > max_s2 ? s2[j] : max_s2;
+    while ((1 << group_log2) < 64 && (1 << group_log2) < max_s2) ++group_log2;
+  }
+  int k = 0;
+  for (int j = 0; j < n_jobs; ++j) {
+    if (s0[j] < 0 || s1[j] < 0 || s2[j] < 0 || s0[j] > 0x7fffffff || s1[j] > 0x7fffffff || s2[j] > 0x7fffffff)
+      return XG_ERR_BAD_SHAPE;
+    const int64_t n_out = dim == 1 ? s0[j] * s2[j] : s0[j] * s1[j];
+    if (n_out == 0) continue;
+    if (inputs[j] == nullptr && s0[j] * s1[j] * s2[j] != 0) return XG_ERR_NULL_PTR;
+    if (outputs[j] == nullptr) return XG_ERR_NULL_PTR;
+    const int64_t per_block = dim == 1 ? 256 : (256 >> group_log2);
+    ComboJob& jb = tbl.job[k++];
+    jb.in = inputs[j];
+    jb.out = outputs[j];
+    jb.s0 = (int32_t)s0[j];
+    jb.s1 = (int32_t)s1[j];
+    jb.s2 = (int32_t)s2[j];
+    jb.block_begin = (int32_t)blocks;
+    blocks += (n_out + per_block - 1) / per_block;
+    if (blocks > 0x7fffffffLL) return XG_ERR_TOO_LARGE;
+  }
+  if (k == 0) return XG_OK;
+  for (int j = k; j < XG_COMBO_SUM_MAX_JOBS; ++j) tbl.job[j] = ComboJob{nullptr, nullptr, 0, 0, 0, 0x7fffffff};
+  if (dim == 1)
+    hipLaunchKernelGGL((combo_sum_kernel<T, 1>), dim3((unsigned)blocks), dim3(256), 0, stream, tbl, k, group_log2);
+  else
+    hipLaunchKernelGGL((combo_sum_kernel<T, 2>), dim3((unsigned)blocks), dim3(256), 0, stream, tbl, k, group_log2);
+  return status_from_hip(hipGetLastError());
+}
+
+}  // namespace
+}  // namespace xg
+
+extern "C" {
+
+int xg_addn(const void* const* inputs, int n, void* out, int64_t numel, int dtype, xg_stream_t stream) {
+  using namespace xg;
+  if (inputs == nullptr || out == nullptr) return XG_ERR_NULL_PTR;
+  if (n < 1 || numel < 0) return XG_ERR_BAD_SHAPE;
+  for (int i = 0; i < n; ++i)
+    if (inputs[i] == nullptr) return XG_ERR_NULL_PTR;
+  if (numel == 0) return XG_OK;
+  hipStream_t st = (hipStream_t)stream;
+  switch (dtype) {
+    case XG_F32:
+      return addn_typed<float>(inputs, n, out, numel, st);
+    case XG_BF16:
+      return addn_typed<bf16_t>(inputs, n, out, numel, st);
+    case XG_F16:
+      return addn_typed<f16_t>(inputs, n, out, numel, st);
+    default:
+      return XG_ERR_BAD_DTYPE;
+  }
+}
+
+int xg_combo_sum(const void* const* inputs, void* const* outputs, const int64_t* s0, const int64_t* s1,
+                 const int64_t* s2, int n_jobs, int dim, int dtype, xg_stream_t stream) {
+  using namespace xg;
+  if (inputs == nullptr || outputs == nullptr || s0 == nullptr || s1 == nullptr || s2 == nullptr)
+    return XG_ERR_NULL_PTR;
+  if (n_jobs < 0) return XG_ERR_BAD_SHAPE;
+  if (n_jobs > XG_COMBO_SUM_MAX_JOBS) return XG_ERR_TOO_LARGE;
+  if (dim != 1 && dim != 2) return XG_ERR_BAD_ARG;
+  if (n_jobs == 0) return XG_OK;
+  hipStream_t st = (hipStream_t)stream;
+  switch (dtype) {
+    case XG_F32:
+      return combo_typed<float>(inputs, outputs, s0, s1, s2, n_jobs, dim, st);
+    case XG_BF16:
+      return combo_typed<bf16_t>(inputs, outputs, s0, s1, s2, n_jobs, dim, st);
+    case XG_F16:
+      return combo_typed<f16_t>(inputs, outputs, s0, s1, s2, n_jobs, dim, st);
+    default:
+      return XG_ERR_BAD_DTYPE;
+  }
+}
+
+}  // extern "C"

@@ -1,0 +1,110 @@
+// Shared device helpers for the gfx950 kernels: 128-bit vector types, dtype
+// conversion, wavefront (64-lane) and workgroup reductions.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/xpu_graph_amd.h"
+
+namespace xg {
+
+constexpr int kWave = 64;
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16_t;
+typedef _Float16 f16_t;
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+
+// Per-dtype traits: a 16-byte vector of VEC elements and conversion to / from fp32.
+template <typename T>
+struct VecOf;
+template <>
+struct VecOf<float> {
+  static constexpr int N = 4;
+  typedef f32x4 type;
+};
+template <>
+struct VecOf<bf16_t> {
+  static constexpr int N = 8;
+  typedef bf16x8 type;
+};
+template <>
+struct VecOf<f16_t> {
+  static constexpr int N = 8;
+  typedef f16x8 type;
+};
+
+__device__ __forceinline__ float to_f32(float v) { return v; }
+__device__ __forceinline__ float to_f32(bf16_t v) { return (float)v; }
+__device__ __forceinline__ float to_f32(f16_t v) { return (float)v; }
+
+template <typename T>
+__device__ __forceinline__ T from_f32(float v) {
+  return (T)v;  // round-to-nearest-even; gfx950 has native f32->bf16 conversion
+}
+
+// 16-byte global load / store.  The NT variants mark the access as streaming
+// (data that is touched once), which keeps it from displacing reused lines.
+template <typename V>
+__device__ __forceinline__ V load_vec(const V* p) {
+  return *p;
+}
+template <typename V>
+__device__ __forceinline__ V load_vec_nt(const V* p) {
+  return __builtin_nontemporal_load(p);
+}
+template <typename V>
+__device__ __forceinline__ void store_vec(V* p, V v) {
+  *p = v;
+}
+template <typename V>
+__device__ __forceinline__ void store_vec_nt(V* p, V v) {
+  __builtin_nontemporal_store(v, p);
+}
+
+// Sum over the low `width` lanes of each aligned lane group (width a power of
+// two <= 64); every lane of the group ends with the total.
+template <int WIDTH = kWave>
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int off = WIDTH / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+  return v;
+}
+template <int WIDTH = kWave>
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int off = WIDTH / 2; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));
+  return v;
+}
+
+// Sum over the THREADS lanes that share one row.  THREADS <= 64: shuffle only.
+// THREADS > 64: per-wave shuffle, then the NW = THREADS/64 partial sums meet in
+// LDS (`red` holds NW floats per row group and is reused after a barrier).
+template <int THREADS>
+__device__ __forceinline__ float group_sum(float v, float* red, int lane_in_row) {
+  if constexpr (THREADS <= kWave) {
+    return wave_sum<THREADS>(v);
+  } else {
+    constexpr int NW = THREADS / kWave;
+    v = wave_sum<kWave>(v);
+    __syncthreads();  // previous use of `red` is over
+    if ((lane_in_row & (kWave - 1)) == 0) red[lane_in_row / kWave] = v;
+    __syncthreads();
+    float t = 0.f;
+#pragma unroll
+    for (int i = 0; i < NW; ++i) t += red[i];
+    return t;
+  }
+}
+
+inline int status_from_hip(hipError_t e) { return e == hipSuccess ? XG_OK : XG_ERR_LAUNCH; }
+
+inline bool aligned_to(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
+
+}  // namespace xg

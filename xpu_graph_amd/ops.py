@@ -1,0 +1,357 @@
+"""``torch.ops.xpu_ops.*``: the custom ops the mi355x target modules call.
+
+Each op has a schema, a Meta (fake-tensor) implementation so that the pass
+pipeline can re-propagate shapes through rewritten graphs, and ONE real
+implementation, registered for the CUDA dispatch key (HIP on ROCm), that hands
+raw device pointers and the current stream to the C-ABI kernel library.  There
+is deliberately no CPU implementation: calling an op on CPU tensors raises
+NotImplementedError from the dispatcher.
+
+Op names follow the reference's convention of a vendor op namespace allowed
+inside device graphs (`xpu_ops`, src/xpu_graph/backends/device_graph.py:26-29).
+"""
+import ctypes
+from typing import List, Optional
+
+import torch
+
+from . import _lib
+from ._lib import XG_BF16, XG_F16, XG_F32
+
+_DTYPE_CODE = {torch.float32: XG_F32, torch.float16: XG_F16, torch.bfloat16: XG_BF16}
+
+_library = torch.library.Library("xpu_ops", "DEF")
+
+_SCHEMAS = [
+    "rms_norm(Tensor x, Tensor? weight, float eps) -> Tensor",
+    "layer_norm(Tensor x, Tensor? weight, Tensor? bias, float eps) -> Tensor",
+    "add_rms_norm(Tensor x, Tensor residual, Tensor? weight, float eps) -> (Tensor, Tensor)",
+    "add_rms_norm_only(Tensor x, Tensor residual, Tensor? weight, float eps) -> Tensor",
+    "add_layer_norm(Tensor x, Tensor residual, Tensor? weight, Tensor? bias, float eps) -> (Tensor, Tensor)",
+    "add_layer_norm_only(Tensor x, Tensor residual, Tensor? weight, Tensor? bias, float eps) -> Tensor",
+    "slice_cat(Tensor src, Tensor table, int chunk_bytes, int out_cols) -> Tensor",
+    "slice_cat_multi(Tensor src, Tensor table, int chunk_bytes, int[] out_cols) -> Tensor[]",
+    "addn(Tensor[] inputs) -> Tensor",
+    "combo_sum(Tensor[] inputs, int dim) -> Tensor[]",
+    "silu_mul(Tensor x) -> Tensor",
+    "silu_mul2(Tensor gate, Tensor up) -> Tensor",
+]
+for _s in _SCHEMAS:
+    _library.define(_s)
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _code(dtype):
+    try:
+        return _DTYPE_CODE[dtype]
+    except KeyError:
+        raise TypeError(f"xpu_ops: dtype {dtype} has no mi355x kernel") from None
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def _rows_2d(x: torch.Tensor):
+    """View x as [rows, cols] with unit column stride without copying when possible."""
+    cols = x.shape[-1]
+    if x.dim() == 2 and x.stride(1) == 1 and x.stride(0) >= cols:
+        return x, x.shape[0], x.stride(0)
+    xc = x if x.is_contiguous() else x.contiguous()
+    rows = xc.numel() // cols if cols else 0
+    return xc, rows, cols
+
+
+def _param_dtype(x_dtype, *params):
+    """Affine parameters are read either in the activation dtype or in fp32."""
+    out = []
+    want = None
+    for p in params:
+        if p is not None and p.dtype != x_dtype:
+            want = torch.float32
+    for p in params:
+        if p is None:
+            out.append(None)
+            continue
+        q = p
+        if want is not None and q.dtype != want:
+            q = q.to(want)
+        out.append(q.contiguous())
+    return out, (want or x_dtype)
+
+
+# ------------------------------------------------------------------- norms
+def _norm_impl(kind, x, residual, weight, bias, eps, want_h):
+    (weight, bias), wb_dtype = _param_dtype(x.dtype, weight, bias)
+    cols = x.shape[-1]
+    for p in (weight, bias):
+        if p is not None and p.numel() != cols:
+            raise ValueError("xpu_ops norm: weight/bias must have the size of the last dimension")
+    x2, rows, xs = _rows_2d(x)
+    y = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+    lib = _lib.lib()
+    dt, wdt = _code(x.dtype), _code(wb_dtype)
+    if x.numel() == 0:
+        if residual is None or not want_h:
+            return y
+        return y, torch.empty_like(y)
+    if residual is None:
+        if kind == "rms":
+            st = lib.xg_rms_norm(_ptr(x2), _ptr(weight), _ptr(y), rows, cols, xs, eps, dt, wdt, _stream())
+        else:
+            st = lib.xg_layer_norm(_ptr(x2), _ptr(weight), _ptr(bias), _ptr(y), rows, cols, xs, eps, dt, wdt, _stream())
+        _lib.check(st, f"xg_{kind}_norm")
+        return y
+    if residual.shape != x.shape or residual.dtype != x.dtype:
+        raise ValueError("xpu_ops add+norm: residual must match x in shape and dtype")
+    r2, _, rs = _rows_2d(residual)
+    h = torch.empty(x.shape, dtype=x.dtype, device=x.device) if want_h else None
+    if kind == "rms":
+        st = lib.xg_add_rms_norm(_ptr(x2), _ptr(r2), _ptr(weight), _ptr(y), _ptr(h), rows, cols, xs, rs, eps, dt, wdt, _stream())
+    else:
+        st = lib.xg_add_layer_norm(
+            _ptr(x2), _ptr(r2), _ptr(weight), _ptr(bias), _ptr(y), _ptr(h), rows, cols, xs, rs, eps, dt, wdt, _stream()
+        )
+    _lib.check(st, f"xg_add_{kind}_norm")
+    return (y, h) if want_h else y
+
+
+def _rms_norm(x, weight, eps):
+    return _norm_impl("rms", x, None, weight, None, eps, False)
+
+
+def _layer_norm(x, weight, bias, eps):
+    return _norm_impl("layer", x, None, weight, bias, eps, False)
+
+
+def _add_rms_norm(x, residual, weight, eps):
+    return _norm_impl("rms", x, residual, weight, None, eps, True)
+
+
+def _add_rms_norm_only(x, residual, weight, eps):
+    return _norm_impl("rms", x, residual, weight, None, eps, False)
+
+
+def _add_layer_norm(x, residual, weight, bias, eps):
+    return _norm_impl("layer", x, residual, weight, bias, eps, True)
+
+
+def _add_layer_norm_only(x, residual, weight, bias, eps):
+    return _norm_impl("layer", x, residual, weight, bias, eps, False)
+
+
+def _like(x):
+    return torch.empty(x.shape, dtype=x.dtype, device=x.device)
+
+
+_library.impl("rms_norm", _rms_norm, "CUDA")
+_library.impl("layer_norm", _layer_norm, "CUDA")
+_library.impl("add_rms_norm", _add_rms_norm, "CUDA")
+_library.impl("add_rms_norm_only", _add_rms_norm_only, "CUDA")
+_library.impl("add_layer_norm", _add_layer_norm, "CUDA")
+_library.impl("add_layer_norm_only", _add_layer_norm_only, "CUDA")
+_library.impl("rms_norm", lambda x, weight, eps: _like(x), "Meta")
+_library.impl("layer_norm", lambda x, weight, bias, eps: _like(x), "Meta")
+_library.impl("add_rms_norm", lambda x, residual, weight, eps: (_like(x), _like(x)), "Meta")
+_library.impl("add_rms_norm_only", lambda x, residual, weight, eps: _like(x), "Meta")
+_library.impl("add_layer_norm", lambda x, residual, weight, bias, eps: (_like(x), _like(x)), "Meta")
+_library.impl("add_layer_norm_only", lambda x, residual, weight, bias, eps: _like(x), "Meta")
+
+
+# --------------------------------------------------------------- slice / cat
+def _slice_cat_multi(src, table, chunk_bytes, out_cols):
+    if src.dim() != 2:
+        raise NotImplementedError("input must be 2d")
+    if src.stride(1) != 1:
+        src = src.contiguous()
+    esz = src.element_size()
+    rows = src.shape[0]
+    outs = [torch.empty((rows, c), dtype=src.dtype, device=src.device) for c in out_cols]
+    n = len(outs)
+    if n > _lib.SLICE_CAT_MAX_OUTS:
+        raise ValueError(f"slice_cat_multi: at most {_lib.SLICE_CAT_MAX_OUTS} outputs per call")
+    if table.dtype != torch.int32 or table.dim() != 2 or table.shape[1] != 4 or not table.is_contiguous():
+        raise ValueError("slice_cat: table must be a contiguous int32 [n_chunks, 4] tensor")
+    if table.device != src.device:
+        raise ValueError("slice_cat: table must live on the source's device")
+    if rows == 0 or table.shape[0] == 0:
+        return outs
+    align = min(chunk_bytes, 4)
+    if (src.stride(0) * esz) % align or src.data_ptr() % align:
+        src = src.contiguous()
+    ptrs = (ctypes.c_void_p * n)(*[o.data_ptr() for o in outs])
+    rbs = (ctypes.c_int64 * n)(*[c * esz for c in out_cols])
+    st = _lib.lib().xg_slice_cat(
+        _ptr(src), src.stride(0) * esz, rows, ptrs, rbs, n, _ptr(table), table.shape[0], chunk_bytes, _stream()
+    )
+    _lib.check(st, "xg_slice_cat")
+    return outs
+
+
+def _slice_cat(src, table, chunk_bytes, out_cols):
+    return _slice_cat_multi(src, table, chunk_bytes, [out_cols])[0]
+
+
+_library.impl("slice_cat", _slice_cat, "CUDA")
+_library.impl("slice_cat_multi", _slice_cat_multi, "CUDA")
+_library.impl(
+    "slice_cat",
+    lambda src, table, chunk_bytes, out_cols: torch.empty((src.shape[0], out_cols), dtype=src.dtype, device=src.device),
+    "Meta",
+)
+_library.impl(
+    "slice_cat_multi",
+    lambda src, table, chunk_bytes, out_cols: [
+        torch.empty((src.shape[0], c), dtype=src.dtype, device=src.device) for c in out_cols
+    ],
+    "Meta",
+)
+
+
+# --------------------------------------------------------------------- sums
+def _addn(inputs: List[torch.Tensor]):
+    if len(inputs) == 0:
+        raise ValueError("addn: needs at least one input")
+    first = inputs[0]
+    ins = []
+    for t in inputs:
+        if t.shape != first.shape or t.dtype != first.dtype:
+            raise ValueError("addn: all inputs must share shape and dtype")
+        ins.append(t if t.is_contiguous() else t.contiguous())
+    out = torch.empty(first.shape, dtype=first.dtype, device=first.device)
+    if out.numel() == 0:
+        return out
+    ptrs = (ctypes.c_void_p * len(ins))(*[t.data_ptr() for t in ins])
+    st = _lib.lib().xg_addn(ptrs, len(ins), _ptr(out), out.numel(), _code(first.dtype), _stream())
+    _lib.check(st, "xg_addn")
+    return out
+
+
+def _combo_sum_shapes(inputs, dim):
+    if dim not in (1, 2):
+        raise ValueError("combo_sum: dim must be 1 or 2")
+    shapes = []
+    for t in inputs:
+        if t.dim() != 3:
+            raise ValueError("combo_sum: inputs must be 3-d")
+        shapes.append((t.shape[0], t.shape[2]) if dim == 1 else (t.shape[0], t.shape[1]))
+    return shapes
+
+
+def _combo_sum(inputs: List[torch.Tensor], dim: int):
+    shapes = _combo_sum_shapes(inputs, dim)
+    if len(inputs) == 0:
+        return []
+    dtype = inputs[0].dtype
+    ins = []
+    for t in inputs:
+        if t.dtype != dtype:
+            raise ValueError("combo_sum: all inputs must share a dtype")
+        ins.append(t if t.is_contiguous() else t.contiguous())
+    outs = [torch.empty(s, dtype=dtype, device=t.device) for s, t in zip(shapes, ins)]
+    lib = _lib.lib()
+    step = _lib.COMBO_SUM_MAX_JOBS
+    for lo in range(0, len(ins), step):
+        part_in, part_out = ins[lo : lo + step], outs[lo : lo + step]
+        n = len(part_in)
+        ip = (ctypes.c_void_p * n)(*[t.data_ptr() for t in part_in])
+        op = (ctypes.c_void_p * n)(*[t.data_ptr() for t in part_out])
+        s0 = (ctypes.c_int64 * n)(*[t.shape[0] for t in part_in])
+        s1 = (ctypes.c_int64 * n)(*[t.shape[1] for t in part_in])
+        s2 = (ctypes.c_int64 * n)(*[t.shape[2] for t in part_in])
+        st = lib.xg_combo_sum(ip, op, s0, s1, s2, n, dim, _code(dtype), _stream())
+        _lib.check(st, "xg_combo_sum")
+    return outs
+
+
+_library.impl("addn", _addn, "CUDA")
+_library.impl("combo_sum", _combo_sum, "CUDA")
+_library.impl("addn", lambda inputs: _like(inputs[0]), "Meta")
+_library.impl(
+    "combo_sum",
+    lambda inputs, dim: [
+        torch.empty(s, dtype=t.dtype, device=t.device) for s, t in zip(_combo_sum_shapes(inputs, dim), inputs)
+    ],
+    "Meta",
+)
+
+
+# ------------------------------------------------------------------- SwiGLU
+def _silu_mul(x):
+    if x.shape[-1] % 2 != 0:
+        raise ValueError("silu_mul: last dimension must be even")
+    d = x.shape[-1] // 2
+    x2, rows, xs = _rows_2d(x)
+    y = torch.empty((*x.shape[:-1], d), dtype=x.dtype, device=x.device)
+    if y.numel() == 0:
+        return y
+    st = _lib.lib().xg_silu_mul(_ptr(x2), _ptr(y), rows, d, xs, _code(x.dtype), _stream())
+    _lib.check(st, "xg_silu_mul")
+    return y
+
+
+def _silu_mul2(gate, up):
+    if gate.shape != up.shape or gate.dtype != up.dtype:
+        raise ValueError("silu_mul2: gate and up must match in shape and dtype")
+    d = gate.shape[-1]
+    g2, rows, gs = _rows_2d(gate)
+    u2, _, us = _rows_2d(up)
+    y = torch.empty(gate.shape, dtype=gate.dtype, device=gate.device)
+    if y.numel() == 0:
+        return y
+    st = _lib.lib().xg_silu_mul2(_ptr(g2), _ptr(u2), _ptr(y), rows, d, gs, us, _code(gate.dtype), _stream())
+    _lib.check(st, "xg_silu_mul2")
+    return y
+
+
+_library.impl("silu_mul", _silu_mul, "CUDA")
+_library.impl("silu_mul2", _silu_mul2, "CUDA")
+_library.impl(
+    "silu_mul",
+    lambda x: torch.empty((*x.shape[:-1], x.shape[-1] // 2), dtype=x.dtype, device=x.device),
+    "Meta",
+)
+_library.impl("silu_mul2", lambda gate, up: _like(gate), "Meta")
+
+
+# ------------------------------------------------------------ slice tables
+def build_slice_table(slice_lists, src_cols, elem_size, src_row_stride=None):
+    """Chunk table for `xg_slice_cat` from static python slice lists.
+
+    slice_lists: one list of (start, end) column ranges per output (already
+    normalised to 0 <= start <= end <= src_cols).  Returns (int32 [n,4] CPU
+    tensor, chunk_bytes, out_cols per output).  The chunk size is the largest
+    power of two <= 16 bytes that divides every slice length in bytes and whose
+    source alignment requirement (min(chunk, 4) bytes) every slice start meets.
+    """
+    import math
+
+    g = 16
+    for sl in slice_lists:
+        for s, e in sl:
+            if not (0 <= s <= e <= src_cols):
+                raise ValueError(f"slice ({s},{e}) outside the source's {src_cols} columns")
+            g = math.gcd(g, (e - s) * elem_size)
+    stride_bytes = (src_row_stride if src_row_stride is not None else src_cols) * elem_size
+    a = math.gcd(16, stride_bytes)
+    for sl in slice_lists:
+        for s, e in sl:
+            if e > s:
+                a = math.gcd(a, s * elem_size)
+    chunk = max(g, 1)
+    if min(chunk, 4) > a:
+        chunk = a
+    rows_out, out_cols = [], []
+    for oid, sl in enumerate(slice_lists):
+        dst = 0
+        for s, e in sl:
+            nbytes = (e - s) * elem_size
+            for k in range(0, nbytes, chunk):
+                rows_out.append((s * elem_size + k, dst + k, oid, 0))
+            dst += nbytes
+        out_cols.append(dst // elem_size)
+    table = torch.tensor(rows_out, dtype=torch.int32).reshape(-1, 4)
+    return table, chunk, out_cols
