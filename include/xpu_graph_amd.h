@@ -171,8 +171,8 @@ int xg_dense_fp8(const void* a_q, const void* b_q, const float* a_scale_dev, con
  * Scaled dot-product attention, optional causal mask, no dropout.
  *   q [B,H,Sq,D], k/v [B,Hkv,Skv,D], out [B,H,Sq,D]; strides in elements for
  *   batch, head and sequence; the D axis has unit stride; D in {64, 128}.
- *   softmax in fp32 with running max; causal aligns the LAST query with the
- *   last key (top-left aligned when Sq == Skv).
+ *   softmax in fp32 with running max; causal hides key j from query i when
+ *   j > i (the is_causal=True convention of torch, top-left aligned).
  * replaces aten.scaled_dot_product_attention as emitted by FusedSDPA
  *   (passes/patterns/common/fuse_scaled_dot_product_attention.py:184-234).
  * ------------------------------------------------------------------------- */

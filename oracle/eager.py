@@ -163,7 +163,7 @@ def causal_sdpa_eager(q, k, v, scale=None):
     scale = (1.0 / math.sqrt(D)) if scale is None else scale
     Sq, Sk = q.shape[-2], k.shape[-2]
     s = torch.matmul(q, k.transpose(-1, -2)) * scale
-    mask = torch.full((Sq, Sk), float("-inf"), device=q.device, dtype=torch.float32).triu(1 + Sk - Sq)
+    mask = torch.full((Sq, Sk), float("-inf"), device=q.device, dtype=torch.float32).triu(1)
     p = torch.softmax(s.float() + mask, dim=-1).to(q.dtype)
     return torch.matmul(p, v)
 

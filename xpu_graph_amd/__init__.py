@@ -1,0 +1,44 @@
+"""xpu_graph for AMD Instinct MI355X: a torch.compile backend whose `mi355x`
+target lowers matched Aten subgraphs to hand-written gfx950 HIP kernels.
+
+    import torch
+    from xpu_graph_amd import XpuGraph, XpuGraphConfig, Target, OptLevel
+
+    backend = XpuGraph(XpuGraphConfig(is_training=False, target=Target.mi355x, opt_level=OptLevel.level2))
+    fast = torch.compile(model, backend=backend)
+
+Public names follow the reference package (src/xpu_graph/__init__.py).
+"""
+from .compiler import XpuGraph, XpuGraphCompiler, XpuGraphRuntimeArtifact
+from .config import OptLevel, Target, XpuGraphConfig
+from .passes.patterns.plugin_pattern import (
+    deregister_plugin_patterns,
+    enable_plugin_patterns,
+    register_plugin_pattern,
+    register_this_as_pattern_constraint,
+    register_this_as_plugin_pattern,
+)
+
+__version__ = "0.1.0"
+
+__all__ = [
+    "XpuGraph",
+    "XpuGraphCompiler",
+    "XpuGraphConfig",
+    "XpuGraphRuntimeArtifact",
+    "Target",
+    "OptLevel",
+    "mi355x_compiler",
+    "register_plugin_pattern",
+    "register_this_as_plugin_pattern",
+    "register_this_as_pattern_constraint",
+    "deregister_plugin_patterns",
+    "enable_plugin_patterns",
+]
+
+
+def mi355x_compiler(is_training=False, opt_level=OptLevel.level2, debug=False, **config_kwargs):
+    """Ready-made backend for the MI355X target (counterpart of the reference's mlu_compiler / npu_compiler
+    convenience constructors, src/xpu_graph/__init__.py:32-154)."""
+    cfg = XpuGraphConfig(is_training=is_training, target=Target.mi355x, opt_level=opt_level, debug=debug, enable_cache=False, **config_kwargs)
+    return XpuGraph(cfg)

@@ -1,0 +1,183 @@
+"""`XpuGraph`: the torch.compile backend.
+
+    compiled = torch.compile(fn, backend=XpuGraph(XpuGraphConfig(is_training=False, target=Target.mi355x,
+                                                               opt_level=OptLevel.level2)))
+
+Dynamo hands over a Torch-IR graph; AOT dispatch lowers it to functional Aten
+IR; the pass pipeline rewrites that graph (on the mi355x target: into calls of
+the gfx950 kernels) and the rewritten GraphModule is what runs.  Entry points
+and their behaviour follow the reference (src/xpu_graph/compiler.py:32-327);
+graph capture goes through `aot_autograd` -- the reference's own path for
+graphs with subclass inputs (compiler.py:138-154) -- because it is the stable
+interface across torch versions.  No vendor compiler is involved: the compiled
+artifact is the FX GraphModule itself.
+"""
+import itertools
+from typing import Callable
+
+import torch
+from torch._dynamo.backends.common import aot_autograd
+from torch._functorch.aot_autograd import make_boxed_func
+
+from .config import Target, XpuGraphConfig, get_partition_fn
+from .fx_utils import FxStage, fakify_tensors
+from .passes.pass_manager import PassManager
+from .passes.patterns.plugin_pattern import __PLUGIN_PATTERN_GROUP__
+from .utils import local_logger, logger, setup_logger
+
+__all__ = ["XpuGraph", "XpuGraphCompiler", "XpuGraphRuntimeArtifact"]
+
+
+class XpuGraphRuntimeArtifact:
+    """What torch.compile calls at run time; honours the boxed calling convention
+    (reference src/xpu_graph/runtime/__init__.py:1-9)."""
+
+    def __init__(self, compiled_func, boxed=None):
+        self._compiled_func = compiled_func
+        # The wrapper AOT returns takes *args yet inherits a `_boxed_call` attribute from the
+        # module it wraps, so the convention is stated by the creator when it is known.
+        self._boxed = getattr(compiled_func, "_boxed_call", False) if boxed is None else boxed
+
+    def __call__(self, *args):
+        if self._boxed:
+            return self._compiled_func(list(args))
+        return self._compiled_func(*args)
+
+
+def _node_census(gm):
+    counts = {}
+    for n in gm.graph.nodes:
+        if n.op in ("call_function", "call_module", "call_method"):
+            counts[str(n.target)] = counts.get(str(n.target), 0) + 1
+    return dict(sorted(counts.items(), key=lambda kv: -kv[1]))
+
+
+class XpuGraph:
+    def __init__(self, config: XpuGraphConfig, cache=None):
+        config._reset_config_with_env()
+        self._config = config
+        setup_logger(config.debug)
+        self._cache = None  # compile-artifact caching is not part of this build
+        self._orig_ctx = {}
+        self._set_context()
+        self._pass_manager = PassManager(config)
+        # plugin patterns run before the built-in ones of their group
+        plugins = __PLUGIN_PATTERN_GROUP__.get(config.target, {})
+        self._pass_manager.get_pattern_manager().insert_patterns(list(itertools.chain.from_iterable(plugins.values())))
+
+    # -- compile one Aten graph ------------------------------------------------------
+    def _get_compiler(self, stage: FxStage):
+        def compile_stage(gm, sample_inputs):
+            with local_logger(stage.name):
+                fake_mode, fake_inputs = fakify_tensors(sample_inputs)
+                with fake_mode:
+                    with local_logger("before"):
+                        logger.debug("before xpu_graph, graph like:\n %s", gm.print_readable(print_output=False))
+                        logger.info(f"xpu_graph passes start {stage}...")
+                    before = _node_census(gm)
+                    out = self._pass_manager(gm, fake_inputs, stage)
+                    with local_logger("after"):
+                        logger.info("xpu_graph passes complete")
+                        logger.debug("after xpu_graph, graph like:\n %s", out.print_readable(print_output=False))
+                    logger.info(f"node statistic: before {before} after {_node_census(out)}")
+                    if self._config.vendor_compiler_config is not None:
+                        logger.warning("vendor_compiler_config is ignored: this backend runs the rewritten graph directly")
+                # AOT's runtime wrappers call the compiled stage with one list of arguments
+                return make_boxed_func(out)
+
+        return compile_stage
+
+    def __call__(self, dynamo_gm, example_inputs, *args, **kwargs):
+        logger.info(f"{self._config}")
+        logger.debug("before compile: graph like:\n %s", dynamo_gm.print_readable(print_output=False))
+        if self._config.is_training:
+            aot_kwargs = {
+                "fw_compiler": self._get_compiler(FxStage.forward),
+                "bw_compiler": self._get_compiler(FxStage.backward),
+                "inference_compiler": self._get_compiler(FxStage.inference),
+                "keep_inference_input_mutations": True,
+            }
+            part = get_partition_fn(self._config.partition_fn)
+            if part is not None:
+                aot_kwargs["partition_fn"] = part
+            compiled = aot_autograd(**aot_kwargs)(dynamo_gm, example_inputs)
+        else:
+            aot_kwargs = {"fw_compiler": self._get_compiler(FxStage.inference), "keep_inference_input_mutations": True}
+            # an inference compiler: trace without autograd whatever the caller's grad mode is
+            with torch.no_grad():
+                compiled = aot_autograd(**aot_kwargs)(dynamo_gm, example_inputs)
+        artifact = XpuGraphRuntimeArtifact(compiled, boxed=False)
+
+        opts = kwargs.get("options") or {}
+        guard_filter_fn = opts.get("guard_filter_fn")
+        ctx = torch._guards.TracingContext.try_get()
+        if guard_filter_fn is not None and ctx is not None:
+            guards = ctx.guards_context.dynamo_guards
+            flags = guard_filter_fn(guards)
+            dropped = torch._guards.GuardsSet({g for g, keep in zip(guards, flags) if not keep})
+            logger.info(f"Removed guards: {list(dropped)}")
+            ctx.guards_context.dynamo_guards = guards - dropped
+        return artifact
+
+    def get_pattern_manager(self):
+        return self._pass_manager.get_pattern_manager()
+
+    def _set_context(self):
+        import torch._inductor.config as inductor_config
+
+        self._orig_ctx["freezing"] = inductor_config.freezing
+        inductor_config.freezing = bool(self._config.freeze and not self._config.is_training)
+
+    def _restore_context(self):
+        import torch._inductor.config as inductor_config
+
+        inductor_config.freezing = self._orig_ctx["freezing"]
+
+
+class XpuGraphCompiler:
+    """Fluent wrapper: XpuGraphCompiler().set_target(...).set_opt_level(...).done(); .compile(model)
+    (reference compiler.py:273-327).  Every config field gets a property and a chained set_<field>."""
+
+    def __init__(self):
+        self._config = XpuGraphConfig(is_training=False)
+        self._config._reset_config_with_env()
+        self._compiler = None
+        self.prior_work()
+
+    def __init_subclass__(cls, **kw):
+        super().__init_subclass__(**kw)
+
+    def prior_work(self):
+        ...
+
+    def done(self):
+        self._compiler = XpuGraph(self._config)
+        return self
+
+    def compile(self, model, *args, backend=None, **kwargs) -> Callable:
+        assert isinstance(self._compiler, XpuGraph), "You should call XpuGraphCompiler.done before XpuGraphCompiler.compile"
+        return torch.compile(model, *args, backend=self._compiler, **kwargs)
+
+
+def _install_config_accessors():
+    import dataclasses
+
+    for f in dataclasses.fields(XpuGraphConfig):
+        name = f.name
+
+        def getter(self, _n=name):
+            return getattr(self._config, _n)
+
+        def setter(self, val, _n=name):
+            setattr(self._config, _n, val)
+            self._compiler = None
+
+        def chained(self, val, _s=setter):
+            _s(self, val)
+            return self
+
+        setattr(XpuGraphCompiler, name, property(getter, setter))
+        setattr(XpuGraphCompiler, f"set_{name}", chained)
+
+
+_install_config_accessors()

@@ -230,11 +230,12 @@ int launch_typed(const NormArgs& a) {
     const int nvec = (int)(a.cols / VN);
     int tpr = tuned_tpr();
     if (tpr == 0) {
-      // Heuristic: the fewest threads per row that keep <= 8 vectors per thread,
-      // preferring whole-wavefront rows (no LDS, no barrier) up to 512 vectors.
+      // Heuristic from measurement on MI355X: short rows stay inside one wavefront
+      // (no LDS, no barrier); from 256 vectors up a 256-thread row with few
+      // vectors per thread streams better than one wavefront with many.
       if (nvec <= 16 * 2)
         tpr = 16;
-      else if (nvec <= 64 * 8)
+      else if (nvec <= 64 * 4)
         tpr = 64;
       else if (nvec <= 256 * 8)
         tpr = 256;

@@ -355,3 +355,140 @@ def build_slice_table(slice_lists, src_cols, elem_size, src_row_stride=None):
         out_cols.append(dst // elem_size)
     table = torch.tensor(rows_out, dtype=torch.int32).reshape(-1, 4)
     return table, chunk, out_cols
+
+
+# ------------------------------------------------------------- dense / SDPA
+_library.define("dense(Tensor x, Tensor weight, bool weight_trans, Tensor? bias, Tensor? residual, str act) -> Tensor")
+_library.define(
+    "dense_fp8(Tensor x_q, Tensor w_q, bool weight_trans, Tensor x_scale, Tensor w_scale, Tensor? bias, str act, ScalarType out_dtype) -> Tensor"
+)
+_library.define("sdpa(Tensor q, Tensor k, Tensor v, bool is_causal, float scale) -> Tensor")
+
+
+def _dense_out_shape(x, weight, weight_trans):
+    if x.dim() != 2 or weight.dim() != 2:
+        raise ValueError("dense: x and weight must be 2-d")
+    k = x.shape[1]
+    n, wk = (weight.shape[0], weight.shape[1]) if weight_trans else (weight.shape[1], weight.shape[0])
+    if wk != k:
+        raise ValueError(f"dense: inner dimensions differ ({k} vs {wk})")
+    return x.shape[0], n, k
+
+
+def _row_major(t):
+    """2-D tensor with unit last stride (copied only when it is not)."""
+    return t if t.stride(-1) == 1 and t.stride(0) >= t.shape[1] else t.contiguous()
+
+
+def _dense(x, weight, weight_trans, bias, residual, act):
+    m, n, k = _dense_out_shape(x, weight, weight_trans)
+    if act not in _lib.ACT_CODES:
+        raise ValueError(f"dense: unknown activation {act!r}")
+    if weight.dtype != x.dtype:
+        raise TypeError("dense: x and weight must share a dtype")
+    x, weight = _row_major(x), _row_major(weight)
+    out = torch.empty((m, n), dtype=x.dtype, device=x.device)
+    if out.numel() == 0:
+        return out
+    bias_dt = _code(x.dtype)
+    if bias is not None:
+        if bias.numel() != n:
+            raise ValueError("dense: bias must have N elements")
+        bias = bias.contiguous()
+        if bias.dtype != x.dtype:
+            bias = bias.float()
+        bias_dt = _code(bias.dtype)
+    ldr = 0
+    if residual is not None:
+        if tuple(residual.shape) != (m, n) or residual.dtype != x.dtype:
+            raise ValueError("dense: residual must be [M, N] in the input dtype")
+        residual = _row_major(residual)
+        ldr = residual.stride(0)
+    st = _lib.lib().xg_dense(
+        _ptr(x), _ptr(weight), _ptr(bias), _ptr(residual), _ptr(out), m, n, k, x.stride(0), weight.stride(0), ldr,
+        1 if weight_trans else 0, _lib.ACT_CODES[act], _code(x.dtype), bias_dt, _stream(),
+    )
+    _lib.check(st, "xg_dense")
+    return out
+
+
+def _dense_meta(x, weight, weight_trans, bias, residual, act):
+    m, n, _ = _dense_out_shape(x, weight, weight_trans)
+    return torch.empty((m, n), dtype=x.dtype, device=x.device)
+
+
+def _dense_fp8(x_q, w_q, weight_trans, x_scale, w_scale, bias, act, out_dtype):
+    m, n, k = _dense_out_shape(x_q, w_q, weight_trans)
+    if x_q.dtype != torch.float8_e4m3fn or w_q.dtype != torch.float8_e4m3fn:
+        raise TypeError("dense_fp8: operands must be float8_e4m3fn")
+    if act not in _lib.ACT_CODES:
+        raise ValueError(f"dense_fp8: unknown activation {act!r}")
+    x_q, w_q = _row_major(x_q), _row_major(w_q)
+    x_scale = x_scale.reshape(-1).float().contiguous()
+    w_scale = w_scale.reshape(-1).float().contiguous()
+    if x_scale.numel() != 1 or w_scale.numel() != n:
+        raise ValueError("dense_fp8: x_scale must have 1 element and w_scale N elements")
+    out = torch.empty((m, n), dtype=out_dtype, device=x_q.device)
+    if out.numel() == 0:
+        return out
+    bias_dt = XG_F32
+    if bias is not None:
+        if bias.numel() != n:
+            raise ValueError("dense_fp8: bias must have N elements")
+        bias = bias.contiguous()
+        if bias.dtype != out_dtype:
+            bias = bias.float()
+        bias_dt = _code(bias.dtype)
+    st = _lib.lib().xg_dense_fp8(
+        _ptr(x_q), _ptr(w_q), _ptr(x_scale), _ptr(w_scale), _ptr(bias), _ptr(out), m, n, k, x_q.stride(0), w_q.stride(0),
+        1 if weight_trans else 0, _lib.ACT_CODES[act], _code(out_dtype), bias_dt, _stream(),
+    )
+    _lib.check(st, "xg_dense_fp8")
+    return out
+
+
+def _dense_fp8_meta(x_q, w_q, weight_trans, x_scale, w_scale, bias, act, out_dtype):
+    m, n, _ = _dense_out_shape(x_q, w_q, weight_trans)
+    return torch.empty((m, n), dtype=out_dtype, device=x_q.device)
+
+
+def _sdpa_check(q, k, v):
+    if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
+        raise ValueError("sdpa: q, k, v must be [B, H, S, D]")
+    if k.shape != v.shape or q.shape[0] != k.shape[0] or q.shape[3] != k.shape[3] or q.shape[1] % max(k.shape[1], 1) != 0:
+        raise ValueError("sdpa: inconsistent q/k/v shapes")
+
+
+def _unit_last(t):
+    return t if t.stride(-1) == 1 else t.contiguous()
+
+
+def _sdpa(q, k, v, is_causal, scale):
+    _sdpa_check(q, k, v)
+    if k.dtype != q.dtype or v.dtype != q.dtype:
+        raise TypeError("sdpa: q, k, v must share a dtype")
+    q, k, v = _unit_last(q), _unit_last(k), _unit_last(v)
+    B, H, Sq, D = q.shape
+    out = torch.empty((B, H, Sq, D), dtype=q.dtype, device=q.device)
+    if out.numel() == 0:
+        return out
+    S3 = ctypes.c_int64 * 3
+    st = _lib.lib().xg_sdpa(
+        _ptr(q), _ptr(k), _ptr(v), _ptr(out), B, H, k.shape[1], Sq, k.shape[2], D, S3(*q.stride()[:3]), S3(*k.stride()[:3]),
+        S3(*v.stride()[:3]), S3(*out.stride()[:3]), scale, 1 if is_causal else 0, _code(q.dtype), _stream(),
+    )
+    _lib.check(st, "xg_sdpa")
+    return out
+
+
+def _sdpa_meta(q, k, v, is_causal, scale):
+    _sdpa_check(q, k, v)
+    return torch.empty(q.shape, dtype=q.dtype, device=q.device)
+
+
+_library.impl("dense", _dense, "CUDA")
+_library.impl("dense", _dense_meta, "Meta")
+_library.impl("dense_fp8", _dense_fp8, "CUDA")
+_library.impl("dense_fp8", _dense_fp8_meta, "Meta")
+_library.impl("sdpa", _sdpa, "CUDA")
+_library.impl("sdpa", _sdpa_meta, "Meta")

@@ -1,0 +1,159 @@
+"""Target-independent clean-up passes that keep graphs canonical for the matchers:
+assertion removal, view->reshape, dead-code elimination, common-subexpression
+elimination and folding of constant subgraphs.
+
+Behaviour follows the reference's passes of the same names
+(src/xpu_graph/passes/{remove_runtime_assertions,view_to_reshape,dce,cse,constant_folding}.py).
+"""
+import torch
+import torch.fx as fx
+import torch.utils._pytree as pytree
+
+from ..fx_utils import FxStage, outside_fake_mode
+from ..utils import logger
+from .optimizer import Optimizer
+
+aten = torch.ops.aten
+_ALL_STAGES = [FxStage.inference, FxStage.pregrad, FxStage.forward, FxStage.backward]
+
+
+class RemoveAssertions(Optimizer):
+    """Drops aten._assert_tensor_metadata nodes: they add users that defeat single-use checks."""
+
+    _support_stages = _ALL_STAGES
+
+    def process(self, gm):
+        if not hasattr(aten, "_assert_tensor_metadata"):
+            return False
+        victims = list(gm.graph.find_nodes(op="call_function", target=aten._assert_tensor_metadata.default))
+        for n in victims:
+            gm.graph.erase_node(n)
+        return bool(victims)
+
+
+class ViewToReshape(Optimizer):
+    """view/_unsafe_view -> reshape: later rewrites may change input strides, reshape stays valid."""
+
+    _support_stages = _ALL_STAGES
+
+    def process(self, gm):
+        changed = False
+        for n in gm.graph.nodes:
+            if n.op == "call_function" and n.target in (aten.view.default, aten._unsafe_view.default):
+                n.target = aten.reshape.default
+                changed = True
+        return changed
+
+
+class Dce(Optimizer):
+    _support_stages = _ALL_STAGES
+
+    def process(self, gm):
+        changed = gm.graph.eliminate_dead_code()
+        used = {n.target for n in gm.graph.nodes if n.op == "get_attr"}
+        for name in [k for k in getattr(gm, "_xg_constants", ()) if k not in used]:
+            delattr(gm, name)
+            gm._xg_constants.remove(name)
+            changed = True
+        return changed
+
+
+def _hashable(x):
+    if isinstance(x, (list, tuple)):
+        return tuple(_hashable(i) for i in x)
+    if isinstance(x, dict):
+        return tuple(sorted((k, _hashable(v)) for k, v in x.items()))
+    if isinstance(x, fx.Node):
+        return ("node", id(x))
+    if isinstance(x, (torch.dtype, torch.device, torch.layout, torch.memory_format, str, int, float, bool, type(None), slice)):
+        return (type(x).__name__, x if not isinstance(x, slice) else (x.start, x.stop, x.step))
+    return ("obj", id(x))
+
+
+class Cse(Optimizer):
+    """Merges repeated pure call_function nodes with identical targets and arguments."""
+
+    _support_stages = _ALL_STAGES
+
+    @staticmethod
+    def _mergeable(node):
+        if node.op != "call_function" or node.is_impure():
+            return False
+        tgt = node.target
+        if isinstance(tgt, torch._ops.OpOverload):
+            if torch.Tag.nondeterministic_seeded in tgt.tags or tgt._schema.is_mutable:
+                return False
+            name = tgt._schema.name
+            # factories and copies return fresh storage that later in-place ops may write
+            if name.startswith("aten::empty") or name in ("aten::clone", "aten::_to_copy", "aten::copy"):
+                return False
+            return True
+        return tgt.__module__ == "_operator"
+
+    def process(self, gm):
+        seen = {}
+        changed = False
+        for node in list(gm.graph.nodes):
+            if not self._mergeable(node):
+                continue
+            key = (node.target, _hashable(node.args), _hashable(node.kwargs))
+            prev = seen.get(key)
+            if prev is None:
+                seen[key] = node
+            else:
+                node.replace_all_uses_with(prev)
+                gm.graph.erase_node(node)
+                changed = True
+        return changed
+
+
+def is_constant(arg, include_params=True):
+    """Python scalars, and get_attr nodes (graph constants; parameters when include_params)."""
+    if isinstance(arg, fx.Node):
+        if arg.op != "get_attr":
+            return False
+        if include_params:
+            return True
+        return arg.target in getattr(arg.graph.owning_module, "_xg_constants", ())
+    return True
+
+
+class ConstantFolding(Optimizer):
+    """Evaluates call_function nodes whose inputs are all constants and stores the
+    result as a module attribute read through get_attr."""
+
+    def __init__(self, folding_params=False):
+        super().__init__()
+        self.folding_params = folding_params
+
+    def process(self, gm):
+        graph = gm.graph
+        anchor = None
+        for anchor in graph.nodes:
+            if anchor.op not in ("placeholder", "get_attr"):
+                break
+        changed = False
+        for node in list(graph.nodes):
+            if node.op != "call_function" or node.is_impure():
+                continue
+            flat, _ = pytree.tree_flatten((node.args, node.kwargs))
+            if not any(isinstance(a, fx.Node) for a in flat):
+                continue  # factory calls stay in the graph: they are cheap and device-bound
+            if not all(is_constant(a, self.folding_params) for a in flat):
+                continue
+            args, kwargs = pytree.tree_map(lambda a: getattr(gm, a.target) if isinstance(a, fx.Node) else a, (node.args, node.kwargs))
+            logger.info(f"start constant folding: {node.name} {node.target}")
+            with outside_fake_mode():
+                value = node.target(*args, **kwargs)
+            if not isinstance(value, torch.Tensor):
+                continue
+            name = f"_xg_folded_{node.name}"
+            gm.register_buffer(name, value, persistent=False)
+            if not hasattr(gm, "_xg_constants"):
+                gm._xg_constants = []
+            gm._xg_constants.append(name)
+            with graph.inserting_before(anchor):
+                const = graph.get_attr(name)
+            node.replace_all_uses_with(const)
+            changed = True
+        return changed

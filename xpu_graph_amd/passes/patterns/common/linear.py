@@ -1,0 +1,57 @@
+"""mm + bias -> addmm (reference src/xpu_graph/passes/patterns/common/fuse_addmm.py:12-90).
+
+Fires when one operand of an add.Tensor is an mm (or 2-D matmul) used only by
+that add and the sum has the mm's shape.  A python-number / symbolic bias
+becomes a scalar_tensor; a bias of another dtype is cast to the input's dtype,
+and the result is cast back if the add had promoted it.
+"""
+import torch
+from torch import fx
+
+from ....config import OptLevel
+from ....fx_utils import FxStage
+from ..pattern import Pattern
+from ..utils.node_utils import aten, is_call, mm_operands, same_shape
+
+
+def match_mm_plus_bias(node):
+    if not is_call(node, aten.add.Tensor):
+        return None
+    for mm, bias in ((node.args[0], node.args[1]), (node.args[1], node.args[0])):
+        ops = mm_operands(mm) if isinstance(mm, fx.Node) else None
+        if ops is None:
+            continue
+        if len(mm.users) != 1 or not same_shape(node.meta["val"].shape, mm.meta["val"].shape):
+            return None
+        return bias, ops[0], ops[1]
+    return None
+
+
+class FusedAddMM(Pattern):
+    _opt_level = OptLevel.level2
+    _support_stages = [FxStage.inference, FxStage.forward, FxStage.pregrad]
+
+    def process(self, gm):
+        g = gm.graph
+        cast = aten.to.dtype if self._current_stage == FxStage.pregrad else aten._to_copy.default
+        changed = False
+        for node in reversed(g.nodes):
+            m = match_mm_plus_bias(node)
+            if m is None:
+                continue
+            bias, x, w = m
+            x_val = x.meta["val"]
+            with g.inserting_before(node):
+                if isinstance(bias, (int, float)) or (isinstance(bias, fx.Node) and not isinstance(bias.meta["val"], torch.Tensor)):
+                    bias = g.create_node(
+                        "call_function", aten.scalar_tensor.default, (bias,), {"dtype": x_val.dtype, "device": x_val.device}, name="bias_constant"
+                    )
+                elif bias.meta["val"].dtype != x_val.dtype:
+                    bias = g.create_node("call_function", cast, (bias,), {"dtype": x_val.dtype}, name="bias_cast")
+                new = g.create_node("call_function", aten.addmm.default, (bias, x, w), name="addmm_replacement")
+                if x_val.dtype != node.meta["val"].dtype:
+                    new = g.create_node("call_function", cast, (new,), {"dtype": node.meta["val"].dtype}, name="input_cast")
+            node.replace_all_uses_with(new)
+            g.erase_node(node)
+            changed = True
+        return changed

@@ -1,0 +1,203 @@
+"""Attention ops -> the flash-style gfx950 kernel.
+
+Handles `aten.scaled_dot_product_attention` (what FusedSDPA emits) and the
+backend-specific ops it decomposes to when the user calls
+F.scaled_dot_product_attention directly.  An additive mask is accepted only if
+it is a compile-time constant equal to the causal mask (-inf or the dtype's
+lowest value strictly above the diagonal, 0 elsewhere); it is then dropped and
+the kernel masks by index.  The reference never detects causality
+(fuse_scaled_dot_product_attention.py:184-234 forwards the mask as attn_mask).
+
+The rewrite also looks through the contiguous clones and 3-D reshapes FusedSDPA
+puts in front of q, k, v: the kernel takes strides, so the [B, H, S, D] views
+are passed as they are.
+"""
+import math
+import operator
+
+import torch
+from torch import fx, nn
+
+from .....config import OptLevel
+from .....fx_utils import outside_fake_mode
+from ...pattern import Pattern, PatternGroup
+from ...utils.node_utils import VIEW_OPS, aten, is_call, is_getitem, same_shape
+
+SDPA_NAME = "mi355x_sdpa"
+_DTYPES = (torch.bfloat16, torch.float16)
+_HEAD_DIMS = (64, 128)
+_MAX_CONST_ELEMS = 1 << 26
+
+
+class SDPAModule(nn.Module):
+    def forward(self, q, k, v, is_causal, scale):
+        return torch.ops.xpu_ops.sdpa(q, k, v, is_causal, scale)
+
+
+def _const_eval(node, memo):
+    """Value of a node computed from no graph input (factories, constants and ops on them), on CPU; None otherwise."""
+    if node in memo:
+        return memo[node]
+    out = None
+    if node.op == "get_attr":
+        obj = node.graph.owning_module
+        for part in node.target.split("."):
+            obj = getattr(obj, part)
+        out = obj.detach().cpu() if isinstance(obj, torch.Tensor) else None
+    elif node.op == "call_function" and isinstance(node.target, torch._ops.OpOverload):
+        v = node.meta.get("val")
+        ok = isinstance(v, torch.Tensor) and all(isinstance(d, int) for d in v.shape) and v.numel() <= _MAX_CONST_ELEMS
+        if ok and torch.Tag.nondeterministic_seeded not in node.target.tags:
+            vals = {}
+            for inp in node.all_input_nodes:
+                vals[inp] = _const_eval(inp, memo)
+                if vals[inp] is None:
+                    ok = False
+                    break
+            if ok:
+                args = fx.map_arg(node.args, lambda n: vals[n])
+                kwargs = dict(fx.map_arg(node.kwargs, lambda n: vals[n]))
+                if "device" in kwargs:
+                    kwargs["device"] = torch.device("cpu")
+                kwargs.pop("pin_memory", None)
+                try:
+                    out = node.target(*args, **kwargs)
+                except Exception:
+                    out = None
+    memo[node] = out
+    return out
+
+
+def is_causal_constant(mask, sq, skv):
+    """True when `mask` is a compile-time constant that broadcasts to the [sq, skv] causal additive mask."""
+    if not isinstance(mask, fx.Node) or not isinstance(sq, int) or not isinstance(skv, int):
+        return False
+    with outside_fake_mode():
+        val = _const_eval(mask, {})
+        if not isinstance(val, torch.Tensor) or not val.dtype.is_floating_point:
+            return False
+        if val.dim() < 2 or val.shape[-2:] != (sq, skv):
+            return False
+        lead = val.reshape(-1, sq, skv)
+        if not all(torch.equal(lead[0], lead[i]) for i in range(1, lead.shape[0])):
+            return False
+        m = lead[0].float()
+        upper = torch.ones(sq, skv, dtype=torch.bool).triu(1)  # key j hidden from query i when j > i, as is_causal=True means
+        lowest = torch.finfo(val.dtype).min
+        masked = m[upper]
+        return bool((m[~upper] == 0).all()) and bool(((masked == float("-inf")) | (masked <= lowest)).all())
+
+
+def _peel_qv(node, dims):
+    """reshape(clone(reshape(x4d, [BH,S,D])), [B,H,S,D]) -> x4d when x4d already has that 4-D shape."""
+    if is_call(node, *VIEW_OPS) and is_call(node.args[0], aten.clone.default):
+        inner = node.args[0].args[0]
+        if is_call(inner, *VIEW_OPS):
+            src = inner.args[0]
+            if isinstance(src, fx.Node) and "val" in src.meta and same_shape(list(src.meta["val"].shape), list(dims)):
+                return src
+    return node
+
+
+def _peel_k(node, dims):
+    """reshape(clone(transpose(reshape(transpose(k4d, -1, -2), [BH,D,S]), -1, -2)), [B,H,S,D]) -> k4d."""
+    if not (is_call(node, *VIEW_OPS) and is_call(node.args[0], aten.clone.default)):
+        return node
+    t1 = node.args[0].args[0]
+    if not is_call(t1, aten.transpose.int) or {t1.args[1], t1.args[2]} not in ({-1, -2}, {1, 2}):
+        return node
+    r = t1.args[0]
+    if not is_call(r, *VIEW_OPS):
+        return node
+    t0 = r.args[0]
+    if not is_call(t0, aten.transpose.int) or {t0.args[1], t0.args[2]} not in ({-1, -2}, {2, 3}):
+        return node
+    src = t0.args[0]
+    if isinstance(src, fx.Node) and "val" in src.meta and same_shape(list(src.meta["val"].shape), list(dims)):
+        return src
+    return node
+
+
+def _supported(q, k, v):
+    vq, vk, vv = (n.meta.get("val") for n in (q, k, v))
+    if not all(isinstance(t, torch.Tensor) and t.dim() == 4 for t in (vq, vk, vv)):
+        return False
+    if vq.dtype not in _DTYPES or vk.dtype != vq.dtype or vv.dtype != vq.dtype:
+        return False
+    B, H, Sq, D = vq.shape
+    if not all(isinstance(d, int) for d in (B, H, Sq, D, *vk.shape, *vv.shape)):
+        return False
+    if D not in _HEAD_DIMS or vk.shape[-1] != D or vv.shape[-1] != D:
+        return False
+    if vk.shape[0] != B or vv.shape != vk.shape or vk.shape[1] == 0 or H % vk.shape[1] != 0:
+        return False
+    return True
+
+
+class FusedCausalSDPA(Pattern):
+    _opt_level = OptLevel.level2
+    _pattern_group = PatternGroup.GROUP1
+
+    def _emit(self, gm, node, q, k, v, causal, scale, replace):
+        if scale is None:
+            scale = 1.0 / math.sqrt(q.meta["val"].shape[-1])
+        if not isinstance(scale, (int, float)):
+            return False
+        with gm.graph.inserting_before(node):
+            new = gm.graph.call_module(SDPA_NAME, args=(q, k, v, bool(causal), float(scale)))
+        replace(new)
+        return True
+
+    def process(self, gm):
+        if not hasattr(gm, SDPA_NAME):
+            gm.add_submodule(SDPA_NAME, SDPAModule())
+        g = gm.graph
+        changed = False
+        backend_ops = {}
+        for name, (drop_idx, causal_idx, bias_idx) in {
+            "_scaled_dot_product_flash_attention": (3, 4, None),
+            "_scaled_dot_product_flash_attention_for_cpu": (3, 4, None),
+            "_scaled_dot_product_efficient_attention": (5, 6, 3),
+            "_scaled_dot_product_cudnn_attention": (5, 6, 3),
+        }.items():
+            op = getattr(aten, name, None)
+            if op is not None:
+                backend_ops[op.default] = (drop_idx, causal_idx, bias_idx)
+
+        for node in reversed(list(g.nodes)):
+            if is_call(node, aten.scaled_dot_product_attention.default):
+                q, k, v = node.args[:3]
+                mask = node.args[3] if len(node.args) > 3 else node.kwargs.get("attn_mask")
+                dropout = node.args[4] if len(node.args) > 4 else node.kwargs.get("dropout_p", 0.0)
+                causal = node.args[5] if len(node.args) > 5 else node.kwargs.get("is_causal", False)
+                scale = node.kwargs.get("scale")
+                if node.kwargs.get("enable_gqa", False) or dropout != 0.0 or not _supported(q, k, v):
+                    continue
+                sq, skv = q.meta["val"].shape[2], k.meta["val"].shape[2]
+                if mask is not None:
+                    if causal or not is_causal_constant(mask, sq, skv):
+                        continue
+                    causal = True
+                q2 = _peel_qv(q, q.meta["val"].shape)
+                k2 = _peel_k(k, k.meta["val"].shape)
+                v2 = _peel_qv(v, v.meta["val"].shape)
+                changed |= self._emit(gm, node, q2, k2, v2, causal, scale, node.replace_all_uses_with)
+            elif node.op == "call_function" and node.target in backend_ops:
+                drop_idx, causal_idx, bias_idx = backend_ops[node.target]
+                users = list(node.users)
+                if not users or not all(is_getitem(u) and u.args[1] == 0 for u in users):
+                    continue
+                args = node.args
+                q, k, v = args[:3]
+                dropout = args[drop_idx] if len(args) > drop_idx else node.kwargs.get("dropout_p", 0.0)
+                causal = args[causal_idx] if len(args) > causal_idx else node.kwargs.get("is_causal", False)
+                bias = (args[bias_idx] if len(args) > bias_idx else None) if bias_idx is not None else node.kwargs.get("attn_mask")
+                if dropout != 0.0 or bias is not None or not _supported(q, k, v):
+                    continue
+
+                def replace(new, users=users):
+                    for u in users:
+                        u.replace_all_uses_with(new)
+
+                changed |= self._emit(gm, node, q, k, v, causal, node.kwargs.get("scale"), replace)
+        return changed

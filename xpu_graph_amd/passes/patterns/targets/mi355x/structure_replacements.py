@@ -1,0 +1,147 @@
+"""Modules the structure patterns substitute on the mi355x target.  Signatures
+are the reference's (passes/patterns/targets/mlu/structure_replacements/
+__init__.py:27-179, dense_layer_modules.py:4-68, norm_modules.py:4-21); bodies
+call `torch.ops.xpu_ops.*`, i.e. the HIP kernels, and nothing else."""
+import torch
+from torch._subclasses.fake_tensor import FakeTensor
+
+from ..... import ops as _xops
+
+_DENSE_DTYPES = (torch.bfloat16, torch.float16)
+
+
+class RMSNormModule(torch.nn.Module):
+    def forward(self, inputs, weight, eps):
+        return torch.ops.xpu_ops.rms_norm(inputs, weight, eps)
+
+
+class LayerNormModule(torch.nn.Module):
+    def forward(self, inputs, weight, bias, eps):
+        return torch.ops.xpu_ops.layer_norm(inputs, weight, bias, eps)
+
+
+class _SliceTables:
+    """Per-(slice list, source layout, device) cache of device-resident chunk tables,
+    so the steady state does no host work beyond a dict lookup."""
+
+    def __init__(self):
+        self._cache = {}
+
+    def get(self, src, slice_lists):
+        key = (tuple(tuple(map(tuple, sl)) for sl in slice_lists), src.shape[1], src.stride(0), src.element_size(), str(src.device))
+        hit = self._cache.get(key)
+        if hit is None:
+            table, chunk, out_cols = _xops.build_slice_table(slice_lists, src.shape[1], src.element_size(), src.stride(0))
+            if isinstance(src, FakeTensor):
+                # shape propagation only: a table of the right shape, nothing cached
+                return torch.empty(table.shape, dtype=torch.int32, device=src.device), chunk, out_cols
+            hit = (table.to(src.device), chunk, out_cols)
+            self._cache[key] = hit
+        return hit
+
+    def __getstate__(self):
+        return {}
+
+    def __setstate__(self, state):
+        self._cache = {}
+
+
+def _check_2d(t):
+    if t.dim() != 2:
+        raise NotImplementedError("input must be 2d")
+    if t.stride(1) != 1:
+        t = t.contiguous()
+    return t
+
+
+class FuseSliceCatSameInputModule(torch.nn.Module):
+    """forward(input2d, [(start, end), ...]) -> [rows, sum(end - start)]"""
+
+    def __init__(self):
+        super().__init__()
+        self._tables = _SliceTables()
+
+    def forward(self, input_tensor, slices):
+        src = _check_2d(input_tensor)
+        table, chunk, out_cols = self._tables.get(src, [slices])
+        return torch.ops.xpu_ops.slice_cat(src, table, chunk, out_cols[0])
+
+
+class FuseSliceCatSameInputModule_v2(torch.nn.Module):
+    """Built with the static table of all slice lists; forward returns one tensor per list, from ONE launch."""
+
+    def __init__(self, many_slices):
+        super().__init__()
+        self.many_slices = [list(map(tuple, sl)) for sl in many_slices]
+        self._tables = _SliceTables()
+
+    def forward(self, input_tensor, many_slices=None):
+        src = _check_2d(input_tensor)
+        lists = self.many_slices
+        step = _xops._lib.SLICE_CAT_MAX_OUTS
+        outs = []
+        for lo in range(0, len(lists), step):
+            part = lists[lo : lo + step]
+            table, chunk, out_cols = self._tables.get(src, part)
+            outs += torch.ops.xpu_ops.slice_cat_multi(src, table, chunk, out_cols)
+        return outs
+
+
+class ComboSumModule(torch.nn.Module):
+    """forward([3-D tensors], [dim]) -> [2-D sums]; one launch for all jobs."""
+
+    def forward(self, input_list, dim):
+        return torch.ops.xpu_ops.combo_sum(list(input_list), dim[0])
+
+
+class DenseLayerModule(torch.nn.Module):
+    """forward(inputs, weight, weight_trans, bias | None, act) -> act(inputs @ W(+T) + bias).
+    A 1-D (or [1, N]) bias is a bias; a 2-D bias is a residual added before the activation."""
+
+    def __init__(self, fast_act=False):
+        super().__init__()
+        self.fast_act = fast_act
+
+    def forward(self, inputs, weight, weight_trans, bias, act):
+        n = weight.shape[-2] if weight_trans else weight.shape[-1]
+        m = inputs.shape[0]
+        residual = None
+        if bias is not None:
+            if bias.dim() == 2 and bias.shape[0] == 1:
+                bias = bias.reshape(-1)
+            if bias.dim() == 1:
+                if bias.shape[0] != n:
+                    bias = bias.broadcast_to((n,)).contiguous()
+            else:
+                residual = bias if tuple(bias.shape) == (m, n) else bias.broadcast_to((m, n)).contiguous()
+                bias = None
+        return torch.ops.xpu_ops.dense(inputs, weight, weight_trans, bias, residual, act)
+
+
+def can_fuse_custom_denselayer(inputs, weight, weight_trans, bias, act_str):
+    """Match-time veto (arguments are FakeTensors): what the MFMA kernel cannot take stays in Aten."""
+    if act_str not in ("none", "relu", "gelu", "silu", "sigmoid"):
+        return False
+    if inputs.dtype not in _DENSE_DTYPES or weight.dtype != inputs.dtype:
+        return False
+    if inputs.dim() != 2 or weight.dim() != 2:
+        return False
+    if bias is not None and (bias.dtype != inputs.dtype or bias.dim() > 2):
+        return False
+    k = inputs.shape[1]
+    n = weight.shape[0] if weight_trans else weight.shape[1]
+    if not (isinstance(k, int) and isinstance(n, int)):
+        return False
+    return k % 8 == 0 and n % 8 == 0 and k > 0 and n > 0
+
+
+def get_structure_replacements(config):
+    return {
+        "CustomRMSNorm": RMSNormModule,
+        "CustomLayerNorm": LayerNormModule,
+        "FusedCatSlice": FuseSliceCatSameInputModule,
+        "FusedSliceStackSum": FuseSliceCatSameInputModule,
+        "FusedMultipleSliceCat": FuseSliceCatSameInputModule_v2,
+        "ComboSum3dInp": ComboSumModule,
+        "CustomDenseLayer": (DenseLayerModule, can_fuse_custom_denselayer),
+    }
