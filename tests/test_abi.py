@@ -1,0 +1,61 @@
+"""The C-ABI library: it is built, loads, and exports exactly the entry points
+include/xpu_graph_amd.h declares (no compute calls here: no GPU needed)."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "xpu_graph_amd.h")
+
+
+def declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(xg_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_declares_the_expected_entry_points():
+    syms = declared_symbols()
+    for s in ("xg_rms_norm", "xg_layer_norm", "xg_add_rms_norm", "xg_add_layer_norm", "xg_slice_cat", "xg_addn",
+              "xg_combo_sum", "xg_silu_mul", "xg_silu_mul2", "xg_dense", "xg_dense_fp8", "xg_sdpa", "xg_copy_bytes",
+              "xg_version", "xg_status_string"):
+        assert s in syms
+
+
+def test_library_exports_every_declared_symbol():
+    from xpu_graph_amd import _lib
+
+    if not _lib.is_built():
+        pytest.fail(f"{_lib.LIB_PATH} not built: run `python -m xpu_graph_amd.build`")
+    handle = ctypes.CDLL(_lib.LIB_PATH)
+    for name in declared_symbols():
+        assert hasattr(handle, name), f"{name} declared in the header but not exported"
+    assert sorted(_lib.exported_symbols()) == declared_symbols()  # the ctypes table covers the whole header
+
+
+def test_status_strings_and_version():
+    from xpu_graph_amd import _lib
+
+    lib = _lib.lib()
+    assert lib.xg_version() >= 100
+    assert lib.xg_status_string(0) == b"ok"
+    assert b"NULL" in lib.xg_status_string(-4)
+    with pytest.raises(_lib.XgError):
+        _lib.check(-2, "demo")
+
+
+def test_argument_validation_needs_no_gpu():
+    """Host-side checks run before any launch, so they can be exercised without a device."""
+    from xpu_graph_amd import _lib
+
+    lib = _lib.lib()
+    assert lib.xg_rms_norm(None, None, None, 4, 8, 8, 1e-6, 0, 0, None) == -4  # NULL x
+    buf = ctypes.create_string_buffer(1024)
+    p = ctypes.cast(buf, ctypes.c_void_p)
+    assert lib.xg_rms_norm(p, None, p, 4, 8, 4, 1e-6, 0, 0, None) == -2  # stride < cols
+    assert lib.xg_rms_norm(p, None, p, 4, 8, 8, 1e-6, 7, 7, None) == -1  # unknown dtype
+    assert lib.xg_rms_norm(p, None, p, 0, 8, 8, 1e-6, 0, 0, None) == 0  # empty: nothing to launch
+    assert lib.xg_copy_bytes(p, p, 24, None) == -2  # not a multiple of 16
+    assert lib.xg_silu_mul(p, p, 2, 8, 8, 0, None) == -2  # row stride < 2*d

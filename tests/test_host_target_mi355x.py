@@ -1,0 +1,260 @@
+"""Graph rewriting for the mi355x target, checked on the CPU: which patterns
+fire and what the rewritten graph calls.  The rewritten graphs are not run
+here -- on CPU tensors the xpu_ops have no implementation and must raise."""
+import math
+import operator
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from xpu_graph_amd import OptLevel, Target, XpuGraph, XpuGraphConfig, mi355x_compiler
+from xpu_graph_amd.test_utils import need_xpu_graph_logs
+
+bf16 = torch.bfloat16
+
+
+@pytest.fixture()
+def backend():
+    return mi355x_compiler()
+
+
+def rewrite(backend, fn, *args, must_fail=True):
+    """Compile fn for the mi355x target on CPU inputs; returns the rewritten graph."""
+    with need_xpu_graph_logs():
+        c = torch.compile(fn, backend=backend)
+        if must_fail:
+            with pytest.raises(NotImplementedError):  # no CPU fallback behind the custom ops
+                c(*args)
+        else:
+            c(*args)
+    return backend.compiled_graphs[-1]
+
+
+def modules_called(gm):
+    return [n.target for n in gm.graph.nodes if n.op == "call_module"]
+
+
+def aten_ops(gm):
+    return [str(n.target) for n in gm.graph.nodes if n.op == "call_function" and n.target is not operator.getitem]
+
+
+def test_c1_rmsnorm_becomes_one_custom_call(caplog, backend):
+    def fn(x, w):
+        return x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + 1e-6) * w
+
+    gm = rewrite(backend, fn, torch.randn(8, 64), torch.randn(64))
+    assert modules_called(gm) == ["custom_rms_norm"] and aten_ops(gm) == []
+    assert "Pattern.CustomRMSNorm changed graph" in caplog.text
+
+
+def test_unweighted_rmsnorm_stays_default(caplog, backend):
+    def fn(x):
+        return x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + 1e-6)
+
+    gm = rewrite(backend, fn, torch.randn(8, 64), must_fail=False)
+    assert modules_called(gm) == ["fused_rms_norm"]  # CustomRMSNorm needs a weight
+
+
+@pytest.mark.parametrize("form", ["library", "decomposed"])
+def test_c2_add_layernorm_two_outputs(caplog, backend, form):
+    def library(x, r, g, b):
+        h = x + r
+        return F.layer_norm(h, (h.shape[-1],), g, b, 1e-5), h
+
+    def decomposed(x, r, g, b):
+        h = x + r
+        hf = h.float()
+        n = ((hf - hf.mean(-1, keepdim=True)) * torch.rsqrt(hf.var(-1, unbiased=False, keepdim=True) + 1e-5)).to(h.dtype)
+        return n * g + b, h
+
+    args = (torch.randn(8, 64).to(bf16), torch.randn(8, 64).to(bf16), torch.randn(64).to(bf16), torch.randn(64).to(bf16))
+    gm = rewrite(backend, {"library": library, "decomposed": decomposed}[form], *args)
+    assert modules_called(gm) == ["mi355x_fused_add_norm"] and aten_ops(gm) == []
+    node = next(n for n in gm.graph.nodes if n.op == "call_module")
+    assert node.args[6] is True and node.args[7] == "layer_norm" and node.args[5] == 1e-5
+    assert "Pattern.FusedAddLayerNorm changed graph" in caplog.text
+
+
+def test_add_rmsnorm_single_output_when_sum_is_private(caplog, backend):
+    def fn(x, r, w):
+        h = (x + r).float()
+        return (h * torch.rsqrt(h.pow(2).mean(-1, keepdim=True) + 1e-6)).to(x.dtype) * w
+
+    args = (torch.randn(4, 32).to(bf16), torch.randn(4, 32).to(bf16), torch.randn(32).to(bf16))
+    gm = rewrite(backend, fn, *args)
+    assert modules_called(gm) == ["mi355x_fused_add_norm"]
+    node = next(n for n in gm.graph.nodes if n.op == "call_module")
+    assert node.args[6] is False and node.args[7] == "rms_norm"
+    assert "Pattern.FusedAddRMSNorm changed graph" in caplog.text
+
+
+def test_add_norm_sum_used_before_norm_keeps_topological_order(backend):
+    def fn(x, r, g, b):
+        h = x + r
+        side = h * 2  # a user of the sum that precedes the norm in graph order
+        return F.layer_norm(h, (h.shape[-1],), g, b, 1e-5), side
+
+    args = (torch.randn(4, 32), torch.randn(4, 32), torch.randn(32), torch.randn(32))
+    gm = rewrite(backend, fn, *args)
+    gm.graph.lint()
+    assert modules_called(gm) == ["mi355x_fused_add_norm"]
+
+
+def test_c3_slice_cat_and_addn(caplog, backend):
+    offs = [7, 100, 40, 200]
+
+    def fn(src, *ts):
+        cat = torch.cat([src[:, o : o + 8] for o in offs], dim=1)
+        acc = ts[0]
+        for t in ts[1:]:
+            acc = acc + t
+        return cat, acc
+
+    ts = [torch.randn(6, 16) for _ in range(6)]
+    gm = rewrite(backend, fn, torch.randn(6, 256), *ts)
+    assert sorted(modules_called(gm)) == ["fuse_slice_cat", "mi355x_addn"]
+    assert "aten.slice.Tensor" not in aten_ops(gm) and "aten.stack.default" not in aten_ops(gm)
+    node = next(n for n in gm.graph.nodes if n.target == "fuse_slice_cat")
+    assert node.args[1] == [(o, o + 8) for o in offs]
+    for p in ("FusedCatSlice", "FusedAddN", "FusedStackSumToAddN", "FoldCat"):
+        assert f"Pattern.{p} changed graph" in caplog.text, p
+
+
+def test_slice_cat_mixed_inputs_int64max_and_negative_end(backend):
+    def fn(src, other):
+        return torch.cat([other, src[:, 3:9], src[:, 20:], src[:, 10:-200], other], dim=-1)
+
+    gm = rewrite(backend, fn, torch.randn(4, 256), torch.randn(4, 5))
+    node = next(n for n in gm.graph.nodes if n.target == "fuse_slice_cat")
+    assert node.args[1] == [(3, 9), (20, 256), (10, 56)]
+    cat = next(n for n in gm.graph.nodes if n.op == "call_function" and "cat" in str(n.target))
+    assert len(cat.args[0]) == 3
+
+
+def test_slice_cat_not_fused_along_rows_or_3d(caplog, backend):
+    def rows(src):
+        return torch.cat([src[0:2], src[4:6]], dim=0)
+
+    def cube(src):
+        return torch.cat([src[:, :, 0:2], src[:, :, 4:6]], dim=2)
+
+    rewrite(backend, rows, torch.randn(8, 8), must_fail=False)
+    rewrite(backend, cube, torch.randn(2, 8, 8), must_fail=False)
+    assert "Pattern.FusedCatSlice changed graph" not in caplog.text
+
+
+def test_multiple_slice_cats_share_one_multi_output_module(caplog, backend):
+    def fn(src):
+        a = torch.cat([src[:, 0:4], src[:, 8:12]], dim=1)
+        b = torch.cat([src[:, 16:20], src[:, 4:8], src[:, 30:32]], dim=1)
+        return a, b
+
+    gm = rewrite(backend, fn, torch.randn(4, 64))
+    mods = modules_called(gm)
+    assert len(mods) == 1 and mods[0].startswith("fuse_slice_cat_v2")
+    assert "Pattern.FusedMultipleSliceCat changed graph" in caplog.text
+    sub = gm.get_submodule(mods[0])
+    assert sub.many_slices == [[(0, 4), (8, 12)], [(16, 20), (4, 8), (30, 32)]]
+
+
+def test_slice_stack_sum_and_combo_sum(caplog, backend):
+    def fn(src):
+        a = torch.stack([src[:, 0:8], src[:, 8:16], src[:, 32:40]], dim=0).sum(dim=0)
+        b = torch.stack([src[:, 40:48], src[:, 16:24]], dim=0).sum(dim=0)
+        return a, b
+
+    gm = rewrite(backend, fn, torch.randn(4, 64))
+    assert "Pattern.FusedSliceStackSum changed graph" in caplog.text
+    assert "Pattern.ComboSum3dInp changed graph" in caplog.text
+    assert "combo_sum" in modules_called(gm)
+
+
+@pytest.mark.parametrize("form", ["mm_add", "linear", "nobias", "relu"])
+def test_c4_dense(caplog, backend, form):
+    x = torch.randn(16, 64).to(bf16)
+    if form == "mm_add":
+        fn, args = (lambda x, w, b: F.silu(x @ w + b)), (x, torch.randn(64, 32).to(bf16), torch.randn(32).to(bf16))
+    elif form == "linear":
+        fn, args = (lambda x, w, b: F.silu(F.linear(x, w, b))), (x, torch.randn(32, 64).to(bf16), torch.randn(32).to(bf16))
+    elif form == "nobias":
+        fn, args = (lambda x, w: x @ w), (x, torch.randn(64, 32).to(bf16))
+    else:
+        fn, args = (lambda x, w, b: F.relu(torch.addmm(b, x, w))), (x, torch.randn(64, 32).to(bf16), torch.randn(16, 32).to(bf16))
+    gm = rewrite(backend, fn, *args)
+    assert modules_called(gm) == ["custom_dense_layer_replacement"]
+    node = next(n for n in gm.graph.nodes if n.op == "call_module")
+    assert node.args[2] is (form == "linear")
+    assert node.args[4] == {"mm_add": "silu", "linear": "silu", "nobias": "none", "relu": "relu"}[form]
+    assert "Pattern.CustomDenseLayer changed graph" in caplog.text
+
+
+def test_dense_constraint_vetoes_fp32_and_odd_sizes(caplog, backend):
+    rewrite(backend, lambda x, w: x @ w, torch.randn(8, 16), torch.randn(16, 8), must_fail=False)  # fp32 stays Aten
+    rewrite(backend, lambda x, w: x @ w, torch.randn(8, 12).to(bf16), torch.randn(12, 8).to(bf16), must_fail=False)
+    assert "Pattern.CustomDenseLayer changed graph" not in caplog.text
+
+
+def test_swiglu_both_forms(caplog, backend):
+    def halves(x):
+        d = x.shape[-1] // 2
+        return F.silu(x[..., :d]) * x[..., d:]
+
+    def pair(a, b):
+        return F.silu(a) * b
+
+    gm = rewrite(backend, halves, torch.randn(4, 64).to(bf16))
+    assert modules_called(gm) == ["mi355x_silu_mul"]
+    gm = rewrite(backend, pair, torch.randn(4, 32).to(bf16), torch.randn(4, 32).to(bf16))
+    assert modules_called(gm) == ["mi355x_silu_mul2"]
+    assert "Pattern.FusedSwiGLU changed graph" in caplog.text
+
+
+def _eager_causal_attention(q, k, v):
+    S, D = q.shape[-2], q.shape[-1]
+    w = torch.matmul(q, k.transpose(2, 3)) / math.sqrt(D)
+    w = w + torch.full((S, S), float("-inf"), dtype=q.dtype).triu(1)
+    w = torch.softmax(w, dim=-1, dtype=torch.float32).to(q.dtype)
+    return torch.matmul(w, v)
+
+
+def test_c5_causal_attention_recognised(caplog, backend):
+    q, k, v = (torch.randn(2, 4, 32, 64).to(bf16) for _ in range(3))
+    gm = rewrite(backend, _eager_causal_attention, q, k, v)
+    assert "Pattern.FusedSDPA changed graph" in caplog.text
+    assert "Pattern.FusedCausalSDPA changed graph" in caplog.text
+    node = next(n for n in gm.graph.nodes if n.target == "mi355x_sdpa")
+    assert node.args[3] is True and abs(node.args[4] - 1 / 8) < 1e-12
+    # q, k, v reach the kernel as the caller's 4-D tensors: no clones, no mask, no softmax left
+    assert all(a.op == "placeholder" for a in node.args[:3])
+    assert not any(s in " ".join(aten_ops(gm)) for s in ("softmax", "full", "triu", "clone", "bmm"))
+
+
+def test_library_sdpa_is_causal_flag(caplog, backend):
+    q, k, v = (torch.randn(2, 4, 32, 64).to(bf16) for _ in range(3))
+    gm = rewrite(backend, lambda q, k, v: F.scaled_dot_product_attention(q, k, v, is_causal=True), q, k, v)
+    node = next(n for n in gm.graph.nodes if n.target == "mi355x_sdpa")
+    assert node.args[3] is True
+
+
+def test_arbitrary_mask_is_not_taken(caplog, backend):
+    def fn(q, k, v, m):
+        w = torch.matmul(q, k.transpose(2, 3)) / 8.0 + m
+        return torch.matmul(torch.softmax(w, dim=-1), v)
+
+    q, k, v = (torch.randn(2, 4, 32, 64).to(bf16) for _ in range(3))
+    gm = rewrite(backend, fn, q, k, v, torch.randn(32, 32).to(bf16), must_fail=False)
+    assert "mi355x_sdpa" not in modules_called(gm)
+    assert "aten.scaled_dot_product_attention.default" in aten_ops(gm)
+
+
+def test_target_none_has_no_structure_patterns(caplog):
+    be = XpuGraph(XpuGraphConfig(is_training=False, opt_level=OptLevel.level2, target=Target.none))
+    names = [str(p) for ps in be.get_pattern_manager()._patterns.values() for p in ps]
+    assert "CustomRMSNorm" not in names and "FusedCatSlice" not in names and "FusedSwiGLU" not in names
+    be2 = mi355x_compiler()
+    names2 = [str(p) for ps in be2.get_pattern_manager()._patterns.values() for p in ps]
+    for want in ("CustomRMSNorm", "CustomLayerNorm", "FusedCatSlice", "FusedMultipleSliceCat", "FusedSliceStackSum",
+                 "ComboSum3dInp", "CustomDenseLayer", "FusedAddLayerNorm", "FusedAddRMSNorm", "FusedSwiGLU",
+                 "FusedStackSumToAddN", "FusedCausalSDPA", "NativeNormToDefault"):
+        assert want in names2, want

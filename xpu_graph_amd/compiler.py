@@ -59,6 +59,7 @@ class XpuGraph:
         setup_logger(config.debug)
         self._cache = None  # compile-artifact caching is not part of this build
         self._orig_ctx = {}
+        self.compiled_graphs = []  # the last few rewritten GraphModules, newest last (inspection / tests)
         self._set_context()
         self._pass_manager = PassManager(config)
         # plugin patterns run before the built-in ones of their group
@@ -82,6 +83,8 @@ class XpuGraph:
                     logger.info(f"node statistic: before {before} after {_node_census(out)}")
                     if self._config.vendor_compiler_config is not None:
                         logger.warning("vendor_compiler_config is ignored: this backend runs the rewritten graph directly")
+                self.compiled_graphs.append(out)
+                del self.compiled_graphs[:-8]
                 # AOT's runtime wrappers call the compiled stage with one list of arguments
                 return make_boxed_func(out)
 

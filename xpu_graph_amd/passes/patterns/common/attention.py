@@ -86,7 +86,7 @@ def match_attention(node):
                 return None
             if is_constant(scale):
                 scale = _const_value(scale)
-        cur = arg(cur, 0)
+        cur = skip_layout_ops(arg(cur, 0))
 
     if is_call(cur, aten.bmm.default):
         q, k = arg(cur, 0), arg(cur, 1)

@@ -107,7 +107,7 @@ _recorder = []
 
 def _as_match_filter(check):
     def match_filter(match, gm, pattern_graph):
-        ok = check(*[p.meta["val"] for p in match.placeholder_nodes])
+        ok = check(*[p.meta["val"] if isinstance(p, fx.Node) else p for p in match.placeholder_nodes])  # literals bind as values
         assert isinstance(ok, bool)
         return ok
 

@@ -88,14 +88,23 @@ def is_causal_constant(mask, sq, skv):
         return bool((m[~upper] == 0).all()) and bool(((masked == float("-inf")) | (masked <= lowest)).all())
 
 
+def _same_attention_problem(src, dims):
+    """src is 4-D [B', H', S, D] with B'*H' == B*H and the same S, D: every (batch, head) pair is an
+    independent attention problem, so how the leading two axes are split does not matter."""
+    if not (isinstance(src, fx.Node) and "val" in src.meta and isinstance(src.meta["val"], torch.Tensor)):
+        return False
+    shp = list(src.meta["val"].shape)
+    if len(shp) != 4 or not all(isinstance(d, int) for d in shp + list(dims)):
+        return False
+    return shp[2:] == list(dims[2:]) and shp[0] * shp[1] == dims[0] * dims[1]
+
+
 def _peel_qv(node, dims):
-    """reshape(clone(reshape(x4d, [BH,S,D])), [B,H,S,D]) -> x4d when x4d already has that 4-D shape."""
+    """reshape(clone(reshape(x4d, [BH,S,D])), [B,H,S,D]) -> x4d."""
     if is_call(node, *VIEW_OPS) and is_call(node.args[0], aten.clone.default):
         inner = node.args[0].args[0]
-        if is_call(inner, *VIEW_OPS):
-            src = inner.args[0]
-            if isinstance(src, fx.Node) and "val" in src.meta and same_shape(list(src.meta["val"].shape), list(dims)):
-                return src
+        if is_call(inner, *VIEW_OPS) and _same_attention_problem(inner.args[0], dims):
+            return inner.args[0]
     return node
 
 
@@ -113,9 +122,7 @@ def _peel_k(node, dims):
     if not is_call(t0, aten.transpose.int) or {t0.args[1], t0.args[2]} not in ({-1, -2}, {2, 3}):
         return node
     src = t0.args[0]
-    if isinstance(src, fx.Node) and "val" in src.meta and same_shape(list(src.meta["val"].shape), list(dims)):
-        return src
-    return node
+    return src if _same_attention_problem(src, dims) else node
 
 
 def _supported(q, k, v):
@@ -181,7 +188,19 @@ class FusedCausalSDPA(Pattern):
                 q2 = _peel_qv(q, q.meta["val"].shape)
                 k2 = _peel_k(k, k.meta["val"].shape)
                 v2 = _peel_qv(v, v.meta["val"].shape)
-                changed |= self._emit(gm, node, q2, k2, v2, causal, scale, node.replace_all_uses_with)
+                lead = {tuple(n.meta["val"].shape[:2]) for n in (q2, k2, v2)}
+                peeled = q2 is not q and k2 is not k and v2 is not v and len(lead) == 1
+                if not peeled:
+                    q2, k2, v2 = q, k, v
+                out_shape = tuple(node.meta["val"].shape)
+
+                def replace(new, old=node, reshape_back=peeled and tuple(q2.meta["val"].shape) != out_shape, shp=out_shape):
+                    if reshape_back:
+                        with gm.graph.inserting_after(new):
+                            new = gm.graph.call_function(aten.reshape.default, (new, shp))
+                    old.replace_all_uses_with(new)
+
+                changed |= self._emit(gm, node, q2, k2, v2, causal, scale, replace)
             elif node.op == "call_function" and node.target in backend_ops:
                 drop_idx, causal_idx, bias_idx = backend_ops[node.target]
                 users = list(node.users)
