@@ -1,0 +1,101 @@
+"""GPU parity of the MFMA dense layer (torch.ops.xpu_ops.dense -> xg_dense)
+against the eager oracle: bf16 / fp16, weight as [K, N] and as [N, K],
+bias / residual / activation variants, ragged edges.  Tolerance rtol 1.6e-2
+against the fp32-computed reference of the same bf16 inputs (atol scaled to the
+accumulation length)."""
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import eager, inputs
+
+pytestmark = pytest.mark.gpu
+
+
+def _ops():
+    import xpu_graph_amd.ops  # noqa: F401
+
+    return torch.ops.xpu_ops
+
+
+def ref32(x, W, weight_trans, bias, residual, act):
+    y = x.float() @ (W.float().t() if weight_trans else W.float())
+    if bias is not None:
+        y = y + bias.float()
+    if residual is not None:
+        y = y + residual.float()
+    return {"none": lambda t: t, "relu": F.relu, "gelu": F.gelu, "silu": F.silu, "sigmoid": torch.sigmoid}[act](y)
+
+
+def close(got, want, k):
+    torch.testing.assert_close(got.float(), want, rtol=1.6e-2, atol=2e-3 * max(1.0, (k / 64) ** 0.5))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("weight_trans", [False, True])
+@pytest.mark.parametrize("M,N,K", [(256, 256, 64), (512, 768, 256), (300, 264, 200), (1, 8, 8), (1000, 1032, 72), (64, 4096, 4096)])
+def test_dense_shapes(device, dtype, weight_trans, M, N, K):
+    g = torch.Generator().manual_seed(M + N + K)
+    x = torch.randn(M, K, generator=g).to(dtype).to(device)
+    W = (torch.randn(N, K, generator=g) / K**0.5).to(dtype).to(device)
+    if not weight_trans:
+        W = W.t().contiguous()
+    b = torch.randn(N, generator=g).to(dtype).to(device)
+    got = _ops().dense(x, W, weight_trans, b, None, "silu")
+    assert got.shape == (M, N) and got.dtype == dtype
+    close(got, ref32(x, W, weight_trans, b, None, "silu"), K)
+    got = _ops().dense(x, W, weight_trans, None, None, "none")
+    close(got, ref32(x, W, weight_trans, None, None, "none"), K)
+
+
+@pytest.mark.parametrize("act", ["none", "relu", "gelu", "silu", "sigmoid"])
+def test_dense_bias_residual_activation(device, act):
+    M, N, K = 320, 520, 136
+    g = torch.Generator().manual_seed(7)
+    x = torch.randn(M, K, generator=g).bfloat16().to(device)
+    W = (0.1 * torch.randn(K, N, generator=g)).bfloat16().to(device)
+    b32 = torch.randn(N, generator=g).to(device)
+    res = torch.randn(M, N, generator=g).bfloat16().to(device)
+    got = _ops().dense(x, W, False, b32, res, act)  # fp32 bias + residual
+    close(got, ref32(x, W, False, b32, res, act), K)
+    got = _ops().dense(x, W, False, None, res, act)
+    close(got, ref32(x, W, False, None, res, act), K)
+
+
+def test_dense_identity_and_strided_views(device):
+    x = torch.randn(256, 128, device=device).bfloat16()
+    eye = torch.eye(128, device=device).bfloat16()
+    assert torch.equal(_ops().dense(x, eye, False, None, None, "none"), x)  # W = I is exact
+    assert torch.equal(_ops().dense(x, eye, True, None, None, "none"), x)
+    big = torch.randn(256, 512, device=device).bfloat16()
+    xv = big[:, 128:256]  # row stride 512
+    Wv = torch.randn(128, 512, device=device).bfloat16()[:, 64:192]
+    close(_ops().dense(xv, Wv, False, None, None, "none"), ref32(xv, Wv, False, None, None, "none"), 128)
+    xt = torch.randn(128, 256, device=device).bfloat16().t()  # column stride != 1: copied by the op
+    close(_ops().dense(xt, eye, False, None, None, "relu"), F.relu(xt.float()), 128)
+
+
+def test_dense_c4_full_size(device):
+    x, W, b = inputs.c4_dense(device=device)
+    got = _ops().dense(x, W, False, b, None, "silu")
+    want = eager.dense_silu_eager(x, W, b)  # the unfused bf16 graph on the same device
+    torch.testing.assert_close(got, want, rtol=1.6e-2, atol=2e-2)
+    rows = torch.tensor([0, 1, 4095, 8191], device=device)
+    close(got[rows], ref32(x[rows], W, False, b, None, "silu"), 4096)
+    Wt = W.t().contiguous()
+    got_t = _ops().dense(x, Wt, True, b, None, "silu")
+    assert torch.equal(got_t, got)  # both weight layouts run the same arithmetic in the same order
+
+
+def test_dense_rejects_what_the_kernel_cannot_take(device):
+    from xpu_graph_amd._lib import XgError
+
+    x = torch.randn(8, 12, device=device).bfloat16()
+    W = torch.randn(12, 8, device=device).bfloat16()
+    with pytest.raises(XgError):
+        _ops().dense(x, W, False, None, None, "none")  # K % 8 != 0
+    with pytest.raises(ValueError):
+        _ops().dense(x, torch.randn(16, 8, device=device).bfloat16(), False, None, None, "none")
+    with pytest.raises(ValueError):
+        _ops().dense(x, W, False, None, None, "tanh")
+    assert _ops().dense(torch.empty(0, 16, device=device).bfloat16(), torch.randn(16, 8, device=device).bfloat16(), False, None, None, "none").shape == (0, 8)
