@@ -56,6 +56,9 @@ def build_library(verbose=True, jobs=None):
     """Compile every kernel source for gfx950 and link the C-ABI shared library."""
     os.makedirs(OBJ_DIR, exist_ok=True)
     srcs = sources()
+    wanted = {os.path.basename(s)[:-4] + ".o" for s in srcs}
+    for stale in set(os.listdir(OBJ_DIR)) - wanted:
+        os.remove(os.path.join(OBJ_DIR, stale))
     jobs = jobs or min(len(srcs), max(1, (os.cpu_count() or 2) - 1), 8)
     if verbose:
         print(f"[xpu_graph_amd.build] hipcc {ARCH}: {len(srcs)} sources, {jobs} jobs", flush=True)

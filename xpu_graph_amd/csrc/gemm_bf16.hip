@@ -1,0 +1,38 @@
+// bf16 instantiation of the dense-layer kernels and the xg_dense entry point.
+#include "gemm_impl.hpp"
+
+namespace xg {
+namespace gemm {
+int launch_f16(const GemmParams& p, bool b_trans, hipStream_t st);  // gemm_f16.hip
+int launch_bf16(const GemmParams& p, bool b_trans, hipStream_t st) {
+  return b_trans ? launch_gemm<bf16_t, bf16_t, BLayout::KMajor>(p, st) : launch_gemm<bf16_t, bf16_t, BLayout::NMajor>(p, st);
+}
+}  // namespace gemm
+}  // namespace xg
+
+extern "C" {
+
+int xg_dense(const void* a, const void* b, const void* bias, const void* residual, void* out, int64_t M, int64_t N,
+             int64_t K, int64_t lda, int64_t ldb, int64_t ldr, int b_trans, int act, int dtype, int bias_dtype,
+             xg_stream_t stream) {
+  using namespace xg;
+  using namespace xg::gemm;
+  if (a == nullptr || b == nullptr || out == nullptr) return XG_ERR_NULL_PTR;
+  if (M < 0 || N <= 0 || K <= 0 || lda < K || (b_trans ? ldb < K : ldb < N) || (residual && ldr < N)) return XG_ERR_BAD_SHAPE;
+  if (M > 0x7fffffff || N > 0x7fffffff || K > 0x7fffffff) return XG_ERR_TOO_LARGE;
+  if (dtype != XG_BF16 && dtype != XG_F16) return XG_ERR_BAD_DTYPE;
+  if (bias && bias_dtype != dtype && bias_dtype != XG_F32) return XG_ERR_BAD_DTYPE;
+  if (act < XG_ACT_NONE || act > XG_ACT_SIGMOID) return XG_ERR_BAD_ARG;
+  // 16-byte operand loads and 16-byte output stores
+  if (K % 8 != 0 || N % 8 != 0 || lda % 8 != 0 || ldb % 8 != 0 || (residual && ldr % 8 != 0)) return XG_ERR_BAD_ALIGN;
+  if (!aligned_to(a, 16) || !aligned_to(b, 16) || !aligned_to(out, 16) || (bias && !aligned_to(bias, 16)) ||
+      (residual && !aligned_to(residual, 16)))
+    return XG_ERR_BAD_ALIGN;
+  if (M == 0) return XG_OK;
+  const GemmParams p = make_params(a, b, bias, residual, out, M, N, K, lda, ldb, ldr, act, bias && bias_dtype == XG_F32);
+  hipStream_t st = (hipStream_t)stream;
+  return dtype == XG_BF16 ? gemm::launch_bf16(p, b_trans != 0, st) : gemm::launch_f16(p, b_trans != 0, st);
+}
+
+
+}  // extern "C"

@@ -1,0 +1,620 @@
+// Shared implementation of the dense-layer kernels (included by gemm_bf16.hip, gemm_f16.hip and
+// gemm_fp8.hip, one translation unit per operand type so that they compile in parallel).
+//
+// Dense layer for gfx950: out = act(A @ B(+T) * scales + bias + residual) on the
+// matrix cores.
+//
+// Tiling: one 256-thread workgroup (4 wavefronts, 2 x 2) owns a 256 x 256 output
+// tile; each wavefront owns 128 x 128 of it as 4 x 4 MFMA tiles of 32 x 32, i.e.
+// 256 fp32 accumulators per lane -- the whole accumulator file at one wavefront
+// per SIMD.  K advances in slabs of 128 BYTES per row (64 bf16/f16 or 128 fp8
+// elements), double-buffered in 128 KiB of LDS.
+//
+// Two kernels share everything but the way a slab reaches LDS:
+//  * gemm_dma_kernel (K a multiple of the slab): `global_load_lds_dwordx4` moves
+//    memory straight into LDS, 1 KiB per wavefront instruction.  The loads of
+//    slab t+1 are issued a few at a time BETWEEN the MFMAs of slab t, as are the
+//    LDS fragment reads of the next k-step, so the matrix pipe never waits for
+//    the wavefront to finish issuing memory instructions.
+//  * gemm_staged_kernel (any K % 8 == 0): slabs pass through registers, which
+//    lets the last, partial slab be zero-filled.
+//
+// LDS layout (K-contiguous operands): row r of a slab is 128 bytes = 8 chunks of
+// 16 bytes; chunk c is stored at c ^ (r & 7) ^ ((r >> 3) & 1), which makes the
+// 16-byte fragment reads of 16 consecutive rows and the row-wise writes conflict
+// free.  Direct-to-LDS loads write 64 lanes x 16 bytes consecutively, so there
+// the permutation is applied on the global side: the lane that lands on
+// physical chunk pc of row r fetches logical chunk pc ^ swz(r).  A [K, N]
+// (N-contiguous) B operand is kept [k][n] in LDS and read with the transposing
+// LDS load of gfx950 (ds_read_b64_tr_b16), so no transpose pass is needed.
+//
+// The MFMA is issued with B's fragment as the first operand, so each lane ends
+// up with 4 CONSECUTIVE output columns of one row, which makes the accumulators
+// cheap to park in LDS; the epilogue (scales, bias, residual, activation,
+// rounding) then runs as a short rolled loop over row-major data and stores
+// 16 bytes per lane, whole 128-byte lines per row.
+//
+// Workgroups are dealt to the 8 XCDs round-robin by the hardware; the block id
+// is remapped so that each XCD works through one contiguous, grouped run of
+// tiles and its L2 sees each operand slab a few times instead of once per CU.
+#pragma once
+#include "xg_common.hpp"
+
+#include <stdlib.h>
+
+#include <type_traits>
+#include <utility>
+
+namespace xg {
+namespace gemm {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef int i32x8 __attribute__((ext_vector_type(8)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(1))) void gvoid;
+typedef __attribute__((address_space(3))) void lvoid;
+typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+
+constexpr int BM = 256, BN = 256;
+constexpr int ROW_BYTES = 128;               // bytes of K per tile row and slab
+constexpr int SLAB_BYTES = BM * ROW_BYTES;   // 32 KiB per operand per stage
+constexpr int STAGE_BYTES = 2 * SLAB_BYTES;  // A slab, then B slab
+constexpr int SMEM_BYTES = 2 * STAGE_BYTES;
+constexpr int kThreads = 256;
+constexpr int kXcds = 8;
+constexpr int kGroupM = 8;
+#ifndef XG_GEMM_LOAD_STEPS
+#define XG_GEMM_LOAD_STEPS 1
+#endif
+
+enum class BLayout { KMajor, NMajor };  // B stored [N, K] (K contiguous) or [K, N] (N contiguous)
+
+struct GemmParams {
+  const void* A;
+  const void* B;
+  const void* bias;
+  const void* res;
+  void* out;
+  const float* a_scale;  // fp8 only
+  const float* b_scale;  // fp8 only
+  int M, N, K;
+  int64_t lda, ldb, ldr;
+  int act;
+  int bias_f32;
+  int tiles_m, tiles_n;
+};
+
+// Compile-time loop: the body receives std::integral_constant indices, so every
+// accumulator access has a constant index and the accumulators stay in registers.
+template <typename F, int... I>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, I...>) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+  static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
+
+template <typename T>
+struct Elem;
+template <>
+struct Elem<bf16_t> {
+  static constexpr int BYTES = 2;
+  static constexpr int KSTEPS = 4;  // 4 x (32x32x16) per 64-element slab
+};
+template <>
+struct Elem<f16_t> {
+  static constexpr int BYTES = 2;
+  static constexpr int KSTEPS = 4;
+};
+template <>
+struct Elem<uint8_t> {  // OCP e4m3
+  static constexpr int BYTES = 1;
+  static constexpr int KSTEPS = 2;  // 2 x (32x32x64) per 128-element slab
+};
+
+// One k-step's operand fragment of a 32-row MFMA tile: 16 bytes per lane for the
+// 16-bit types, 32 bytes per lane for fp8.
+template <typename T>
+struct Frag {
+  u32x4 v;
+};
+template <>
+struct Frag<uint8_t> {
+  u32x4 lo, hi;
+};
+
+__device__ __forceinline__ f32x16 mma(const Frag<bf16_t>& a, const Frag<bf16_t>& b, f32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a.v), __builtin_bit_cast(bf16x8, b.v), c, 0, 0, 0);
+}
+__device__ __forceinline__ f32x16 mma(const Frag<f16_t>& a, const Frag<f16_t>& b, f32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a.v), __builtin_bit_cast(f16x8, b.v), c, 0, 0, 0);
+}
+__device__ __forceinline__ f32x16 mma(const Frag<uint8_t>& a, const Frag<uint8_t>& b, f32x16 c) {
+  const i32x8 x = {(int)a.lo.x, (int)a.lo.y, (int)a.lo.z, (int)a.lo.w, (int)a.hi.x, (int)a.hi.y, (int)a.hi.z, (int)a.hi.w};
+  const i32x8 y = {(int)b.lo.x, (int)b.lo.y, (int)b.lo.z, (int)b.lo.w, (int)b.hi.x, (int)b.hi.y, (int)b.hi.z, (int)b.hi.w};
+  // format 0 = e4m3 for both operands; scale exponents 127 = 2^0
+  return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(x, y, c, 0, 0, 0, 127, 0, 127);
+}
+
+__device__ __forceinline__ int swz(int row) { return (row & 7) ^ ((row >> 3) & 1); }
+
+// XCD-aware, grouped tile order.
+__device__ __forceinline__ void tile_of_block(const GemmParams& p, int& tm, int& tn) {
+  const int nb = gridDim.x;
+  const int bid = blockIdx.x;
+  const int xcd = bid % kXcds, local = bid / kXcds;
+  const int base = nb / kXcds, extra = nb % kXcds;
+  const int tile = xcd * base + (xcd < extra ? xcd : extra) + local;
+  const int per_group = kGroupM * p.tiles_n;
+  const int group = tile / per_group;
+  const int first_m = group * kGroupM;
+  const int gsz = (p.tiles_m - first_m) < kGroupM ? (p.tiles_m - first_m) : kGroupM;
+  const int in_group = tile % per_group;
+  tm = first_m + in_group % gsz;
+  tn = in_group / gsz;
+}
+
+// Lane coordinates shared by the fragment reads and the epilogue.
+struct Lane {
+  int tid, lane, wave, wm, wn, l32, half, p16, blk;
+  int fsw;    // swz() of this lane's fragment row
+  int tr_sw;  // granule permutation of the transposing read
+  int a_row[4], b_row[4];
+  __device__ __forceinline__ Lane() {
+    tid = threadIdx.x;
+    lane = tid & 63;
+    wave = tid >> 6;
+    wm = wave >> 1;
+    wn = wave & 1;
+    l32 = lane & 31;
+    half = lane >> 5;
+    p16 = lane & 15;
+    blk = (lane >> 4) & 1;
+    fsw = swz(l32);
+    tr_sw = (p16 >> 2) | (half << 2);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      a_row[i] = (wm * 128 + i * 32 + l32) * ROW_BYTES;
+      b_row[i] = (wn * 128 + i * 32 + l32) * ROW_BYTES;
+    }
+  }
+};
+
+// Fragments of k-step ks from the slabs at a_s / b_s.
+template <typename T, BLayout BL>
+__device__ __forceinline__ void read_frags(const Lane& L, const char* a_s, const char* b_s, int ks, Frag<T> (&fa)[4],
+                                           Frag<T> (&fb)[4]) {
+  if constexpr (Elem<T>::BYTES == 2) {
+    const int ch = ((ks * 2 + L.half) ^ L.fsw) << 4;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) fa[i].v = *reinterpret_cast<const u32x4*>(a_s + L.a_row[i] + ch);
+    if constexpr (BL == BLayout::KMajor) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) fb[j].v = *reinterpret_cast<const u32x4*>(b_s + L.b_row[j] + ch);
+    } else {
+      // slab is [64 k][256 n]: a 16-lane group reads a 4(k) x 16(n) block and gets it back transposed
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int gran = ((L.wn * 4 + j) ^ L.tr_sw) & 7;
+        const int col = (gran << 6) + (L.blk << 5) + ((L.p16 & 3) << 3);
+        const int row0 = ks * 16 + L.half * 8 + (L.p16 >> 2);
+        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(b_s + row0 * (BN * 2) + col));
+        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(b_s + (row0 + 4) * (BN * 2) + col));
+        const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
+        fb[j].v = u32x4{l2.x, l2.y, h2.x, h2.y};
+      }
+    }
+  } else {
+    // fp8: a k-step is 64 elements; each lane half supplies 32 consecutive bytes (2 chunks)
+    const int ch0 = ((ks * 4 + L.half * 2) ^ L.fsw) << 4, ch1 = ((ks * 4 + L.half * 2 + 1) ^ L.fsw) << 4;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      fa[i].lo = *reinterpret_cast<const u32x4*>(a_s + L.a_row[i] + ch0);
+      fa[i].hi = *reinterpret_cast<const u32x4*>(a_s + L.a_row[i] + ch1);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      fb[j].lo = *reinterpret_cast<const u32x4*>(b_s + L.b_row[j] + ch0);
+      fb[j].hi = *reinterpret_cast<const u32x4*>(b_s + L.b_row[j] + ch1);
+    }
+  }
+}
+
+template <typename T>
+__device__ __forceinline__ void mma_step(f32x16 (&acc)[4][4], const Frag<T> (&fa)[4], const Frag<T> (&fb)[4]) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = mma(fb[j], fa[i], acc[i][j]);
+}
+
+// ---- epilogue -------------------------------------------------------------------------
+// Runs per wavefront, in two halves of 64 output columns, through the wavefront's own 32 KiB of
+// LDS (the slabs are dead by then):
+//   1. park the raw fp32 accumulators of the half (16-byte stores, constant register indices);
+//   2. a ROLLED loop re-reads them row-major -- 8 lanes x 8 columns cover a 64-column row
+//      segment, 8 rows per pass -- applies scale, bias, residual and activation, rounds, and
+//      writes 16 bytes per lane (one full 128-byte line per row).
+// All the arithmetic therefore exists once, in a loop a few dozen instructions long, instead of
+// 256 unrolled copies; the per-lane bias and scale values are loop invariant.
+template <typename OT, int ACT>
+__device__ __forceinline__ void epilogue_rows(const GemmParams& p, const char* park, int lane, int m_base, int n, bool n_ok,
+                                              const float (&sv)[8], const float (&bv)[8]) {
+  typedef OT O8 __attribute__((ext_vector_type(8)));
+  const int c = lane & 7, rr = lane >> 3;
+  for (int it = 0; it < 16; ++it) {
+    const int row = it * 8 + rr;
+    const int m = m_base + row;
+    const f32x4 lo = *reinterpret_cast<const f32x4*>(park + row * 256 + (((2 * c) ^ (row & 15)) << 4));
+    const f32x4 hi = *reinterpret_cast<const f32x4*>(park + row * 256 + (((2 * c + 1) ^ (row & 15)) << 4));
+    if (!(n_ok && m < p.M)) continue;
+    float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = v[e] * sv[e] + bv[e];
+    if (p.res) {
+      const O8 r = *reinterpret_cast<const O8*>(reinterpret_cast<const OT*>(p.res) + (int64_t)m * p.ldr + n);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] += to_f32(r[e]);
+    }
+    O8 o;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      float t = v[e];
+      if constexpr (ACT == XG_ACT_RELU) t = fmaxf(t, 0.f);
+      if constexpr (ACT == XG_ACT_GELU) t = 0.5f * t * (1.f + erff(t * 0.70710678118654752f));
+      if constexpr (ACT == XG_ACT_SILU) t = t / (1.f + __expf(-t));
+      if constexpr (ACT == XG_ACT_SIGMOID) t = 1.f / (1.f + __expf(-t));
+      o[e] = from_f32<OT>(t);
+    }
+    *reinterpret_cast<O8*>(reinterpret_cast<OT*>(p.out) + (int64_t)m * p.N + n) = o;
+  }
+}
+
+template <typename OT>
+__device__ __forceinline__ void epilogue(const GemmParams& p, const Lane& L, f32x16 (&acc)[4][4], char* smem, int m0,
+                                         int n0) {
+  typedef OT O8 __attribute__((ext_vector_type(8)));
+  char* park = smem + L.wave * (128 * 64 * 4);
+  const float a_sc = p.a_scale ? *p.a_scale : 1.f;
+  const int m_base = m0 + L.wm * 128;
+  static_for<2>([&](auto H) {
+    constexpr int h = decltype(H)::value;
+    // 1. park: row = i*32 + l32, 16-byte chunk = jj*8 + g*2 + half, xor-ed with the row to spread the banks
+    static_for<2>([&](auto JJ) {
+      static_for<4>([&](auto G) {
+        static_for<4>([&](auto I) {
+          constexpr int jj = decltype(JJ)::value, g = decltype(G)::value, i = decltype(I)::value;
+          const int row = i * 32 + L.l32;
+          const int chunk = (jj * 8 + g * 2 + L.half) ^ (row & 15);
+          const f32x16& a = acc[i][h * 2 + jj];
+          *reinterpret_cast<f32x4*>(park + row * 256 + (chunk << 4)) = f32x4{a[4 * g], a[4 * g + 1], a[4 * g + 2], a[4 * g + 3]};
+        });
+      });
+    });
+    // 2. this lane's 8 columns of the half, and their scale / bias
+    const int n = n0 + L.wn * 128 + h * 64 + (L.lane & 7) * 8;
+    const bool n_ok = n < p.N;  // N % 8 == 0: the 8 columns are in or out together
+    float sv[8], bv[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      sv[e] = a_sc;
+      bv[e] = 0.f;
+    }
+    if (n_ok && p.b_scale) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) sv[e] = a_sc * p.b_scale[n + e];
+    }
+    if (n_ok && p.bias) {
+      if (p.bias_f32) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) bv[e] = reinterpret_cast<const float*>(p.bias)[n + e];
+      } else {
+        const O8 t = *reinterpret_cast<const O8*>(reinterpret_cast<const OT*>(p.bias) + n);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) bv[e] = to_f32(t[e]);
+      }
+    }
+    switch (p.act) {  // uniform; each case is the same short loop with one activation inlined
+      case XG_ACT_RELU:
+        epilogue_rows<OT, XG_ACT_RELU>(p, park, L.lane, m_base, n, n_ok, sv, bv);
+        break;
+      case XG_ACT_GELU:
+        epilogue_rows<OT, XG_ACT_GELU>(p, park, L.lane, m_base, n, n_ok, sv, bv);
+        break;
+      case XG_ACT_SILU:
+        epilogue_rows<OT, XG_ACT_SILU>(p, park, L.lane, m_base, n, n_ok, sv, bv);
+        break;
+      case XG_ACT_SIGMOID:
+        epilogue_rows<OT, XG_ACT_SIGMOID>(p, park, L.lane, m_base, n, n_ok, sv, bv);
+        break;
+      default:
+        epilogue_rows<OT, XG_ACT_NONE>(p, park, L.lane, m_base, n, n_ok, sv, bv);
+        break;
+    }
+  });
+}
+
+__device__ __forceinline__ void zero_acc(f32x16 (&acc)[4][4]) {
+  const f32x16 zero = {};
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = zero;
+}
+
+// ---- kernel 1: direct global -> LDS ------------------------------------------------------
+// T: operand element type (bf16_t, f16_t, or uint8_t for OCP e4m3); OT: output / bias / residual type.
+template <typename T, typename OT, BLayout BL>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_dma_kernel(GemmParams p) {
+  extern __shared__ __align__(16) char smem[];
+  constexpr int EB = Elem<T>::BYTES;
+  constexpr int KSTEPS = Elem<T>::KSTEPS;
+  constexpr int SLAB_K = ROW_BYTES / EB;
+  // The next slab's 16 direct loads all go out during the first k-steps of the current slab, so that
+  // the remaining steps cover their latency before the wait at the slab's end.
+  constexpr int LOAD_STEPS = XG_GEMM_LOAD_STEPS;
+  constexpr int PER_STEP = 16 / LOAD_STEPS;
+  static_assert(BL == BLayout::KMajor || EB == 2, "the transposing LDS read is wired for 16-bit elements only");
+
+  int tm, tn;
+  tile_of_block(p, tm, tn);
+  const int m0 = tm * BM, n0 = tn * BN;
+  const Lane L;
+
+  // Per-lane byte offsets of the 8 + 8 direct loads of a slab, relative to the slab's
+  // (uniform) base address; the host guarantees they fit in 31 bits.
+  uint32_t a_off[8], b_off[8];
+  {
+    const int lrow = L.lane >> 3;
+    const int lc = (L.lane & 7) ^ lrow ^ (L.wave & 1);  // logical chunk this lane fetches (see header)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int r = j * 32 + L.wave * 8 + lrow;
+      int gr = m0 + r;
+      gr = gr < p.M ? gr : p.M - 1;  // rows past the edge re-read the last row; their results are never stored
+      a_off[j] = (uint32_t)(((int64_t)gr * p.lda) * EB + lc * 16);
+      if constexpr (BL == BLayout::KMajor) {
+        int gn = n0 + r;
+        gn = gn < p.N ? gn : p.N - 1;
+        b_off[j] = (uint32_t)(((int64_t)gn * p.ldb) * EB + lc * 16);
+      } else {
+        const int kr = j * 8 + L.wave * 2 + L.half;
+        const int pc32 = L.lane & 31;
+        const int sw = ((L.wave * 2 + L.half) & 3) | ((j & 1) << 2);
+        const int gran = ((pc32 >> 2) ^ sw) & 7;
+        int gc = n0 + (gran * 4 + (pc32 & 3)) * 8;
+        gc = gc < p.N ? gc : (p.N - 8);  // N % 8 == 0 is checked on the host
+        b_off[j] = (uint32_t)(((int64_t)kr * p.ldb + gc) * EB);
+      }
+    }
+  }
+  const int64_t a_step = ROW_BYTES;
+  const int64_t b_step = BL == BLayout::KMajor ? (int64_t)ROW_BYTES : (int64_t)SLAB_K * p.ldb * EB;
+
+  // load number q (0..15) of the slab whose operand bases are a_g / b_g, into `stage`
+  auto issue = [&](int q, const char* a_g, const char* b_g, int stage) {
+    char* dst = smem + stage * STAGE_BYTES + L.wave * 1024 + (q & 7) * 4096 + (q < 8 ? 0 : SLAB_BYTES);
+    const char* src = q < 8 ? a_g + a_off[q & 7] : b_g + b_off[q & 7];
+    __builtin_amdgcn_global_load_lds((const gvoid*)src, (lvoid*)dst, 16, 0, 0);
+  };
+
+  f32x16 acc[4][4];
+  zero_acc(acc);
+
+  const int KT = p.K / SLAB_K;
+  const char* a_g = reinterpret_cast<const char*>(p.A);
+  const char* b_g = reinterpret_cast<const char*>(p.B);
+  static_for<16>([&](auto Q) { issue(decltype(Q)::value, a_g, b_g, 0); });
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+
+  // One slab of math.  PREFETCH: also issue the next slab's direct loads, spread over the k-steps.
+  auto slab = [&](auto PREFETCH, int stage, const char* a_next, const char* b_next) {
+    constexpr bool prefetch = decltype(PREFETCH)::value;
+    const char* a_s = smem + stage * STAGE_BYTES;
+    const char* b_s = a_s + SLAB_BYTES;
+    Frag<T> fa[2][4], fb[2][4];
+    read_frags<T, BL>(L, a_s, b_s, 0, fa[0], fb[0]);
+    __builtin_amdgcn_sched_barrier(0);
+    static_for<KSTEPS>([&](auto KS) {
+      constexpr int ks = decltype(KS)::value;
+      constexpr bool more = ks + 1 < KSTEPS;
+      if constexpr (more) read_frags<T, BL>(L, a_s, b_s, ks + 1, fa[(ks + 1) & 1], fb[(ks + 1) & 1]);
+      if constexpr (prefetch && ks < LOAD_STEPS)
+        static_for<PER_STEP>([&](auto Q) { issue(ks * PER_STEP + decltype(Q)::value, a_next, b_next, stage ^ 1); });
+      mma_step<T>(acc, fa[ks & 1], fb[ks & 1]);
+      // Issue order inside the step: the next step's LDS reads and the direct loads are threaded
+      // between pairs of MFMAs instead of queueing in front of them.
+      constexpr int reads = more ? (EB == 1 ? 16 : (BL == BLayout::KMajor ? 8 : 12)) : 0;
+      constexpr int loads = (prefetch && ks < LOAD_STEPS) ? PER_STEP : 0;
+      static_for<8>([&](auto R) {
+        constexpr int r = decltype(R)::value;
+        constexpr int rd = reads / 8 + (r < reads % 8 ? 1 : 0);
+        constexpr int ld = loads / 8 + (r < loads % 8 ? 1 : 0);
+        if constexpr (rd > 0) __builtin_amdgcn_sched_group_barrier(0x100, rd, 0);  // LDS reads
+        if constexpr (ld > 0) __builtin_amdgcn_sched_group_barrier(0x020, ld, 0);  // memory reads
+        __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);                         // MFMA
+      });
+      __builtin_amdgcn_sched_barrier(0);  // keep each step's reads and math inside the step
+    });
+  };
+
+  for (int kt = 0; kt + 1 < KT; ++kt) {
+    a_g += a_step;
+    b_g += b_step;
+    slab(std::true_type{}, kt & 1, a_g, b_g);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wavefront's share of the next slab has landed
+    __syncthreads();                                   // ... and everybody else's
+  }
+  slab(std::false_type{}, (KT - 1) & 1, a_g, b_g);
+  __syncthreads();  // the slabs are dead: the epilogue reuses LDS
+
+  epilogue<OT>(p, L, acc, smem, m0, n0);
+}
+
+// ---- kernel 2: slabs staged through registers (any K) --------------------------------------
+template <typename T, typename OT, BLayout BL>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_staged_kernel(GemmParams p) {
+  extern __shared__ __align__(16) char smem[];
+  constexpr int EB = Elem<T>::BYTES;
+  constexpr int KSTEPS = Elem<T>::KSTEPS;
+  constexpr int SLAB_K = ROW_BYTES / EB;
+  static_assert(BL == BLayout::KMajor || EB == 2, "the transposing LDS read is wired for 16-bit elements only");
+
+  int tm, tn;
+  tile_of_block(p, tm, tn);
+  const int m0 = tm * BM, n0 = tn * BN;
+  const Lane L;
+  const int tid = L.tid;
+
+  // K-major operand: thread covers chunk c8 of rows r0 + 32 j (8 threads = one 128-byte row).
+  const int c8 = tid & 7, r0 = tid >> 3;
+  const char* a_ptr[8];
+  const char* b_ptr[8];
+  int a_lds[8], b_lds[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const int r = r0 + 32 * j;
+    int gr = m0 + r;
+    gr = gr < p.M ? gr : p.M - 1;
+    a_ptr[j] = reinterpret_cast<const char*>(p.A) + ((int64_t)gr * p.lda) * EB + c8 * 16;
+    a_lds[j] = r * ROW_BYTES + ((c8 ^ swz(r)) << 4);
+  }
+  if constexpr (BL == BLayout::KMajor) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int r = r0 + 32 * j;
+      int gr = n0 + r;
+      gr = gr < p.N ? gr : p.N - 1;
+      b_ptr[j] = reinterpret_cast<const char*>(p.B) + ((int64_t)gr * p.ldb) * EB + c8 * 16;
+      b_lds[j] = r * ROW_BYTES + ((c8 ^ swz(r)) << 4);
+    }
+  } else {
+    // N-major operand: slab is [64 k][256 n]; thread covers 16-byte chunk c32 (8 columns) of k rows kr0 + 8 j.
+    const int c32 = tid & 31, kr0 = tid >> 5;
+    int gc = n0 + c32 * 8;
+    gc = gc < p.N ? gc : (p.N - 8);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int kr = kr0 + 8 * j;
+      b_ptr[j] = reinterpret_cast<const char*>(p.B) + ((int64_t)kr * p.ldb + gc) * EB;
+      const int sw = (kr & 3) | (((kr >> 3) & 1) << 2);
+      b_lds[j] = kr * (BN * EB) + ((((c32 >> 2) ^ sw) & 7) << 6) + ((c32 & 3) << 4);
+    }
+  }
+
+  u32x4 ga[8], gb[8];
+  auto load_slab = [&](int kt) {
+    const int k_left = p.K - kt * SLAB_K;  // elements of K still valid from this slab's start
+    const int64_t koff = (int64_t)kt * ROW_BYTES;
+    const int64_t boff = BL == BLayout::KMajor ? koff : (int64_t)kt * SLAB_K * p.ldb * EB;
+    if (k_left >= SLAB_K) {  // uniform: a whole slab, no per-load predicate
+#pragma unroll
+      for (int j = 0; j < 8; ++j) ga[j] = *reinterpret_cast<const u32x4*>(a_ptr[j] + koff);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) gb[j] = *reinterpret_cast<const u32x4*>(b_ptr[j] + boff);
+    } else {  // the last, partial slab: chunks past K read as zero
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        ga[j] = (c8 * (16 / EB) < k_left) ? *reinterpret_cast<const u32x4*>(a_ptr[j] + koff) : u32x4{0, 0, 0, 0};
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const bool ok = BL == BLayout::KMajor ? (c8 * (16 / EB) < k_left) : ((tid >> 5) + 8 * j < k_left);
+        gb[j] = ok ? *reinterpret_cast<const u32x4*>(b_ptr[j] + boff) : u32x4{0, 0, 0, 0};
+      }
+    }
+  };
+  auto store_slab = [&](int stage) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) *reinterpret_cast<u32x4*>(smem + stage * STAGE_BYTES + a_lds[j]) = ga[j];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) *reinterpret_cast<u32x4*>(smem + stage * STAGE_BYTES + SLAB_BYTES + b_lds[j]) = gb[j];
+  };
+
+  f32x16 acc[4][4];
+  zero_acc(acc);
+
+  const int KT = (p.K + SLAB_K - 1) / SLAB_K;
+  load_slab(0);
+  store_slab(0);
+  __syncthreads();
+  if (KT > 1) load_slab(1);
+
+  for (int kt = 0; kt < KT; ++kt) {
+    const int stage = kt & 1;
+    const char* a_s = smem + stage * STAGE_BYTES;
+    const char* b_s = a_s + SLAB_BYTES;
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) {
+      Frag<T> fa[4], fb[4];
+      read_frags<T, BL>(L, a_s, b_s, ks, fa, fb);
+      mma_step<T>(acc, fa, fb);
+      if (ks == 0 && kt + 1 < KT) store_slab(stage ^ 1);  // slab kt+1: registers -> the idle LDS stage
+      if (ks == 1 && kt + 2 < KT) load_slab(kt + 2);      // slab kt+2: memory -> registers
+    }
+    __syncthreads();
+  }
+
+  epilogue<OT>(p, L, acc, smem, m0, n0);
+}
+
+template <typename K>
+int set_smem_once(K kernel) {
+  static hipError_t st = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES);
+  return st == hipSuccess ? XG_OK : XG_ERR_LAUNCH;
+}
+
+template <typename K>
+int launch_kernel(K kernel, const GemmParams& p, hipStream_t stream) {
+  if (int st = set_smem_once(kernel)) return st;
+  const int64_t tiles = (int64_t)p.tiles_m * p.tiles_n;
+  if (tiles > 0x7fffffffLL) return XG_ERR_TOO_LARGE;
+  hipLaunchKernelGGL(kernel, dim3((unsigned)tiles), dim3(kThreads), SMEM_BYTES, stream, p);
+  return status_from_hip(hipGetLastError());
+}
+
+// The direct-to-LDS kernel needs whole slabs and 31-bit operand offsets.
+template <typename T>
+bool dma_ok(const GemmParams& p, BLayout bl) {
+  constexpr int EB = Elem<T>::BYTES;
+  constexpr int SLAB_K = ROW_BYTES / EB;
+  static const bool off = getenv("XG_GEMM_NO_DMA") != nullptr;
+  if (off || p.K % SLAB_K != 0) return false;
+  const int64_t lim = 0x7fffffffLL;
+  const int64_t a_bytes = ((int64_t)p.M * p.lda) * EB;
+  const int64_t b_bytes = bl == BLayout::KMajor ? ((int64_t)p.N * p.ldb) * EB : ((int64_t)SLAB_K * p.ldb + p.N) * EB;
+  return a_bytes < lim && b_bytes < lim;
+}
+
+template <typename T, typename OT, BLayout BL>
+int launch_gemm(const GemmParams& p, hipStream_t stream) {
+  if (dma_ok<T>(p, BL)) return launch_kernel(gemm_dma_kernel<T, OT, BL>, p, stream);
+  return launch_kernel(gemm_staged_kernel<T, OT, BL>, p, stream);
+}
+
+inline GemmParams make_params(const void* a, const void* b, const void* bias, const void* residual, void* out, int64_t M,
+                       int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldr, int act, bool bias_f32) {
+  GemmParams p{};
+  p.A = a;
+  p.B = b;
+  p.bias = bias;
+  p.res = residual;
+  p.out = out;
+  p.a_scale = nullptr;
+  p.b_scale = nullptr;
+  p.M = (int)M;
+  p.N = (int)N;
+  p.K = (int)K;
+  p.lda = lda;
+  p.ldb = ldb;
+  p.ldr = ldr;
+  p.act = act;
+  p.bias_f32 = bias_f32 ? 1 : 0;
+  p.tiles_m = (int)((M + BM - 1) / BM);
+  p.tiles_n = (int)((N + BN - 1) / BN);
+  return p;
+}
+
+}  // namespace gemm
+}  // namespace xg
