@@ -15,7 +15,9 @@
 //    memory straight into LDS, 1 KiB per wavefront instruction.  The loads of
 //    slab t+1 are issued a few at a time BETWEEN the MFMAs of slab t, as are the
 //    LDS fragment reads of the next k-step, so the matrix pipe never waits for
-//    the wavefront to finish issuing memory instructions.
+//    the wavefront to finish issuing memory instructions.  One 4-byte touch per
+//    128-byte line warms L2 for slab t+2, because one slab of math is too short
+//    to cover an L2 miss.
 //  * gemm_staged_kernel (any K % 8 == 0): slabs pass through registers, which
 //    lets the last, partial slab be zero-filled.
 //
@@ -399,6 +401,28 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
     __builtin_amdgcn_global_load_lds((const gvoid*)src, (lvoid*)dst, 16, 0, 0);
   };
 
+  // L2 warm-up two slabs ahead: one 4-byte touch per 128-byte line.  A row panel is shared by the
+  // tiles of a tile row and a B panel by the tiles of a tile column that run on the same XCD at
+  // the same time, so only one tile of each group needs to touch them.
+  const bool pf_a = (tn & 3) == 0, pf_b = (tm & 7) == 0;
+  const char* pfa_ptr;
+  const char* pfb_ptr;
+  {
+    int gr = m0 + L.tid;
+    gr = gr < p.M ? gr : p.M - 1;
+    pfa_ptr = reinterpret_cast<const char*>(p.A) + ((int64_t)gr * p.lda) * EB;
+    if constexpr (BL == BLayout::KMajor) {
+      int gn = n0 + L.tid;
+      gn = gn < p.N ? gn : p.N - 1;
+      pfb_ptr = reinterpret_cast<const char*>(p.B) + ((int64_t)gn * p.ldb) * EB;
+    } else {
+      int gc = n0 + (L.tid & 3) * 64;
+      gc = gc < p.N ? gc : (p.N - 8);
+      pfb_ptr = reinterpret_cast<const char*>(p.B) + ((int64_t)(L.tid >> 2) * p.ldb + gc) * EB;
+    }
+  }
+  uint32_t pf_sink = 0, pf_va = 0, pf_vb = 0;
+
   f32x16 acc[4][4];
   zero_acc(acc);
 
@@ -410,7 +434,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
   __syncthreads();
 
   // One slab of math.  PREFETCH: also issue the next slab's direct loads, spread over the k-steps.
-  auto slab = [&](auto PREFETCH, int stage, const char* a_next, const char* b_next) {
+  auto slab = [&](auto PREFETCH, int stage, const char* a_next, const char* b_next, int64_t pf_koff, int64_t pf_boff, bool do_pf) {
     constexpr bool prefetch = decltype(PREFETCH)::value;
     const char* a_s = smem + stage * STAGE_BYTES;
     const char* b_s = a_s + SLAB_BYTES;
@@ -423,6 +447,11 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
       if constexpr (more) read_frags<T, BL>(L, a_s, b_s, ks + 1, fa[(ks + 1) & 1], fb[(ks + 1) & 1]);
       if constexpr (prefetch && ks < LOAD_STEPS)
         static_for<PER_STEP>([&](auto Q) { issue(ks * PER_STEP + decltype(Q)::value, a_next, b_next, stage ^ 1); });
+      if constexpr (prefetch && ks == LOAD_STEPS) {
+        pf_sink ^= pf_va ^ pf_vb;  // last slab's touches: long since returned
+        if (do_pf && pf_a) pf_va = *reinterpret_cast<const uint32_t*>(pfa_ptr + pf_koff);
+        if (do_pf && pf_b) pf_vb = *reinterpret_cast<const uint32_t*>(pfb_ptr + pf_boff);
+      }
       mma_step<T>(acc, fa[ks & 1], fb[ks & 1]);
       // Issue order inside the step: the next step's LDS reads and the direct loads are threaded
       // between pairs of MFMAs instead of queueing in front of them.
@@ -443,13 +472,14 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
   for (int kt = 0; kt + 1 < KT; ++kt) {
     a_g += a_step;
     b_g += b_step;
-    slab(std::true_type{}, kt & 1, a_g, b_g);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wavefront's share of the next slab has landed
+    slab(std::true_type{}, kt & 1, a_g, b_g, (int64_t)(kt + 2) * a_step, (int64_t)(kt + 2) * b_step, kt + 2 < KT);
+    asm volatile("s_waitcnt vmcnt(2)" ::: "memory");  // all but the two newest (the L2 touches) have landed
     __syncthreads();                                   // ... and everybody else's
   }
-  slab(std::false_type{}, (KT - 1) & 1, a_g, b_g);
+  slab(std::false_type{}, (KT - 1) & 1, a_g, b_g, 0, 0, false);
   __syncthreads();  // the slabs are dead: the epilogue reuses LDS
 
+  if (pf_sink == 0x9e3779b9u && pf_va == 0x7f4a7c15u) reinterpret_cast<uint32_t*>(p.out)[0] = pf_vb;  // keeps the touches alive
   epilogue<OT>(p, L, acc, smem, m0, n0);
 }
 
