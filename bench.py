@@ -113,6 +113,8 @@ class AddLayerNormC2(Workload):
     dtype = "bf16"
     kernel = "norm_rows_kernel<bf16,bf16,LAYER>"
     work = 4 * 8192 * 4096 * 2 + 2 * 4096 * 2
+    # HBM bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE, scaled by a 64 MiB copy (profiles/membound_fused_ops_bench.md)
+    traffic = 268.6e6
 
     def setup(self, torch, dev):
         from oracle import inputs
@@ -156,6 +158,7 @@ class RmsNormC1(Workload):
     dtype = "f32"
     kernel = "norm_rows_kernel<f32,f32,RMS>"
     work = 2 * 2048 * 4096 * 4 + 4096 * 4
+    traffic = 67.3e6
 
     def setup(self, torch, dev):
         from oracle import inputs
@@ -194,6 +197,7 @@ class SliceCatC3a(Workload):
     dtype = "b32"
     kernel = "slice_cat_kernel<16>"
     work = 2 * 4096 * 2048 * 4 + 64 * 8
+    traffic = 96.9e6  # unaligned 128-byte slices straddle two 128-byte lines on the read side
 
     def setup(self, torch, dev):
         from oracle import inputs
@@ -236,6 +240,7 @@ class AddNC3b(Workload):
     dtype = "f32"
     kernel = "addn_kernel<f32>"
     work = 33 * 4096 * 256 * 4
+    traffic = 138.4e6
 
     def setup(self, torch, dev):
         from oracle import inputs
