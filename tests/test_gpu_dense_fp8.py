@@ -1,0 +1,96 @@
+"""GPU parity of the fp8 (OCP e4m3) dense layer (torch.ops.xpu_ops.dense_fp8 ->
+xg_dense_fp8): activations quantised per tensor, weights per output channel,
+fp32 accumulation, scales / bias / activation in the epilogue.  The reference
+has no fp8 path; the oracle is the dequantised fp32 product (exact for the
+same quantised operands), tolerance rtol 1.6e-2."""
+import json
+import os
+
+import pytest
+import torch
+
+from oracle import eager, inputs
+
+pytestmark = pytest.mark.gpu
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+def _ops():
+    import xpu_graph_amd.ops  # noqa: F401
+
+    return torch.ops.xpu_ops
+
+
+def quantised(M, N, K, device, seed):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(M, K, generator=g)
+    W = torch.randn(K, N, generator=g) / K**0.5
+    b = 0.1 * torch.randn(N, generator=g)
+    x_q, s_x = eager.quantize_fp8_per_tensor(x)
+    W_q, s_w = eager.quantize_fp8_per_out_channel(W)
+    return x_q.to(device), W_q.to(device), s_x.to(device), s_w.to(device), b.to(device)
+
+
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("M,N,K", [(256, 256, 128), (512, 768, 256), (300, 264, 208), (1, 8, 16), (1000, 1032, 80), (64, 2048, 4096)])
+def test_dense_fp8_shapes(device, out_dtype, M, N, K):
+    x_q, W_q, s_x, s_w, b = quantised(M, N, K, device, seed=M + N + K)
+    w_nk = W_q.t().contiguous()  # the kernel takes the weight as [N, K]
+    got = _ops().dense_fp8(x_q, w_nk, True, s_x, s_w, b, "silu", out_dtype)
+    assert got.shape == (M, N) and got.dtype == out_dtype
+    want = eager.dense_fp8_silu_eager(x_q, W_q, s_x, s_w, b)
+    torch.testing.assert_close(got.float(), want, rtol=1.6e-2, atol=2e-3)
+    got = _ops().dense_fp8(x_q, w_nk, True, s_x, s_w, None, "none", out_dtype)
+    want = (x_q.float() @ W_q.float()) * s_x * s_w
+    torch.testing.assert_close(got.float(), want, rtol=1.6e-2, atol=2e-3)
+
+
+def test_dense_fp8_accumulation_precision(device):
+    """The e4m3 MFMA adds its 64 products per instruction with a shortened aligned mantissa: measured error
+    is about 2^-13 of the largest product, far inside the fp8 tolerance but not fp32-exact.  Pin that bound."""
+    x_q, W_q, _, _, _ = quantised(512, 512, 4096, device, seed=2)
+    one = torch.ones(1, device=device)
+    got = _ops().dense_fp8(x_q, W_q.t().contiguous(), True, one, one.expand(512).contiguous(), None, "none", torch.float32)
+    exact = x_q.double() @ W_q.double()
+    weight = x_q.double().abs() @ W_q.double().abs()
+    assert ((got.double() - exact).abs() / weight).max().item() < 1e-4
+
+
+def test_dense_fp8_decodes_every_code(device):
+    """Every finite e4m3 code times 1.0 comes back as the value the format defines (known-answer table)."""
+    with open(os.path.join(GOLDEN, "fp8_e4m3fn_kat.json")) as f:
+        kat = json.load(f)
+    codes = torch.arange(256, dtype=torch.uint8)
+    finite = (codes & 0x7F) != 0x7F
+    a = torch.zeros(256, 16, dtype=torch.uint8)
+    a[:, 3] = torch.where(finite, codes, torch.zeros_like(codes))
+    w = torch.zeros(8, 16, dtype=torch.uint8)
+    w[5, 3] = 0x38  # 1.0
+    one = torch.ones(1, device=device)
+    got = _ops().dense_fp8(a.view(torch.float8_e4m3fn).to(device), w.view(torch.float8_e4m3fn).to(device), True, one, one.expand(8), None, "none", torch.float32)
+    want = a[:, 3].view(torch.float8_e4m3fn).float()
+    assert torch.equal(got[:, 5].cpu(), want)
+    assert torch.count_nonzero(got[:, :5]) == 0 and torch.count_nonzero(got[:, 6:]) == 0
+    for code, val in zip(kat["codes"], kat["decoded"]):  # the committed known answers, through the MFMA decode
+        assert got[code, 5].item() == val
+
+
+def test_dense_fp8_c4_full_size(device):
+    x, W, b = inputs.c4_dense(device=device)
+    x_q, s_x = eager.quantize_fp8_per_tensor(x)
+    W_q, s_w = eager.quantize_fp8_per_out_channel(W)
+    got = _ops().dense_fp8(x_q, W_q.t().contiguous(), True, s_x, s_w, b, "silu", torch.bfloat16)
+    rows = torch.arange(0, 8192, 61, device=device)  # a row sample keeps the fp32 reference small
+    want = eager.dense_fp8_silu_eager(x_q[rows], W_q, s_x, s_w, b)
+    torch.testing.assert_close(got[rows].float(), want, rtol=1.6e-2, atol=2e-3)
+    # against the unquantised layer: per-tensor / per-channel e4m3 keeps about two significant digits
+    full = eager.dense_silu_eager(x[rows], W, b).float()
+    err = (got[rows].float() - full).abs().mean() / full.abs().mean()
+    assert err < 0.08
+
+
+def test_dense_fp8_rejects_kn_weight(device):
+    x_q, W_q, s_x, s_w, b = quantised(64, 64, 64, device, seed=1)
+    with pytest.raises(Exception):
+        _ops().dense_fp8(x_q, W_q, False, s_x, s_w, b, "none", torch.bfloat16)

@@ -1,0 +1,137 @@
+"""GPU parity of the attention kernel (torch.ops.xpu_ops.sdpa -> xg_sdpa).
+
+Reference: softmax(q k^T * scale + mask) v evaluated in fp32 on the SAME bf16 /
+fp16 inputs (the oracle's formula with no intermediate rounding), tolerance
+rtol 1.6e-2 with an absolute floor of one bf16 ulp of the value range; the
+oracle itself (which rounds the scores and probabilities to the storage dtype,
+as the HF eager form does) is compared at the same tolerance.  Cases follow the
+reference's tests/common/test_fuse_sdpa.py:14-610: self and cross attention,
+unequal lengths, half precision, plus what the kernel adds: causal masking by
+index, grouped heads, strided [B, S, H, D] views, ragged tails.
+"""
+import math
+
+import pytest
+import torch
+
+from oracle import eager
+
+pytestmark = pytest.mark.gpu
+
+
+def _ops():
+    import xpu_graph_amd.ops  # noqa: F401
+
+    return torch.ops.xpu_ops
+
+
+def ref32(q, k, v, causal, scale):
+    qf, kf, vf = q.float(), k.float(), v.float()
+    rep = q.shape[1] // k.shape[1]
+    if rep > 1:
+        kf = kf.repeat_interleave(rep, dim=1)
+        vf = vf.repeat_interleave(rep, dim=1)
+    s = torch.matmul(qf, kf.transpose(-1, -2)) * scale
+    if causal:
+        Sq, Sk = q.shape[-2], k.shape[-2]
+        s = s + torch.full((Sq, Sk), float("-inf"), device=q.device).triu(1)
+    return torch.matmul(torch.softmax(s, dim=-1), vf)
+
+
+def close(got, want):
+    torch.testing.assert_close(got.float(), want, rtol=1.6e-2, atol=8e-3)
+
+
+def make(B, H, Hkv, Sq, Skv, D, dtype, device, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    q = torch.randn(B, H, Sq, D, generator=g).to(dtype).to(device)
+    k = torch.randn(B, Hkv, Skv, D, generator=g).to(dtype).to(device)
+    v = torch.randn(B, Hkv, Skv, D, generator=g).to(dtype).to(device)
+    return q, k, v
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("D", [128, 64])
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("Sq,Skv", [(256, 256), (128, 64), (1, 1), (1, 300), (129, 65), (200, 333), (333, 200), (64, 1000)])
+def test_sdpa_shapes(device, dtype, D, causal, Sq, Skv):
+    q, k, v = make(2, 3, 3, Sq, Skv, D, dtype, device, seed=Sq + Skv + D)
+    scale = 1.0 / math.sqrt(D)
+    got = _ops().sdpa(q, k, v, causal, scale)
+    assert got.shape == q.shape and got.dtype == dtype
+    close(got, ref32(q, k, v, causal, scale))
+
+
+def test_sdpa_matches_oracle_causal(device):
+    q, k, v = make(1, 4, 4, 512, 512, 128, torch.bfloat16, device, seed=5)
+    got = _ops().sdpa(q, k, v, True, 1.0 / math.sqrt(128))
+    # the eager form rounds scores and probabilities to bf16 (up to one ulp of |out| <= 4), hence the wider floor
+    torch.testing.assert_close(got.float(), eager.causal_sdpa_eager(q, k, v).float(), rtol=1.6e-2, atol=2e-2)
+
+
+def test_sdpa_grouped_heads_and_strided_views(device):
+    B, S, H, Hkv, D = 2, 320, 8, 2, 128
+    g = torch.Generator().manual_seed(11)
+    # [B, S, H, D] storage viewed as [B, H, S, D], as a projection followed by view + transpose leaves it
+    q = torch.randn(B, S, H, D, generator=g).bfloat16().to(device).transpose(1, 2)
+    k = torch.randn(B, S, Hkv, D, generator=g).bfloat16().to(device).transpose(1, 2)
+    v = torch.randn(B, S, Hkv, D, generator=g).bfloat16().to(device).transpose(1, 2)
+    assert not q.is_contiguous()
+    for causal in (True, False):
+        close(_ops().sdpa(q, k, v, causal, 0.1), ref32(q, k, v, causal, 0.1))
+
+
+@pytest.mark.parametrize("scale", [-0.2, 0.0, 1.0])
+def test_sdpa_scale_sign_and_zero(device, scale):
+    q, k, v = make(1, 2, 2, 192, 192, 64, torch.bfloat16, device, seed=3)
+    q = q * 0.3
+    for causal in (True, False):
+        close(_ops().sdpa(q, k, v, causal, scale), ref32(q, k, v, causal, scale))
+
+
+def test_sdpa_invariants(device):
+    """What the mathematics fixes regardless of size: rows of the softmax sum to one (v = const gives const);
+    causal row 0 returns v[0]; one-hot attention (huge aligned scores) returns the selected value row exactly."""
+    B, H, S, D = 1, 2, 384, 128
+    q, k, v = make(B, H, H, S, S, D, torch.bfloat16, device, seed=9)
+    ones = torch.full_like(v, 0.75)
+    for causal in (True, False):
+        out = _ops().sdpa(q, k, ones, causal, 0.09)
+        assert torch.equal(out, ones)
+    out = _ops().sdpa(q, k, v, True, 0.09)
+    assert torch.equal(out[:, :, 0], v[:, :, 0])
+    # keys = +-1 codes of their index; query i = 16 * code(i): score(i, i) = 16 * D, every other score is lower by
+    # at least 32, so after the softmax only key i survives in bf16
+    idx = torch.arange(S, device=device)
+    bits = ((idx[:, None] >> torch.arange(9, device=device)[None, :]) & 1).float() * 2 - 1  # [S, 9]
+    code = bits.repeat(1, D // 9 + 1)[:, :D]
+    kk = code.bfloat16().expand(B, H, S, D).contiguous()
+    qq = (16 * code).bfloat16().expand(B, H, S, D).contiguous()
+    for causal in (True, False):
+        out = _ops().sdpa(qq, kk, v, causal, 1.0)
+        assert torch.equal(out, v)
+
+
+def test_sdpa_c5_full_size(device):
+    """The attention of benchmark config 5: B 4, 32 heads, S 2048, D 128, causal, bf16."""
+    B, H, S, D = 4, 32, 2048, 128
+    q, k, v = make(B, H, H, S, S, D, torch.bfloat16, device, seed=1)
+    scale = 1.0 / math.sqrt(D)
+    got = _ops().sdpa(q, k, v, True, scale)
+    for b in range(B):  # reference one batch at a time: 32 x 2048 x 2048 fp32 scores = 512 MiB
+        close(got[b : b + 1], ref32(q[b : b + 1], k[b : b + 1], v[b : b + 1], True, scale))
+    ones = torch.ones_like(v)
+    assert torch.equal(_ops().sdpa(q, k, ones, True, scale), ones)
+
+
+def test_sdpa_rejects_what_the_kernel_cannot_take(device):
+    q, k, v = make(1, 2, 2, 64, 64, 128, torch.bfloat16, device)
+    with pytest.raises(Exception):
+        _ops().sdpa(q.float(), k.float(), v.float(), False, 1.0)  # fp32 has no kernel
+    q96, k96, v96 = make(1, 2, 2, 64, 64, 96, torch.bfloat16, device)
+    with pytest.raises(Exception):
+        _ops().sdpa(q96, k96, v96, False, 1.0)  # head dim 96
+    with pytest.raises(Exception):
+        _ops().sdpa(q, k[:, :1], v, False, 1.0)  # k / v disagree
+    empty = _ops().sdpa(q[:, :, :0], k, v, False, 1.0)
+    assert empty.shape == (1, 2, 0, 128)

@@ -1,0 +1,376 @@
+// Scaled dot-product attention for gfx950: one pass over the keys with a running
+// maximum (flash-attention forward), optional causal mask, no dropout.
+//
+// Work split
+//   workgroup = 4 waves = 128 query rows of one (batch, head); wave w owns rows
+//   32w..32w+31.  Keys / values stream through LDS in tiles of 64 rows, moved by
+//   `global_load_lds_dwordx4` (no register staging) into two stages, so the tile
+//   of step j+1 lands while step j is computed; one barrier per step.
+//
+// Transposed products: everything a query row needs stays in one lane
+//   S^T = K Q^T   : MFMA 32x32x16 with the K tile as the A operand and the
+//                   register-resident Q rows as B.  The result puts query
+//                   (lane % 32) in the lane and 16 of a tile's 32 keys in its 16
+//                   accumulator registers; lanes l and l^32 share a query.
+//   softmax       : row maximum = per-lane max + ONE cross-lane exchange; the
+//                   correction factor and the row sum are per-lane scalars.
+//   O^T += V^T P^T: V^T tile as A, the probabilities as B.  The k index of an
+//                   MFMA may be permuted freely as long as A and B agree, so the
+//                   k slots are chosen to be exactly the keys a lane already
+//                   holds: P never moves between lanes and never touches LDS.
+//                   The matching V^T fragment (8 keys x 1 head-dim column per
+//                   lane) comes from two `ds_read_b64_tr_b16` reads.
+//
+// LDS layout: row-major [64 keys][D] per tile, 16-byte chunks XOR-swizzled by a
+// function of the row so that the 16-lane groups of the K reads (same chunk, 16
+// rows) and the 8-row x 64-byte footprints of the transposing V reads spread over
+// all banks.  The swizzle is applied to the GLOBAL address of each lane of the
+// direct load, since its LDS side is fixed (lane i -> base + 16 i).
+#include "xg_common.hpp"
+
+#include <math.h>
+#include <stdlib.h>
+
+#include <type_traits>
+#include <utility>
+
+namespace xg {
+namespace sdpa {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef short s16x8 __attribute__((ext_vector_type(8)));
+typedef __attribute__((address_space(1))) void gvoid;
+typedef __attribute__((address_space(3))) void lvoid;
+typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+
+constexpr int BQ = 128;   // query rows per workgroup
+constexpr int BKV = 64;   // key rows per step
+constexpr int kThreads = 256;
+
+struct Params {
+  const void* q;
+  const void* k;
+  const void* v;
+  void* o;
+  int B, H, Hkv, Sq, Skv;
+  int64_t qs[3], ks[3], vs[3], os[3];  // element strides of batch, head, sequence
+  float c;                             // scale * log2(e)
+  int causal;
+  int n_qb;   // query blocks per (batch, head)
+  int order;  // 0: heaviest query blocks of ALL heads first; 1: head after head inside each XCD
+};
+
+template <typename F, int... I>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, I...>) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+  static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
+
+template <typename T>
+struct Vec8;
+template <>
+struct Vec8<bf16_t> {
+  typedef bf16x8 type;
+};
+template <>
+struct Vec8<f16_t> {
+  typedef f16x8 type;
+};
+
+__device__ __forceinline__ f32x16 mma(bf16x8 a, bf16x8 b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
+__device__ __forceinline__ f32x16 mma(f16x8 a, f16x8 b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0); }
+
+// Chunk swizzles (16-byte chunks within a row of D elements).
+template <int D>
+__device__ __forceinline__ int swz_k(int r) {
+  if constexpr (D == 128) return r & 15;  // 256-byte rows: 16 rows x one chunk -> 16 distinct bank groups
+  else return (r >> 1) & 7;               // 128-byte rows: two rows per 256 bytes
+}
+template <int D>
+__device__ __forceinline__ int swz_v(int r) {
+  // the transposing read touches 8 consecutive rows x 4 aligned chunks: rows must move the GROUP of four
+  if constexpr (D == 128) return ((r & 3) << 2) | ((r >> 2) & 3);
+  else return (((r >> 1) & 1) << 2) | ((r >> 2) & 3);
+}
+
+template <typename T, int D>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void sdpa_fwd_kernel(Params p) {
+  typedef typename Vec8<T>::type V8;
+  constexpr int RB = D * 2;          // bytes per tile row
+  constexpr int CH = RB / 16;        // chunks per row
+  constexpr int TILE = BKV * RB;     // one K or V tile
+  constexpr int STAGE = 2 * TILE;    // K tile, then V tile
+  constexpr int KK = D / 16;         // k-steps of Q K^T
+  constexpr int DT = D / 32;         // 32-row tiles of O^T
+  constexpr int LPW = CH / 4;        // direct loads per wave per tile (1 KiB each)
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l32 = lane & 31, h = lane >> 5;
+
+  // ---- which (batch, head, query block).  Blocks are dealt round-robin to the 8 XCDs, so with the
+  // number of heads a multiple of 8 both orders keep all query blocks of a head on ONE XCD (one L2).
+  int bh, qb;
+  {
+    const int id = blockIdx.x, nbh = p.B * p.H;
+    if (p.order == 1 && (nbh & 7) == 0) {
+      const int xcd = id & 7, slot = id >> 3;
+      bh = (slot / p.n_qb) * 8 + xcd;
+      qb = p.n_qb - 1 - slot % p.n_qb;
+    } else {
+      bh = id % nbh;
+      qb = p.n_qb - 1 - id / nbh;  // causal: late query blocks have the most keys, start them first
+    }
+  }
+  const int b = bh / p.H, head = bh % p.H, hkv = head / (p.H / p.Hkv);
+  const int q0 = qb * BQ;
+  const int qrow = q0 + 32 * wave + l32;  // this lane's query
+
+  // ---- Q rows into registers, in B-operand order: lane holds Q[q][16 kk + 8 h .. +8]
+  V8 qf[KK];
+  {
+    const int qr = qrow < p.Sq ? qrow : p.Sq - 1;
+    const T* qg = reinterpret_cast<const T*>(p.q) + (int64_t)b * p.qs[0] + (int64_t)head * p.qs[1] + (int64_t)qr * p.qs[2];
+    static_for<KK>([&](auto KI) {
+      constexpr int kk = decltype(KI)::value;
+      qf[kk] = *reinterpret_cast<const V8*>(qg + 16 * kk + 8 * h);
+    });
+  }
+
+  // ---- direct-load bookkeeping: load i of this wave fills LDS bytes [(wave*LPW+i)*1024, +1024) of a tile
+  const char* kg = reinterpret_cast<const char*>(p.k) + ((int64_t)b * p.ks[0] + (int64_t)hkv * p.ks[1]) * 2;
+  const char* vg = reinterpret_cast<const char*>(p.v) + ((int64_t)b * p.vs[0] + (int64_t)hkv * p.vs[1]) * 2;
+  int ld_row[LPW], ld_kc[LPW], ld_vc[LPW];
+  static_for<LPW>([&](auto I) {
+    constexpr int i = decltype(I)::value;
+    const int pos = (wave * LPW + i) * 1024 + lane * 16;
+    const int row = pos / RB, pc = (pos % RB) >> 4;
+    ld_row[i] = row;
+    ld_kc[i] = (pc ^ swz_k<D>(row)) << 4;
+    ld_vc[i] = (pc ^ swz_v<D>(row)) << 4;
+  });
+  const int64_t k_row_bytes = p.ks[2] * 2, v_row_bytes = p.vs[2] * 2;
+  auto issue = [&](int j, int stage) {
+    static_for<LPW>([&](auto I) {
+      constexpr int i = decltype(I)::value;
+      int r = j * BKV + ld_row[i];
+      r = r < p.Skv ? r : p.Skv - 1;  // rows past the end repeat the last key; they are masked below
+      char* kd = smem + stage * STAGE + (wave * LPW + i) * 1024;
+      __builtin_amdgcn_global_load_lds((const gvoid*)(kg + r * k_row_bytes + ld_kc[i]), (lvoid*)kd, 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((const gvoid*)(vg + r * v_row_bytes + ld_vc[i]), (lvoid*)(kd + TILE), 16, 0, 0);
+    });
+  };
+
+  // ---- number of key tiles this workgroup visits
+  int n_steps = (p.Skv + BKV - 1) / BKV;
+  if (p.causal) {
+    int q_last = q0 + BQ - 1;
+    q_last = q_last < p.Sq ? q_last : p.Sq - 1;
+    const int lim = q_last / BKV + 1;
+    n_steps = n_steps < lim ? n_steps : lim;
+  }
+  const int qw_min = q0 + 32 * wave, qw_max = qw_min + 31;
+
+  // ---- per-lane LDS read offsets
+  const int kx = swz_k<D>(l32);  // same for both 32-row tiles of a K tile
+  const int a16 = lane & 15, b16 = (lane >> 4) & 1;
+
+  f32x16 o_acc[DT];
+  static_for<DT>([&](auto I) {
+    o_acc[decltype(I)::value] = f32x16{0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  });
+  float m_run = -INFINITY, l_run = 0.f;
+
+  issue(0, 0);
+  for (int j = 0; j < n_steps; ++j) {
+    const int stage = j & 1;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's part of tile j has landed
+    __syncthreads();                                  // ... everyone's has, and everyone is done with tile j-1
+    if (j + 1 < n_steps) issue(j + 1, stage ^ 1);
+    const int kv0 = j * BKV;
+    if (p.causal && kv0 > qw_max) continue;  // this wave's queries see none of these keys (wave-uniform)
+
+    const char* k_s = smem + stage * STAGE;
+    const char* v_s = k_s + TILE;
+
+    // S^T tile: s[t][v] = <key 32t + 8(v/4) + 4h + v%4 , query l32>
+    f32x16 s[2];
+    static_for<2>([&](auto TI) {
+      constexpr int t = decltype(TI)::value;
+      s[t] = f32x16{0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      static_for<KK>([&](auto KI) {
+        constexpr int kk = decltype(KI)::value;
+        const int off = (32 * t + l32) * RB + (((2 * kk + h) ^ kx) << 4);
+        const V8 kf = *reinterpret_cast<const V8*>(k_s + off);
+        s[t] = mma(kf, qf[kk], s[t]);
+      });
+    });
+
+    // scores are s * c in the exponent's base-2 scale.  Tiles that cross the diagonal or the end of
+    // the keys are scaled and masked explicitly (cc = 1 afterwards); all others fold c into the FMA.
+    float cc = p.c;
+    const bool need_mask = (p.causal && kv0 + BKV - 1 > qw_min) || (kv0 + BKV > p.Skv);
+    if (need_mask) {
+      int lim = p.Skv - 1;  // last visible key of this lane's query
+      if (p.causal) lim = lim < qrow ? lim : qrow;
+      const int rel = lim - kv0 - 4 * h;
+      static_for<2>([&](auto TI) {
+        constexpr int t = decltype(TI)::value;
+        static_for<16>([&](auto VI) {
+          constexpr int v = decltype(VI)::value;
+          constexpr int key = 32 * t + 8 * (v / 4) + (v % 4);
+          s[t][v] = key > rel ? -INFINITY : s[t][v] * cc;
+        });
+      });
+      cc = 1.f;
+    }
+    float mx = s[0][0];
+    if (cc >= 0.f) {
+      static_for<2>([&](auto TI) { static_for<16>([&](auto VI) { mx = fmaxf(mx, s[decltype(TI)::value][decltype(VI)::value]); }); });
+    } else {
+      static_for<2>([&](auto TI) { static_for<16>([&](auto VI) { mx = fminf(mx, s[decltype(TI)::value][decltype(VI)::value]); }); });
+    }
+    float mt = mx * cc;
+    mt = fmaxf(mt, __shfl_xor(mt, 32, kWave));
+    const float m_new = fmaxf(m_run, mt);
+    const float m_use = m_new == -INFINITY ? 0.f : m_new;  // a row with no visible key yet
+    const float alpha = __builtin_amdgcn_exp2f(m_run - m_use);
+    float psum = 0.f;
+    static_for<2>([&](auto TI) {
+      constexpr int t = decltype(TI)::value;
+      static_for<16>([&](auto VI) {
+        constexpr int v = decltype(VI)::value;
+        const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(s[t][v], cc, -m_use));
+        s[t][v] = e;
+        psum += e;
+      });
+    });
+    l_run = l_run * alpha + psum;
+    m_run = m_new;
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {
+      static_for<DT>([&](auto I) { o_acc[decltype(I)::value] *= alpha; });
+    }
+
+    // O^T += V^T P^T.  k-step (t, st) uses keys 32t + 16st + {4h..4h+3} and 32t + 16st + 8 + {4h..4h+3}:
+    // exactly registers 8st..8st+7 of s[t] in this lane.
+    static_for<2>([&](auto TI) {
+      constexpr int t = decltype(TI)::value;
+      static_for<2>([&](auto SI) {
+        constexpr int st = decltype(SI)::value;
+        V8 pf;
+        static_for<8>([&](auto JI) {
+          constexpr int jj = decltype(JI)::value;
+          pf[jj] = (T)s[t][8 * st + jj];
+        });
+        static_for<DT>([&](auto DI) {
+          constexpr int dt = decltype(DI)::value;
+          // lane a16 of a 16-lane group addresses key row (a16/4), head-dim columns 4(a16%4)..+3 of the group's
+          // 16 columns; the transposing read returns, for result slot e, key row e at column a16.
+          const int r0 = 32 * t + 16 * st + 4 * h + (a16 >> 2);
+          const int r1 = r0 + 8;
+          const int chunk = 4 * dt + 2 * b16 + ((a16 & 3) >> 1);
+          const int sub = (a16 & 1) << 3;
+          const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(v_s + r0 * RB + ((chunk ^ swz_v<D>(r0)) << 4) + sub));
+          const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(v_s + r1 * RB + ((chunk ^ swz_v<D>(r1)) << 4) + sub));
+          const s16x8 both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+          o_acc[dt] = mma(__builtin_bit_cast(V8, both), pf, o_acc[dt]);
+        });
+      });
+    });
+  }
+
+  // ---- normalise and write: O[q][d] = O^T[d][q] / l.  The tile is parked in LDS (per wave) so that
+  // global stores are 16 bytes per lane and whole rows per 16 lanes.
+  const float l_tot = l_run + __shfl_xor(l_run, 32, kWave);
+  const float inv = 1.f / l_tot;
+  __syncthreads();  // all waves are done reading K / V tiles
+  char* park = smem + wave * (32 * RB);
+  static_for<DT>([&](auto DI) {
+    constexpr int dt = decltype(DI)::value;
+    static_for<4>([&](auto GI) {
+      constexpr int g = decltype(GI)::value;
+      typedef T t4 __attribute__((ext_vector_type(4)));
+      t4 w;
+      static_for<4>([&](auto EI) {
+        constexpr int e = decltype(EI)::value;
+        w[e] = (T)(o_acc[dt][4 * g + e] * inv);
+      });
+      // columns 32dt + 8g + 4h .. +3 of row l32: chunk 4dt + g, upper or lower 8 bytes
+      *reinterpret_cast<t4*>(park + l32 * RB + (((4 * dt + g) ^ swz_k<D>(l32)) << 4) + 8 * h) = w;
+    });
+  });
+  __syncthreads();
+  T* og = reinterpret_cast<T*>(p.o) + (int64_t)b * p.os[0] + (int64_t)head * p.os[1];
+  static_for<RB / 32>([&](auto I) {
+    constexpr int i = decltype(I)::value;
+    const int pos = i * 1024 + lane * 16;
+    const int row = pos / RB, pc = (pos % RB) >> 4;
+    const int c = pc ^ swz_k<D>(row);
+    const u32x4 val = *reinterpret_cast<const u32x4*>(park + pos);
+    const int qr = q0 + 32 * wave + row;
+    if (qr < p.Sq) *reinterpret_cast<u32x4*>(og + (int64_t)qr * p.os[2] + c * 8) = val;
+  });
+}
+
+template <typename T, int D>
+int launch(const Params& p, hipStream_t stream) {
+  constexpr int SMEM = 2 * 2 * BKV * D * 2;
+  auto kernel = sdpa_fwd_kernel<T, D>;
+  static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, SMEM);
+  if (attr != hipSuccess) return XG_ERR_LAUNCH;
+  const int64_t blocks = (int64_t)p.B * p.H * p.n_qb;
+  hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(kThreads), SMEM, stream, p);
+  return status_from_hip(hipGetLastError());
+}
+
+}  // namespace sdpa
+}  // namespace xg
+
+extern "C" int xg_sdpa(const void* q, const void* k, const void* v, void* out, int64_t B, int64_t H, int64_t Hkv, int64_t Sq,
+                       int64_t Skv, int64_t D, const int64_t q_strides[3], const int64_t k_strides[3], const int64_t v_strides[3],
+                       const int64_t o_strides[3], float scale, int causal, int dtype, xg_stream_t stream) {
+  using namespace xg;
+  if (dtype != XG_BF16 && dtype != XG_F16) return XG_ERR_BAD_DTYPE;
+  if (B < 0 || H < 0 || Hkv < 0 || Sq < 0 || Skv < 0) return XG_ERR_BAD_SHAPE;
+  if (D != 64 && D != 128) return XG_ERR_BAD_SHAPE;
+  if (B == 0 || H == 0 || Sq == 0) return XG_OK;
+  if (Hkv == 0 || H % Hkv != 0 || Skv == 0) return XG_ERR_BAD_SHAPE;
+  if (!q || !k || !v || !out || !q_strides || !k_strides || !v_strides || !o_strides) return XG_ERR_NULL_PTR;
+  if (!(scale == scale) || fabsf(scale) > 3.0e38f) return XG_ERR_BAD_ARG;
+  if (Sq > (1 << 30) || Skv > (1 << 30)) return XG_ERR_TOO_LARGE;
+  const int64_t n_qb = (Sq + sdpa::BQ - 1) / sdpa::BQ;
+  if (B * H > (1 << 24) || B * H * n_qb > 0x7fffffffLL) return XG_ERR_TOO_LARGE;
+  if (!aligned_to(q, 16) || !aligned_to(k, 16) || !aligned_to(v, 16) || !aligned_to(out, 16)) return XG_ERR_BAD_ALIGN;
+  sdpa::Params p;
+  for (int i = 0; i < 3; ++i) {
+    if (q_strides[i] < 0 || k_strides[i] < 0 || v_strides[i] < 0 || o_strides[i] < 0) return XG_ERR_BAD_SHAPE;
+    if (q_strides[i] % 8 || k_strides[i] % 8 || v_strides[i] % 8 || o_strides[i] % 8) return XG_ERR_BAD_ALIGN;
+    p.qs[i] = q_strides[i];
+    p.ks[i] = k_strides[i];
+    p.vs[i] = v_strides[i];
+    p.os[i] = o_strides[i];
+  }
+  p.q = q;
+  p.k = k;
+  p.v = v;
+  p.o = out;
+  p.B = (int)B;
+  p.H = (int)H;
+  p.Hkv = (int)Hkv;
+  p.Sq = (int)Sq;
+  p.Skv = (int)Skv;
+  p.c = scale * 1.44269504088896340736f;
+  p.causal = causal ? 1 : 0;
+  p.n_qb = (int)n_qb;
+  p.order = 0;
+  if (const char* e = getenv("XG_SDPA_ORDER")) p.order = atoi(e) == 1 ? 1 : 0;
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  if (dtype == XG_BF16) return D == 128 ? sdpa::launch<bf16_t, 128>(p, st) : sdpa::launch<bf16_t, 64>(p, st);
+  return D == 128 ? sdpa::launch<f16_t, 128>(p, st) : sdpa::launch<f16_t, 64>(p, st);
+}
