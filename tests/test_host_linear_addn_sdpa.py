@@ -225,3 +225,25 @@ def test_clone_feeding_output_is_kept():
     x = torch.randn(3)
     y = torch.compile(fn, backend=be)(x)
     assert torch.equal(x, y) and y.data_ptr() != x.data_ptr()
+
+
+def test_output_clone_of_private_intermediate_is_dropped():
+    """Beyond the reference: the copy left over from cat([t]) of a fresh intermediate is removed even at a
+    graph output, while clones that keep two outputs (or an output and an input) apart stay."""
+    be = XpuGraph(XpuGraphConfig(is_training=False))
+    x = torch.randn(4, 16)
+
+    def single(x):
+        return torch.cat([torch.cat([x[:, 0:4], x[:, 8:12]], dim=1)], dim=1)
+
+    assert torch.equal(torch.compile(single, backend=be)(x), single(x))
+    assert "aten.clone.default" not in [str(n.target) for n in be.compiled_graphs[-1].graph.nodes]
+
+    def aliased(x):
+        y = x + 1
+        return y, y.clone(), x.clone(), x[:, :4].clone()
+
+    got = torch.compile(aliased, backend=be)(x)
+    for a, b in zip(got, aliased(x)):
+        assert torch.equal(a, b)
+    assert got[0].data_ptr() != got[1].data_ptr() and got[2].data_ptr() != x.data_ptr() and got[3].data_ptr() != x.data_ptr()

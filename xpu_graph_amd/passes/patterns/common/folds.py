@@ -166,19 +166,47 @@ class FoldCat(Pattern):
 
 
 class FoldClone(Pattern):
-    """clone(x, preserve_format) -> x unless the clone's storage reaches a graph output."""
+    """clone(x, preserve_format) -> x unless the clone's storage reaches a graph output.
+
+    One case beyond the reference: a clone that IS a graph output is still dropped when x is a contiguous
+    intermediate with storage of its own (not an input's, not a parameter's) that reaches no other output;
+    nobody can then tell the copy from the original.  This is what is left of cat([fused]) once a whole
+    slice/cat group has become a single kernel call, and the copy would double that kernel's memory traffic.
+    """
 
     _support_stages = [FxStage.inference]
 
+    @staticmethod
+    def _private_intermediate(gm, clone, out_nodes):
+        src = clone.args[0]
+        key = _storage_key(src)
+        if key is None or src.op not in ("call_module", "call_function"):
+            return False
+        for n in gm.graph.nodes:
+            if n.op in ("placeholder", "get_attr") and _storage_key(n) == key:
+                return False
+        if any(o is not clone and _storage_key(o) == key for o in out_nodes):
+            return False
+        fmt = clone.kwargs.get("memory_format", torch.preserve_format)
+        return fmt in (torch.preserve_format, torch.contiguous_format) and src.meta["val"].is_contiguous()
+
     def process(self, gm):
         outs = _output_storages(gm)
+        out_nodes = list(list(gm.graph.nodes)[-1].all_input_nodes)
         changed = False
         for n in [n for n in gm.graph.nodes if is_call(n, aten.clone.default)]:
             key = _storage_key(n)
-            if key is None or key in outs:
+            if key is None:
                 continue
             src = n.args[0]
             if not isinstance(src.meta.get("val"), torch.Tensor):
+                continue
+            if key in outs:
+                if n in out_nodes and self._private_intermediate(gm, n, out_nodes):
+                    n.replace_all_uses_with(src)
+                    gm.graph.erase_node(n)
+                    out_nodes = list(list(gm.graph.nodes)[-1].all_input_nodes)
+                    changed = True
                 continue
             if n.kwargs.get("memory_format", torch.preserve_format) == torch.preserve_format:
                 n.replace_all_uses_with(src)
