@@ -272,8 +272,210 @@ class AddNC3b(Workload):
         return (lambda: fn(*ts)), how
 
 
+class DenseC4(Workload):
+    name = "C4 dense + bias + SiLU bf16 M8192 K4096 N11008"
+    bound = "mfma"
+    dtype = "bf16"
+    unit = "TFLOP/s"
+    kernel = "gemm_dma_kernel<bf16,[K,N] weight>"
+    work = 2 * 8192 * 4096 * 11008
+    n_sets = 3
+    cpu_rows = 512
+
+    def setup(self, torch, dev):
+        from oracle import inputs
+        from xpu_graph_amd import _lib
+
+        self.torch = torch
+        self.sets = [inputs.c4_dense(device=dev, seed=i) for i in range(self.n_sets)]
+        self.outs = [torch.empty(8192, 11008, device=dev, dtype=torch.bfloat16) for _ in range(self.n_sets)]
+        self.lib = _lib.lib()
+        self.st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def op_call(self, i):
+        x, W, b = self.sets[i]
+        return self.torch.ops.xpu_ops.dense(x, W, False, b, None, "silu")
+
+    def abi_call(self, i):
+        x, W, b = self.sets[i]
+        self.lib.xg_dense(_p(x), _p(W), _p(b), None, _p(self.outs[i]), 8192, 11008, 4096, 4096, 11008, 0, 0, 3, 2, 2, self.st)
+
+    def check(self, torch):
+        x, W, b = self.sets[0]
+        rows = torch.arange(0, 8192, 97, device=x.device)
+        want = torch.nn.functional.silu(x[rows].float() @ W.float() + b.float())
+        torch.testing.assert_close(self.op_call(0)[rows].float(), want, rtol=1.6e-2, atol=2e-2)
+
+    def cpu_fn(self, torch):
+        from oracle import eager, inputs
+
+        x, W, b = inputs.c4_dense(M=self.cpu_rows, device="cpu", seed=0)
+        fn, how = _default_path_compile(eager.dense_silu_eager)
+        return (lambda: fn(x, W, b)), how + f", first {self.cpu_rows} of 8192 rows"
+
+    @property
+    def cpu_work(self):
+        return self.work * self.cpu_rows / 8192
+
+
+class DenseFp8C4(DenseC4):
+    name = "C4 dense + bias + SiLU fp8 e4m3 (per-tensor x, per-channel W) M8192 K4096 N11008"
+    dtype = "fp8"
+    kernel = "gemm_dma_kernel<e4m3,[N,K] weight>"
+
+    def setup(self, torch, dev):
+        from oracle import eager, inputs
+        from xpu_graph_amd import _lib
+
+        self.torch = torch
+        self.sets = []
+        for i in range(self.n_sets):
+            x, W, b = inputs.c4_dense(device=dev, seed=i)
+            x_q, s_x = eager.quantize_fp8_per_tensor(x)
+            W_q, s_w = eager.quantize_fp8_per_out_channel(W)
+            self.sets.append((x_q, W_q.t().contiguous(), s_x, s_w.contiguous(), b))
+            if i == 0:
+                self.W_q0 = W_q
+        self.outs = [torch.empty(8192, 11008, device=dev, dtype=torch.bfloat16) for _ in range(self.n_sets)]
+        self.lib = _lib.lib()
+        self.st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def op_call(self, i):
+        x_q, w_nk, s_x, s_w, b = self.sets[i]
+        return self.torch.ops.xpu_ops.dense_fp8(x_q, w_nk, True, s_x, s_w, b, "silu", self.torch.bfloat16)
+
+    def abi_call(self, i):
+        x_q, w_nk, s_x, s_w, b = self.sets[i]
+        self.lib.xg_dense_fp8(_p(x_q), _p(w_nk), _p(s_x), _p(s_w), _p(b), _p(self.outs[i]), 8192, 11008, 4096, 4096, 4096, 1, 3, 2, 2, self.st)
+
+    def check(self, torch):
+        from oracle import eager
+
+        x_q, w_nk, s_x, s_w, b = self.sets[0]
+        rows = torch.arange(0, 8192, 97, device=x_q.device)
+        want = eager.dense_fp8_silu_eager(x_q[rows], self.W_q0, s_x, s_w, b)
+        torch.testing.assert_close(self.op_call(0)[rows].float(), want, rtol=1.6e-2, atol=2e-3)
+        del self.W_q0
+
+    def cpu_fn(self, torch):
+        from oracle import eager, inputs
+
+        x, W, b = inputs.c4_dense(M=self.cpu_rows, device="cpu", seed=0)
+        x_q, s_x = eager.quantize_fp8_per_tensor(x)
+        W_q, s_w = eager.quantize_fp8_per_out_channel(W)
+        return (lambda: eager.dense_fp8_silu_eager(x_q, W_q, s_x, s_w, b)), f"eager dequantise + fp32 matmul, first {self.cpu_rows} of 8192 rows"
+
+
+class SdpaC5(Workload):
+    name = "C5 causal attention bf16 B4 H32 S2048 D128"
+    bound = "mfma"
+    dtype = "bf16"
+    unit = "TFLOP/s"
+    kernel = "sdpa_fwd_kernel<bf16,128>"
+    work = 4 * 4 * 32 * 2048 * 2048 * 128 // 2  # two matmuls, lower triangle only
+    n_sets = 3
+    cpu_heads = 8
+
+    def setup(self, torch, dev):
+        from xpu_graph_amd import _lib
+
+        self.torch = torch
+        g = torch.Generator().manual_seed(0)
+        self.sets = [tuple(torch.randn(4, 32, 2048, 128, generator=g).bfloat16().to(dev) for _ in range(3)) for _ in range(self.n_sets)]
+        self.outs = [torch.empty_like(s[0]) for s in self.sets]
+        self.lib = _lib.lib()
+        self.st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        self.strides = (ctypes.c_int64 * 3)(32 * 2048 * 128, 2048 * 128, 128)
+        self.scale = ctypes.c_float(128**-0.5)
+
+    def op_call(self, i):
+        q, k, v = self.sets[i]
+        return self.torch.ops.xpu_ops.sdpa(q, k, v, True, 128**-0.5)
+
+    def abi_call(self, i):
+        q, k, v = self.sets[i]
+        s = self.strides
+        self.lib.xg_sdpa(_p(q), _p(k), _p(v), _p(self.outs[i]), 4, 32, 32, 2048, 2048, 128, s, s, s, s, self.scale, 1, 2, self.st)
+
+    def check(self, torch):
+        from oracle import eager
+
+        q, k, v = (t[:1, :4] for t in self.sets[0])
+        got = self.op_call(0)[:1, :4]
+        torch.testing.assert_close(got.float(), eager.causal_sdpa_eager(q.float(), k.float(), v.float()), rtol=1.6e-2, atol=8e-3)
+
+    def cpu_fn(self, torch):
+        from oracle import eager
+
+        g = torch.Generator().manual_seed(0)
+        q, k, v = (torch.randn(1, self.cpu_heads, 2048, 128, generator=g).bfloat16() for _ in range(3))
+        fn, how = _default_path_compile(eager.causal_sdpa_eager)
+        return (lambda: fn(q, k, v)), how + f", {self.cpu_heads} of 128 (batch, head) pairs"
+
+    @property
+    def cpu_work(self):
+        return self.work * self.cpu_heads / 128
+
+
+class LlamaBlockC5(Workload):
+    name = "C5 Llama decoder block bf16 B4 S2048 hidden4096 H32 inter11008, torch.compile(mi355x) end to end"
+    bound = "mfma"
+    dtype = "bf16"
+    unit = "TFLOP/s"
+    kernel = "whole compiled block (7 dense, attention, 3 norm / gate kernels, eager RoPE)"
+    work = 2 * 8192 * (4 * 4096 * 4096 + 3 * 4096 * 11008) + 4 * 4 * 32 * 2048 * 2048 * 128 // 2
+    n_sets = 1
+    cpu_tokens = 256
+
+    def setup(self, torch, dev):
+        from oracle import eager, inputs
+        from xpu_graph_amd import mi355x_compiler
+
+        self.torch = torch
+        self.x, self.p = inputs.c5_llama_block(device=dev)
+        self.names = sorted(self.p)
+        names = self.names
+
+        def block(x, *ws):
+            return eager.llama_block_eager(x, dict(zip(names, ws)), n_heads=32)
+
+        self.eager_fn = block
+        self.fn = torch.compile(block, backend=mi355x_compiler(), dynamic=False)
+        self.ws = [self.p[n] for n in names]
+
+    def op_call(self, i):
+        with self.torch.no_grad():
+            return self.fn(self.x, *self.ws)
+
+    abi_call = op_call
+
+    def check(self, torch):
+        got = self.op_call(0)
+        with torch.no_grad():
+            want = self.eager_fn(self.x, *self.ws)
+            self.eager_ms = _events_time(torch, lambda i: self.eager_fn(self.x, *self.ws), 1, 5, 2) * 1e3
+        assert (got.float() - want.float()).abs().mean().item() < 2e-2
+
+    def cpu_fn(self, torch):
+        from oracle import eager, inputs
+
+        x, p = inputs.c5_llama_block(B=1, S=self.cpu_tokens, device="cpu")
+        fn, how = _default_path_compile(lambda x: eager.llama_block_eager(x, p, n_heads=32))
+
+        def run():
+            with torch.no_grad():
+                return fn(x)
+
+        return run, how + f", B1 S{self.cpu_tokens} (1/32 of the tokens)"
+
+    @property
+    def cpu_work(self):
+        t = self.cpu_tokens
+        return 2 * t * (4 * 4096 * 4096 + 3 * 4096 * 11008) + 4 * 32 * t * t * 128 // 2
+
+
 HEADLINE = AddLayerNormC2
-OTHERS = [RmsNormC1, SliceCatC3a, AddNC3b]
+OTHERS = [RmsNormC1, SliceCatC3a, AddNC3b, DenseC4, DenseFp8C4, SdpaC5, LlamaBlockC5]
 
 
 def run_workload(torch, dev, wl, steps, warmup, with_cpu=True):
@@ -281,8 +483,9 @@ def run_workload(torch, dev, wl, steps, warmup, with_cpu=True):
     wl.check(torch)
     peak = HBM_PEAK_GBPS if wl.bound == "hbm" else (FP8_PEAK_TFLOPS if wl.dtype == "fp8" else BF16_PEAK_TFLOPS)
     scale = 1e9 if wl.bound == "hbm" else 1e12
-    t_op = _wall_time(torch, wl.op_call, N_SETS, steps, warmup)
-    t_k = _events_time(torch, wl.abi_call, N_SETS, max(steps, 100), max(warmup, 20))
+    n_sets = getattr(wl, "n_sets", N_SETS)
+    t_op = _wall_time(torch, wl.op_call, n_sets, steps, warmup)
+    t_k = _events_time(torch, wl.abi_call, n_sets, max(steps, 100), max(warmup, 20))
     res = {
         "workload": wl.name,
         "dtype": wl.dtype,
@@ -304,12 +507,14 @@ def run_workload(torch, dev, wl, steps, warmup, with_cpu=True):
         fn, how = wl.cpu_fn(torch)
         t_cpu, n = _cpu_time(fn)
         res["cpu_baseline"] = {
-            "value": wl.work / t_cpu / scale,
+            "value": getattr(wl, "cpu_work", wl.work) / t_cpu / scale,
             "unit": res["unit"],
             "cores": torch.get_num_threads(),
             "kind": "port",
-            "sample": f"{n} timed runs of the full-size workload through {how}, median {t_cpu * 1e3:.2f} ms",
+            "sample": f"{n} timed runs of {'a bounded sample' if hasattr(wl, 'cpu_work') else 'the full-size workload'} through {how}, median {t_cpu * 1e3:.2f} ms",
         }
+    if hasattr(wl, "eager_ms"):
+        res["eager_gpu_ms"] = wl.eager_ms
     return res
 
 
@@ -330,7 +535,13 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py needs a GPU (the mi355x path has no CPU fallback)", file=sys.stderr)
         sys.exit(1)
+    import logging
+
     import xpu_graph_amd.ops  # noqa: F401
+
+    for handler in logging.getLogger("xpu_graph").handlers:  # stdout carries the one JSON line only
+        if isinstance(handler, logging.StreamHandler):
+            handler.setStream(sys.stderr)
 
     torch.set_num_threads(min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16"))))
     dev = torch.device("cuda:0")
