@@ -84,6 +84,7 @@ struct GemmParams {
   int act;
   int bias_f32;
   int tiles_m, tiles_n;
+  int pf_dist;  // how many slabs ahead the L2 warm-up touches run
 };
 
 // Compile-time loop: the body receives std::integral_constant indices, so every
@@ -472,9 +473,19 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
   for (int kt = 0; kt + 1 < KT; ++kt) {
     a_g += a_step;
     b_g += b_step;
-    slab(std::true_type{}, kt & 1, a_g, b_g, (int64_t)(kt + 2) * a_step, (int64_t)(kt + 2) * b_step, kt + 2 < KT);
-    asm volatile("s_waitcnt vmcnt(2)" ::: "memory");  // all but the two newest (the L2 touches) have landed
-    __syncthreads();                                   // ... and everybody else's
+    const bool do_pf = kt + p.pf_dist < KT;
+    slab(std::true_type{}, kt & 1, a_g, b_g, (int64_t)(kt + p.pf_dist) * a_step, (int64_t)(kt + p.pf_dist) * b_step, do_pf);
+    // Every direct load of the next slab must have landed; only the L2 touches, which are the newest
+    // memory reads of this wave, may stay in flight.  How many there are is uniform over the workgroup.
+    const int touches = do_pf ? (int)pf_a + (int)pf_b : 0;
+    if (touches == 2) {
+      asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
+    } else if (touches == 1) {
+      asm volatile("s_waitcnt vmcnt(1)" ::: "memory");
+    } else {
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
+    __syncthreads();  // ... and everybody else's
   }
   slab(std::false_type{}, (KT - 1) & 1, a_g, b_g, 0, 0, false);
   __syncthreads();  // the slabs are dead: the epilogue reuses LDS
@@ -642,6 +653,8 @@ inline GemmParams make_params(const void* a, const void* b, const void* bias, co
   p.act = act;
   p.bias_f32 = bias_f32 ? 1 : 0;
   p.tiles_m = (int)((M + BM - 1) / BM);
+  static const int pf_env = getenv("XG_GEMM_PF") ? atoi(getenv("XG_GEMM_PF")) : 2;
+  p.pf_dist = pf_env < 1 ? 1 : (pf_env > 16 ? 16 : pf_env);
   p.tiles_n = (int)((N + BN - 1) / BN);
   return p;
 }

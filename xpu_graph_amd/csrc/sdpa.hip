@@ -143,32 +143,43 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
     });
   }
 
-  // ---- direct-load bookkeeping: load i of this wave fills LDS bytes [(wave*LPW+i)*1024, +1024) of a tile
+  // ---- direct-load bookkeeping: load i of this wave fills LDS bytes [(wave*LPW+i)*1024, +1024) of a tile.
+  // The global address is a workgroup-uniform tile base plus a 32-bit per-lane offset that does not change
+  // from tile to tile (row within the tile x row stride + swizzled chunk), so a step costs no address math.
   const char* kg = reinterpret_cast<const char*>(p.k) + ((int64_t)b * p.ks[0] + (int64_t)hkv * p.ks[1]) * 2;
   const char* vg = reinterpret_cast<const char*>(p.v) + ((int64_t)b * p.vs[0] + (int64_t)hkv * p.vs[1]) * 2;
-  int ld_row[LPW], ld_kc[LPW], ld_vc[LPW];
-  static_for<LPW>([&](auto I) {
-    constexpr int i = decltype(I)::value;
-    const int pos = (wave * LPW + i) * 1024 + lane * 16;
-    const int row = pos / RB, pc = (pos % RB) >> 4;
-    ld_row[i] = row;
-    ld_kc[i] = (pc ^ swz_k<D>(row)) << 4;
-    ld_vc[i] = (pc ^ swz_v<D>(row)) << 4;
-  });
-  const int64_t k_row_bytes = p.ks[2] * 2, v_row_bytes = p.vs[2] * 2;
-  auto issue = [&](int j, int stage) {
+  const uint32_t k_row_bytes = (uint32_t)(p.ks[2] * 2), v_row_bytes = (uint32_t)(p.vs[2] * 2);
+  uint32_t k_off[LPW], v_off[LPW];
+  auto lane_offsets = [&](int rows_valid) {  // rows at or past rows_valid repeat the last valid row; they are masked below
     static_for<LPW>([&](auto I) {
       constexpr int i = decltype(I)::value;
-      int r = j * BKV + ld_row[i];
-      r = r < p.Skv ? r : p.Skv - 1;  // rows past the end repeat the last key; they are masked below
+      const int pos = (wave * LPW + i) * 1024 + lane * 16;
+      int row = pos / RB;
+      const int pc = (pos % RB) >> 4;
+      const int kc = (pc ^ swz_k<D>(row)) << 4, vc = (pc ^ swz_v<D>(row)) << 4;
+      row = row < rows_valid ? row : rows_valid - 1;
+      k_off[i] = (uint32_t)row * k_row_bytes + kc;
+      v_off[i] = (uint32_t)row * v_row_bytes + vc;
+    });
+  };
+  lane_offsets(BKV);
+  const int n_tiles_all = (p.Skv + BKV - 1) / BKV;
+  const int rows_last = p.Skv - (n_tiles_all - 1) * BKV;  // valid rows of the last key tile
+  auto issue = [&](int j, auto STAGE_IDX) {
+    constexpr int stage = decltype(STAGE_IDX)::value;
+    if (j == n_tiles_all - 1 && rows_last < BKV) lane_offsets(rows_last);  // at most once: it is the last tile
+    const char* kt = kg + (int64_t)j * BKV * k_row_bytes;
+    const char* vt = vg + (int64_t)j * BKV * v_row_bytes;
+    static_for<LPW>([&](auto I) {
+      constexpr int i = decltype(I)::value;
       char* kd = smem + stage * STAGE + (wave * LPW + i) * 1024;
-      __builtin_amdgcn_global_load_lds((const gvoid*)(kg + r * k_row_bytes + ld_kc[i]), (lvoid*)kd, 16, 0, 0);
-      __builtin_amdgcn_global_load_lds((const gvoid*)(vg + r * v_row_bytes + ld_vc[i]), (lvoid*)(kd + TILE), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((const gvoid*)(kt + k_off[i]), (lvoid*)kd, 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((const gvoid*)(vt + v_off[i]), (lvoid*)(kd + TILE), 16, 0, 0);
     });
   };
 
   // ---- number of key tiles this workgroup visits
-  int n_steps = (p.Skv + BKV - 1) / BKV;
+  int n_steps = n_tiles_all;
   if (p.causal) {
     int q_last = q0 + BQ - 1;
     q_last = q_last < p.Sq ? q_last : p.Sq - 1;
@@ -177,24 +188,29 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
   }
   const int qw_min = q0 + 32 * wave, qw_max = qw_min + 31;
 
-  // ---- per-lane LDS read offsets
+  // ---- per-lane parts of the LDS read addresses (everything else is a compile-time offset)
   const int kx = swz_k<D>(l32);  // same for both 32-row tiles of a K tile
   const int a16 = lane & 15, b16 = (lane >> 4) & 1;
+  const int v_row = 4 * h + (a16 >> 2);                          // key row (mod 16) this lane addresses for the V^T fragments
+  const int v_chunk = 2 * b16 + ((a16 & 3) >> 1), v_sub = (a16 & 1) << 3;
 
   f32x16 o_acc[DT];
   static_for<DT>([&](auto I) {
     o_acc[decltype(I)::value] = f32x16{0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   });
+  // m_run is the exponent reference of the running sums, not necessarily the true running maximum: it is
+  // moved only when a row's maximum exceeds it by more than kSlack (in log2 units), so probabilities stay
+  // below 2^kSlack and the accumulator rescale is skipped on most tiles.  The result is the same quotient.
+  constexpr float kSlack = 8.f;
   float m_run = -INFINITY, l_run = 0.f;
 
-  issue(0, 0);
-  for (int j = 0; j < n_steps; ++j) {
-    const int stage = j & 1;
+  auto step = [&](auto STAGE_IDX, int j) {
+    constexpr int stage = decltype(STAGE_IDX)::value;
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's part of tile j has landed
     __syncthreads();                                  // ... everyone's has, and everyone is done with tile j-1
-    if (j + 1 < n_steps) issue(j + 1, stage ^ 1);
+    if (j + 1 < n_steps) issue(j + 1, std::integral_constant<int, stage ^ 1>{});
     const int kv0 = j * BKV;
-    if (p.causal && kv0 > qw_max) continue;  // this wave's queries see none of these keys (wave-uniform)
+    if (p.causal && kv0 > qw_max) return;  // this wave's queries see none of these keys (wave-uniform)
 
     const char* k_s = smem + stage * STAGE;
     const char* v_s = k_s + TILE;
@@ -206,8 +222,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
       s[t] = f32x16{0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
       static_for<KK>([&](auto KI) {
         constexpr int kk = decltype(KI)::value;
-        const int off = (32 * t + l32) * RB + (((2 * kk + h) ^ kx) << 4);
-        const V8 kf = *reinterpret_cast<const V8*>(k_s + off);
+        const int off = l32 * RB + (((2 * kk + h) ^ kx) << 4);
+        const V8 kf = *reinterpret_cast<const V8*>(k_s + 32 * t * RB + off);
         s[t] = mma(kf, qf[kk], s[t]);
       });
     });
@@ -238,7 +254,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
     }
     float mt = mx * cc;
     mt = fmaxf(mt, __shfl_xor(mt, 32, kWave));
-    const float m_new = fmaxf(m_run, mt);
+    const float m_new = mt > m_run + kSlack ? mt : m_run;  // -inf + slack = -inf: the first visible key always moves it
     const float m_use = m_new == -INFINITY ? 0.f : m_new;  // a row with no visible key yet
     const float alpha = __builtin_amdgcn_exp2f(m_run - m_use);
     float psum = 0.f;
@@ -251,11 +267,12 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
         psum += e;
       });
     });
-    l_run = l_run * alpha + psum;
-    m_run = m_new;
-    if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {
+    if (__builtin_amdgcn_ballot_w64(m_new != m_run) != 0) {
+      l_run *= alpha;
       static_for<DT>([&](auto I) { o_acc[decltype(I)::value] *= alpha; });
     }
+    l_run += psum;
+    m_run = m_new;
 
     // O^T += V^T P^T.  k-step (t, st) uses keys 32t + 16st + {4h..4h+3} and 32t + 16st + 8 + {4h..4h+3}:
     // exactly registers 8st..8st+7 of s[t] in this lane.
@@ -272,17 +289,22 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
           constexpr int dt = decltype(DI)::value;
           // lane a16 of a 16-lane group addresses key row (a16/4), head-dim columns 4(a16%4)..+3 of the group's
           // 16 columns; the transposing read returns, for result slot e, key row e at column a16.
-          const int r0 = 32 * t + 16 * st + 4 * h + (a16 >> 2);
-          const int r1 = r0 + 8;
-          const int chunk = 4 * dt + 2 * b16 + ((a16 & 3) >> 1);
-          const int sub = (a16 & 1) << 3;
-          const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(v_s + r0 * RB + ((chunk ^ swz_v<D>(r0)) << 4) + sub));
-          const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(v_s + r1 * RB + ((chunk ^ swz_v<D>(r1)) << 4) + sub));
+          const int off0 = v_row * RB + (((4 * dt + v_chunk) ^ swz_v<D>(v_row)) << 4) + v_sub;
+          const int off1 = (v_row + 8) * RB + (((4 * dt + v_chunk) ^ swz_v<D>(v_row + 8)) << 4) + v_sub;
+          const char* base = v_s + (32 * t + 16 * st) * RB;
+          const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(base + off0));
+          const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(base + off1));
           const s16x8 both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
           o_acc[dt] = mma(__builtin_bit_cast(V8, both), pf, o_acc[dt]);
         });
       });
     });
+  };
+
+  issue(0, std::integral_constant<int, 0>{});
+  for (int j = 0; j < n_steps; j += 2) {
+    step(std::integral_constant<int, 0>{}, j);
+    if (j + 1 < n_steps) step(std::integral_constant<int, 1>{}, j + 1);
   }
 
   // ---- normalise and write: O[q][d] = O^T[d][q] / l.  The tile is parked in LDS (per wave) so that
@@ -356,6 +378,8 @@ extern "C" int xg_sdpa(const void* q, const void* k, const void* v, void* out, i
     p.vs[i] = v_strides[i];
     p.os[i] = o_strides[i];
   }
+  // per-lane tile offsets are 32-bit: 64 rows of K / V must span less than 2 GiB
+  if (k_strides[2] > (1 << 23) || v_strides[2] > (1 << 23)) return XG_ERR_TOO_LARGE;
   p.q = q;
   p.k = k;
   p.v = v;
