@@ -12,12 +12,15 @@
 //
 // Two kernels share everything but the way a slab reaches LDS:
 //  * gemm_dma_kernel (K a multiple of the slab): `global_load_lds_dwordx4` moves
-//    memory straight into LDS, 1 KiB per wavefront instruction.  The loads of
-//    slab t+1 are issued a few at a time BETWEEN the MFMAs of slab t, as are the
-//    LDS fragment reads of the next k-step, so the matrix pipe never waits for
-//    the wavefront to finish issuing memory instructions.  One 4-byte touch per
-//    128-byte line warms L2 for slab t+2, because one slab of math is too short
-//    to cover an L2 miss.
+//    memory straight into LDS, 1 KiB per wavefront instruction.  The source is
+//    written in issue order: exactly one direct load and / or one LDS fragment
+//    read sits in front of each MFMA, so the matrix pipe never waits for the
+//    wavefront to finish issuing memory instructions.  The pipeline is rotated by
+//    one k-step: the wait-and-barrier that hands slab t+1 over sits in front of
+//    the LAST k-step of slab t (whose fragments are already in registers), so the
+//    first fragments of slab t+1 and the loads of slab t+2 go out under that
+//    step's MFMAs.  One 4-byte touch per 128-byte line warms L2 one slab further
+//    ahead, because one slab of math is too short to cover an L2 miss.
 //  * gemm_staged_kernel (any K % 8 == 0): slabs pass through registers, which
 //    lets the last, partial slab be zero-filled.
 //
@@ -65,9 +68,6 @@ constexpr int SMEM_BYTES = 2 * STAGE_BYTES;
 constexpr int kThreads = 256;
 constexpr int kXcds = 8;
 constexpr int kGroupM = 8;
-#ifndef XG_GEMM_LOAD_STEPS
-#define XG_GEMM_LOAD_STEPS 1
-#endif
 
 enum class BLayout { KMajor, NMajor };  // B stored [N, K] (K contiguous) or [K, N] (N contiguous)
 
@@ -184,44 +184,45 @@ struct Lane {
   }
 };
 
-// Fragments of k-step ks from the slabs at a_s / b_s.
-template <typename T, BLayout BL>
-__device__ __forceinline__ void read_frags(const Lane& L, const char* a_s, const char* b_s, int ks, Frag<T> (&fa)[4],
-                                           Frag<T> (&fb)[4]) {
+// Unit U (0..3: A tile row U, 4..7: B tile column U-4) of the fragments of k-step ks from the slabs at a_s / b_s.
+template <typename T, BLayout BL, int U>
+__device__ __forceinline__ void read_unit(const Lane& L, const char* a_s, const char* b_s, int ks, Frag<T> (&fa)[4],
+                                          Frag<T> (&fb)[4]) {
   if constexpr (Elem<T>::BYTES == 2) {
     const int ch = ((ks * 2 + L.half) ^ L.fsw) << 4;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) fa[i].v = *reinterpret_cast<const u32x4*>(a_s + L.a_row[i] + ch);
-    if constexpr (BL == BLayout::KMajor) {
-#pragma unroll
-      for (int j = 0; j < 4; ++j) fb[j].v = *reinterpret_cast<const u32x4*>(b_s + L.b_row[j] + ch);
+    if constexpr (U < 4) {
+      fa[U].v = *reinterpret_cast<const u32x4*>(a_s + L.a_row[U] + ch);
+    } else if constexpr (BL == BLayout::KMajor) {
+      fb[U - 4].v = *reinterpret_cast<const u32x4*>(b_s + L.b_row[U - 4] + ch);
     } else {
       // slab is [64 k][256 n]: a 16-lane group reads a 4(k) x 16(n) block and gets it back transposed
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int gran = ((L.wn * 4 + j) ^ L.tr_sw) & 7;
-        const int col = (gran << 6) + (L.blk << 5) + ((L.p16 & 3) << 3);
-        const int row0 = ks * 16 + L.half * 8 + (L.p16 >> 2);
-        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(b_s + row0 * (BN * 2) + col));
-        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(b_s + (row0 + 4) * (BN * 2) + col));
-        const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
-        fb[j].v = u32x4{l2.x, l2.y, h2.x, h2.y};
-      }
+      constexpr int j = U - 4;
+      const int gran = ((L.wn * 4 + j) ^ L.tr_sw) & 7;
+      const int col = (gran << 6) + (L.blk << 5) + ((L.p16 & 3) << 3);
+      const int row0 = ks * 16 + L.half * 8 + (L.p16 >> 2);
+      const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(b_s + row0 * (BN * 2) + col));
+      const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(b_s + (row0 + 4) * (BN * 2) + col));
+      const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
+      fb[j].v = u32x4{l2.x, l2.y, h2.x, h2.y};
     }
   } else {
     // fp8: a k-step is 64 elements; each lane half supplies 32 consecutive bytes (2 chunks)
     const int ch0 = ((ks * 4 + L.half * 2) ^ L.fsw) << 4, ch1 = ((ks * 4 + L.half * 2 + 1) ^ L.fsw) << 4;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      fa[i].lo = *reinterpret_cast<const u32x4*>(a_s + L.a_row[i] + ch0);
-      fa[i].hi = *reinterpret_cast<const u32x4*>(a_s + L.a_row[i] + ch1);
-    }
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      fb[j].lo = *reinterpret_cast<const u32x4*>(b_s + L.b_row[j] + ch0);
-      fb[j].hi = *reinterpret_cast<const u32x4*>(b_s + L.b_row[j] + ch1);
+    if constexpr (U < 4) {
+      fa[U].lo = *reinterpret_cast<const u32x4*>(a_s + L.a_row[U] + ch0);
+      fa[U].hi = *reinterpret_cast<const u32x4*>(a_s + L.a_row[U] + ch1);
+    } else {
+      fb[U - 4].lo = *reinterpret_cast<const u32x4*>(b_s + L.b_row[U - 4] + ch0);
+      fb[U - 4].hi = *reinterpret_cast<const u32x4*>(b_s + L.b_row[U - 4] + ch1);
     }
   }
+}
+
+// All fragments of k-step ks.
+template <typename T, BLayout BL>
+__device__ __forceinline__ void read_frags(const Lane& L, const char* a_s, const char* b_s, int ks, Frag<T> (&fa)[4],
+                                           Frag<T> (&fb)[4]) {
+  static_for<8>([&](auto U) { read_unit<T, BL, decltype(U)::value>(L, a_s, b_s, ks, fa, fb); });
 }
 
 template <typename T>
@@ -354,10 +355,6 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
   constexpr int EB = Elem<T>::BYTES;
   constexpr int KSTEPS = Elem<T>::KSTEPS;
   constexpr int SLAB_K = ROW_BYTES / EB;
-  // The next slab's 16 direct loads all go out during the first k-steps of the current slab, so that
-  // the remaining steps cover their latency before the wait at the slab's end.
-  constexpr int LOAD_STEPS = XG_GEMM_LOAD_STEPS;
-  constexpr int PER_STEP = 16 / LOAD_STEPS;
   static_assert(BL == BLayout::KMajor || EB == 2, "the transposing LDS read is wired for 16-bit elements only");
 
   int tm, tn;
@@ -394,17 +391,25 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
   }
   const int64_t a_step = ROW_BYTES;
   const int64_t b_step = BL == BLayout::KMajor ? (int64_t)ROW_BYTES : (int64_t)SLAB_K * p.ldb * EB;
+  const int wave_u = __builtin_amdgcn_readfirstlane(L.wave);  // LDS destinations of direct loads are wavefront-uniform
+  const char* const a_base = reinterpret_cast<const char*>(p.A);
+  const char* const b_base = reinterpret_cast<const char*>(p.B);
 
-  // load number q (0..15) of the slab whose operand bases are a_g / b_g, into `stage`
-  auto issue = [&](int q, const char* a_g, const char* b_g, int stage) {
-    char* dst = smem + stage * STAGE_BYTES + L.wave * 1024 + (q & 7) * 4096 + (q < 8 ? 0 : SLAB_BYTES);
-    const char* src = q < 8 ? a_g + a_off[q & 7] : b_g + b_off[q & 7];
-    __builtin_amdgcn_global_load_lds((const gvoid*)src, (lvoid*)dst, 16, 0, 0);
+  // load number Q (0..15) of slab kt into `stage`: uniform slab base + 32-bit lane offset
+  auto issue = [&](auto Q, int kt, int stage) {
+    constexpr int q = decltype(Q)::value;
+    char* dst = smem + stage * STAGE_BYTES + wave_u * 1024 + (q & 7) * 4096 + (q < 8 ? 0 : SLAB_BYTES);
+    // The empty asm keeps the lane offset a 32-bit register up to this point, so that the load takes the
+    // "uniform 64-bit base + 32-bit lane offset" addressing form instead of a 64-bit add per lane.
+    uint32_t off = q < 8 ? a_off[q & 7] : b_off[q & 7];
+    asm volatile("" : "+v"(off));
+    const char* base = q < 8 ? a_base + kt * a_step : b_base + kt * b_step;
+    __builtin_amdgcn_global_load_lds((const gvoid*)(base + off), (lvoid*)dst, 16, 0, 0);
   };
 
-  // L2 warm-up two slabs ahead: one 4-byte touch per 128-byte line.  A row panel is shared by the
-  // tiles of a tile row and a B panel by the tiles of a tile column that run on the same XCD at
-  // the same time, so only one tile of each group needs to touch them.
+  // L2 warm-up: one 4-byte touch per 128-byte line.  A row panel is shared by the tiles of a tile
+  // row and a B panel by the tiles of a tile column that run on the same XCD at the same time, so
+  // only one tile of each group needs to touch them.
   const bool pf_a = (tn & 3) == 0, pf_b = (tm & 7) == 0;
   const char* pfa_ptr;
   const char* pfb_ptr;
@@ -426,68 +431,105 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
 
   f32x16 acc[4][4];
   zero_acc(acc);
+  Frag<T> fa[2][4], fb[2][4];
+  static_assert(KSTEPS % 2 == 0, "the fragment double buffer assumes that a slab starts in buffer 0");
 
+  // Issue plan of the 16 direct loads of a slab.  The address unit of a CU moves 64 bytes per clock, so
+  // the 4 x 16 loads of a slab keep it busy for half a slab of math, and the instruction stream is in
+  // order: a load that finds the queue full holds up the MFMAs behind it.  The loads are therefore spread
+  // out, the first half in the last k-step of slab t-2 (right after the barrier that frees the stage), the
+  // rest early in slab t-1, so that at least one k-step of math (16-bit types) separates the last load
+  // from the barrier that needs it.  Measured on C4: K-contiguous weights are fastest with a load in
+  // front of every second MFMA; for the [K, N] layout, whose transposing fragment reads keep LDS busier,
+  // the loads must stay clear of the MFMAs that carry the fragment reads (the first eight of a k-step).
+  struct Plan {
+    int early[16];    // load to issue in front of MFMA idx of the LAST k-step (of slab t-2), or -1
+    int late[3][16];  // same for k-steps 0..2 (of slab t-1)
+    int n_early;
+  };
+  constexpr Plan plan = []() constexpr {
+    Plan P{};
+    for (int i = 0; i < 16; ++i) {
+      P.early[i] = -1;
+      for (int k = 0; k < 3; ++k) P.late[k][i] = -1;
+    }
+    int q = 0;
+    if (BL == BLayout::KMajor) {
+      for (int i = 0; i < 16; i += 2) P.early[i] = q++;
+      for (int i = 0; i < 16; i += 2) P.late[0][i] = q++;
+    } else {
+      for (int i = 8; i < 16; ++i) P.early[i] = q++;
+      for (int i = 8; i < 12; ++i) P.late[0][i] = q++;
+      for (int i = 8; i < 12; ++i) P.late[1][i] = q++;
+    }
+    P.n_early = 8;
+    return P;
+  }();
+  static_assert(KSTEPS >= 2 && (BL == BLayout::KMajor || KSTEPS >= 3), "late loads need a k-step that is not the last");
   const int KT = p.K / SLAB_K;
-  const char* a_g = reinterpret_cast<const char*>(p.A);
-  const char* b_g = reinterpret_cast<const char*>(p.B);
-  static_for<16>([&](auto Q) { issue(decltype(Q)::value, a_g, b_g, 0); });
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  static_for<16>([&](auto Q) { issue(Q, 0, 0); });
+  if (KT > 1) {
+    static_for<plan.n_early>([&](auto Q) { issue(Q, 1, 1); });
+    static_assert(plan.n_early == 8, "the wait below leaves exactly the early loads of slab 1 in flight");
+    asm volatile("s_waitcnt vmcnt(8)" ::: "memory");  // slab 0 has landed
+  } else {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  }
   __syncthreads();
+  read_frags<T, BL>(L, smem, smem + SLAB_BYTES, 0, fa[0], fb[0]);
 
-  // One slab of math.  PREFETCH: also issue the next slab's direct loads, spread over the k-steps.
-  auto slab = [&](auto PREFETCH, int stage, const char* a_next, const char* b_next, int64_t pf_koff, int64_t pf_boff, bool do_pf) {
-    constexpr bool prefetch = decltype(PREFETCH)::value;
+  // One slab of math, written in issue order.  NEXT: slab kt+1 exists (hand it over in front of the last
+  // k-step and fetch its first fragments under that step); NEXT2: slab kt+2 exists (its direct loads go
+  // into this slab's stage, which is free once every wavefront is past the barrier).
+  auto slab = [&](auto NEXT, auto NEXT2, int kt) {
+    constexpr bool next = decltype(NEXT)::value, next2 = decltype(NEXT2)::value;
+    const int stage = kt & 1;
     const char* a_s = smem + stage * STAGE_BYTES;
     const char* b_s = a_s + SLAB_BYTES;
-    Frag<T> fa[2][4], fb[2][4];
-    read_frags<T, BL>(L, a_s, b_s, 0, fa[0], fb[0]);
-    __builtin_amdgcn_sched_barrier(0);
+    const char* a_n = smem + (stage ^ 1) * STAGE_BYTES;
+    const char* b_n = a_n + SLAB_BYTES;
     static_for<KSTEPS>([&](auto KS) {
       constexpr int ks = decltype(KS)::value;
-      constexpr bool more = ks + 1 < KSTEPS;
-      if constexpr (more) read_frags<T, BL>(L, a_s, b_s, ks + 1, fa[(ks + 1) & 1], fb[(ks + 1) & 1]);
-      if constexpr (prefetch && ks < LOAD_STEPS)
-        static_for<PER_STEP>([&](auto Q) { issue(ks * PER_STEP + decltype(Q)::value, a_next, b_next, stage ^ 1); });
-      if constexpr (prefetch && ks == LOAD_STEPS) {
-        pf_sink ^= pf_va ^ pf_vb;  // last slab's touches: long since returned
-        if (do_pf && pf_a) pf_va = *reinterpret_cast<const uint32_t*>(pfa_ptr + pf_koff);
-        if (do_pf && pf_b) pf_vb = *reinterpret_cast<const uint32_t*>(pfb_ptr + pf_boff);
+      constexpr bool last_step = ks + 1 == KSTEPS;
+      if constexpr (last_step && next) {
+        // This step's fragments are in registers, so nothing of slab kt is read from LDS any more, and
+        // every direct load of slab kt+1 must have landed (the L2 touches are older than its last loads).
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
       }
-      mma_step<T>(acc, fa[ks & 1], fb[ks & 1]);
-      // Issue order inside the step: the next step's LDS reads and the direct loads are threaded
-      // between pairs of MFMAs instead of queueing in front of them.
-      constexpr int reads = more ? (EB == 1 ? 16 : (BL == BLayout::KMajor ? 8 : 12)) : 0;
-      constexpr int loads = (prefetch && ks < LOAD_STEPS) ? PER_STEP : 0;
-      static_for<8>([&](auto R) {
-        constexpr int r = decltype(R)::value;
-        constexpr int rd = reads / 8 + (r < reads % 8 ? 1 : 0);
-        constexpr int ld = loads / 8 + (r < loads % 8 ? 1 : 0);
-        if constexpr (rd > 0) __builtin_amdgcn_sched_group_barrier(0x100, rd, 0);  // LDS reads
-        if constexpr (ld > 0) __builtin_amdgcn_sched_group_barrier(0x020, ld, 0);  // memory reads
-        __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);                         // MFMA
+      static_for<16>([&](auto IDX) {
+        constexpr int idx = decltype(IDX)::value;
+        constexpr int i = idx / 4, j = idx % 4;
+        if constexpr (!last_step) {
+          if constexpr (idx < 8) read_unit<T, BL, idx>(L, a_s, b_s, ks + 1, fa[(ks + 1) & 1], fb[(ks + 1) & 1]);
+        } else if constexpr (next) {
+          if constexpr (idx < 8) read_unit<T, BL, idx>(L, a_n, b_n, 0, fa[0], fb[0]);
+        }
+        // direct loads: the rest of slab kt+1 early in this slab, the head of slab kt+2 after the barrier
+        if constexpr (next && !last_step) {
+          constexpr int q = plan.late[ks < 3 ? ks : 0][idx];
+          if constexpr (q >= 0 && q < 16) issue(std::integral_constant<int, (q >= 0 ? q : 0)>{}, kt + 1, stage ^ 1);
+        }
+        if constexpr (next2 && last_step) {
+          constexpr int q = plan.early[idx];
+          if constexpr (q >= 0) issue(std::integral_constant<int, (q >= 0 ? q : 0)>{}, kt + 2, stage);
+        }
+        acc[i][j] = mma(fb[ks & 1][j], fa[ks & 1][i], acc[i][j]);
+        __builtin_amdgcn_sched_barrier(0);  // keep the issue order of the source
       });
-      __builtin_amdgcn_sched_barrier(0);  // keep each step's reads and math inside the step
     });
+    if constexpr (next2) {
+      pf_sink ^= pf_va ^ pf_vb;  // the previous touches: long since returned
+      const bool do_pf = kt + 1 + p.pf_dist < KT;
+      if (do_pf && pf_a) pf_va = *reinterpret_cast<const uint32_t*>(pfa_ptr + (int64_t)(kt + 1 + p.pf_dist) * a_step);
+      if (do_pf && pf_b) pf_vb = *reinterpret_cast<const uint32_t*>(pfb_ptr + (int64_t)(kt + 1 + p.pf_dist) * b_step);
+    }
   };
 
-  for (int kt = 0; kt + 1 < KT; ++kt) {
-    a_g += a_step;
-    b_g += b_step;
-    const bool do_pf = kt + p.pf_dist < KT;
-    slab(std::true_type{}, kt & 1, a_g, b_g, (int64_t)(kt + p.pf_dist) * a_step, (int64_t)(kt + p.pf_dist) * b_step, do_pf);
-    // Every direct load of the next slab must have landed; only the L2 touches, which are the newest
-    // memory reads of this wave, may stay in flight.  How many there are is uniform over the workgroup.
-    const int touches = do_pf ? (int)pf_a + (int)pf_b : 0;
-    if (touches == 2) {
-      asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
-    } else if (touches == 1) {
-      asm volatile("s_waitcnt vmcnt(1)" ::: "memory");
-    } else {
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    }
-    __syncthreads();  // ... and everybody else's
-  }
-  slab(std::false_type{}, (KT - 1) & 1, a_g, b_g, 0, 0, false);
+  for (int kt = 0; kt + 2 < KT; ++kt) slab(std::true_type{}, std::true_type{}, kt);
+  if (KT > 1) slab(std::true_type{}, std::false_type{}, KT - 2);
+  slab(std::false_type{}, std::false_type{}, KT - 1);
   __syncthreads();  // the slabs are dead: the epilogue reuses LDS
 
   if (pf_sink == 0x9e3779b9u && pf_va == 0x7f4a7c15u) reinterpret_cast<uint32_t*>(p.out)[0] = pf_vb;  // keeps the touches alive
