@@ -434,103 +434,162 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
   Frag<T> fa[2][4], fb[2][4];
   static_assert(KSTEPS % 2 == 0, "the fragment double buffer assumes that a slab starts in buffer 0");
 
-  // Issue plan of the 16 direct loads of a slab.  The address unit of a CU moves 64 bytes per clock, so
-  // the 4 x 16 loads of a slab keep it busy for half a slab of math, and the instruction stream is in
-  // order: a load that finds the queue full holds up the MFMAs behind it.  The loads are therefore spread
-  // out, the first half in the last k-step of slab t-2 (right after the barrier that frees the stage), the
-  // rest early in slab t-1, so that at least one k-step of math (16-bit types) separates the last load
-  // from the barrier that needs it.  Measured on C4: K-contiguous weights are fastest with a load in
-  // front of every second MFMA; for the [K, N] layout, whose transposing fragment reads keep LDS busier,
-  // the loads must stay clear of the MFMAs that carry the fragment reads (the first eight of a k-step).
-  struct Plan {
-    int early[16];    // load to issue in front of MFMA idx of the LAST k-step (of slab t-2), or -1
-    int late[3][16];  // same for k-steps 0..2 (of slab t-1)
-    int n_early;
-  };
-  constexpr Plan plan = []() constexpr {
-    Plan P{};
-    for (int i = 0; i < 16; ++i) {
-      P.early[i] = -1;
-      for (int k = 0; k < 3; ++k) P.late[k][i] = -1;
-    }
-    int q = 0;
-    if (BL == BLayout::KMajor) {
-      for (int i = 0; i < 16; i += 2) P.early[i] = q++;
-      for (int i = 0; i < 16; i += 2) P.late[0][i] = q++;
-    } else {
-      for (int i = 8; i < 16; ++i) P.early[i] = q++;
-      for (int i = 8; i < 12; ++i) P.late[0][i] = q++;
-      for (int i = 8; i < 12; ++i) P.late[1][i] = q++;
-    }
-    P.n_early = 8;
-    return P;
-  }();
-  static_assert(KSTEPS >= 2 && (BL == BLayout::KMajor || KSTEPS >= 3), "late loads need a k-step that is not the last");
   const int KT = p.K / SLAB_K;
-  static_for<16>([&](auto Q) { issue(Q, 0, 0); });
-  if (KT > 1) {
-    static_for<plan.n_early>([&](auto Q) { issue(Q, 1, 1); });
-    static_assert(plan.n_early == 8, "the wait below leaves exactly the early loads of slab 1 in flight");
-    asm volatile("s_waitcnt vmcnt(8)" ::: "memory");  // slab 0 has landed
-  } else {
+  if constexpr (BL == BLayout::NMajor) {
+    // ---- [K, N] weights: the transposing fragment reads keep LDS close to saturated, and direct loads
+    // that share a k-step with them stall.  Measured best here: all 16 loads of slab t+1 go out in the
+    // first k-step of slab t, one barrier at the end of the slab, the compiler's issue order inside a step.
+    static_for<16>([&](auto Q) { issue(Q, 0, 0); });
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  }
-  __syncthreads();
-  read_frags<T, BL>(L, smem, smem + SLAB_BYTES, 0, fa[0], fb[0]);
-
-  // One slab of math, written in issue order.  NEXT: slab kt+1 exists (hand it over in front of the last
-  // k-step and fetch its first fragments under that step); NEXT2: slab kt+2 exists (its direct loads go
-  // into this slab's stage, which is free once every wavefront is past the barrier).
-  auto slab = [&](auto NEXT, auto NEXT2, int kt) {
-    constexpr bool next = decltype(NEXT)::value, next2 = decltype(NEXT2)::value;
-    const int stage = kt & 1;
-    const char* a_s = smem + stage * STAGE_BYTES;
-    const char* b_s = a_s + SLAB_BYTES;
-    const char* a_n = smem + (stage ^ 1) * STAGE_BYTES;
-    const char* b_n = a_n + SLAB_BYTES;
-    static_for<KSTEPS>([&](auto KS) {
-      constexpr int ks = decltype(KS)::value;
-      constexpr bool last_step = ks + 1 == KSTEPS;
-      if constexpr (last_step && next) {
-        // This step's fragments are in registers, so nothing of slab kt is read from LDS any more, and
-        // every direct load of slab kt+1 must have landed (the L2 touches are older than its last loads).
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();
-      }
-      static_for<16>([&](auto IDX) {
-        constexpr int idx = decltype(IDX)::value;
-        constexpr int i = idx / 4, j = idx % 4;
-        if constexpr (!last_step) {
-          if constexpr (idx < 8) read_unit<T, BL, idx>(L, a_s, b_s, ks + 1, fa[(ks + 1) & 1], fb[(ks + 1) & 1]);
-        } else if constexpr (next) {
-          if constexpr (idx < 8) read_unit<T, BL, idx>(L, a_n, b_n, 0, fa[0], fb[0]);
+    __syncthreads();
+    auto slab = [&](auto PREFETCH, int kt) {
+      constexpr bool prefetch = decltype(PREFETCH)::value;
+      const int stage = kt & 1;
+      const char* a_s = smem + stage * STAGE_BYTES;
+      const char* b_s = a_s + SLAB_BYTES;
+      read_frags<T, BL>(L, a_s, b_s, 0, fa[0], fb[0]);
+      __builtin_amdgcn_sched_barrier(0);
+      static_for<KSTEPS>([&](auto KS) {
+        constexpr int ks = decltype(KS)::value;
+        constexpr bool more = ks + 1 < KSTEPS;
+        if constexpr (more) read_frags<T, BL>(L, a_s, b_s, ks + 1, fa[(ks + 1) & 1], fb[(ks + 1) & 1]);
+        if constexpr (prefetch && ks == 0) static_for<16>([&](auto Q) { issue(Q, kt + 1, stage ^ 1); });
+        if constexpr (prefetch && ks == 1) {
+          pf_sink ^= pf_va ^ pf_vb;  // the previous touches: long since returned
+          const bool do_pf = kt + p.pf_dist < KT;
+          if (do_pf && pf_a) pf_va = *reinterpret_cast<const uint32_t*>(pfa_ptr + (int64_t)(kt + p.pf_dist) * a_step);
+          if (do_pf && pf_b) pf_vb = *reinterpret_cast<const uint32_t*>(pfb_ptr + (int64_t)(kt + p.pf_dist) * b_step);
         }
-        // direct loads: the rest of slab kt+1 early in this slab, the head of slab kt+2 after the barrier
-        if constexpr (next && !last_step) {
-          constexpr int q = plan.late[ks < 3 ? ks : 0][idx];
-          if constexpr (q >= 0 && q < 16) issue(std::integral_constant<int, (q >= 0 ? q : 0)>{}, kt + 1, stage ^ 1);
-        }
-        if constexpr (next2 && last_step) {
-          constexpr int q = plan.early[idx];
-          if constexpr (q >= 0) issue(std::integral_constant<int, (q >= 0 ? q : 0)>{}, kt + 2, stage);
-        }
-        acc[i][j] = mma(fb[ks & 1][j], fa[ks & 1][i], acc[i][j]);
-        __builtin_amdgcn_sched_barrier(0);  // keep the issue order of the source
+        mma_step<T>(acc, fa[ks & 1], fb[ks & 1]);
+        // scheduling hints: thread the next step's LDS reads and the direct loads between pairs of MFMAs
+        constexpr int reads = more ? 12 : 0;
+        constexpr int loads = (prefetch && ks == 0) ? 16 : 0;
+        static_for<8>([&](auto R) {
+          constexpr int r = decltype(R)::value;
+          constexpr int rd = reads / 8 + (r < reads % 8 ? 1 : 0);
+          constexpr int ld = loads / 8 + (r < loads % 8 ? 1 : 0);
+          if constexpr (rd > 0) __builtin_amdgcn_sched_group_barrier(0x100, rd, 0);  // LDS reads
+          if constexpr (ld > 0) __builtin_amdgcn_sched_group_barrier(0x020, ld, 0);  // memory reads
+          __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);                         // MFMA
+        });
+        __builtin_amdgcn_sched_barrier(0);  // keep each step's reads and math inside the step
       });
-    });
-    if constexpr (next2) {
-      pf_sink ^= pf_va ^ pf_vb;  // the previous touches: long since returned
-      const bool do_pf = kt + 1 + p.pf_dist < KT;
-      if (do_pf && pf_a) pf_va = *reinterpret_cast<const uint32_t*>(pfa_ptr + (int64_t)(kt + 1 + p.pf_dist) * a_step);
-      if (do_pf && pf_b) pf_vb = *reinterpret_cast<const uint32_t*>(pfb_ptr + (int64_t)(kt + 1 + p.pf_dist) * b_step);
+    };
+    for (int kt = 0; kt + 1 < KT; ++kt) {
+      slab(std::true_type{}, kt);
+      // Every direct load of the next slab must have landed; only the L2 touches, which are the newest
+      // memory reads of this wave, may stay in flight.  How many there are is uniform over the workgroup.
+      const int touches = kt + p.pf_dist < KT ? (int)pf_a + (int)pf_b : 0;
+      if (touches == 2) {
+        asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
+      } else if (touches == 1) {
+        asm volatile("s_waitcnt vmcnt(1)" ::: "memory");
+      } else {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      }
+      __syncthreads();  // ... and everybody else's
     }
-  };
+    slab(std::false_type{}, KT - 1);
+    __syncthreads();  // the slabs are dead: the epilogue reuses LDS
+  } else {
+    // Issue plan of the 16 direct loads of a slab.  The address unit of a CU moves 64 bytes per clock, so
+    // the 4 x 16 loads of a slab keep it busy for half a slab of math, and the instruction stream is in
+    // order: a load that finds the queue full holds up the MFMAs behind it.  The loads are therefore spread
+    // out, the first half in the last k-step of slab t-2 (right after the barrier that frees the stage), the
+    // rest early in slab t-1, so that at least one k-step of math (16-bit types) separates the last load
+    // from the barrier that needs it.  Measured on C4: K-contiguous weights are fastest with a load in
+    // front of every second MFMA; for the [K, N] layout, whose transposing fragment reads keep LDS busier,
+    // the loads must stay clear of the MFMAs that carry the fragment reads (the first eight of a k-step).
+    struct Plan {
+      int early[16];    // load to issue in front of MFMA idx of the LAST k-step (of slab t-2), or -1
+      int late[3][16];  // same for k-steps 0..2 (of slab t-1)
+      int n_early;
+    };
+    constexpr Plan plan = []() constexpr {
+      Plan P{};
+      for (int i = 0; i < 16; ++i) {
+        P.early[i] = -1;
+        for (int k = 0; k < 3; ++k) P.late[k][i] = -1;
+      }
+      int q = 0;
+      if (BL == BLayout::KMajor) {
+        for (int i = 0; i < 16; i += 2) P.early[i] = q++;
+        for (int i = 0; i < 16; i += 2) P.late[0][i] = q++;
+      } else {
+        for (int i = 8; i < 16; ++i) P.early[i] = q++;
+        for (int i = 8; i < 12; ++i) P.late[0][i] = q++;
+        for (int i = 8; i < 12; ++i) P.late[1][i] = q++;
+      }
+      P.n_early = 8;
+      return P;
+    }();
+    static_assert(KSTEPS >= 2 && (BL == BLayout::KMajor || KSTEPS >= 3), "late loads need a k-step that is not the last");
+    static_for<16>([&](auto Q) { issue(Q, 0, 0); });
+    if (KT > 1) {
+      static_for<plan.n_early>([&](auto Q) { issue(Q, 1, 1); });
+      static_assert(plan.n_early == 8, "the wait below leaves exactly the early loads of slab 1 in flight");
+      asm volatile("s_waitcnt vmcnt(8)" ::: "memory");  // slab 0 has landed
+    } else {
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
+    __syncthreads();
+    read_frags<T, BL>(L, smem, smem + SLAB_BYTES, 0, fa[0], fb[0]);
 
-  for (int kt = 0; kt + 2 < KT; ++kt) slab(std::true_type{}, std::true_type{}, kt);
-  if (KT > 1) slab(std::true_type{}, std::false_type{}, KT - 2);
-  slab(std::false_type{}, std::false_type{}, KT - 1);
-  __syncthreads();  // the slabs are dead: the epilogue reuses LDS
+    // One slab of math, written in issue order.  NEXT: slab kt+1 exists (hand it over in front of the last
+    // k-step and fetch its first fragments under that step); NEXT2: slab kt+2 exists (its direct loads go
+    // into this slab's stage, which is free once every wavefront is past the barrier).
+    auto slab = [&](auto NEXT, auto NEXT2, int kt) {
+      constexpr bool next = decltype(NEXT)::value, next2 = decltype(NEXT2)::value;
+      const int stage = kt & 1;
+      const char* a_s = smem + stage * STAGE_BYTES;
+      const char* b_s = a_s + SLAB_BYTES;
+      const char* a_n = smem + (stage ^ 1) * STAGE_BYTES;
+      const char* b_n = a_n + SLAB_BYTES;
+      static_for<KSTEPS>([&](auto KS) {
+        constexpr int ks = decltype(KS)::value;
+        constexpr bool last_step = ks + 1 == KSTEPS;
+        if constexpr (last_step && next) {
+          // This step's fragments are in registers, so nothing of slab kt is read from LDS any more, and
+          // every direct load of slab kt+1 must have landed (the L2 touches are older than its last loads).
+          asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+          asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+          __syncthreads();
+        }
+        static_for<16>([&](auto IDX) {
+          constexpr int idx = decltype(IDX)::value;
+          constexpr int i = idx / 4, j = idx % 4;
+          if constexpr (!last_step) {
+            if constexpr (idx < 8) read_unit<T, BL, idx>(L, a_s, b_s, ks + 1, fa[(ks + 1) & 1], fb[(ks + 1) & 1]);
+          } else if constexpr (next) {
+            if constexpr (idx < 8) read_unit<T, BL, idx>(L, a_n, b_n, 0, fa[0], fb[0]);
+          }
+          // direct loads: the rest of slab kt+1 early in this slab, the head of slab kt+2 after the barrier
+          if constexpr (next && !last_step) {
+            constexpr int q = plan.late[ks < 3 ? ks : 0][idx];
+            if constexpr (q >= 0 && q < 16) issue(std::integral_constant<int, (q >= 0 ? q : 0)>{}, kt + 1, stage ^ 1);
+          }
+          if constexpr (next2 && last_step) {
+            constexpr int q = plan.early[idx];
+            if constexpr (q >= 0) issue(std::integral_constant<int, (q >= 0 ? q : 0)>{}, kt + 2, stage);
+          }
+          acc[i][j] = mma(fb[ks & 1][j], fa[ks & 1][i], acc[i][j]);
+          __builtin_amdgcn_sched_barrier(0);  // keep the issue order of the source
+        });
+      });
+      if constexpr (next2) {
+        pf_sink ^= pf_va ^ pf_vb;  // the previous touches: long since returned
+        const bool do_pf = kt + 1 + p.pf_dist < KT;
+        if (do_pf && pf_a) pf_va = *reinterpret_cast<const uint32_t*>(pfa_ptr + (int64_t)(kt + 1 + p.pf_dist) * a_step);
+        if (do_pf && pf_b) pf_vb = *reinterpret_cast<const uint32_t*>(pfb_ptr + (int64_t)(kt + 1 + p.pf_dist) * b_step);
+      }
+    };
+
+    for (int kt = 0; kt + 2 < KT; ++kt) slab(std::true_type{}, std::true_type{}, kt);
+    if (KT > 1) slab(std::true_type{}, std::false_type{}, KT - 2);
+    slab(std::false_type{}, std::false_type{}, KT - 1);
+    __syncthreads();  // the slabs are dead: the epilogue reuses LDS
+
+  }
 
   if (pf_sink == 0x9e3779b9u && pf_va == 0x7f4a7c15u) reinterpret_cast<uint32_t*>(p.out)[0] = pf_vb;  // keeps the touches alive
   epilogue<OT>(p, L, acc, smem, m0, n0);
