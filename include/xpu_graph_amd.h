@@ -182,6 +182,18 @@ int xg_sdpa(const void* q, const void* k, const void* v, void* out, int64_t B, i
             xg_stream_t stream);
 
 /* ---------------------------------------------------------------------------
+ * Rotary position embedding, rotate-half convention:
+ *   out = x * cos + cat(-x[..., D/2:], x[..., :D/2]) * sin      (fp32 math, one rounding)
+ *   x, out [B,H,S,D] with element strides for batch, head, sequence (D has unit stride, D % 16 == 0);
+ *   cos, sin [S,D] tables with row stride `table_stride`, dtype `table_dtype` = `dtype` or XG_F32.
+ * No counterpart in the reference (it has no rotary-embedding pattern): replaces the eager
+ *   mul / slice / neg / cat / mul / add subgraph of the Llama block of benchmark config 5.
+ * ------------------------------------------------------------------------- */
+int xg_rope(const void* x, const void* cos_table, const void* sin_table, void* out, int64_t B, int64_t H, int64_t S,
+            int64_t D, const int64_t x_strides[3], const int64_t o_strides[3], int64_t table_stride, int dtype,
+            int table_dtype, xg_stream_t stream);
+
+/* ---------------------------------------------------------------------------
  * Plain device copy of `bytes` bytes (16-byte aligned), used as the known-size
  * yardstick that scales the FETCH_SIZE / WRITE_SIZE profiler counters.
  * ------------------------------------------------------------------------- */

@@ -112,7 +112,8 @@ def test_c5_llama_block(device, B, S):
     out, mods, rest = run(fn, x, *[p[n] for n in names])
     print("llama block modules:", mods)
     print("llama block remaining aten:", rest)
-    assert "mi355x_sdpa" in mods
+    assert "mi355x_sdpa" in mods and mods.count("mi355x_rope") == 2
+    assert not any(k in t for t in rest for k in ("clone", "aten.cat", "aten.neg")), rest  # no layout copies, no unfused rotary math
     heavy = [t for t in rest if any(k in t for k in ("aten.mm", "aten.bmm", "aten.addmm", "softmax", "aten.matmul"))]
     assert heavy == [], heavy  # every matmul and the softmax went to custom kernels
     # A block is a chain of some twenty bf16 roundings; eager and fused round at different places, so both are

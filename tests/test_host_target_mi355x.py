@@ -258,3 +258,54 @@ def test_target_none_has_no_structure_patterns(caplog):
                  "ComboSum3dInp", "CustomDenseLayer", "FusedAddLayerNorm", "FusedAddRMSNorm", "FusedSwiGLU",
                  "FusedStackSumToAddN", "FusedCausalSDPA", "NativeNormToDefault"):
         assert want in names2, want
+
+
+def _rope_fn(q, cos, sin):
+    d = q.shape[-1] // 2
+    return q * cos + torch.cat([-q[..., d:], q[..., :d]], dim=-1) * sin
+
+
+def test_rope_rotate_half_becomes_one_call(caplog, backend):
+    q = torch.randn(2, 16, 4, 64).to(bf16).transpose(1, 2)  # [B, H, S, D] view of [B, S, H, D] storage
+    cos, sin = torch.randn(16, 64).to(bf16), torch.randn(16, 64).to(bf16)
+    gm = rewrite(backend, _rope_fn, q, cos, sin)
+    assert modules_called(gm) == ["mi355x_rope"] and aten_ops(gm) == []
+    assert "Pattern.FusedRoPE changed graph" in caplog.text
+    node = next(n for n in gm.graph.nodes if n.op == "call_module")
+    assert node.meta["val"].stride() == q.stride()  # written in the layout it was read in
+
+
+def test_rope_not_taken_for_other_rotations_or_mixed_dtypes(caplog, backend):
+    q = torch.randn(2, 4, 16, 64).to(bf16)
+    cos, sin = torch.randn(16, 64).to(bf16), torch.randn(16, 64).to(bf16)
+
+    def quarter(q, cos, sin):  # rotates by a quarter of the head dim: not the rotate-half form
+        return q * cos + torch.cat([-q[..., 16:], q[..., :16]], dim=-1) * sin
+
+    def no_neg(q, cos, sin):
+        return q * cos + torch.cat([q[..., 32:], q[..., :32]], dim=-1) * sin
+
+    for fn, args in ((quarter, (q, cos, sin)), (no_neg, (q, cos, sin)), (_rope_fn, (q, cos.float(), sin.float())), (_rope_fn, (q, cos[None].expand(2, 16, 64)[:, None], sin[None].expand(2, 16, 64)[:, None]))):
+        gm = rewrite(backend, fn, *args, must_fail=False)
+        assert "mi355x_rope" not in modules_called(gm)
+
+
+def test_llama_block_graph_has_no_layout_copies(backend):
+    """q / k go through rope in the projection's own layout, attention writes [B, S, H, D], so the transposes
+    around it are views and the contiguous() copy in front of the output projection disappears; the rotary
+    tables are folded to constants."""
+    from oracle import eager, inputs
+
+    for batch in (1, 3):  # with a batch, the traced batched matmuls carry extra contiguous copies of q, k^T and v
+        torch._dynamo.reset()  # a recompile for a new batch size would otherwise trace the batch as a symbol
+        x, p = inputs.c5_llama_block(B=batch, S=32, hidden=512, inter=256, device="cpu")
+        names = sorted(p)
+
+        def fn(x, *ws):
+            return eager.llama_block_eager(x, dict(zip(names, ws)), n_heads=8)
+
+        gm = rewrite(mi355x_compiler(), fn, x, *[p[n] for n in names])
+        mods = modules_called(gm)
+        assert mods.count("mi355x_rope") == 2 and "mi355x_sdpa" in mods
+        left = aten_ops(gm)
+        assert not any(k in t for t in left for k in ("clone", "cat", "neg", "cos", "sin", "arange", "softmax", "aten.mm", "aten.bmm")), left

@@ -363,6 +363,7 @@ _library.define(
     "dense_fp8(Tensor x_q, Tensor w_q, bool weight_trans, Tensor x_scale, Tensor w_scale, Tensor? bias, str act, ScalarType out_dtype) -> Tensor"
 )
 _library.define("sdpa(Tensor q, Tensor k, Tensor v, bool is_causal, float scale) -> Tensor")
+_library.define("rope(Tensor x, Tensor cos, Tensor sin) -> Tensor")
 
 
 def _dense_out_shape(x, weight, weight_trans):
@@ -463,13 +464,32 @@ def _unit_last(t):
     return t if t.stride(-1) == 1 else t.contiguous()
 
 
+def _dense_strides_ok(t):
+    """Strides describe a permutation of a contiguous block (no overlap, no gaps)."""
+    dims = sorted(((st, sz) for st, sz in zip(t.stride(), t.shape) if sz != 1), key=lambda d: d[0])
+    expect = 1
+    for st, sz in dims:
+        if st != expect:
+            return False
+        expect *= sz
+    return True
+
+
+def _empty_like_layout(t):
+    """Output buffer in the layout of `t` when that layout is dense with a unit last stride (e.g. [B, S, H, D]
+    storage viewed as [B, H, S, D]): what follows -- usually transpose(1, 2).reshape(B, S, H*D) -- is then a view."""
+    if t.stride(-1) == 1 and _dense_strides_ok(t):
+        return torch.empty_strided(t.shape, t.stride(), dtype=t.dtype, device=t.device)
+    return torch.empty(t.shape, dtype=t.dtype, device=t.device)
+
+
 def _sdpa(q, k, v, is_causal, scale):
     _sdpa_check(q, k, v)
     if k.dtype != q.dtype or v.dtype != q.dtype:
         raise TypeError("sdpa: q, k, v must share a dtype")
     q, k, v = _unit_last(q), _unit_last(k), _unit_last(v)
     B, H, Sq, D = q.shape
-    out = torch.empty((B, H, Sq, D), dtype=q.dtype, device=q.device)
+    out = _empty_like_layout(q)
     if out.numel() == 0:
         return out
     S3 = ctypes.c_int64 * 3
@@ -483,7 +503,44 @@ def _sdpa(q, k, v, is_causal, scale):
 
 def _sdpa_meta(q, k, v, is_causal, scale):
     _sdpa_check(q, k, v)
-    return torch.empty(q.shape, dtype=q.dtype, device=q.device)
+    return _empty_like_layout(_unit_last(q))
+
+
+def _rope_check(x, cos, sin):
+    if x.dim() != 4:
+        raise ValueError("rope: x must be [B, H, S, D]")
+    S, D = x.shape[2], x.shape[3]
+    if D % 16 != 0:
+        raise ValueError("rope: head dim must be a multiple of 16")
+    for t in (cos, sin):
+        if t.dim() < 2 or tuple(t.shape[-2:]) != (S, D) or any(d != 1 for d in t.shape[:-2]):
+            raise ValueError("rope: cos / sin must be [S, D] tables (leading dims of size 1 allowed)")
+    if cos.dtype != sin.dtype or cos.dtype not in (x.dtype, torch.float32):
+        raise TypeError("rope: cos / sin must share a dtype, that of x or float32")
+
+
+def _rope(x, cos, sin):
+    _rope_check(x, cos, sin)
+    x = _unit_last(x)
+    B, H, S, D = x.shape
+    out = _empty_like_layout(x)
+    if out.numel() == 0:
+        return out
+    cos2, sin2 = cos.reshape(S, D), sin.reshape(S, D)
+    if cos2.stride(1) != 1 or sin2.stride() != cos2.stride():
+        cos2, sin2 = cos2.contiguous(), sin2.contiguous()
+    S3 = ctypes.c_int64 * 3
+    st = _lib.lib().xg_rope(
+        _ptr(x), _ptr(cos2), _ptr(sin2), _ptr(out), B, H, S, D, S3(*x.stride()[:3]), S3(*out.stride()[:3]), cos2.stride(0),
+        _code(x.dtype), _code(cos2.dtype), _stream(),
+    )
+    _lib.check(st, "xg_rope")
+    return out
+
+
+def _rope_meta(x, cos, sin):
+    _rope_check(x, cos, sin)
+    return _empty_like_layout(_unit_last(x))
 
 
 _library.impl("dense", _dense, "CUDA")
@@ -492,3 +549,5 @@ _library.impl("dense_fp8", _dense_fp8, "CUDA")
 _library.impl("dense_fp8", _dense_fp8_meta, "Meta")
 _library.impl("sdpa", _sdpa, "CUDA")
 _library.impl("sdpa", _sdpa_meta, "Meta")
+_library.impl("rope", _rope, "CUDA")
+_library.impl("rope", _rope_meta, "Meta")

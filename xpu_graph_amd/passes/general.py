@@ -126,6 +126,19 @@ class ConstantFolding(Optimizer):
         super().__init__()
         self.folding_params = folding_params
 
+    @staticmethod
+    def _foldable_factory(node):
+        """A call with no tensor input (arange, full, ...) folds like any other constant expression -- position
+        tables and masks are built from them -- unless its value is not a function of its arguments."""
+        tgt = node.target
+        if not isinstance(tgt, torch._ops.OpOverload):
+            return False
+        name = tgt._schema.name
+        if torch.Tag.nondeterministic_seeded in tgt.tags or name.startswith("aten::empty") or name.startswith("aten::new_empty"):
+            return False
+        val = node.meta.get("val")
+        return isinstance(val, torch.Tensor) and all(isinstance(d, int) for d in val.shape)
+
     def process(self, gm):
         graph = gm.graph
         anchor = None
@@ -137,9 +150,9 @@ class ConstantFolding(Optimizer):
             if node.op != "call_function" or node.is_impure():
                 continue
             flat, _ = pytree.tree_flatten((node.args, node.kwargs))
-            if not any(isinstance(a, fx.Node) for a in flat):
-                continue  # factory calls stay in the graph: they are cheap and device-bound
             if not all(is_constant(a, self.folding_params) for a in flat):
+                continue
+            if not any(isinstance(a, fx.Node) for a in flat) and not self._foldable_factory(node):
                 continue
             args, kwargs = pytree.tree_map(lambda a: getattr(gm, a.target) if isinstance(a, fx.Node) else a, (node.args, node.kwargs))
             logger.info(f"start constant folding: {node.name} {node.target}")

@@ -208,7 +208,10 @@ class FoldClone(Pattern):
                     out_nodes = list(list(gm.graph.nodes)[-1].all_input_nodes)
                     changed = True
                 continue
-            if n.kwargs.get("memory_format", torch.preserve_format) == torch.preserve_format:
+            fmt = n.kwargs.get("memory_format", torch.preserve_format)
+            # also: a copy into the contiguous format of something that already is contiguous (one case beyond the
+            # reference; it is what remains of transpose(1, 2).contiguous() once a kernel writes [B, S, H, D] directly)
+            if fmt == torch.preserve_format or (fmt == torch.contiguous_format and src.meta["val"].is_contiguous()):
                 n.replace_all_uses_with(src)
                 gm.graph.erase_node(n)
                 changed = True

@@ -99,26 +99,34 @@ def _same_attention_problem(src, dims):
     return shp[2:] == list(dims[2:]) and shp[0] * shp[1] == dims[0] * dims[1]
 
 
+def _through_clone(node):
+    """The contiguous copy FusedSDPA inserts may already have been folded away."""
+    return node.args[0] if is_call(node, aten.clone.default) else node
+
+
 def _peel_qv(node, dims):
-    """reshape(clone(reshape(x4d, [BH,S,D])), [B,H,S,D]) -> x4d."""
-    if is_call(node, *VIEW_OPS) and is_call(node.args[0], aten.clone.default):
-        inner = node.args[0].args[0]
-        if is_call(inner, *VIEW_OPS) and _same_attention_problem(inner.args[0], dims):
-            return inner.args[0]
-    return node
+    """reshape(clone(reshape(x4d, [BH,S,D])), [B,H,S,D]) -> x4d.  Reshapes reinterpret row-major order and clones
+    copy, so any chain of them that ends in a 4-D tensor with the same S, D and number of heads is looked through
+    (the clone, or one of the reshapes, may already have been folded away)."""
+    cur, found = node, node
+    while is_call(cur, *VIEW_OPS) or is_call(cur, aten.clone.default):
+        cur = cur.args[0]
+        if _same_attention_problem(cur, dims):
+            found = cur  # keep going: a copy further up is looked through as well
+    return found
 
 
 def _peel_k(node, dims):
     """reshape(clone(transpose(reshape(transpose(k4d, -1, -2), [BH,D,S]), -1, -2)), [B,H,S,D]) -> k4d."""
-    if not (is_call(node, *VIEW_OPS) and is_call(node.args[0], aten.clone.default)):
+    if not is_call(node, *VIEW_OPS):
         return node
-    t1 = node.args[0].args[0]
+    t1 = _through_clone(node.args[0])
     if not is_call(t1, aten.transpose.int) or {t1.args[1], t1.args[2]} not in ({-1, -2}, {1, 2}):
         return node
     r = t1.args[0]
     if not is_call(r, *VIEW_OPS):
         return node
-    t0 = r.args[0]
+    t0 = _through_clone(r.args[0])  # batched matmul materialises k^T when k is a strided view
     if not is_call(t0, aten.transpose.int) or {t0.args[1], t0.args[2]} not in ({-1, -2}, {2, 3}):
         return node
     src = t0.args[0]
