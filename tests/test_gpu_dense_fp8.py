@@ -94,3 +94,21 @@ def test_dense_fp8_rejects_kn_weight(device):
     x_q, W_q, s_x, s_w, b = quantised(64, 64, 64, device, seed=1)
     with pytest.raises(Exception):
         _ops().dense_fp8(x_q, W_q, False, s_x, s_w, b, "none", torch.bfloat16)
+
+
+def test_fp8_dense_plugin_pattern_end_to_end(device):
+    """The user's eager fp8 layer, compiled for the mi355x target with the plugin pattern registered, runs on the
+    fp8 MFMA kernel and agrees with the same eager function (reference plugin API: plugin_pattern.py:114-284)."""
+    from xpu_graph_amd import enable_plugin_patterns, mi355x_compiler, plugins
+
+    M, N, K = 512, 1024, 2048
+    x_q, W_q, s_x, s_w, b = quantised(M, N, K, device, seed=4)
+    w_nk = W_q.t().contiguous()
+    b16 = b.bfloat16()
+    with enable_plugin_patterns():
+        plugins.register_fp8_dense(plugins.fp8_linear_silu_eager, act="silu")
+        be = mi355x_compiler()
+        got = torch.compile(plugins.fp8_linear_silu_eager, backend=be, dynamic=False)(x_q, w_nk, s_x, s_w, b16)
+    assert any("dense_fp8" in str(n.target) for n in be.compiled_graphs[-1].graph.nodes)
+    want = plugins.fp8_linear_silu_eager(x_q, w_nk, s_x, s_w, b16)
+    torch.testing.assert_close(got.float(), want.float(), rtol=1.6e-2, atol=4e-3)

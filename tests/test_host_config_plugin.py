@@ -178,3 +178,29 @@ def test_plugin_registry_is_keyed_by_target():
 def test_public_api_names():
     for name in ("XpuGraph", "XpuGraphConfig", "Target", "OptLevel", "mi355x_compiler", "register_plugin_pattern", "XpuGraphCompiler"):
         assert hasattr(xpu_graph_amd, name)
+
+
+def test_fp8_dense_plugin_pattern_rewrites_user_function():
+    """The fp8 dense layer reaches the kernel library as a plugin pattern on the mi355x target."""
+    from xpu_graph_amd import mi355x_compiler, plugins
+
+    def layer(x_q, w_q, s_x, s_w, b, extra):
+        return plugins.fp8_linear_silu_eager(x_q, w_q, s_x, s_w, b) + extra
+
+    x_q, w_q, s_x, s_w, b = plugins.example_fp8_inputs(16, 24, 64)
+    extra = torch.zeros(16, 24, dtype=torch.bfloat16)
+    with enable_plugin_patterns():
+        plugins.register_fp8_dense(plugins.fp8_linear_silu_eager, act="silu")
+        be = mi355x_compiler()
+        with pytest.raises(NotImplementedError):  # rewritten to the custom op, which has no CPU implementation
+            torch.compile(layer, backend=be)(x_q, w_q, s_x, s_w, b, extra)
+        gm = be.compiled_graphs[-1]
+        targets = [str(n.target) for n in gm.graph.nodes if n.op == "call_function"]
+        assert any("dense_fp8" in t for t in targets) and not any("aten.mm" in t or "silu" in t for t in targets), targets
+        # K not a multiple of 16: the constraint vetoes the match and the eager subgraph stays (and runs on the CPU)
+        torch._dynamo.reset()
+        be = mi355x_compiler()
+        x8, w8, s1, sn, bb = plugins.example_fp8_inputs(16, 24, 40)
+        got = torch.compile(layer, backend=be)(x8, w8, s1, sn, bb, extra)
+        torch.testing.assert_close(got, layer(x8, w8, s1, sn, bb, extra))
+        assert not any("dense_fp8" in str(n.target) for n in be.compiled_graphs[-1].graph.nodes)
