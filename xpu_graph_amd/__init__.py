@@ -11,6 +11,7 @@ Public names follow the reference package (src/xpu_graph/__init__.py).
 """
 from .compiler import XpuGraph, XpuGraphCompiler, XpuGraphRuntimeArtifact
 from .config import OptLevel, Target, XpuGraphConfig
+from .device_graph_runner import GraphRunner, HIPGraphRunner
 from .passes.patterns.plugin_pattern import (
     deregister_plugin_patterns,
     enable_plugin_patterns,
@@ -29,6 +30,8 @@ __all__ = [
     "Target",
     "OptLevel",
     "mi355x_compiler",
+    "GraphRunner",
+    "HIPGraphRunner",
     "register_plugin_pattern",
     "register_this_as_plugin_pattern",
     "register_this_as_pattern_constraint",
