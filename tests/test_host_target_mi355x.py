@@ -309,3 +309,30 @@ def test_llama_block_graph_has_no_layout_copies(backend):
         assert mods.count("mi355x_rope") == 2 and "mi355x_sdpa" in mods
         left = aten_ops(gm)
         assert not any(k in t for t in left for k in ("clone", "cat", "neg", "cos", "sin", "arange", "softmax", "aten.mm", "aten.bmm")), left
+
+
+def test_residual_add_moves_into_the_dense_epilogue(caplog, backend):
+    def fn(x, w, r):
+        return F.linear(x, w).view(2, 8, 32) + r  # output projection, reshaped, plus residual
+
+    x, w, r = torch.randn(16, 64).to(bf16), torch.randn(32, 64).to(bf16), torch.randn(2, 8, 32).to(bf16)
+    gm = rewrite(backend, fn, x, w, r)
+    assert "Pattern.FusedDenseResidual changed graph" in caplog.text
+    assert modules_called(gm) == ["custom_dense_layer_replacement"] and "aten.add.Tensor" not in aten_ops(gm)
+    node = next(n for n in gm.graph.nodes if n.op == "call_module")
+    assert tuple(node.args[3].meta["val"].shape) == (16, 32)  # the residual, viewed as [M, N]
+
+
+def test_residual_not_fused_when_dense_has_other_users_or_an_activation(backend):
+    def two_users(x, w, r):
+        y = F.linear(x, w)
+        return y + r, y
+
+    def activated(x, w, r):
+        return F.silu(F.linear(x, w)) + r
+
+    x, w, r = torch.randn(16, 64).to(bf16), torch.randn(32, 64).to(bf16), torch.randn(16, 32).to(bf16)
+    for fn in (two_users, activated):
+        gm = rewrite(mi355x_compiler(), fn, x, w, r)
+        assert "aten.add.Tensor" in aten_ops(gm)
+        torch._dynamo.reset()
