@@ -80,7 +80,7 @@ struct GemmParams {
   const float* a_scale;  // fp8 only
   const float* b_scale;  // fp8 only
   int M, N, K;
-  int64_t lda, ldb, ldr;
+  int64_t lda, ldb, ldr, ldc;  // row strides in elements of A, B, the residual and the output
   int act;
   int bias_f32;
   int tiles_m, tiles_n;
@@ -164,7 +164,8 @@ struct Lane {
   int fsw;    // swz() of this lane's fragment row
   int tr_sw;  // granule permutation of the transposing read
   int a_row[4], b_row[4];
-  __device__ __forceinline__ Lane() {
+  // ni: 32-row A units per wave (4: 256-row tile, 2: 128-row tile)
+  __device__ __forceinline__ explicit Lane(int ni = 4) {
     tid = threadIdx.x;
     lane = tid & 63;
     wave = tid >> 6;
@@ -178,7 +179,7 @@ struct Lane {
     tr_sw = (p16 >> 2) | (half << 2);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      a_row[i] = (wm * 128 + i * 32 + l32) * ROW_BYTES;
+      a_row[i] = (wm * ni * 32 + i * 32 + l32) * ROW_BYTES;
       b_row[i] = (wn * 128 + i * 32 + l32) * ROW_BYTES;
     }
   }
@@ -218,17 +219,20 @@ __device__ __forceinline__ void read_unit(const Lane& L, const char* a_s, const 
   }
 }
 
-// All fragments of k-step ks.
-template <typename T, BLayout BL>
+// All fragments of k-step ks (NI A units, 4 B units).
+template <typename T, BLayout BL, int NI = 4>
 __device__ __forceinline__ void read_frags(const Lane& L, const char* a_s, const char* b_s, int ks, Frag<T> (&fa)[4],
                                            Frag<T> (&fb)[4]) {
-  static_for<8>([&](auto U) { read_unit<T, BL, decltype(U)::value>(L, a_s, b_s, ks, fa, fb); });
+  static_for<8>([&](auto U) {
+    constexpr int u = decltype(U)::value;
+    if constexpr (u >= 4 || u < NI) read_unit<T, BL, u>(L, a_s, b_s, ks, fa, fb);
+  });
 }
 
-template <typename T>
+template <typename T, int NI = 4>
 __device__ __forceinline__ void mma_step(f32x16 (&acc)[4][4], const Frag<T> (&fa)[4], const Frag<T> (&fb)[4]) {
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < NI; ++i)
 #pragma unroll
     for (int j = 0; j < 4; ++j) acc[i][j] = mma(fb[j], fa[i], acc[i][j]);
 }
@@ -244,10 +248,10 @@ __device__ __forceinline__ void mma_step(f32x16 (&acc)[4][4], const Frag<T> (&fa
 // 256 unrolled copies; the per-lane bias and scale values are loop invariant.
 template <typename OT, int ACT>
 __device__ __forceinline__ void epilogue_rows(const GemmParams& p, const char* park, int lane, int m_base, int n, bool n_ok,
-                                              const float (&sv)[8], const float (&bv)[8]) {
+                                              const float (&sv)[8], const float (&bv)[8], int passes) {
   typedef OT O8 __attribute__((ext_vector_type(8)));
   const int c = lane & 7, rr = lane >> 3;
-  for (int it = 0; it < 16; ++it) {
+  for (int it = 0; it < passes; ++it) {
     const int row = it * 8 + rr;
     const int m = m_base + row;
     const f32x4 lo = *reinterpret_cast<const f32x4*>(park + row * 256 + (((2 * c) ^ (row & 15)) << 4));
@@ -271,23 +275,23 @@ __device__ __forceinline__ void epilogue_rows(const GemmParams& p, const char* p
       if constexpr (ACT == XG_ACT_SIGMOID) t = 1.f / (1.f + __expf(-t));
       o[e] = from_f32<OT>(t);
     }
-    *reinterpret_cast<O8*>(reinterpret_cast<OT*>(p.out) + (int64_t)m * p.N + n) = o;
+    *reinterpret_cast<O8*>(reinterpret_cast<OT*>(p.out) + (int64_t)m * p.ldc + n) = o;
   }
 }
 
-template <typename OT>
+template <typename OT, int NI = 4>
 __device__ __forceinline__ void epilogue(const GemmParams& p, const Lane& L, f32x16 (&acc)[4][4], char* smem, int m0,
                                          int n0) {
   typedef OT O8 __attribute__((ext_vector_type(8)));
   char* park = smem + L.wave * (128 * 64 * 4);
   const float a_sc = p.a_scale ? *p.a_scale : 1.f;
-  const int m_base = m0 + L.wm * 128;
+  const int m_base = m0 + L.wm * (NI * 32);
   static_for<2>([&](auto H) {
     constexpr int h = decltype(H)::value;
     // 1. park: row = i*32 + l32, 16-byte chunk = jj*8 + g*2 + half, xor-ed with the row to spread the banks
     static_for<2>([&](auto JJ) {
       static_for<4>([&](auto G) {
-        static_for<4>([&](auto I) {
+        static_for<NI>([&](auto I) {
           constexpr int jj = decltype(JJ)::value, g = decltype(G)::value, i = decltype(I)::value;
           const int row = i * 32 + L.l32;
           const int chunk = (jj * 8 + g * 2 + L.half) ^ (row & 15);
@@ -321,19 +325,19 @@ __device__ __forceinline__ void epilogue(const GemmParams& p, const Lane& L, f32
     }
     switch (p.act) {  // uniform; each case is the same short loop with one activation inlined
       case XG_ACT_RELU:
-        epilogue_rows<OT, XG_ACT_RELU>(p, park, L.lane, m_base, n, n_ok, sv, bv);
+        epilogue_rows<OT, XG_ACT_RELU>(p, park, L.lane, m_base, n, n_ok, sv, bv, NI * 4);
         break;
       case XG_ACT_GELU:
-        epilogue_rows<OT, XG_ACT_GELU>(p, park, L.lane, m_base, n, n_ok, sv, bv);
+        epilogue_rows<OT, XG_ACT_GELU>(p, park, L.lane, m_base, n, n_ok, sv, bv, NI * 4);
         break;
       case XG_ACT_SILU:
-        epilogue_rows<OT, XG_ACT_SILU>(p, park, L.lane, m_base, n, n_ok, sv, bv);
+        epilogue_rows<OT, XG_ACT_SILU>(p, park, L.lane, m_base, n, n_ok, sv, bv, NI * 4);
         break;
       case XG_ACT_SIGMOID:
-        epilogue_rows<OT, XG_ACT_SIGMOID>(p, park, L.lane, m_base, n, n_ok, sv, bv);
+        epilogue_rows<OT, XG_ACT_SIGMOID>(p, park, L.lane, m_base, n, n_ok, sv, bv, NI * 4);
         break;
       default:
-        epilogue_rows<OT, XG_ACT_NONE>(p, park, L.lane, m_base, n, n_ok, sv, bv);
+        epilogue_rows<OT, XG_ACT_NONE>(p, park, L.lane, m_base, n, n_ok, sv, bv, NI * 4);
         break;
     }
   });
@@ -349,7 +353,8 @@ __device__ __forceinline__ void zero_acc(f32x16 (&acc)[4][4]) {
 
 // ---- kernel 1: direct global -> LDS ------------------------------------------------------
 // T: operand element type (bf16_t, f16_t, or uint8_t for OCP e4m3); OT: output / bias / residual type.
-template <typename T, typename OT, BLayout BL>
+// NI: 32-row A units per wave: 4 = 256 x 256 tile, 2 = 128 x 256 tile (used for the last, partial round of tiles).
+template <typename T, typename OT, BLayout BL, int NI = 4>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_dma_kernel(GemmParams p) {
   extern __shared__ __align__(16) char smem[];
   constexpr int EB = Elem<T>::BYTES;
@@ -359,8 +364,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
 
   int tm, tn;
   tile_of_block(p, tm, tn);
-  const int m0 = tm * BM, n0 = tn * BN;
-  const Lane L;
+  const int m0 = tm * (NI * 64), n0 = tn * BN;
+  const Lane L(NI);
 
   // Per-lane byte offsets of the 8 + 8 direct loads of a slab, relative to the slab's
   // (uniform) base address; the host guarantees they fit in 31 bits.
@@ -398,6 +403,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
   // load number Q (0..15) of slab kt into `stage`: uniform slab base + 32-bit lane offset
   auto issue = [&](auto Q, int kt, int stage) {
     constexpr int q = decltype(Q)::value;
+    if constexpr (q < 8 && q >= 2 * NI) return;  // a 128-row tile has only 4 A loads per wave
     char* dst = smem + stage * STAGE_BYTES + wave_u * 1024 + (q & 7) * 4096 + (q < 8 ? 0 : SLAB_BYTES);
     // The empty asm keeps the lane offset a 32-bit register up to this point, so that the load takes the
     // "uniform 64-bit base + 32-bit lane offset" addressing form instead of a 64-bit add per lane.
@@ -447,12 +453,12 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
       const int stage = kt & 1;
       const char* a_s = smem + stage * STAGE_BYTES;
       const char* b_s = a_s + SLAB_BYTES;
-      read_frags<T, BL>(L, a_s, b_s, 0, fa[0], fb[0]);
+      read_frags<T, BL, NI>(L, a_s, b_s, 0, fa[0], fb[0]);
       __builtin_amdgcn_sched_barrier(0);
       static_for<KSTEPS>([&](auto KS) {
         constexpr int ks = decltype(KS)::value;
         constexpr bool more = ks + 1 < KSTEPS;
-        if constexpr (more) read_frags<T, BL>(L, a_s, b_s, ks + 1, fa[(ks + 1) & 1], fb[(ks + 1) & 1]);
+        if constexpr (more) read_frags<T, BL, NI>(L, a_s, b_s, ks + 1, fa[(ks + 1) & 1], fb[(ks + 1) & 1]);
         if constexpr (prefetch && ks == 0) static_for<16>([&](auto Q) { issue(Q, kt + 1, stage ^ 1); });
         if constexpr (prefetch && ks == 1) {
           pf_sink ^= pf_va ^ pf_vb;  // the previous touches: long since returned
@@ -460,17 +466,17 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
           if (do_pf && pf_a) pf_va = *reinterpret_cast<const uint32_t*>(pfa_ptr + (int64_t)(kt + p.pf_dist) * a_step);
           if (do_pf && pf_b) pf_vb = *reinterpret_cast<const uint32_t*>(pfb_ptr + (int64_t)(kt + p.pf_dist) * b_step);
         }
-        mma_step<T>(acc, fa[ks & 1], fb[ks & 1]);
+        mma_step<T, NI>(acc, fa[ks & 1], fb[ks & 1]);
         // scheduling hints: thread the next step's LDS reads and the direct loads between pairs of MFMAs
-        constexpr int reads = more ? 12 : 0;
-        constexpr int loads = (prefetch && ks == 0) ? 16 : 0;
+        constexpr int reads = more ? NI + 8 : 0;
+        constexpr int loads = (prefetch && ks == 0) ? 8 + 2 * NI : 0;
         static_for<8>([&](auto R) {
           constexpr int r = decltype(R)::value;
           constexpr int rd = reads / 8 + (r < reads % 8 ? 1 : 0);
           constexpr int ld = loads / 8 + (r < loads % 8 ? 1 : 0);
           if constexpr (rd > 0) __builtin_amdgcn_sched_group_barrier(0x100, rd, 0);  // LDS reads
           if constexpr (ld > 0) __builtin_amdgcn_sched_group_barrier(0x020, ld, 0);  // memory reads
-          __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);                         // MFMA
+          __builtin_amdgcn_sched_group_barrier(0x008, NI / 2, 0);                    // MFMA
         });
         __builtin_amdgcn_sched_barrier(0);  // keep each step's reads and math inside the step
       });
@@ -527,13 +533,18 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
     static_for<16>([&](auto Q) { issue(Q, 0, 0); });
     if (KT > 1) {
       static_for<plan.n_early>([&](auto Q) { issue(Q, 1, 1); });
-      static_assert(plan.n_early == 8, "the wait below leaves exactly the early loads of slab 1 in flight");
-      asm volatile("s_waitcnt vmcnt(8)" ::: "memory");  // slab 0 has landed
+      // slab 0 has landed when only the early loads of slab 1 (the A loads that exist for this tile height) are in flight
+      static_assert(plan.n_early == 8 && BL == BLayout::KMajor, "the waits below count the early loads of slab 1");
+      if constexpr (NI == 4) {
+        asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+      } else {
+        asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+      }
     } else {
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     }
     __syncthreads();
-    read_frags<T, BL>(L, smem, smem + SLAB_BYTES, 0, fa[0], fb[0]);
+    read_frags<T, BL, NI>(L, smem, smem + SLAB_BYTES, 0, fa[0], fb[0]);
 
     // One slab of math, written in issue order.  NEXT: slab kt+1 exists (hand it over in front of the last
     // k-step and fetch its first fragments under that step); NEXT2: slab kt+2 exists (its direct loads go
@@ -558,10 +569,9 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
         static_for<16>([&](auto IDX) {
           constexpr int idx = decltype(IDX)::value;
           constexpr int i = idx / 4, j = idx % 4;
-          if constexpr (!last_step) {
-            if constexpr (idx < 8) read_unit<T, BL, idx>(L, a_s, b_s, ks + 1, fa[(ks + 1) & 1], fb[(ks + 1) & 1]);
-          } else if constexpr (next) {
-            if constexpr (idx < 8) read_unit<T, BL, idx>(L, a_n, b_n, 0, fa[0], fb[0]);
+          if constexpr (idx < 8 && (idx >= 4 || idx < NI)) {  // units 0..3 are A tile rows: a 128-row tile has two
+            if constexpr (!last_step) read_unit<T, BL, idx>(L, a_s, b_s, ks + 1, fa[(ks + 1) & 1], fb[(ks + 1) & 1]);
+            else if constexpr (next) read_unit<T, BL, idx>(L, a_n, b_n, 0, fa[0], fb[0]);
           }
           // direct loads: the rest of slab kt+1 early in this slab, the head of slab kt+2 after the barrier
           if constexpr (next && !last_step) {
@@ -572,7 +582,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
             constexpr int q = plan.early[idx];
             if constexpr (q >= 0) issue(std::integral_constant<int, (q >= 0 ? q : 0)>{}, kt + 2, stage);
           }
-          acc[i][j] = mma(fb[ks & 1][j], fa[ks & 1][i], acc[i][j]);
+          if constexpr (i < NI) acc[i][j] = mma(fb[ks & 1][j], fa[ks & 1][i], acc[i][j]);
           __builtin_amdgcn_sched_barrier(0);  // keep the issue order of the source
         });
       });
@@ -592,7 +602,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
   }
 
   if (pf_sink == 0x9e3779b9u && pf_va == 0x7f4a7c15u) reinterpret_cast<uint32_t*>(p.out)[0] = pf_vb;  // keeps the touches alive
-  epilogue<OT>(p, L, acc, smem, m0, n0);
+  epilogue<OT, NI>(p, L, acc, smem, m0, n0);
 }
 
 // ---- kernel 2: slabs staged through registers (any K) --------------------------------------
@@ -729,10 +739,59 @@ bool dma_ok(const GemmParams& p, BLayout bl) {
   return a_bytes < lim && b_bytes < lim;
 }
 
+inline int cu_count() {
+  static const int n = [] {
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+      cus = 256;
+    return cus;
+  }();
+  return n;
+}
+
+// A launch of tm x tn tiles on C compute units runs ceil(tm tn / C) rounds, and the last one may be mostly empty
+// (C4: 1376 tiles on 256 CUs = 5.4 rounds, paid as 6).  When the tiles past the last full round are at most half a
+// round, the tile columns they make up are computed by a SECOND launch of 128 x 256 tiles instead: twice as many
+// workgroups of half the work fill the machine once, for about 0.55 of a round.  Returns how many tile columns the
+// 256 x 256 launch keeps (tn: no split).
+inline int full_tile_columns(int tm, int tn) {
+  static const bool off = getenv("XG_GEMM_NO_SPLIT") != nullptr;
+  const int cus = cu_count();
+  int g = tm, c = cus;  // gcd
+  while (c) {
+    const int t = g % c;
+    g = c;
+    c = t;
+  }
+  const int col_step = cus / g;  // tile columns per whole number of rounds
+  const int keep = tn / col_step * col_step;
+  const int tail_tiles = tm * (tn - keep);
+  if (off || keep == 0 || keep == tn || 2 * tail_tiles > cus) return tn;
+  return keep;
+}
+
 template <typename T, typename OT, BLayout BL>
 int launch_gemm(const GemmParams& p, hipStream_t stream) {
-  if (dma_ok<T>(p, BL)) return launch_kernel(gemm_dma_kernel<T, OT, BL>, p, stream);
-  return launch_kernel(gemm_staged_kernel<T, OT, BL>, p, stream);
+  if (!dma_ok<T>(p, BL)) return launch_kernel(gemm_staged_kernel<T, OT, BL>, p, stream);
+  const int keep = full_tile_columns(p.tiles_m, p.tiles_n);
+  if (keep == p.tiles_n) return launch_kernel(gemm_dma_kernel<T, OT, BL, 4>, p, stream);
+  // columns [0, keep * BN): full tiles; the rest: 128-row tiles on operand pointers moved to the split column
+  constexpr int EB = Elem<T>::BYTES;
+  const int64_t n_split = (int64_t)keep * BN;
+  GemmParams full = p;
+  full.N = (int)n_split;
+  full.tiles_n = keep;
+  if (int st = launch_kernel(gemm_dma_kernel<T, OT, BL, 4>, full, stream)) return st;
+  GemmParams rest = p;
+  rest.N = p.N - (int)n_split;
+  rest.tiles_n = p.tiles_n - keep;
+  rest.tiles_m = (p.M + 127) / 128;
+  rest.B = reinterpret_cast<const char*>(p.B) + (BL == BLayout::KMajor ? n_split * p.ldb * EB : n_split * EB);
+  if (p.bias) rest.bias = reinterpret_cast<const char*>(p.bias) + n_split * (p.bias_f32 ? 4 : (int64_t)sizeof(OT));
+  if (p.b_scale) rest.b_scale = p.b_scale + n_split;
+  if (p.res) rest.res = reinterpret_cast<const char*>(p.res) + n_split * (int64_t)sizeof(OT);
+  rest.out = reinterpret_cast<char*>(p.out) + n_split * (int64_t)sizeof(OT);
+  return launch_kernel(gemm_dma_kernel<T, OT, BL, 2>, rest, stream);
 }
 
 inline GemmParams make_params(const void* a, const void* b, const void* bias, const void* residual, void* out, int64_t M,
@@ -751,6 +810,7 @@ inline GemmParams make_params(const void* a, const void* b, const void* bias, co
   p.lda = lda;
   p.ldb = ldb;
   p.ldr = ldr;
+  p.ldc = N;
   p.act = act;
   p.bias_f32 = bias_f32 ? 1 : 0;
   p.tiles_m = (int)((M + BM - 1) / BM);
