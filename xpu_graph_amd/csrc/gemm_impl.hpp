@@ -143,9 +143,7 @@ __device__ __forceinline__ f32x16 mma(const Frag<uint8_t>& a, const Frag<uint8_t
 __device__ __forceinline__ int swz(int row) { return (row & 7) ^ ((row >> 3) & 1); }
 
 // XCD-aware, grouped tile order.
-__device__ __forceinline__ void tile_of_block(const GemmParams& p, int& tm, int& tn) {
-  const int nb = gridDim.x;
-  const int bid = blockIdx.x;
+__device__ __forceinline__ void tile_of_block(const GemmParams& p, int bid, int nb, int& tm, int& tn) {
   const int xcd = bid % kXcds, local = bid / kXcds;
   const int base = nb / kXcds, extra = nb % kXcds;
   const int tile = xcd * base + (xcd < extra ? xcd : extra) + local;
@@ -354,16 +352,16 @@ __device__ __forceinline__ void zero_acc(f32x16 (&acc)[4][4]) {
 // ---- kernel 1: direct global -> LDS ------------------------------------------------------
 // T: operand element type (bf16_t, f16_t, or uint8_t for OCP e4m3); OT: output / bias / residual type.
 // NI: 32-row A units per wave: 4 = 256 x 256 tile, 2 = 128 x 256 tile (used for the last, partial round of tiles).
-template <typename T, typename OT, BLayout BL, int NI = 4>
-__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_dma_kernel(GemmParams p) {
-  extern __shared__ __align__(16) char smem[];
+// bid / nb: this workgroup's index among the nb workgroups that share the tile grid of p.
+template <typename T, typename OT, BLayout BL, int NI>
+__device__ __forceinline__ void gemm_dma_tile(const GemmParams& p, int bid, int nb, char* smem) {
   constexpr int EB = Elem<T>::BYTES;
   constexpr int KSTEPS = Elem<T>::KSTEPS;
   constexpr int SLAB_K = ROW_BYTES / EB;
   static_assert(BL == BLayout::KMajor || EB == 2, "the transposing LDS read is wired for 16-bit elements only");
 
   int tm, tn;
-  tile_of_block(p, tm, tn);
+  tile_of_block(p, bid, nb, tm, tn);
   const int m0 = tm * (NI * 64), n0 = tn * BN;
   const Lane L(NI);
 
@@ -605,6 +603,26 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
   epilogue<OT, NI>(p, L, acc, smem, m0, n0);
 }
 
+template <typename T, typename OT, BLayout BL>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_dma_kernel(GemmParams p) {
+  extern __shared__ __align__(16) char smem[];
+  gemm_dma_tile<T, OT, BL, 4>(p, blockIdx.x, gridDim.x, smem);
+}
+
+// One launch for two tile grids: the first n_full workgroups compute the 256 x 256 tiles of `full`, the others the
+// 128 x 256 tiles of `rest` (the tile columns past the last full round), which start as soon as compute units free up.
+template <typename T, typename OT, BLayout BL>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_dma_split_kernel(GemmParams full, GemmParams rest,
+                                                                                                                    int n_full) {
+  extern __shared__ __align__(16) char smem[];
+  const int bid = blockIdx.x;  // uniform
+  if (bid < n_full) {
+    gemm_dma_tile<T, OT, BL, 4>(full, bid, n_full, smem);
+  } else {
+    gemm_dma_tile<T, OT, BL, 2>(rest, bid - n_full, (int)gridDim.x - n_full, smem);
+  }
+}
+
 // ---- kernel 2: slabs staged through registers (any K) --------------------------------------
 template <typename T, typename OT, BLayout BL>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_staged_kernel(GemmParams p) {
@@ -615,7 +633,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
   static_assert(BL == BLayout::KMajor || EB == 2, "the transposing LDS read is wired for 16-bit elements only");
 
   int tm, tn;
-  tile_of_block(p, tm, tn);
+  tile_of_block(p, blockIdx.x, gridDim.x, tm, tn);
   const int m0 = tm * BM, n0 = tn * BN;
   const Lane L;
   const int tid = L.tid;
@@ -751,9 +769,9 @@ inline int cu_count() {
 
 // A launch of tm x tn tiles on C compute units runs ceil(tm tn / C) rounds, and the last one may be mostly empty
 // (C4: 1376 tiles on 256 CUs = 5.4 rounds, paid as 6).  When the tiles past the last full round are at most half a
-// round, the tile columns they make up are computed by a SECOND launch of 128 x 256 tiles instead: twice as many
-// workgroups of half the work fill the machine once, for about 0.55 of a round.  Returns how many tile columns the
-// 256 x 256 launch keeps (tn: no split).
+// round, the tile columns they make up are computed as 128 x 256 tiles instead: twice as many workgroups of half
+// the work fill the machine once, for about 0.55 of a round.  Returns how many tile columns the
+// full-size tiles keep (tn: no split).
 inline int full_tile_columns(int tm, int tn) {
   static const bool off = getenv("XG_GEMM_NO_SPLIT") != nullptr;
   const int cus = cu_count();
@@ -774,14 +792,13 @@ template <typename T, typename OT, BLayout BL>
 int launch_gemm(const GemmParams& p, hipStream_t stream) {
   if (!dma_ok<T>(p, BL)) return launch_kernel(gemm_staged_kernel<T, OT, BL>, p, stream);
   const int keep = full_tile_columns(p.tiles_m, p.tiles_n);
-  if (keep == p.tiles_n) return launch_kernel(gemm_dma_kernel<T, OT, BL, 4>, p, stream);
+  if (keep == p.tiles_n) return launch_kernel(gemm_dma_kernel<T, OT, BL>, p, stream);
   // columns [0, keep * BN): full tiles; the rest: 128-row tiles on operand pointers moved to the split column
   constexpr int EB = Elem<T>::BYTES;
   const int64_t n_split = (int64_t)keep * BN;
   GemmParams full = p;
   full.N = (int)n_split;
   full.tiles_n = keep;
-  if (int st = launch_kernel(gemm_dma_kernel<T, OT, BL, 4>, full, stream)) return st;
   GemmParams rest = p;
   rest.N = p.N - (int)n_split;
   rest.tiles_n = p.tiles_n - keep;
@@ -791,7 +808,12 @@ int launch_gemm(const GemmParams& p, hipStream_t stream) {
   if (p.b_scale) rest.b_scale = p.b_scale + n_split;
   if (p.res) rest.res = reinterpret_cast<const char*>(p.res) + n_split * (int64_t)sizeof(OT);
   rest.out = reinterpret_cast<char*>(p.out) + n_split * (int64_t)sizeof(OT);
-  return launch_kernel(gemm_dma_kernel<T, OT, BL, 2>, rest, stream);
+  auto kernel = gemm_dma_split_kernel<T, OT, BL>;
+  if (int st = set_smem_once(kernel)) return st;
+  const int64_t n_full = (int64_t)full.tiles_m * full.tiles_n, n_rest = (int64_t)rest.tiles_m * rest.tiles_n;
+  if (n_full + n_rest > 0x7fffffffLL) return XG_ERR_TOO_LARGE;
+  hipLaunchKernelGGL(kernel, dim3((unsigned)(n_full + n_rest)), dim3(kThreads), SMEM_BYTES, stream, full, rest, (int)n_full);
+  return status_from_hip(hipGetLastError());
 }
 
 inline GemmParams make_params(const void* a, const void* b, const void* bias, const void* residual, void* out, int64_t M,
