@@ -277,7 +277,7 @@ class DenseC4(Workload):
     bound = "mfma"
     dtype = "bf16"
     unit = "TFLOP/s"
-    kernel = "gemm_dma_kernel<bf16,[K,N] weight>"
+    kernel = "gemm_dma_split_kernel<bf16,[K,N] weight> (256x256 tiles + 128x256 tiles for the last partial round)"
     work = 2 * 8192 * 4096 * 11008
     n_sets = 3
     cpu_rows = 512
@@ -321,7 +321,7 @@ class DenseC4(Workload):
 class DenseFp8C4(DenseC4):
     name = "C4 dense + bias + SiLU fp8 e4m3 (per-tensor x, per-channel W) M8192 K4096 N11008"
     dtype = "fp8"
-    kernel = "gemm_dma_kernel<e4m3,[N,K] weight>"
+    kernel = "gemm_dma_split_kernel<e4m3,[N,K] weight>"
 
     def setup(self, torch, dev):
         from oracle import eager, inputs
