@@ -392,7 +392,10 @@ extern "C" int xg_sdpa(const void* q, const void* k, const void* v, void* out, i
   p.c = scale * 1.44269504088896340736f;
   p.causal = causal ? 1 : 0;
   p.n_qb = (int)n_qb;
-  p.order = 0;
+  // Measured (B4 H32 D128): without a mask, or with many query blocks per head, walking head after head inside
+  // each XCD is faster (S2048 non-causal 290 vs 315 us, S8192 causal 558 vs 575 us); short causal problems want
+  // the heaviest query blocks of all heads first (S2048 causal 176 vs 205 us).
+  p.order = (!p.causal || n_qb >= 32) ? 1 : 0;
   if (const char* e = getenv("XG_SDPA_ORDER")) p.order = atoi(e) == 1 ? 1 : 0;
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   if (dtype == XG_BF16) return D == 128 ? sdpa::launch<bf16_t, 128>(p, st) : sdpa::launch<bf16_t, 64>(p, st);
