@@ -279,6 +279,8 @@ class DenseC4(Workload):
     unit = "TFLOP/s"
     kernel = "gemm_dma_split_kernel<bf16,[K,N] weight> (256x256 tiles + 128x256 tiles for the last partial round)"
     work = 2 * 8192 * 4096 * 11008
+    # FETCH_SIZE / WRITE_SIZE per launch (profiles/mfma_kernels_bench.md): each XCD's L2 pulls its own copy of the operand panels
+    traffic = 1312.3e6
     n_sets = 3
     cpu_rows = 512
 
@@ -322,6 +324,7 @@ class DenseFp8C4(DenseC4):
     name = "C4 dense + bias + SiLU fp8 e4m3 (per-tensor x, per-channel W) M8192 K4096 N11008"
     dtype = "fp8"
     kernel = "gemm_dma_split_kernel<e4m3,[N,K] weight>"
+    traffic = None
 
     def setup(self, torch, dev):
         from oracle import eager, inputs
@@ -373,6 +376,7 @@ class SdpaC5(Workload):
     unit = "TFLOP/s"
     kernel = "sdpa_fwd_kernel<bf16,128>"
     work = 4 * 4 * 32 * 2048 * 2048 * 128 // 2  # two matmuls, lower triangle only
+    traffic = 700.3e6
     n_sets = 3
     cpu_heads = 8
 
@@ -422,7 +426,8 @@ class LlamaBlockC5(Workload):
     bound = "mfma"
     dtype = "bf16"
     unit = "TFLOP/s"
-    kernel = "whole compiled block (7 dense, attention, 3 norm / gate kernels, eager RoPE)"
+    kernel = "whole compiled block (7 dense, attention, 2 rotary, 3 norm / gate kernels)"
+    traffic = None
     work = 2 * 8192 * (4 * 4096 * 4096 + 3 * 4096 * 11008) + 4 * 4 * 32 * 2048 * 2048 * 128 // 2
     n_sets = 1
     cpu_tokens = 256
