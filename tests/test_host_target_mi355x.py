@@ -336,3 +336,41 @@ def test_residual_not_fused_when_dense_has_other_users_or_an_activation(backend)
         gm = rewrite(mi355x_compiler(), fn, x, w, r)
         assert "aten.add.Tensor" in aten_ops(gm)
         torch._dynamo.reset()
+
+
+@pytest.mark.parametrize("form", ["bmm", "bmm_act", "bmm_bias", "baddbmm", "residual", "w_trans"])
+def test_batch_dense_layer(caplog, backend, form):
+    """bmm (+ bias | residual) (+ activation) -> one batched dense call
+    (reference tests/mlu/test_custom_batchdenselayer.py; structure/custom_denselayer.py:102-128)."""
+    B, M, K, N = 3, 16, 64, 32
+    x = torch.randn(B, M, K).to(bf16)
+    w = torch.randn(B, K, N).to(bf16)
+    wt = torch.randn(B, N, K).to(bf16)
+    bias = torch.randn(B, 1, N).to(bf16)
+    res = torch.randn(B, M, N).to(bf16)
+    fns = {
+        "bmm": (lambda x, w: torch.bmm(x, w), (x, w), False, "none"),
+        "bmm_act": (lambda x, w: F.gelu(torch.bmm(x, w)), (x, w), False, "gelu"),
+        "bmm_bias": (lambda x, w, b: F.silu(torch.bmm(x, w) + b), (x, w, bias), False, "silu"),
+        "baddbmm": (lambda x, w, b: torch.baddbmm(b, x, w), (x, w, bias), False, "none"),
+        "residual": (lambda x, w, r: torch.bmm(x, w) + r, (x, w, res), False, "none"),
+        "w_trans": (lambda x, w: torch.relu(torch.bmm(x, w.transpose(1, 2))), (x, wt), True, "relu"),
+    }
+    fn, args, trans, act = fns[form]
+    gm = rewrite(backend, fn, *args)
+    assert "Pattern.CustomBatchDenseLayer changed graph" in caplog.text
+    assert modules_called(gm) == ["custom_batch_dense_layer_replacement"]
+    assert not any(k in t for t in aten_ops(gm) for k in ("bmm", "gelu", "silu", "relu", "aten.add"))
+    node = next(n for n in gm.graph.nodes if n.op == "call_module")
+    assert node.args[2] is trans and node.args[4] == act
+    assert (node.args[3] is None) == (len(args) == 2)
+
+
+def test_batch_dense_layer_vetoes(backend):
+    x32, w32 = torch.randn(2, 8, 16), torch.randn(2, 16, 8)
+    gm = rewrite(mi355x_compiler(), lambda x, w: torch.bmm(x, w), x32, w32, must_fail=False)  # fp32 stays on Aten
+    assert modules_called(gm) == []
+    torch._dynamo.reset()
+    x, w = torch.randn(2, 8, 12).to(bf16), torch.randn(2, 12, 8).to(bf16)  # K not a multiple of 8
+    gm = rewrite(mi355x_compiler(), lambda x, w: torch.bmm(x, w), x, w, must_fail=False)
+    assert modules_called(gm) == []

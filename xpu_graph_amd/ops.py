@@ -359,6 +359,7 @@ def build_slice_table(slice_lists, src_cols, elem_size, src_row_stride=None):
 
 # ------------------------------------------------------------- dense / SDPA
 _library.define("dense(Tensor x, Tensor weight, bool weight_trans, Tensor? bias, Tensor? residual, str act) -> Tensor")
+_library.define("dense_batched(Tensor x, Tensor weight, bool weight_trans, Tensor? bias, Tensor? residual, str act) -> Tensor")
 _library.define(
     "dense_fp8(Tensor x_q, Tensor w_q, bool weight_trans, Tensor x_scale, Tensor w_scale, Tensor? bias, str act, ScalarType out_dtype) -> Tensor"
 )
@@ -381,14 +382,14 @@ def _row_major(t):
     return t if t.stride(-1) == 1 and t.stride(0) >= t.shape[1] else t.contiguous()
 
 
-def _dense(x, weight, weight_trans, bias, residual, act):
+def _dense_into(x, weight, weight_trans, bias, residual, act, out):
+    """One xg_dense launch writing the contiguous [M, N] tensor `out`."""
     m, n, k = _dense_out_shape(x, weight, weight_trans)
     if act not in _lib.ACT_CODES:
         raise ValueError(f"dense: unknown activation {act!r}")
     if weight.dtype != x.dtype:
         raise TypeError("dense: x and weight must share a dtype")
     x, weight = _row_major(x), _row_major(weight)
-    out = torch.empty((m, n), dtype=x.dtype, device=x.device)
     if out.numel() == 0:
         return out
     bias_dt = _code(x.dtype)
@@ -411,6 +412,42 @@ def _dense(x, weight, weight_trans, bias, residual, act):
     )
     _lib.check(st, "xg_dense")
     return out
+
+
+def _dense(x, weight, weight_trans, bias, residual, act):
+    m, n, _ = _dense_out_shape(x, weight, weight_trans)
+    return _dense_into(x, weight, weight_trans, bias, residual, act, torch.empty((m, n), dtype=x.dtype, device=x.device))
+
+
+def _dense_batched_shape(x, weight, weight_trans):
+    if x.dim() != 3 or weight.dim() != 3 or x.shape[0] != weight.shape[0]:
+        raise ValueError("dense_batched: x must be [B, M, K] and weight [B, K, N] (or [B, N, K] with weight_trans)")
+    k = x.shape[2]
+    wk, n = (weight.shape[2], weight.shape[1]) if weight_trans else (weight.shape[1], weight.shape[2])
+    if wk != k:
+        raise ValueError("dense_batched: inner dimensions differ")
+    return x.shape[0], x.shape[1], n
+
+
+def _dense_batched(x, weight, weight_trans, bias, residual, act):
+    """One dense launch per batch entry, on slices of the operands (no copies for contiguous batches).
+    bias: [N] shared or [B, N] per batch; residual: [B, M, N]."""
+    b, m, n = _dense_batched_shape(x, weight, weight_trans)
+    out = torch.empty((b, m, n), dtype=x.dtype, device=x.device)
+    if bias is not None and bias.dim() == 2 and bias.shape[0] != b:
+        raise ValueError("dense_batched: a 2-D bias must be [B, N]")
+    if residual is not None and tuple(residual.shape) != (b, m, n):
+        raise ValueError("dense_batched: residual must be [B, M, N]")
+    for i in range(b):
+        bi = None if bias is None else (bias if bias.dim() == 1 else bias[i])
+        ri = None if residual is None else residual[i]
+        _dense_into(x[i], weight[i], weight_trans, bi, ri, act, out[i])
+    return out
+
+
+def _dense_batched_meta(x, weight, weight_trans, bias, residual, act):
+    b, m, n = _dense_batched_shape(x, weight, weight_trans)
+    return torch.empty((b, m, n), dtype=x.dtype, device=x.device)
 
 
 def _dense_meta(x, weight, weight_trans, bias, residual, act):
@@ -545,6 +582,8 @@ def _rope_meta(x, cos, sin):
 
 _library.impl("dense", _dense, "CUDA")
 _library.impl("dense", _dense_meta, "Meta")
+_library.impl("dense_batched", _dense_batched, "CUDA")
+_library.impl("dense_batched", _dense_batched_meta, "Meta")
 _library.impl("dense_fp8", _dense_fp8, "CUDA")
 _library.impl("dense_fp8", _dense_fp8_meta, "Meta")
 _library.impl("sdpa", _sdpa, "CUDA")

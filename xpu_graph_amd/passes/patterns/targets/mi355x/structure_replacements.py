@@ -135,6 +135,54 @@ def can_fuse_custom_denselayer(inputs, weight, weight_trans, bias, act_str):
     return k % 8 == 0 and n % 8 == 0 and k > 0 and n > 0
 
 
+class BatchDenseLayerModule(torch.nn.Module):
+    """forward(inputs [B,M,K], weight [B,K,N] | [B,N,K], weight_trans, bias | None, act): a bias of the output's
+    shape is a residual, anything else must broadcast to [B, 1, N]
+    (reference targets/mlu/structure_replacements/dense_layer_modules.py:71-111)."""
+
+    def forward(self, inputs, weight, weight_trans, bias, act):
+        b, m, _ = inputs.shape
+        n = weight.shape[-2] if weight_trans else weight.shape[-1]
+        residual = None
+        if bias is not None:
+            if tuple(bias.shape) == (b, m, n) and m != 1:
+                residual, bias = bias, None
+            elif bias.dim() == 1 or all(d == 1 for d in bias.shape[:-1]):
+                bias = bias.reshape(-1)
+                if bias.shape[0] != n:
+                    bias = bias.broadcast_to((n,)).contiguous()
+            else:
+                bias = bias.broadcast_to((b, 1, n)).reshape(b, n)
+        return torch.ops.xpu_ops.dense_batched(inputs, weight, weight_trans, bias, residual, act)
+
+
+def can_fuse_custom_batch_denselayer(inputs, weight, weight_trans, bias, act_str):
+    """Match-time veto (FakeTensors): 3-D operands of a 16-bit type with static, 8-aligned K and N."""
+    if act_str not in ("none", "relu", "gelu", "silu", "sigmoid"):
+        return False
+    if inputs.dim() != 3 or weight.dim() != 3 or inputs.dtype not in _DENSE_DTYPES or weight.dtype != inputs.dtype:
+        return False
+    dims = (*inputs.shape, *weight.shape)
+    if not all(isinstance(d, int) for d in dims) or inputs.shape[0] != weight.shape[0]:
+        return False
+    k = inputs.shape[2]
+    n = weight.shape[1] if weight_trans else weight.shape[2]
+    if bias is not None:
+        b, m = inputs.shape[0], inputs.shape[1]
+        if bias.dtype != inputs.dtype or not all(isinstance(d, int) for d in bias.shape):
+            return False
+        try:
+            if tuple(torch.broadcast_shapes(tuple(bias.shape), (b, m, n))) != (b, m, n):
+                return False
+        except RuntimeError:
+            return False
+        if tuple(bias.shape) != (b, m, n) and bias.dim() == 3 and bias.shape[1] != 1:
+            return False  # varies along M without being a full residual
+        if bias.dim() == 2 and bias.shape[0] != 1:
+            return False  # [M, N]-shaped bias: neither per-batch nor shared
+    return k % 8 == 0 and n % 8 == 0 and k > 0 and n > 0
+
+
 def get_structure_replacements(config):
     return {
         "CustomRMSNorm": RMSNormModule,
@@ -144,4 +192,5 @@ def get_structure_replacements(config):
         "FusedMultipleSliceCat": FuseSliceCatSameInputModule_v2,
         "ComboSum3dInp": ComboSumModule,
         "CustomDenseLayer": (DenseLayerModule, can_fuse_custom_denselayer),
+        "CustomBatchDenseLayer": (BatchDenseLayerModule, can_fuse_custom_batch_denselayer),
     }
