@@ -140,6 +140,22 @@ __device__ __forceinline__ f32x16 mma(const Frag<uint8_t>& a, const Frag<uint8_t
   return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(x, y, c, 0, 0, 0, 127, 0, 127);
 }
 
+// L2 warm-up touch: a 4-byte load whose result is never read.  It is written as inline asm so that the compiler
+// does not track it: a tracked load is waited for (together with every direct load issued before it) where its
+// value is handed to the next loop iteration.  All touches write `sink`, which must stay live until a vmcnt(0)
+// wait has passed.
+__device__ __forceinline__ void touch(const char* ptr, uint32_t& sink) {
+  asm volatile("global_load_dword %0, %1, off" : "+v"(sink) : "v"(ptr) : "memory");
+}
+
+// Workgroup barrier without the memory fence of __syncthreads(), which waits for EVERY outstanding memory
+// operation, the L2 touches included.  The caller waits for what it needs with explicit s_waitcnt.
+__device__ __forceinline__ void barrier_only() {
+  __builtin_amdgcn_sched_barrier(0);
+  asm volatile("s_barrier" ::: "memory");
+  __builtin_amdgcn_sched_barrier(0);
+}
+
 __device__ __forceinline__ int swz(int row) { return (row & 7) ^ ((row >> 3) & 1); }
 
 // XCD-aware, grouped tile order.
@@ -431,7 +447,7 @@ __device__ __forceinline__ void gemm_dma_tile(const GemmParams& p, int bid, int 
       pfb_ptr = reinterpret_cast<const char*>(p.B) + ((int64_t)(L.tid >> 2) * p.ldb + gc) * EB;
     }
   }
-  uint32_t pf_sink = 0, pf_va = 0, pf_vb = 0;
+  uint32_t pf_sink = 0;  // every touch lands here; never read
 
   f32x16 acc[4][4];
   zero_acc(acc);
@@ -459,10 +475,9 @@ __device__ __forceinline__ void gemm_dma_tile(const GemmParams& p, int bid, int 
         if constexpr (more) read_frags<T, BL, NI>(L, a_s, b_s, ks + 1, fa[(ks + 1) & 1], fb[(ks + 1) & 1]);
         if constexpr (prefetch && ks == 0) static_for<16>([&](auto Q) { issue(Q, kt + 1, stage ^ 1); });
         if constexpr (prefetch && ks == 1) {
-          pf_sink ^= pf_va ^ pf_vb;  // the previous touches: long since returned
           const bool do_pf = kt + p.pf_dist < KT;
-          if (do_pf && pf_a) pf_va = *reinterpret_cast<const uint32_t*>(pfa_ptr + (int64_t)(kt + p.pf_dist) * a_step);
-          if (do_pf && pf_b) pf_vb = *reinterpret_cast<const uint32_t*>(pfb_ptr + (int64_t)(kt + p.pf_dist) * b_step);
+          if (do_pf && pf_a) touch(pfa_ptr + (int64_t)(kt + p.pf_dist) * a_step, pf_sink);
+          if (do_pf && pf_b) touch(pfb_ptr + (int64_t)(kt + p.pf_dist) * b_step, pf_sink);
         }
         mma_step<T, NI>(acc, fa[ks & 1], fb[ks & 1]);
         // scheduling hints: thread the next step's LDS reads and the direct loads between pairs of MFMAs
@@ -491,7 +506,8 @@ __device__ __forceinline__ void gemm_dma_tile(const GemmParams& p, int bid, int 
       } else {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       }
-      __syncthreads();  // ... and everybody else's
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // this wave's fragment reads of the slab are done
+      barrier_only();                                     // ... and everybody else's loads and reads
     }
     slab(std::false_type{}, KT - 1);
     __syncthreads();  // the slabs are dead: the epilogue reuses LDS
@@ -528,6 +544,7 @@ __device__ __forceinline__ void gemm_dma_tile(const GemmParams& p, int bid, int 
       return P;
     }();
     static_assert(KSTEPS >= 2 && (BL == BLayout::KMajor || KSTEPS >= 3), "late loads need a k-step that is not the last");
+    static_assert(BL == BLayout::KMajor, "the touches below are placed for a plan whose late loads all sit in k-step 0");
     static_for<16>([&](auto Q) { issue(Q, 0, 0); });
     if (KT > 1) {
       static_for<plan.n_early>([&](auto Q) { issue(Q, 1, 1); });
@@ -554,15 +571,30 @@ __device__ __forceinline__ void gemm_dma_tile(const GemmParams& p, int bid, int 
       const char* b_s = a_s + SLAB_BYTES;
       const char* a_n = smem + (stage ^ 1) * STAGE_BYTES;
       const char* b_n = a_n + SLAB_BYTES;
+      // The L2 touches of this slab go out after its last direct load (the late loads all sit in k-step 0), so
+      // that the hand-over can leave them in flight; how many there are is uniform over the workgroup.
+      const bool do_pf = next && kt + 1 + p.pf_dist < KT;
+      const int touches = do_pf ? (int)pf_a + (int)pf_b : 0;
       static_for<KSTEPS>([&](auto KS) {
         constexpr int ks = decltype(KS)::value;
         constexpr bool last_step = ks + 1 == KSTEPS;
+        if constexpr (ks == 1 && next) {
+          if (do_pf && pf_a) touch(pfa_ptr + (int64_t)(kt + 1 + p.pf_dist) * a_step, pf_sink);
+          if (do_pf && pf_b) touch(pfb_ptr + (int64_t)(kt + 1 + p.pf_dist) * b_step, pf_sink);
+        }
         if constexpr (last_step && next) {
           // This step's fragments are in registers, so nothing of slab kt is read from LDS any more, and
-          // every direct load of slab kt+1 must have landed (the L2 touches are older than its last loads).
+          // every direct load of slab kt+1 must have landed; only the touches, the newest memory reads of this
+          // wave, may stay in flight.
           asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-          asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-          __syncthreads();
+          if (touches == 2) {
+            asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
+          } else if (touches == 1) {
+            asm volatile("s_waitcnt vmcnt(1)" ::: "memory");
+          } else {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+          }
+          barrier_only();
         }
         static_for<16>([&](auto IDX) {
           constexpr int idx = decltype(IDX)::value;
@@ -584,12 +616,6 @@ __device__ __forceinline__ void gemm_dma_tile(const GemmParams& p, int bid, int 
           __builtin_amdgcn_sched_barrier(0);  // keep the issue order of the source
         });
       });
-      if constexpr (next2) {
-        pf_sink ^= pf_va ^ pf_vb;  // the previous touches: long since returned
-        const bool do_pf = kt + 1 + p.pf_dist < KT;
-        if (do_pf && pf_a) pf_va = *reinterpret_cast<const uint32_t*>(pfa_ptr + (int64_t)(kt + 1 + p.pf_dist) * a_step);
-        if (do_pf && pf_b) pf_vb = *reinterpret_cast<const uint32_t*>(pfb_ptr + (int64_t)(kt + 1 + p.pf_dist) * b_step);
-      }
     };
 
     for (int kt = 0; kt + 2 < KT; ++kt) slab(std::true_type{}, std::true_type{}, kt);
@@ -599,7 +625,7 @@ __device__ __forceinline__ void gemm_dma_tile(const GemmParams& p, int bid, int 
 
   }
 
-  if (pf_sink == 0x9e3779b9u && pf_va == 0x7f4a7c15u) reinterpret_cast<uint32_t*>(p.out)[0] = pf_vb;  // keeps the touches alive
+  asm volatile("s_waitcnt vmcnt(0)" : "+v"(pf_sink)::"memory");  // the last touches have landed: their register is free again
   epilogue<OT, NI>(p, L, acc, smem, m0, n0);
 }
 
