@@ -19,8 +19,14 @@
 //    one k-step: the wait-and-barrier that hands slab t+1 over sits in front of
 //    the LAST k-step of slab t (whose fragments are already in registers), so the
 //    first fragments of slab t+1 and the loads of slab t+2 go out under that
-//    step's MFMAs.  One 4-byte touch per 128-byte line warms L2 one slab further
-//    ahead, because one slab of math is too short to cover an L2 miss.
+//    step's MFMAs.  One 4-byte touch per 128-byte line warms L2 further ahead,
+//    because one slab of math is too short to cover an L2 miss.  Every wait of
+//    the loop is explicit: the touches and the transposing LDS reads are issued
+//    as inline asm, because the compiler would otherwise wait for ALL loads in
+//    flight at the loop's back edge (a tracked touch) and in front of every
+//    transposing read (which it cannot tell apart from the stage being loaded),
+//    and the hand-over barrier is a bare s_barrier, without the fence of
+//    __syncthreads() that waits for the touches as well.
 //  * gemm_staged_kernel (any K % 8 == 0): slabs pass through registers, which
 //    lets the last, partial slab be zero-filled.
 //
@@ -156,6 +162,14 @@ __device__ __forceinline__ void barrier_only() {
   __builtin_amdgcn_sched_barrier(0);
 }
 
+// s_waitcnt as a real instruction rather than inline asm, so that the compiler's own wait insertion knows about it.
+// gfx9 encoding: vmcnt = bits 3:0 and 15:14, expcnt = 6:4, lgkmcnt = 11:8; a field at its maximum does not wait.
+template <int N>
+__device__ __forceinline__ void wait_vm() {
+  __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));
+}
+__device__ __forceinline__ void wait_lgkm0() { __builtin_amdgcn_s_waitcnt(0xC07F); }
+
 __device__ __forceinline__ int swz(int row) { return (row & 7) ^ ((row >> 3) & 1); }
 
 // XCD-aware, grouped tile order.
@@ -200,7 +214,11 @@ struct Lane {
 };
 
 // Unit U (0..3: A tile row U, 4..7: B tile column U-4) of the fragments of k-step ks from the slabs at a_s / b_s.
-template <typename T, BLayout BL, int U>
+// RAW_TR: issue the transposing reads of a [K, N] operand as inline asm.  The compiler holds back a read that it
+// knows to be an LDS access until every direct load in flight has landed (it cannot tell that those go to the other
+// stage), which would stall the wave right after it has sent the next slab's loads.  The price: it does not wait
+// for the result either -- the caller must (wait_lgkm0) before the fragments are used.
+template <typename T, BLayout BL, int U, bool RAW_TR = false>
 __device__ __forceinline__ void read_unit(const Lane& L, const char* a_s, const char* b_s, int ks, Frag<T> (&fa)[4],
                                           Frag<T> (&fb)[4]) {
   if constexpr (Elem<T>::BYTES == 2) {
@@ -215,9 +233,18 @@ __device__ __forceinline__ void read_unit(const Lane& L, const char* a_s, const 
       const int gran = ((L.wn * 4 + j) ^ L.tr_sw) & 7;
       const int col = (gran << 6) + (L.blk << 5) + ((L.p16 & 3) << 3);
       const int row0 = ks * 16 + L.half * 8 + (L.p16 >> 2);
-      const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(b_s + row0 * (BN * 2) + col));
-      const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(b_s + (row0 + 4) * (BN * 2) + col));
-      const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
+      u32x2 l2, h2;
+      if constexpr (RAW_TR) {
+        const uint32_t addr = (uint32_t)(size_t)(lvoid*)(b_s + row0 * (BN * 2) + col);
+        static_assert(4 * BN * 2 == 2048, "byte offset of the second half of the fragment");
+        asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(l2) : "v"(addr) : "memory");
+        asm volatile("ds_read_b64_tr_b16 %0, %1 offset:2048" : "=v"(h2) : "v"(addr) : "memory");
+      } else {
+        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(b_s + row0 * (BN * 2) + col));
+        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(b_s + (row0 + 4) * (BN * 2) + col));
+        l2 = __builtin_bit_cast(u32x2, lo);
+        h2 = __builtin_bit_cast(u32x2, hi);
+      }
       fb[j].v = u32x4{l2.x, l2.y, h2.x, h2.y};
     }
   } else {
@@ -234,12 +261,12 @@ __device__ __forceinline__ void read_unit(const Lane& L, const char* a_s, const 
 }
 
 // All fragments of k-step ks (NI A units, 4 B units).
-template <typename T, BLayout BL, int NI = 4>
+template <typename T, BLayout BL, int NI = 4, bool RAW_TR = false>
 __device__ __forceinline__ void read_frags(const Lane& L, const char* a_s, const char* b_s, int ks, Frag<T> (&fa)[4],
                                            Frag<T> (&fb)[4]) {
   static_for<8>([&](auto U) {
     constexpr int u = decltype(U)::value;
-    if constexpr (u >= 4 || u < NI) read_unit<T, BL, u>(L, a_s, b_s, ks, fa, fb);
+    if constexpr (u >= 4 || u < NI) read_unit<T, BL, u, RAW_TR>(L, a_s, b_s, ks, fa, fb);
   });
 }
 
@@ -455,175 +482,106 @@ __device__ __forceinline__ void gemm_dma_tile(const GemmParams& p, int bid, int 
   static_assert(KSTEPS % 2 == 0, "the fragment double buffer assumes that a slab starts in buffer 0");
 
   const int KT = p.K / SLAB_K;
-  if constexpr (BL == BLayout::NMajor) {
-    // ---- [K, N] weights: the transposing fragment reads keep LDS close to saturated, and direct loads
-    // that share a k-step with them stall.  Measured best here: all 16 loads of slab t+1 go out in the
-    // first k-step of slab t, one barrier at the end of the slab, the compiler's issue order inside a step.
-    static_for<16>([&](auto Q) { issue(Q, 0, 0); });
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-    auto slab = [&](auto PREFETCH, int kt) {
-      constexpr bool prefetch = decltype(PREFETCH)::value;
-      const int stage = kt & 1;
-      const char* a_s = smem + stage * STAGE_BYTES;
-      const char* b_s = a_s + SLAB_BYTES;
-      read_frags<T, BL, NI>(L, a_s, b_s, 0, fa[0], fb[0]);
-      __builtin_amdgcn_sched_barrier(0);
-      static_for<KSTEPS>([&](auto KS) {
-        constexpr int ks = decltype(KS)::value;
-        constexpr bool more = ks + 1 < KSTEPS;
-        if constexpr (more) read_frags<T, BL, NI>(L, a_s, b_s, ks + 1, fa[(ks + 1) & 1], fb[(ks + 1) & 1]);
-        if constexpr (prefetch && ks == 0) static_for<16>([&](auto Q) { issue(Q, kt + 1, stage ^ 1); });
-        if constexpr (prefetch && ks == 1) {
-          const bool do_pf = kt + p.pf_dist < KT;
-          if (do_pf && pf_a) touch(pfa_ptr + (int64_t)(kt + p.pf_dist) * a_step, pf_sink);
-          if (do_pf && pf_b) touch(pfb_ptr + (int64_t)(kt + p.pf_dist) * b_step, pf_sink);
-        }
-        mma_step<T, NI>(acc, fa[ks & 1], fb[ks & 1]);
-        // scheduling hints: thread the next step's LDS reads and the direct loads between pairs of MFMAs
-        constexpr int reads = more ? NI + 8 : 0;
-        constexpr int loads = (prefetch && ks == 0) ? 8 + 2 * NI : 0;
-        static_for<8>([&](auto R) {
-          constexpr int r = decltype(R)::value;
-          constexpr int rd = reads / 8 + (r < reads % 8 ? 1 : 0);
-          constexpr int ld = loads / 8 + (r < loads % 8 ? 1 : 0);
-          if constexpr (rd > 0) __builtin_amdgcn_sched_group_barrier(0x100, rd, 0);  // LDS reads
-          if constexpr (ld > 0) __builtin_amdgcn_sched_group_barrier(0x020, ld, 0);  // memory reads
-          __builtin_amdgcn_sched_group_barrier(0x008, NI / 2, 0);                    // MFMA
-        });
-        __builtin_amdgcn_sched_barrier(0);  // keep each step's reads and math inside the step
-      });
-    };
-    for (int kt = 0; kt + 1 < KT; ++kt) {
-      slab(std::true_type{}, kt);
-      // Every direct load of the next slab must have landed; only the L2 touches, which are the newest
-      // memory reads of this wave, may stay in flight.  How many there are is uniform over the workgroup.
-      const int touches = kt + p.pf_dist < KT ? (int)pf_a + (int)pf_b : 0;
-      if (touches == 2) {
-        asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
-      } else if (touches == 1) {
-        asm volatile("s_waitcnt vmcnt(1)" ::: "memory");
-      } else {
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-      }
-      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // this wave's fragment reads of the slab are done
-      barrier_only();                                     // ... and everybody else's loads and reads
-    }
-    slab(std::false_type{}, KT - 1);
-    __syncthreads();  // the slabs are dead: the epilogue reuses LDS
-  } else {
-    // Issue plan of the 16 direct loads of a slab.  The address unit of a CU moves 64 bytes per clock, so
-    // the 4 x 16 loads of a slab keep it busy for half a slab of math, and the instruction stream is in
-    // order: a load that finds the queue full holds up the MFMAs behind it.  The loads are therefore spread
-    // out, the first half in the last k-step of slab t-2 (right after the barrier that frees the stage), the
-    // rest early in slab t-1, so that at least one k-step of math (16-bit types) separates the last load
-    // from the barrier that needs it.  Measured on C4: K-contiguous weights are fastest with a load in
-    // front of every second MFMA; for the [K, N] layout, whose transposing fragment reads keep LDS busier,
-    // the loads must stay clear of the MFMAs that carry the fragment reads (the first eight of a k-step).
-    struct Plan {
-      int early[16];    // load to issue in front of MFMA idx of the LAST k-step (of slab t-2), or -1
-      int late[3][16];  // same for k-steps 0..2 (of slab t-1)
-      int n_early;
-    };
-    constexpr Plan plan = []() constexpr {
-      Plan P{};
-      for (int i = 0; i < 16; ++i) {
-        P.early[i] = -1;
-        for (int k = 0; k < 3; ++k) P.late[k][i] = -1;
-      }
-      int q = 0;
-      if (BL == BLayout::KMajor) {
-        for (int i = 0; i < 16; i += 2) P.early[i] = q++;
-        for (int i = 0; i < 16; i += 2) P.late[0][i] = q++;
-      } else {
-        for (int i = 8; i < 16; ++i) P.early[i] = q++;
-        for (int i = 8; i < 12; ++i) P.late[0][i] = q++;
-        for (int i = 8; i < 12; ++i) P.late[1][i] = q++;
-      }
-      P.n_early = 8;
-      return P;
-    }();
-    static_assert(KSTEPS >= 2 && (BL == BLayout::KMajor || KSTEPS >= 3), "late loads need a k-step that is not the last");
-    static_assert(BL == BLayout::KMajor, "the touches below are placed for a plan whose late loads all sit in k-step 0");
-    static_for<16>([&](auto Q) { issue(Q, 0, 0); });
-    if (KT > 1) {
-      static_for<plan.n_early>([&](auto Q) { issue(Q, 1, 1); });
-      // slab 0 has landed when only the early loads of slab 1 (the A loads that exist for this tile height) are in flight
-      static_assert(plan.n_early == 8 && BL == BLayout::KMajor, "the waits below count the early loads of slab 1");
-      if constexpr (NI == 4) {
-        asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
-      } else {
-        asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
-      }
+  // Issue plan of the 16 direct loads of a slab.  The instruction stream of a wave is in order and the CU's
+  // address unit moves 64 bytes per clock, so a direct load holds up the MFMAs behind it for a few clocks; the
+  // loads are spread out, one in front of every second MFMA: the first half in the last k-step of slab t-2
+  // (right after the barrier that frees the stage), the rest in the first k-step of slab t-1, so that at least
+  // one k-step of math (16-bit types) separates the last load from the barrier that needs it.
+  struct Plan {
+    int early[16];  // load to issue in front of MFMA idx of the LAST k-step (of slab t-2), or -1
+    int late[16];   // same for k-step 0 (of slab t-1)
+    int n_early;
+  };
+  constexpr Plan plan = []() constexpr {
+    Plan P{};
+    for (int i = 0; i < 16; ++i) P.early[i] = P.late[i] = -1;
+    int q = 0;
+    for (int i = 0; i < 16; i += 2) P.early[i] = q++;
+    for (int i = 0; i < 16; i += 2) P.late[i] = q++;
+    P.n_early = 8;
+    return P;
+  }();
+  static_assert(KSTEPS >= 2, "the late loads need a k-step that is not the last");
+  static_for<16>([&](auto Q) { issue(Q, 0, 0); });
+  if (KT > 1) {
+    static_for<plan.n_early>([&](auto Q) { issue(Q, 1, 1); });
+    // slab 0 has landed when only the early loads of slab 1 (the A loads that exist for this tile height) are in flight
+    static_assert(plan.n_early == 8, "the waits below count the early loads of slab 1");
+    if constexpr (NI == 4) {
+      wait_vm<8>();
     } else {
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      wait_vm<4>();
     }
-    __syncthreads();
-    read_frags<T, BL, NI>(L, smem, smem + SLAB_BYTES, 0, fa[0], fb[0]);
-
-    // One slab of math, written in issue order.  NEXT: slab kt+1 exists (hand it over in front of the last
-    // k-step and fetch its first fragments under that step); NEXT2: slab kt+2 exists (its direct loads go
-    // into this slab's stage, which is free once every wavefront is past the barrier).
-    auto slab = [&](auto NEXT, auto NEXT2, int kt) {
-      constexpr bool next = decltype(NEXT)::value, next2 = decltype(NEXT2)::value;
-      const int stage = kt & 1;
-      const char* a_s = smem + stage * STAGE_BYTES;
-      const char* b_s = a_s + SLAB_BYTES;
-      const char* a_n = smem + (stage ^ 1) * STAGE_BYTES;
-      const char* b_n = a_n + SLAB_BYTES;
-      // The L2 touches of this slab go out after its last direct load (the late loads all sit in k-step 0), so
-      // that the hand-over can leave them in flight; how many there are is uniform over the workgroup.
-      const bool do_pf = next && kt + 1 + p.pf_dist < KT;
-      const int touches = do_pf ? (int)pf_a + (int)pf_b : 0;
-      static_for<KSTEPS>([&](auto KS) {
-        constexpr int ks = decltype(KS)::value;
-        constexpr bool last_step = ks + 1 == KSTEPS;
-        if constexpr (ks == 1 && next) {
-          if (do_pf && pf_a) touch(pfa_ptr + (int64_t)(kt + 1 + p.pf_dist) * a_step, pf_sink);
-          if (do_pf && pf_b) touch(pfb_ptr + (int64_t)(kt + 1 + p.pf_dist) * b_step, pf_sink);
-        }
-        if constexpr (last_step && next) {
-          // This step's fragments are in registers, so nothing of slab kt is read from LDS any more, and
-          // every direct load of slab kt+1 must have landed; only the touches, the newest memory reads of this
-          // wave, may stay in flight.
-          asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-          if (touches == 2) {
-            asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
-          } else if (touches == 1) {
-            asm volatile("s_waitcnt vmcnt(1)" ::: "memory");
-          } else {
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-          }
-          barrier_only();
-        }
-        static_for<16>([&](auto IDX) {
-          constexpr int idx = decltype(IDX)::value;
-          constexpr int i = idx / 4, j = idx % 4;
-          if constexpr (idx < 8 && (idx >= 4 || idx < NI)) {  // units 0..3 are A tile rows: a 128-row tile has two
-            if constexpr (!last_step) read_unit<T, BL, idx>(L, a_s, b_s, ks + 1, fa[(ks + 1) & 1], fb[(ks + 1) & 1]);
-            else if constexpr (next) read_unit<T, BL, idx>(L, a_n, b_n, 0, fa[0], fb[0]);
-          }
-          // direct loads: the rest of slab kt+1 early in this slab, the head of slab kt+2 after the barrier
-          if constexpr (next && !last_step) {
-            constexpr int q = plan.late[ks < 3 ? ks : 0][idx];
-            if constexpr (q >= 0 && q < 16) issue(std::integral_constant<int, (q >= 0 ? q : 0)>{}, kt + 1, stage ^ 1);
-          }
-          if constexpr (next2 && last_step) {
-            constexpr int q = plan.early[idx];
-            if constexpr (q >= 0) issue(std::integral_constant<int, (q >= 0 ? q : 0)>{}, kt + 2, stage);
-          }
-          if constexpr (i < NI) acc[i][j] = mma(fb[ks & 1][j], fa[ks & 1][i], acc[i][j]);
-          __builtin_amdgcn_sched_barrier(0);  // keep the issue order of the source
-        });
-      });
-    };
-
-    for (int kt = 0; kt + 2 < KT; ++kt) slab(std::true_type{}, std::true_type{}, kt);
-    if (KT > 1) slab(std::true_type{}, std::false_type{}, KT - 2);
-    slab(std::false_type{}, std::false_type{}, KT - 1);
-    __syncthreads();  // the slabs are dead: the epilogue reuses LDS
-
+  } else {
+    wait_vm<0>();
   }
+  barrier_only();
+  read_frags<T, BL, NI>(L, smem, smem + SLAB_BYTES, 0, fa[0], fb[0]);
+
+  // One slab of math, written in issue order.  NEXT: slab kt+1 exists (hand it over in front of the last
+  // k-step and fetch its first fragments under that step); NEXT2: slab kt+2 exists (its direct loads go
+  // into this slab's stage, which is free once every wavefront is past the barrier).
+  auto slab = [&](auto NEXT, auto NEXT2, int kt) {
+    constexpr bool next = decltype(NEXT)::value, next2 = decltype(NEXT2)::value;
+    const int stage = kt & 1;
+    const char* a_s = smem + stage * STAGE_BYTES;
+    const char* b_s = a_s + SLAB_BYTES;
+    const char* a_n = smem + (stage ^ 1) * STAGE_BYTES;
+    const char* b_n = a_n + SLAB_BYTES;
+    // The L2 touches of this slab go out after its last direct load (the late loads all sit in k-step 0), so
+    // that the hand-over can leave them in flight; how many there are is uniform over the workgroup.
+    const bool do_pf = next && kt + 1 + p.pf_dist < KT;
+    const int touches = do_pf ? (int)pf_a + (int)pf_b : 0;
+    static_for<KSTEPS>([&](auto KS) {
+      constexpr int ks = decltype(KS)::value;
+      constexpr bool last_step = ks + 1 == KSTEPS;
+      // the transposing reads are not tracked by the compiler: this step's fragments, read under the previous
+      // step, are in registers once the LDS queue is empty (it has had at least eight MFMAs to drain)
+      if constexpr (BL == BLayout::NMajor) wait_lgkm0();
+      if constexpr (ks == 1 && next) {
+        if (do_pf && pf_a) touch(pfa_ptr + (int64_t)(kt + 1 + p.pf_dist) * a_step, pf_sink);
+        if (do_pf && pf_b) touch(pfb_ptr + (int64_t)(kt + 1 + p.pf_dist) * b_step, pf_sink);
+      }
+      if constexpr (last_step && next) {
+        // This step's fragments are in registers, so nothing of slab kt is read from LDS any more, and
+        // every direct load of slab kt+1 must have landed; only the touches, the newest memory reads of this
+        // wave, may stay in flight.
+        wait_lgkm0();
+        if (touches == 2) {
+          wait_vm<2>();
+        } else if (touches == 1) {
+          wait_vm<1>();
+        } else {
+          wait_vm<0>();
+        }
+        barrier_only();
+      }
+      static_for<16>([&](auto IDX) {
+        constexpr int idx = decltype(IDX)::value;
+        constexpr int i = idx / 4, j = idx % 4;
+        if constexpr (idx < 8 && (idx >= 4 || idx < NI)) {  // units 0..3 are A tile rows: a 128-row tile has two
+          if constexpr (!last_step) read_unit<T, BL, idx, true>(L, a_s, b_s, ks + 1, fa[(ks + 1) & 1], fb[(ks + 1) & 1]);
+          else if constexpr (next) read_unit<T, BL, idx, true>(L, a_n, b_n, 0, fa[0], fb[0]);
+        }
+        // direct loads: the rest of slab kt+1 early in this slab, the head of slab kt+2 after the barrier
+        if constexpr (next && ks == 0 && !last_step) {
+          constexpr int q = plan.late[idx];
+          if constexpr (q >= 0) issue(std::integral_constant<int, (q >= 0 ? q : 0)>{}, kt + 1, stage ^ 1);
+        }
+        if constexpr (next2 && last_step) {
+          constexpr int q = plan.early[idx];
+          if constexpr (q >= 0) issue(std::integral_constant<int, (q >= 0 ? q : 0)>{}, kt + 2, stage);
+        }
+        if constexpr (i < NI) acc[i][j] = mma(fb[ks & 1][j], fa[ks & 1][i], acc[i][j]);
+        __builtin_amdgcn_sched_barrier(0);  // keep the issue order of the source
+      });
+    });
+  };
+
+  for (int kt = 0; kt + 2 < KT; ++kt) slab(std::true_type{}, std::true_type{}, kt);
+  if (KT > 1) slab(std::true_type{}, std::false_type{}, KT - 2);
+  slab(std::false_type{}, std::false_type{}, KT - 1);
+  __syncthreads();  // the slabs are dead: the epilogue reuses LDS
 
   asm volatile("s_waitcnt vmcnt(0)" : "+v"(pf_sink)::"memory");  // the last touches have landed: their register is free again
   epilogue<OT, NI>(p, L, acc, smem, m0, n0);
