@@ -20,13 +20,13 @@
 //    the LAST k-step of slab t (whose fragments are already in registers), so the
 //    first fragments of slab t+1 and the loads of slab t+2 go out under that
 //    step's MFMAs.  One 4-byte touch per 128-byte line warms L2 further ahead,
-//    because one slab of math is too short to cover an L2 miss.  Every wait of
-//    the loop is explicit: the touches and the transposing LDS reads are issued
+//    because one slab of math is too short to cover an L2 miss.  Every memory
+//    wait of the loop is explicit: the direct loads and the touches are issued
 //    as inline asm, because the compiler would otherwise wait for ALL loads in
 //    flight at the loop's back edge (a tracked touch) and in front of every
-//    transposing read (which it cannot tell apart from the stage being loaded),
-//    and the hand-over barrier is a bare s_barrier, without the fence of
-//    __syncthreads() that waits for the touches as well.
+//    transposing read (which it cannot prove disjoint from the stage being
+//    loaded), and the hand-over barrier is a bare s_barrier, without the fence
+//    of __syncthreads() that waits for the touches as well.
 //  * gemm_staged_kernel (any K % 8 == 0): slabs pass through registers, which
 //    lets the last, partial slab be zero-filled.
 //
@@ -214,11 +214,7 @@ struct Lane {
 };
 
 // Unit U (0..3: A tile row U, 4..7: B tile column U-4) of the fragments of k-step ks from the slabs at a_s / b_s.
-// RAW_TR: issue the transposing reads of a [K, N] operand as inline asm.  The compiler holds back a read that it
-// knows to be an LDS access until every direct load in flight has landed (it cannot tell that those go to the other
-// stage), which would stall the wave right after it has sent the next slab's loads.  The price: it does not wait
-// for the result either -- the caller must (wait_lgkm0) before the fragments are used.
-template <typename T, BLayout BL, int U, bool RAW_TR = false>
+template <typename T, BLayout BL, int U>
 __device__ __forceinline__ void read_unit(const Lane& L, const char* a_s, const char* b_s, int ks, Frag<T> (&fa)[4],
                                           Frag<T> (&fb)[4]) {
   if constexpr (Elem<T>::BYTES == 2) {
@@ -233,18 +229,9 @@ __device__ __forceinline__ void read_unit(const Lane& L, const char* a_s, const 
       const int gran = ((L.wn * 4 + j) ^ L.tr_sw) & 7;
       const int col = (gran << 6) + (L.blk << 5) + ((L.p16 & 3) << 3);
       const int row0 = ks * 16 + L.half * 8 + (L.p16 >> 2);
-      u32x2 l2, h2;
-      if constexpr (RAW_TR) {
-        const uint32_t addr = (uint32_t)(size_t)(lvoid*)(b_s + row0 * (BN * 2) + col);
-        static_assert(4 * BN * 2 == 2048, "byte offset of the second half of the fragment");
-        asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(l2) : "v"(addr) : "memory");
-        asm volatile("ds_read_b64_tr_b16 %0, %1 offset:2048" : "=v"(h2) : "v"(addr) : "memory");
-      } else {
-        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(b_s + row0 * (BN * 2) + col));
-        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(b_s + (row0 + 4) * (BN * 2) + col));
-        l2 = __builtin_bit_cast(u32x2, lo);
-        h2 = __builtin_bit_cast(u32x2, hi);
-      }
+      const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(b_s + row0 * (BN * 2) + col));
+      const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(b_s + (row0 + 4) * (BN * 2) + col));
+      const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
       fb[j].v = u32x4{l2.x, l2.y, h2.x, h2.y};
     }
   } else {
@@ -261,12 +248,12 @@ __device__ __forceinline__ void read_unit(const Lane& L, const char* a_s, const 
 }
 
 // All fragments of k-step ks (NI A units, 4 B units).
-template <typename T, BLayout BL, int NI = 4, bool RAW_TR = false>
+template <typename T, BLayout BL, int NI = 4>
 __device__ __forceinline__ void read_frags(const Lane& L, const char* a_s, const char* b_s, int ks, Frag<T> (&fa)[4],
                                            Frag<T> (&fb)[4]) {
   static_for<8>([&](auto U) {
     constexpr int u = decltype(U)::value;
-    if constexpr (u >= 4 || u < NI) read_unit<T, BL, u, RAW_TR>(L, a_s, b_s, ks, fa, fb);
+    if constexpr (u >= 4 || u < NI) read_unit<T, BL, u>(L, a_s, b_s, ks, fa, fb);
   });
 }
 
@@ -446,12 +433,9 @@ __device__ __forceinline__ void gemm_dma_tile(const GemmParams& p, int bid, int 
     constexpr int q = decltype(Q)::value;
     if constexpr (q < 8 && q >= 2 * NI) return;  // a 128-row tile has only 4 A loads per wave
     char* dst = smem + stage * STAGE_BYTES + wave_u * 1024 + (q & 7) * 4096 + (q < 8 ? 0 : SLAB_BYTES);
-    // The empty asm keeps the lane offset a 32-bit register up to this point, so that the load takes the
-    // "uniform 64-bit base + 32-bit lane offset" addressing form instead of a 64-bit add per lane.
-    uint32_t off = q < 8 ? a_off[q & 7] : b_off[q & 7];
-    asm volatile("" : "+v"(off));
+    const uint32_t off = q < 8 ? a_off[q & 7] : b_off[q & 7];
     const char* base = q < 8 ? a_base + kt * a_step : b_base + kt * b_step;
-    __builtin_amdgcn_global_load_lds((const gvoid*)(base + off), (lvoid*)dst, 16, 0, 0);
+    load_to_lds16(base, off, (uint32_t)(size_t)(lvoid*)dst);
   };
 
   // L2 warm-up: one 4-byte touch per 128-byte line.  A row panel is shared by the tiles of a tile
@@ -537,7 +521,6 @@ __device__ __forceinline__ void gemm_dma_tile(const GemmParams& p, int bid, int 
       constexpr bool last_step = ks + 1 == KSTEPS;
       // the transposing reads are not tracked by the compiler: this step's fragments, read under the previous
       // step, are in registers once the LDS queue is empty (it has had at least eight MFMAs to drain)
-      if constexpr (BL == BLayout::NMajor) wait_lgkm0();
       if constexpr (ks == 1 && next) {
         if (do_pf && pf_a) touch(pfa_ptr + (int64_t)(kt + 1 + p.pf_dist) * a_step, pf_sink);
         if (do_pf && pf_b) touch(pfb_ptr + (int64_t)(kt + 1 + p.pf_dist) * b_step, pf_sink);
@@ -560,8 +543,8 @@ __device__ __forceinline__ void gemm_dma_tile(const GemmParams& p, int bid, int 
         constexpr int idx = decltype(IDX)::value;
         constexpr int i = idx / 4, j = idx % 4;
         if constexpr (idx < 8 && (idx >= 4 || idx < NI)) {  // units 0..3 are A tile rows: a 128-row tile has two
-          if constexpr (!last_step) read_unit<T, BL, idx, true>(L, a_s, b_s, ks + 1, fa[(ks + 1) & 1], fb[(ks + 1) & 1]);
-          else if constexpr (next) read_unit<T, BL, idx, true>(L, a_n, b_n, 0, fa[0], fb[0]);
+          if constexpr (!last_step) read_unit<T, BL, idx>(L, a_s, b_s, ks + 1, fa[(ks + 1) & 1], fb[(ks + 1) & 1]);
+          else if constexpr (next) read_unit<T, BL, idx>(L, a_n, b_n, 0, fa[0], fb[0]);
         }
         // direct loads: the rest of slab kt+1 early in this slab, the head of slab kt+2 after the barrier
         if constexpr (next && ks == 0 && !last_step) {

@@ -173,8 +173,10 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
     static_for<LPW>([&](auto I) {
       constexpr int i = decltype(I)::value;
       char* kd = smem + stage * STAGE + (wave * LPW + i) * 1024;
-      __builtin_amdgcn_global_load_lds((const gvoid*)(kt + k_off[i]), (lvoid*)kd, 16, 0, 0);
-      __builtin_amdgcn_global_load_lds((const gvoid*)(vt + v_off[i]), (lvoid*)(kd + TILE), 16, 0, 0);
+      // inline-asm loads: the compiler must not know of LDS writes in flight, or it holds the transposing V reads
+      // of THIS tile back until the loads of the next one have landed
+      load_to_lds16(kt, k_off[i], (uint32_t)(size_t)(lvoid*)kd);
+      load_to_lds16(vt, v_off[i], (uint32_t)(size_t)(lvoid*)(kd + TILE));
     });
   };
 
@@ -206,7 +208,10 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
 
   auto step = [&](auto STAGE_IDX, int j) {
     constexpr int stage = decltype(STAGE_IDX)::value;
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's part of tile j has landed
+    // this wave's part of tile j has landed.  A real s_waitcnt (vmcnt(0), the other counters at their maximum)
+    // rather than inline asm: the compiler then knows that the Q rows loaded above have arrived too, and does
+    // not count them down against the (untracked) direct loads inside the loop
+    __builtin_amdgcn_s_waitcnt(0x0F70);
     __syncthreads();                                  // ... everyone's has, and everyone is done with tile j-1
     if (j + 1 < n_steps) issue(j + 1, std::integral_constant<int, stage ^ 1>{});
     const int kv0 = j * BKV;

@@ -103,6 +103,14 @@ __device__ __forceinline__ float group_sum(float v, float* red, int lane_in_row)
   }
 }
 
+// 16 bytes per lane from global memory straight into LDS: lane i's data lands at lds_base + 16 i.  `base` and
+// `lds_base` are wave-uniform.  Issued as inline asm so that the compiler does not know of LDS writes in flight:
+// it would otherwise hold back LDS reads it cannot prove disjoint (the transposing reads) until every direct load
+// in flight has landed.  The caller orders loads and reads with s_waitcnt vmcnt and a barrier.
+__device__ __forceinline__ void load_to_lds16(const void* base, uint32_t lane_off, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_base), "v"(lane_off), "s"(base) : "memory", "m0");
+}
+
 inline int status_from_hip(hipError_t e) { return e == hipSuccess ? XG_OK : XG_ERR_LAUNCH; }
 
 inline bool aligned_to(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
