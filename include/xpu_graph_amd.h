@@ -133,6 +133,20 @@ int xg_combo_sum(const void* const* inputs, void* const* outputs, const int64_t*
                  const int64_t* s2, int n_jobs, int dim, int dtype, xg_stream_t stream);
 
 /* ---------------------------------------------------------------------------
+ * slice -> sum -> cat: out[b, i * cols + c] = sum over r in [starts[i], ends[i]) of
+ * x[b, r, c]; x is [batch, rows, cols] with unit column stride and the given batch
+ * and row strides (elements), out is a contiguous [batch, n_slices * cols]; fp32
+ * accumulate in row order, one rounding.  `starts` / `ends` are HOST arrays of
+ * n_slices <= XG_SLICE_SUM_MAX_SLICES row bounds inside [0, rows].
+ * replaces torch_mlu_triton::fuse_slice_sum_cat as called by SliceSumCatOperation
+ *   (passes/patterns/targets/mlu/fuse_sum_cat.py:73-115).
+ * ------------------------------------------------------------------------- */
+#define XG_SLICE_SUM_MAX_SLICES 64
+int xg_slice_sum_cat(const void* x, void* out, int64_t batch, int64_t rows, int64_t cols, int64_t x_batch_stride,
+                     int64_t x_row_stride, const int32_t* starts, const int32_t* ends, int n_slices, int dtype,
+                     xg_stream_t stream);
+
+/* ---------------------------------------------------------------------------
  * SwiGLU gate: y[r, c] = silu(x[r, c]) * x[r, d + c], x is [rows, 2d] with row
  * stride x_stride, y is contiguous [rows, d]; fp32 math.
  * replaces torch_npu_triton::fused_silu_mul

@@ -107,6 +107,18 @@ def combo_sum_eager(inputs, dim):
     return [t.sum(dim=dim) for t in inputs]
 
 
+def fused_slice_eager(src, starts, width):
+    """The slices FusedSlice gathers (passes/patterns/structure/fuse_slice.py:75-121), stacked as FuseSliceModule
+    returns them (targets/mlu/structure_replacements/__init__.py:21-47): [n, *src.shape[:-1], width]."""
+    return torch.stack([src[..., s : s + width] for s in starts], dim=0)
+
+
+def slice_sum_cat_eager(x, slice_param):
+    """cat of row-slice sums of one 3-D tensor, the graph FusedCatSum matches
+    (passes/patterns/targets/mlu/fuse_sum_cat.py:118-252; tests/mlu/test_slice_sum_cat.py:13-20)."""
+    return torch.cat([torch.sum(x[:, a:b, :], dim=[1]) for a, b in slice_param], dim=1)
+
+
 # --- C4: dense layer ----------------------------------------------------------------
 def dense_silu_eager(x, W, b):
     """BASELINE config 4: F.silu(x @ W + b); the graph FusedAddMM + CustomDenseLayer

@@ -19,7 +19,7 @@ def declared_symbols():
 def test_header_declares_the_expected_entry_points():
     syms = declared_symbols()
     for s in ("xg_rms_norm", "xg_layer_norm", "xg_add_rms_norm", "xg_add_layer_norm", "xg_slice_cat", "xg_addn",
-              "xg_combo_sum", "xg_silu_mul", "xg_silu_mul2", "xg_dense", "xg_dense_fp8", "xg_sdpa", "xg_rope", "xg_copy_bytes",
+              "xg_combo_sum", "xg_slice_sum_cat", "xg_silu_mul", "xg_silu_mul2", "xg_dense", "xg_dense_fp8", "xg_sdpa", "xg_rope", "xg_copy_bytes",
               "xg_version", "xg_status_string"):
         assert s in syms
 
@@ -58,4 +58,10 @@ def test_argument_validation_needs_no_gpu():
     assert lib.xg_rms_norm(p, None, p, 4, 8, 8, 1e-6, 7, 7, None) == -1  # unknown dtype
     assert lib.xg_rms_norm(p, None, p, 0, 8, 8, 1e-6, 0, 0, None) == 0  # empty: nothing to launch
     assert lib.xg_copy_bytes(p, p, 24, None) == -2  # not a multiple of 16
+    i32 = ctypes.c_int32 * 3
+    assert lib.xg_slice_sum_cat(p, p, 2, 4, 8, 32, 8, None, None, 3, 0, None) == -4  # NULL bounds
+    assert lib.xg_slice_sum_cat(p, p, 2, 4, 8, 32, 4, i32(0, 0, 0), i32(1, 2, 3), 3, 0, None) == -2  # row stride < cols
+    assert lib.xg_slice_sum_cat(p, p, 2, 4, 8, 32, 8, i32(0, 0, 0), i32(1, 2, 5), 3, 0, None) == -2  # end past the rows
+    assert lib.xg_slice_sum_cat(p, p, 2, 4, 8, 32, 8, i32(0, 0, 0), i32(1, 2, 3), 3, 9, None) == -1  # unknown dtype
+    assert lib.xg_slice_sum_cat(p, p, 0, 4, 8, 32, 8, i32(0, 0, 0), i32(1, 2, 3), 3, 0, None) == 0  # empty batch
     assert lib.xg_silu_mul(p, p, 2, 8, 8, 0, None) == -2  # row stride < 2*d

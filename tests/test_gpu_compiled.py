@@ -128,3 +128,41 @@ def test_c5_llama_block(device, B, S):
     print(f"llama block B{B} S{S}: mean |err| fused {err_fused.mean().item():.4g} eager {err_eager.mean().item():.4g}; max fused {err_fused.max().item():.4g} eager {err_eager.max().item():.4g}")
     assert err_fused.mean().item() <= 1.05 * err_eager.mean().item()
     torch.testing.assert_close(out.float(), want_f32, rtol=1.6e-2, atol=err_eager.max().item())
+
+
+@pytest.mark.parametrize("rank", [2, 3])
+def test_fused_slice_compiled(device, rank):
+    """Equally wide slices of one tensor, each with a consumer (reference tests/mlu/test_fuse_slice.py:43-60, 128-147):
+    one gather per width, results bit-identical to eager."""
+    starts = [12573, 11984, 11562, 9782, 9727, 9745, 9763, 9773, 9805, 9822, 10283, 10736]
+
+    def fn(x):
+        return [x[..., s : s + 4] + 1 for s in starts] + [x[..., s : s + 32] * 2 for s in starts[:5]]
+
+    x = torch.randn(*((64, 43106) if rank == 2 else (10, 12, 43106)), device=device)
+    out, mods, rest = run(fn, x)
+    assert mods == ["fused_slice_0", "fused_slice_1"] and "aten.slice.Tensor" not in rest
+    for got, want in zip(out, fn(x)):
+        assert torch.equal(got, want)
+
+
+@pytest.mark.parametrize("form", ["alone", "between", "with_other_sum"])
+def test_slice_sum_cat_compiled(device, form):
+    """tests/mlu/test_slice_sum_cat.py:13-58 (fn0, fn2, fn3) on the mi355x target."""
+    params = [(0, 2), (0, 4), (0, 8), (0, 16)]
+    x = torch.rand(86, 32, 32, device=device).half()
+    other2 = torch.rand(86, 32, device=device).half()
+    other3 = torch.rand(86, 32, 32, device=device).half()
+
+    def fn(x, other):
+        sums = [torch.sum(x[:, a:b, :], dim=[1]) for a, b in params]
+        if form == "between":
+            sums = [other] + sums + [other]
+        elif form == "with_other_sum":
+            sums = sums + [torch.sum(other, dim=[1])]
+        return torch.cat(sums, dim=1)
+
+    other = other3 if form == "with_other_sum" else other2
+    out, mods, rest = run(fn, x, other)
+    assert mods == ["mi355x_slice_sum_cat_0"] and "aten.slice.Tensor" not in rest
+    torch.testing.assert_close(out, fn(x, other), rtol=1.6e-2, atol=1e-3)

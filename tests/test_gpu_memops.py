@@ -131,3 +131,64 @@ def test_silu_mul(device, rows, d, dtype):
         torch.testing.assert_close(got, eager.silu_mul_eager(x), rtol=1.6e-2, atol=1e-2)
     got2 = _ops().silu_mul2(x[:, :d], x[:, d:])
     assert torch.equal(got2, got)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("n_slices,width", [(12, 64), (56, 32), (12, 4), (3, 1)])
+def test_fused_slice_module_bit_exact(device, dtype, n_slices, width):
+    """The FusedSlice module ([n, rows, width] gather, one launch per 32 slices) against plain slicing; starts are
+    arbitrary element offsets as in the reference's tests (tests/mlu/test_fuse_slice.py:13-147)."""
+    from xpu_graph_amd.passes.patterns.targets.mi355x.structure_replacements import FuseSliceModule
+
+    g = torch.Generator().manual_seed(n_slices * 1000 + width)
+    src = torch.randn(31, 43106, generator=g).to(dtype).to(device)
+    starts = torch.randint(0, 43106 - width, (n_slices,), generator=g).tolist()
+    got = FuseSliceModule(starts)(src, width)
+    assert got.shape == (n_slices, 31, width)
+    for k, s0 in enumerate(starts):
+        assert torch.equal(got[k], src[:, s0 : s0 + width]), (k, s0)
+
+
+def test_fused_slice_module_3d_and_strided(device):
+    from xpu_graph_amd.passes.patterns.targets.mi355x.structure_replacements import FuseSliceModule
+
+    src = torch.randn(5, 12, 4310, device=device)
+    starts = [1257, 1198, 1156, 978, 972]
+    got = FuseSliceModule(starts)(src, 4)
+    assert got.shape == (5, 5, 12, 4)
+    for k, s0 in enumerate(starts):
+        assert torch.equal(got[k], src[:, :, s0 : s0 + 4])
+    wide = torch.randn(64, 512, device=device)
+    view = wide[:, 128:384]  # row stride 512, 256 columns
+    got = FuseSliceModule([0, 100, 200])(view, 56)
+    for k, s0 in enumerate([0, 100, 200]):
+        assert torch.equal(got[k], view[:, s0 : s0 + 56])
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("batch", [86, 512])
+def test_slice_sum_cat_op(device, dtype, batch):
+    """The shapes of the reference's test (tests/mlu/test_slice_sum_cat.py:67-84) plus slices that do not start at
+    row 0, an empty one, a strided source and a column count that forces the scalar path."""
+    x = torch.rand(batch, 32, 32, device=device).to(dtype)
+    tol = F32 if dtype == torch.float32 else dict(rtol=1.6e-2, atol=1e-3)
+    for params in ([(0, 2), (0, 4), (0, 8), (0, 16)], [(3, 9), (0, 32), (31, 32), (5, 5), (16, 20)]):
+        got = _ops().slice_sum_cat(x, [a for a, _ in params], [b for _, b in params])
+        torch.testing.assert_close(got, eager.slice_sum_cat_eager(x, params), **tol)
+    wide = torch.rand(batch, 40, 48, device=device).to(dtype)
+    view = wide[:, 4:36, 8:40]  # batch stride 1920, row stride 48, 32 columns
+    got = _ops().slice_sum_cat(view, [0, 0, 7], [2, 32, 9])
+    torch.testing.assert_close(got, eager.slice_sum_cat_eager(view, [(0, 2), (0, 32), (7, 9)]), **tol)
+    odd = torch.rand(batch, 12, 13, device=device).to(dtype)
+    got = _ops().slice_sum_cat(odd, [0, 2, 4], [12, 3, 11])
+    torch.testing.assert_close(got, eager.slice_sum_cat_eager(odd, [(0, 12), (2, 3), (4, 11)]), **tol)
+
+
+def test_slice_sum_cat_rejects(device):
+    x = torch.rand(4, 8, 16, device=device)
+    with pytest.raises(RuntimeError, match="xg_slice_sum_cat"):
+        _ops().slice_sum_cat(x, [0, 0, 0], [2, 4, 9])  # end past the rows
+    with pytest.raises(ValueError):
+        _ops().slice_sum_cat(x, list(range(65)), list(range(65)))
+    with pytest.raises(NotImplementedError):
+        _ops().slice_sum_cat(x[0], [0], [1])

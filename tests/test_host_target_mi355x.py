@@ -144,6 +144,103 @@ def test_slice_cat_not_fused_along_rows_or_3d(caplog, backend):
     assert "Pattern.FusedCatSlice changed graph" not in caplog.text
 
 
+def test_fused_slice_groups_by_source_and_width(caplog, backend):
+    """>= 3 equally wide last-dim slices of one source become one gather; the slabs are taken with select
+    (reference tests/mlu/test_fuse_slice.py:24-33: two widths -> two modules)."""
+
+    def fn(x):
+        a = [x[:, s : s + 64] + 1 for s in (0, 64, 128, 192)]
+        b = [x[:, s : s + 128] * 2 for s in (256, 384, 512)]
+        return a + b + [x[:, 700:710] + 1]
+
+    gm = rewrite(backend, fn, torch.randn(6, 1024))
+    mods = modules_called(gm)
+    assert mods == ["fused_slice_0", "fused_slice_1"]
+    assert gm.get_submodule("fused_slice_0").slices_index == [0, 64, 128, 192]
+    assert gm.get_submodule("fused_slice_1").slices_index == [256, 384, 512]
+    calls = {n.target: n for n in gm.graph.nodes if n.op == "call_module"}
+    assert calls["fused_slice_0"].args[1] == 64 and calls["fused_slice_1"].args[1] == 128
+    assert tuple(calls["fused_slice_1"].meta["val"].shape) == (3, 6, 128)
+    assert aten_ops(gm).count("aten.select.int") == 7 and aten_ops(gm).count("aten.slice.Tensor") == 1
+    assert "Pattern.FusedSlice changed graph" in caplog.text
+
+
+def test_fused_slice_3d_source_and_open_ends(backend):
+    def fn(x):
+        return [x[:, :, s:e] + 1 for s, e in ((0, 4), (-4, None), (10, 14), (20, -76))]
+
+    gm = rewrite(backend, fn, torch.randn(2, 3, 100))
+    (name,) = modules_called(gm)
+    assert gm.get_submodule(name).slices_index == [0, 96, 10, 20]
+    call = next(n for n in gm.graph.nodes if n.op == "call_module")
+    assert tuple(call.meta["val"].shape) == (4, 2, 3, 4)
+
+
+def test_fused_slice_vetoes(caplog, backend):
+    def two(x):  # fewer than three of one width
+        return x[:, 0:8] + 1, x[:, 8:16] + 1, x[:, 16:32] + 1
+
+    def views_only(x):  # slices that only feed the output stay views
+        return x[:, 0:8], x[:, 8:16], x[:, 16:24]
+
+    def rows(x):  # not the last dim
+        return x[0:2] + 1, x[2:4] + 1, x[4:6] + 1
+
+    def stepped(x):
+        return x[:, 0:8:2] + 1, x[:, 8:16:2] + 1, x[:, 16:24:2] + 1
+
+    for fn in (two, views_only, rows, stepped):
+        rewrite(backend, fn, torch.randn(8, 64), must_fail=False)
+    assert "Pattern.FusedSlice changed graph" not in caplog.text
+
+
+def test_slice_sum_cat_run_inside_a_cat(caplog, backend):
+    """>= 3 consecutive sum(dim 1) of row slices of one 3-D tensor among a cat's inputs become one call; the other
+    inputs stay (reference tests/mlu/test_slice_sum_cat.py:13-41)."""
+    params = [(0, 2), (0, 4), (0, 8), (0, 16)]
+
+    def fn(x, other):
+        sums = [torch.sum(x[:, a:b, :], dim=[1]) for a, b in params]
+        return torch.cat([other] + sums + [other], dim=1)
+
+    gm = rewrite(backend, fn, torch.randn(6, 32, 32), torch.randn(6, 32))
+    (name,) = modules_called(gm)
+    assert name == "mi355x_slice_sum_cat_0" and gm.get_submodule(name).slice_param == params
+    call = next(n for n in gm.graph.nodes if n.op == "call_module")
+    assert tuple(call.meta["val"].shape) == (6, 4 * 32)
+    cat = next(n for n in gm.graph.nodes if n.op == "call_function" and "cat" in str(n.target))
+    assert len(cat.args[0]) == 3 and cat.args[0][1] is call
+    assert "aten.sum.dim_IntList" not in aten_ops(gm) and "aten.slice.Tensor" not in aten_ops(gm)
+    assert "Pattern.FusedCatSum changed graph" in caplog.text
+
+
+def test_slice_sum_cat_alone_and_vetoes(caplog, backend):
+    def whole(x):  # the run is the whole cat: no cat is left
+        return torch.cat([x[:, a:b, :].sum(1) for a, b in ((1, 3), (0, 4), (2, 8))], dim=-1)
+
+    gm = rewrite(backend, whole, torch.randn(5, 8, 16))
+    assert modules_called(gm) == ["mi355x_slice_sum_cat_0"] and aten_ops(gm) == []
+    assert gm.get_submodule("mi355x_slice_sum_cat_0").slice_param == [(1, 3), (0, 4), (2, 8)]
+    caplog.clear()
+
+    def two(x):
+        return torch.cat([x[:, 0:2, :].sum(1), x[:, 0:4, :].sum(1)], dim=1)
+
+    def keepdim(x):
+        return torch.cat([x[:, 0:a, :].sum(1, keepdim=True) for a in (2, 4, 6)], dim=-1)
+
+    def other_dim(x):
+        return torch.cat([x[:, :, 0:a].sum(2) for a in (2, 4, 6)], dim=1)
+
+    def shared(x):  # a slice with a second user must survive
+        s = x[:, 0:2, :]
+        return torch.cat([s.sum(1), x[:, 0:4, :].sum(1), x[:, 0:6, :].sum(1)], dim=1), s
+
+    for fn in (two, keepdim, other_dim, shared):
+        rewrite(backend, fn, torch.randn(5, 8, 16), must_fail=False)
+    assert "Pattern.FusedCatSum changed graph" not in caplog.text
+
+
 def test_multiple_slice_cats_share_one_multi_output_module(caplog, backend):
     def fn(src):
         a = torch.cat([src[:, 0:4], src[:, 8:12]], dim=1)

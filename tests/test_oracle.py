@@ -95,6 +95,26 @@ def test_addn_is_left_to_right_fp32():
         np.testing.assert_allclose(np64(o), np64(t).sum(axis=1), rtol=1e-6)
 
 
+def test_fused_slice_and_slice_sum_cat_brute_force():
+    src = torch.arange(3 * 4 * 50, dtype=torch.float32).reshape(3, 4, 50)
+    starts = [7, 0, 46, 13]
+    got = eager.fused_slice_eager(src, starts, 4)
+    assert got.shape == (4, 3, 4, 4)
+    for k, s0 in enumerate(starts):
+        for a in range(3):
+            for b in range(4):
+                assert got[k, a, b].tolist() == [float(a * 200 + b * 50 + s0 + c) for c in range(4)]
+    x = torch.arange(2 * 6 * 3, dtype=torch.float32).reshape(2, 6, 3)
+    params = [(0, 2), (0, 6), (3, 4), (2, 2)]
+    out = eager.slice_sum_cat_eager(x, params)
+    want = [[sum(float(x[b, r, c]) for r in range(a, e)) for a, e in params for c in range(3)] for b in range(2)]
+    assert out.tolist() == want
+    # prefix sums telescope: the slice (a, e) is the difference of two slices that start at row 0
+    y = torch.randn(4, 16, 8, dtype=torch.float64)
+    full = eager.slice_sum_cat_eager(y, [(0, 5), (0, 12), (5, 12)])
+    np.testing.assert_allclose(full[:, 16:24].numpy(), (full[:, 8:16] - full[:, 0:8]).numpy(), rtol=1e-12, atol=1e-12)
+
+
 def test_dense_against_numpy_and_identity():
     x, W, b = inputs.c4_dense(16, 32, 24, dtype=torch.float32)
     z = np64(x) @ np64(W) + np64(b)

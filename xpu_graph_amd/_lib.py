@@ -15,6 +15,7 @@ LIB_PATH = os.path.join(_HERE, "libxpu_graph_amd.so")
 XG_F32, XG_F16, XG_BF16, XG_FP8_E4M3 = 0, 1, 2, 3
 ACT_CODES = {"none": 0, "relu": 1, "gelu": 2, "silu": 3, "sigmoid": 4}
 SLICE_CAT_MAX_OUTS = 32
+SLICE_SUM_MAX_SLICES = 64
 COMBO_SUM_MAX_JOBS = 64
 
 _lock = threading.Lock()
@@ -50,6 +51,10 @@ _SIGNATURES = {
         [c_void_p, c_int64, c_int64, ctypes.POINTER(c_void_p), ctypes.POINTER(c_int64), c_int, c_void_p, c_int64, c_int, c_void_p],
     ),
     "xg_addn": (c_int, [ctypes.POINTER(c_void_p), c_int, c_void_p, c_int64, c_int, c_void_p]),
+    "xg_slice_sum_cat": (
+        c_int,
+        [c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64, ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(ctypes.c_int32), c_int, c_int, c_void_p],
+    ),
     "xg_combo_sum": (
         c_int,
         [

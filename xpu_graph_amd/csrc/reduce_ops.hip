@@ -204,6 +204,76 @@ int combo_typed(const void* const* inputs, void* const* outputs, const int64_t* 
   return status_from_hip(hipGetLastError());
 }
 
+// ---- slice -> sum(dim 1) -> cat ------------------------------------------------------------
+// out[b, i * C + c] = sum over r in [start_i, end_i) of x[b, r, c], fp32 accumulate in row order, one rounding.
+// One thread per (batch, slice, VEC columns); the row loop reads VEC * sizeof(T) bytes per lane per row, rows of
+// overlapping slices come from cache.  The slice bounds travel in the kernel arguments.
+struct SliceSumTable {
+  int32_t start[XG_SLICE_SUM_MAX_SLICES];
+  int32_t end[XG_SLICE_SUM_MAX_SLICES];
+};
+
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void slice_sum_cat_kernel(const T* __restrict__ x, T* __restrict__ out, SliceSumTable tbl,
+                                                             int n_slices, int64_t batch, int cvecs, int64_t x_bs,
+                                                             int64_t x_rs, int64_t total) {
+  typedef T VT __attribute__((ext_vector_type(VEC)));
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= total) return;
+  const int cv = (int)(idx % cvecs);
+  const int64_t t = idx / cvecs;
+  const int i = (int)(t % n_slices);
+  const int64_t b = t / n_slices;
+  const T* p = x + b * x_bs + (int64_t)cv * VEC;
+  float acc[VEC];
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) acc[e] = 0.f;
+  const int r1 = tbl.end[i];
+  for (int r = tbl.start[i]; r < r1; ++r) {
+    if constexpr (VEC == 1) {
+      acc[0] += to_f32(p[(int64_t)r * x_rs]);
+    } else {
+      const VT v = *reinterpret_cast<const VT*>(p + (int64_t)r * x_rs);
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) acc[e] += to_f32(v[e]);
+    }
+  }
+  T* o = out + (b * n_slices + i) * ((int64_t)cvecs * VEC) + (int64_t)cv * VEC;
+  if constexpr (VEC == 1) {
+    o[0] = from_f32<T>(acc[0]);
+  } else {
+    VT w;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) w[e] = from_f32<T>(acc[e]);
+    *reinterpret_cast<VT*>(o) = w;
+  }
+}
+
+template <typename T>
+int slice_sum_typed(const void* x, void* out, int64_t batch, int64_t rows, int64_t cols, int64_t x_bs, int64_t x_rs,
+                    const int32_t* starts, const int32_t* ends, int n, hipStream_t stream) {
+  SliceSumTable tbl;
+  for (int i = 0; i < XG_SLICE_SUM_MAX_SLICES; ++i) tbl.start[i] = tbl.end[i] = 0;
+  for (int i = 0; i < n; ++i) {
+    if (starts[i] < 0 || ends[i] < starts[i] || ends[i] > rows) return XG_ERR_BAD_SHAPE;
+    tbl.start[i] = starts[i];
+    tbl.end[i] = ends[i];
+  }
+  constexpr int V = 16 / (int)sizeof(T);
+  const bool vec = cols % V == 0 && x_bs % V == 0 && x_rs % V == 0 && aligned_to(x, 16) && aligned_to(out, 16);
+  const int64_t cvecs = vec ? cols / V : cols;
+  const int64_t total = batch * n * cvecs;
+  const int64_t blocks = (total + 255) / 256;
+  if (cvecs > 0x7fffffffLL || blocks > 0x7fffffffLL) return XG_ERR_TOO_LARGE;
+  if (vec)
+    hipLaunchKernelGGL((slice_sum_cat_kernel<T, V>), dim3((unsigned)blocks), dim3(256), 0, stream, (const T*)x, (T*)out, tbl, n,
+                       batch, (int)cvecs, x_bs, x_rs, total);
+  else
+    hipLaunchKernelGGL((slice_sum_cat_kernel<T, 1>), dim3((unsigned)blocks), dim3(256), 0, stream, (const T*)x, (T*)out, tbl, n,
+                       batch, (int)cvecs, x_bs, x_rs, total);
+  return status_from_hip(hipGetLastError());
+}
+
 }  // namespace
 }  // namespace xg
 
@@ -246,6 +316,28 @@ int xg_combo_sum(const void* const* inputs, void* const* outputs, const int64_t*
       return combo_typed<bf16_t>(inputs, outputs, s0, s1, s2, n_jobs, dim, st);
     case XG_F16:
       return combo_typed<f16_t>(inputs, outputs, s0, s1, s2, n_jobs, dim, st);
+    default:
+      return XG_ERR_BAD_DTYPE;
+  }
+}
+
+int xg_slice_sum_cat(const void* x, void* out, int64_t batch, int64_t rows, int64_t cols, int64_t x_batch_stride,
+                     int64_t x_row_stride, const int32_t* starts, const int32_t* ends, int n_slices, int dtype,
+                     xg_stream_t stream) {
+  using namespace xg;
+  if (starts == nullptr || ends == nullptr) return XG_ERR_NULL_PTR;
+  if (batch < 0 || rows < 0 || cols < 0 || n_slices < 0 || x_row_stride < cols || x_batch_stride < 0) return XG_ERR_BAD_SHAPE;
+  if (n_slices > XG_SLICE_SUM_MAX_SLICES) return XG_ERR_TOO_LARGE;
+  if (batch == 0 || cols == 0 || n_slices == 0) return XG_OK;
+  if (x == nullptr || out == nullptr) return XG_ERR_NULL_PTR;
+  hipStream_t st = (hipStream_t)stream;
+  switch (dtype) {
+    case XG_F32:
+      return slice_sum_typed<float>(x, out, batch, rows, cols, x_batch_stride, x_row_stride, starts, ends, n_slices, st);
+    case XG_BF16:
+      return slice_sum_typed<bf16_t>(x, out, batch, rows, cols, x_batch_stride, x_row_stride, starts, ends, n_slices, st);
+    case XG_F16:
+      return slice_sum_typed<f16_t>(x, out, batch, rows, cols, x_batch_stride, x_row_stride, starts, ends, n_slices, st);
     default:
       return XG_ERR_BAD_DTYPE;
   }

@@ -31,8 +31,10 @@ _SCHEMAS = [
     "add_layer_norm_only(Tensor x, Tensor residual, Tensor? weight, Tensor? bias, float eps) -> Tensor",
     "slice_cat(Tensor src, Tensor table, int chunk_bytes, int out_cols) -> Tensor",
     "slice_cat_multi(Tensor src, Tensor table, int chunk_bytes, int[] out_cols) -> Tensor[]",
+    "slice_stack(Tensor src, Tensor[] tables, int[] chunk_bytes, int slice_len, int num) -> Tensor",
     "addn(Tensor[] inputs) -> Tensor",
     "combo_sum(Tensor[] inputs, int dim) -> Tensor[]",
+    "slice_sum_cat(Tensor x, int[] starts, int[] ends) -> Tensor",
     "silu_mul(Tensor x) -> Tensor",
     "silu_mul2(Tensor gate, Tensor up) -> Tensor",
 ]
@@ -195,7 +197,46 @@ def _slice_cat(src, table, chunk_bytes, out_cols):
     return _slice_cat_multi(src, table, chunk_bytes, [out_cols])[0]
 
 
+def _slice_stack(src, tables, chunk_bytes, slice_len, num):
+    """[num, rows, slice_len]: slab k holds one column slice of `src`.  tables[g] places the slices
+    [g * MAX_OUTS, (g + 1) * MAX_OUTS) as the outputs of one `xg_slice_cat` launch; every output pointer is a slab
+    of the ONE result buffer."""
+    if src.dim() != 2:
+        raise NotImplementedError("input must be 2d")
+    if src.stride(1) != 1:
+        src = src.contiguous()
+    esz = src.element_size()
+    rows = src.shape[0]
+    out = torch.empty((num, rows, slice_len), dtype=src.dtype, device=src.device)
+    step = _lib.SLICE_CAT_MAX_OUTS
+    if len(tables) != (num + step - 1) // step or len(chunk_bytes) != len(tables):
+        raise ValueError("slice_stack: one table and one chunk size per group of outputs")
+    if out.numel() == 0:
+        return out
+    align = min(min(chunk_bytes), 4)
+    if (src.stride(0) * esz) % align or src.data_ptr() % align:
+        src = src.contiguous()
+    slab = rows * slice_len * esz
+    for g, (table, chunk) in enumerate(zip(tables, chunk_bytes)):
+        n = min(step, num - g * step)
+        if table.dtype != torch.int32 or table.dim() != 2 or table.shape[1] != 4 or not table.is_contiguous():
+            raise ValueError("slice_stack: tables must be contiguous int32 [n_chunks, 4] tensors")
+        if table.device != src.device:
+            raise ValueError("slice_stack: tables must live on the source's device")
+        ptrs = (ctypes.c_void_p * n)(*[out.data_ptr() + (g * step + k) * slab for k in range(n)])
+        rbs = (ctypes.c_int64 * n)(*([slice_len * esz] * n))
+        st = _lib.lib().xg_slice_cat(_ptr(src), src.stride(0) * esz, rows, ptrs, rbs, n, _ptr(table), table.shape[0], chunk, _stream())
+        _lib.check(st, "xg_slice_cat")
+    return out
+
+
 _library.impl("slice_cat", _slice_cat, "CUDA")
+_library.impl("slice_stack", _slice_stack, "CUDA")
+_library.impl(
+    "slice_stack",
+    lambda src, tables, chunk_bytes, slice_len, num: torch.empty((num, src.shape[0], slice_len), dtype=src.dtype, device=src.device),
+    "Meta",
+)
 _library.impl("slice_cat_multi", _slice_cat_multi, "CUDA")
 _library.impl(
     "slice_cat",
@@ -269,6 +310,36 @@ def _combo_sum(inputs: List[torch.Tensor], dim: int):
 
 _library.impl("addn", _addn, "CUDA")
 _library.impl("combo_sum", _combo_sum, "CUDA")
+
+
+def _slice_sum_cat(x, starts, ends):
+    """x [B, R, C] -> [B, n * C]; block i = x[:, starts[i]:ends[i], :].sum(1)."""
+    if x.dim() != 3:
+        raise NotImplementedError("input must be 3d")
+    if len(starts) != len(ends) or len(starts) == 0:
+        raise ValueError("slice_sum_cat: one (start, end) pair per slice, at least one")
+    if len(starts) > _lib.SLICE_SUM_MAX_SLICES:
+        raise ValueError(f"slice_sum_cat: at most {_lib.SLICE_SUM_MAX_SLICES} slices per call")
+    if x.stride(2) != 1 or x.stride(1) < x.shape[2]:
+        x = x.contiguous()
+    B, R, C = x.shape
+    n = len(starts)
+    out = torch.empty((B, n * C), dtype=x.dtype, device=x.device)
+    if out.numel() == 0:
+        return out
+    s_arr = (ctypes.c_int32 * n)(*starts)
+    e_arr = (ctypes.c_int32 * n)(*ends)
+    st = _lib.lib().xg_slice_sum_cat(_ptr(x), _ptr(out), B, R, C, x.stride(0), x.stride(1), s_arr, e_arr, n, _code(x.dtype), _stream())
+    _lib.check(st, "xg_slice_sum_cat")
+    return out
+
+
+_library.impl("slice_sum_cat", _slice_sum_cat, "CUDA")
+_library.impl(
+    "slice_sum_cat",
+    lambda x, starts, ends: torch.empty((x.shape[0], len(starts) * x.shape[2]), dtype=x.dtype, device=x.device),
+    "Meta",
+)
 _library.impl("addn", lambda inputs: _like(inputs[0]), "Meta")
 _library.impl(
     "combo_sum",

@@ -87,6 +87,32 @@ class FuseSliceCatSameInputModule_v2(torch.nn.Module):
         return outs
 
 
+class FuseSliceModule(torch.nn.Module):
+    """Built with the start columns of equally wide slices of ONE source (last dim); forward(input, slice_len) ->
+    [n_slices, *input.shape[:-1], slice_len], slab k = input[..., start_k : start_k + slice_len]
+    (reference FuseSliceModule, structure_replacements/__init__.py:21-47).  One launch per 32 slices, every slab
+    written straight into the one result buffer."""
+
+    def __init__(self, slices_index):
+        super().__init__()
+        self.slices_index = [int(s) for s in slices_index]
+        self._tables = _SliceTables()
+
+    def forward(self, input_tensor, slice_len):
+        lead = list(input_tensor.shape[:-1])
+        src = input_tensor if input_tensor.dim() == 2 else input_tensor.reshape(-1, input_tensor.shape[-1])
+        src = _check_2d(src)
+        step = _xops._lib.SLICE_CAT_MAX_OUTS
+        tables, chunks = [], []
+        for lo in range(0, len(self.slices_index), step):
+            part = [[(s, s + slice_len)] for s in self.slices_index[lo : lo + step]]
+            table, chunk, _ = self._tables.get(src, part)
+            tables.append(table)
+            chunks.append(chunk)
+        out = torch.ops.xpu_ops.slice_stack(src, tables, chunks, slice_len, len(self.slices_index))
+        return out.view([len(self.slices_index)] + lead + [slice_len])
+
+
 class ComboSumModule(torch.nn.Module):
     """forward([3-D tensors], [dim]) -> [2-D sums]; one launch for all jobs."""
 
@@ -190,6 +216,7 @@ def get_structure_replacements(config):
         "FusedCatSlice": FuseSliceCatSameInputModule,
         "FusedSliceStackSum": FuseSliceCatSameInputModule,
         "FusedMultipleSliceCat": FuseSliceCatSameInputModule_v2,
+        "FusedSlice": FuseSliceModule,
         "ComboSum3dInp": ComboSumModule,
         "CustomDenseLayer": (DenseLayerModule, can_fuse_custom_denselayer),
         "CustomBatchDenseLayer": (BatchDenseLayerModule, can_fuse_custom_batch_denselayer),
