@@ -166,3 +166,29 @@ def test_slice_sum_cat_compiled(device, form):
     out, mods, rest = run(fn, x, other)
     assert mods == ["mi355x_slice_sum_cat_0"] and "aten.slice.Tensor" not in rest
     torch.testing.assert_close(out, fn(x, other), rtol=1.6e-2, atol=1e-3)
+
+
+def test_compile_cache_round_trip_runs_the_kernels(device, tmp_path, caplog):
+    """What the artifact cache hands back after a reload still calls the HIP kernels and computes the same
+    (reference tests/common/test_cache.py:14-55, here on the mi355x target)."""
+    from xpu_graph_amd.test_utils import need_xpu_graph_logs
+
+    src, slices = inputs.c3_slice_cat(rows=512, device=device)
+    x, r, g, b = inputs.c2_add_layernorm(rows=512, device=device)
+
+    def fn(src, x, r, g, b):
+        y, h = eager.add_layernorm_eager(x, r, g, b, 1e-5)
+        return eager.slice_cat_eager(src, slices), y, h
+
+    backend = mi355x_compiler(cache=tmp_path)
+    outs = []
+    with need_xpu_graph_logs(), torch.no_grad():
+        for _ in range(2):
+            outs.append(torch.compile(fn, backend=backend, dynamic=False)(src, x, r, g, b))
+            torch._dynamo.reset()
+    assert caplog.text.count("Save cache in location") == 1 and caplog.text.count("Use cache in location") == 1
+    mods = [n.target for n in backend.compiled_graphs[-1].graph.nodes if n.op == "call_module"]
+    assert sorted(mods) == ["fuse_slice_cat", "mi355x_fused_add_norm"]
+    for a, c in zip(outs[0], outs[1]):
+        assert torch.equal(a, c)
+    assert torch.equal(outs[1][0], eager.slice_cat_eager(src, slices))

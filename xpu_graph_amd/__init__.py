@@ -9,6 +9,9 @@ target lowers matched Aten subgraphs to hand-written gfx950 HIP kernels.
 
 Public names follow the reference package (src/xpu_graph/__init__.py).
 """
+import os
+
+from .cache import XpuGraphCache, XpuGraphLocalCache, default_cache, no_cache
 from .compiler import XpuGraph, XpuGraphCompiler, XpuGraphRuntimeArtifact
 from .config import OptLevel, Target, XpuGraphConfig
 from .device_graph_runner import GraphRunner, HIPGraphRunner
@@ -27,6 +30,10 @@ __all__ = [
     "XpuGraphCompiler",
     "XpuGraphConfig",
     "XpuGraphRuntimeArtifact",
+    "XpuGraphCache",
+    "XpuGraphLocalCache",
+    "default_cache",
+    "no_cache",
     "Target",
     "OptLevel",
     "mi355x_compiler",
@@ -40,8 +47,13 @@ __all__ = [
 ]
 
 
-def mi355x_compiler(is_training=False, opt_level=OptLevel.level2, debug=False, **config_kwargs):
+def mi355x_compiler(is_training=False, opt_level=OptLevel.level2, debug=False, cache=None, **config_kwargs):
     """Ready-made backend for the MI355X target (counterpart of the reference's mlu_compiler / npu_compiler
-    convenience constructors, src/xpu_graph/__init__.py:32-154)."""
-    cfg = XpuGraphConfig(is_training=is_training, target=Target.mi355x, opt_level=opt_level, debug=debug, enable_cache=False, **config_kwargs)
-    return XpuGraph(cfg)
+    convenience constructors, src/xpu_graph/__init__.py:32-154).  `cache`: None (no compile-artifact cache), a
+    directory, or an XpuGraphCache."""
+    if isinstance(cache, (str, os.PathLike)):
+        cache = XpuGraphLocalCache(cache)
+    cfg = XpuGraphConfig(
+        is_training=is_training, target=Target.mi355x, opt_level=opt_level, debug=debug, enable_cache=cache is not None, **config_kwargs
+    )
+    return XpuGraph(cfg, cache)

@@ -13,12 +13,14 @@ interface across torch versions.  No vendor compiler is involved: the compiled
 artifact is the FX GraphModule itself.
 """
 import itertools
+import pickle
 from typing import Callable
 
 import torch
 from torch._dynamo.backends.common import aot_autograd
 from torch._functorch.aot_autograd import make_boxed_func
 
+from .cache import SerializableArtifact, SerializableGraphModule, XpuGraphCache, default_cache
 from .config import Target, XpuGraphConfig, get_partition_fn
 from .fx_utils import FxStage, fakify_tensors
 from .passes.pass_manager import PassManager
@@ -57,7 +59,8 @@ class XpuGraph:
         config._reset_config_with_env()
         self._config = config
         setup_logger(config.debug)
-        self._cache = None  # compile-artifact caching is not part of this build
+        # reference compiler.py:43: a cache object counts only when the configuration enables caching
+        self._cache = (cache if cache is not None else default_cache()) if config.enable_cache else None
         self._orig_ctx = {}
         self.compiled_graphs = []  # the last few rewritten GraphModules, newest last (inspection / tests)
         self._set_context()
@@ -71,6 +74,15 @@ class XpuGraph:
         def compile_stage(gm, sample_inputs):
             with local_logger(stage.name):
                 fake_mode, fake_inputs = fakify_tensors(sample_inputs)
+                hashkey = None
+                if self._cache is not None:
+                    hashkey = self._cache.cache_key(gm, fake_inputs, self._config, stage)
+                    cached = self._cache.load_artifact(hashkey)
+                    if cached is not None:
+                        assert isinstance(cached, SerializableArtifact)
+                        self.compiled_graphs.append(cached.artifact)
+                        del self.compiled_graphs[:-8]
+                        return make_boxed_func(cached.artifact)
                 with fake_mode:
                     with local_logger("before"):
                         logger.debug("before xpu_graph, graph like:\n %s", gm.print_readable(print_output=False))
@@ -83,6 +95,12 @@ class XpuGraph:
                     logger.info(f"node statistic: before {before} after {_node_census(out)}")
                     if self._config.vendor_compiler_config is not None:
                         logger.warning("vendor_compiler_config is ignored: this backend runs the rewritten graph directly")
+                if hashkey is not None:
+                    try:
+                        # what runs is the re-loaded artifact, i.e. what a later process would get
+                        out = self._cache.save_artifact(hashkey, SerializableGraphModule(out)).artifact
+                    except (NotImplementedError, TypeError, AttributeError, pickle.PicklingError) as e:
+                        logger.warning(f"Artifact is not serializable ({e}), skip cache.")
                 self.compiled_graphs.append(out)
                 del self.compiled_graphs[:-8]
                 # AOT's runtime wrappers call the compiled stage with one list of arguments

@@ -98,6 +98,20 @@ class XpuGraphConfig:
             self.partition_fn = get_partition_fn(os.getenv(ENV.partition_fn))
 
 
+_cache_dir = os.getenv(ENV.cache_dir)
+
+
+def get_cache_dir():
+    """XPUGRAPH_CACHE_DIR, or a fresh temporary directory that is then exported under that name so that child
+    processes share it (reference config.py:134-145)."""
+    global _cache_dir
+    if _cache_dir is None:
+        _cache_dir = tempfile.mkdtemp(prefix="xpugraph_")
+        os.environ[ENV.cache_dir] = _cache_dir
+        logger.debug(f"Use {_cache_dir} as default local cache")
+    return _cache_dir
+
+
 _dump_dir = os.getenv(ENV.dump_dir)
 
 

@@ -33,6 +33,14 @@ def need_xpu_graph_logs():
 
 @contextlib.contextmanager
 def skip_xpu_graph_cache(backend):
-    """Force recompilation (this build keeps no compile-artifact cache; only Dynamo's code cache is reset)."""
-    torch._dynamo.reset_code_caches()
-    yield
+    """Force recompilation: Dynamo's code cache is reset and the backend's artifact cache is swapped for the base
+    class, which stores nothing (reference test_utils.py:120-130)."""
+    from .cache import XpuGraphCache
+
+    saved = backend._cache
+    try:
+        torch._dynamo.reset_code_caches()
+        backend._cache = XpuGraphCache() if saved is not None else None
+        yield
+    finally:
+        backend._cache = saved
