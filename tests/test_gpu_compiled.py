@@ -192,3 +192,29 @@ def test_compile_cache_round_trip_runs_the_kernels(device, tmp_path, caplog):
     for a, c in zip(outs[0], outs[1]):
         assert torch.equal(a, c)
     assert torch.equal(outs[1][0], eager.slice_cat_eager(src, slices))
+
+
+def test_interceptor_on_the_mi355x_target(device, caplog, tmp_path, monkeypatch):
+    """The run-time guard compares the HIP path with the Dynamo graph on every call: silent at the bf16 tolerance,
+    loud when the tolerance is set far below bf16 rounding."""
+    from xpu_graph_amd import OptLevel, Target, XpuGraph, XpuGraphConfig
+    from xpu_graph_amd.test_utils import need_xpu_graph_logs
+
+    monkeypatch.setattr("xpu_graph_amd.config._dump_dir", str(tmp_path))
+    x, W, b = inputs.c4_dense(512, 1024, 768, device=device)
+
+    def run_with(tol):
+        cfg = XpuGraphConfig(is_training=False, target=Target.mi355x, opt_level=OptLevel.level2, enable_cache=False, enable_interceptor=tol)
+        backend = XpuGraph(cfg)
+        with torch.no_grad():
+            out = torch.compile(eager.dense_silu_eager, backend=backend, dynamic=False)(x, W, b)
+        mods = [n.target for n in backend.compiled_graphs[-1].graph.nodes if n.op == "call_module"]
+        assert mods == ["custom_dense_layer_replacement"]
+        return out
+
+    with need_xpu_graph_logs():
+        out = run_with("rtol=1.6e-2,atol=2e-2")
+        assert "Monitored inference" in caplog.text and "diverges" not in caplog.text
+        torch.testing.assert_close(out, eager.dense_silu_eager(x, W, b), rtol=1.6e-2, atol=2e-2)
+        run_with("rtol=0,atol=1e-7")  # the fused epilogue rounds once, eager three times: not bit-identical
+    assert "The inference pass diverges" in caplog.text

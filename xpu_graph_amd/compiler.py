@@ -128,6 +128,21 @@ class XpuGraph:
             with torch.no_grad():
                 compiled = aot_autograd(**aot_kwargs)(dynamo_gm, example_inputs)
         artifact = XpuGraphRuntimeArtifact(compiled, boxed=False)
+        if self._config.enable_interceptor is not None:
+            import os
+
+            from .interceptor import intercept
+
+            logger.info("Wrapping compiled function with interceptor")
+            tctx = torch._guards.TracingContext.try_get()
+            artifact = intercept(
+                artifact,
+                golden_fn=dynamo_gm,
+                fw_metadata=getattr(tctx, "fw_metadata", None) if tctx is not None else None,
+                is_training=self._config.is_training,
+                mark=os.environ.get("RANK", "0"),
+                config_str=self._config.enable_interceptor,
+            )
 
         opts = kwargs.get("options") or {}
         guard_filter_fn = opts.get("guard_filter_fn")
