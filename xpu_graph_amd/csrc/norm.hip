@@ -45,11 +45,12 @@ __global__ __launch_bounds__((TPR > 256 ? TPR : 256)) void norm_rows_kernel(
   constexpr int BLOCK = TPR > 256 ? TPR : 256;
   constexpr int RPB = BLOCK / TPR;  // rows per block
   constexpr int NW = TPR > kWave ? TPR / kWave : 1;
-  __shared__ float red_all[RPB * NW];
+  __shared__ float red_all[2 * RPB * NW];  // one buffer per reduction: each is written and read once
 
   const int group = threadIdx.x / TPR;
   const int lir = threadIdx.x % TPR;  // lane in row
   float* red = red_all + group * NW;
+  float* red2 = red_all + (RPB + group) * NW;
   int64_t row = (int64_t)blockIdx.x * RPB + group;
   const bool row_ok = row < rows;
   if (!row_ok) row = rows - 1;  // keep every lane alive for the barriers; stores are masked below
@@ -97,7 +98,7 @@ __global__ __launch_bounds__((TPR > 256 ? TPR : 256)) void norm_rows_kernel(
         for (int j = 0; j < VN; ++j) s += to_f32(hv[i][j]);
       }
     }
-    mean = group_sum<TPR>(s, red, lir) * inv_cols;
+    mean = group_sum<TPR, true>(s, red, lir) * inv_cols;
   }
   float ss = 0.f;
 #pragma unroll
@@ -110,7 +111,7 @@ __global__ __launch_bounds__((TPR > 256 ? TPR : 256)) void norm_rows_kernel(
       }
     }
   }
-  const float rstd = rsqrtf(group_sum<TPR>(ss, red, lir) * inv_cols + eps);
+  const float rstd = rsqrtf(group_sum<TPR, true>(ss, red2, lir) * inv_cols + eps);
 
   if (!row_ok) return;
   V* yr = reinterpret_cast<V*>(y + row * (int64_t)nvec * VN);

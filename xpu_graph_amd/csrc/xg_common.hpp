@@ -4,6 +4,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 #include "../../include/xpu_graph_amd.h"
 
 namespace xg {
@@ -69,12 +71,29 @@ __device__ __forceinline__ void store_vec_nt(V* p, V v) {
 }
 
 // Sum over the low `width` lanes of each aligned lane group (width a power of
-// two <= 64); every lane of the group ends with the total.
+// two <= 64); every lane of the group ends with the total.  Inside a row of 16
+// lanes the exchange is done by the DPP modifiers of the adds themselves (quad
+// permutes, then the two row mirrors); only the steps across rows go through
+// the LDS crossbar.
 template <int WIDTH = kWave>
 __device__ __forceinline__ float wave_sum(float v) {
+#ifdef XG_PLAIN_SHUFFLE
 #pragma unroll
   for (int off = WIDTH / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
   return v;
+#else
+  auto dpp = [](float x, auto CTRL) {
+    constexpr int ctrl = decltype(CTRL)::value;
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), ctrl, 0xF, 0xF, true));
+  };
+  if constexpr (WIDTH >= 2) v += dpp(v, std::integral_constant<int, 0xB1>{});   // quad_perm [1,0,3,2]: lane ^ 1
+  if constexpr (WIDTH >= 4) v += dpp(v, std::integral_constant<int, 0x4E>{});   // quad_perm [2,3,0,1]: lane ^ 2
+  if constexpr (WIDTH >= 8) v += dpp(v, std::integral_constant<int, 0x141>{});  // row_half_mirror: 7 - lane within 8
+  if constexpr (WIDTH >= 16) v += dpp(v, std::integral_constant<int, 0x140>{}); // row_mirror: 15 - lane within 16
+#pragma unroll
+  for (int off = 16; off < WIDTH; off <<= 1) v += __shfl_xor(v, off, kWave);
+  return v;
+#endif
 }
 template <int WIDTH = kWave>
 __device__ __forceinline__ float wave_max(float v) {
@@ -86,14 +105,16 @@ __device__ __forceinline__ float wave_max(float v) {
 // Sum over the THREADS lanes that share one row.  THREADS <= 64: shuffle only.
 // THREADS > 64: per-wave shuffle, then the NW = THREADS/64 partial sums meet in
 // LDS (`red` holds NW floats per row group and is reused after a barrier).
-template <int THREADS>
+// FRESH: `red` has not been read since the last barrier (first use, or a buffer of its own), so the
+// barrier that protects an earlier reader can be left out.
+template <int THREADS, bool FRESH = false>
 __device__ __forceinline__ float group_sum(float v, float* red, int lane_in_row) {
   if constexpr (THREADS <= kWave) {
     return wave_sum<THREADS>(v);
   } else {
     constexpr int NW = THREADS / kWave;
     v = wave_sum<kWave>(v);
-    __syncthreads();  // previous use of `red` is over
+    if constexpr (!FRESH) __syncthreads();  // previous use of `red` is over
     if ((lane_in_row & (kWave - 1)) == 0) red[lane_in_row / kWave] = v;
     __syncthreads();
     float t = 0.f;
