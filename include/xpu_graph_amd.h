@@ -159,6 +159,19 @@ int xg_silu_mul2(const void* gate, const void* up, void* y, int64_t rows, int64_
                  int64_t up_stride, int dtype, xg_stream_t stream);
 
 /* ---------------------------------------------------------------------------
+ * Gated dense layer (SwiGLU): out[M, N] = silu(a w_gate^T) * (a w_up^T), both
+ * weights [N, K] with unit K stride and row stride ldb, a [M, K] with row stride
+ * lda, out contiguous [M, N]; bf16 or f16, fp32 accumulation; each projection is
+ * rounded to `dtype` before the gate is applied, so the result is bit-identical
+ * to two xg_dense calls followed by xg_silu_mul2.  K must be a multiple of 64.
+ * No counterpart in the reference: it fuses what its test writes as two linear
+ * layers and a silu * mul (tests/npu/test_silu_mul.py:8-16 after two
+ * CustomDenseLayer calls, structure/custom_denselayer.py:46-128).
+ * ------------------------------------------------------------------------- */
+int xg_dense_glu(const void* a, const void* w_gate, const void* w_up, void* out, int64_t M, int64_t N, int64_t K,
+                 int64_t lda, int64_t ldb, int dtype, xg_stream_t stream);
+
+/* ---------------------------------------------------------------------------
  * Dense layer: out[M,N] = act(a[M,K] @ B + bias (+ residual)), fp32 accumulate.
  *   a: row-major, row stride lda.  B is [K,N] row-major with row stride ldb when
  *   b_trans == 0, or the transpose of a row-major [N,K] (row stride ldb) when

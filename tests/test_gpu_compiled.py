@@ -113,6 +113,7 @@ def test_c5_llama_block(device, B, S):
     print("llama block modules:", mods)
     print("llama block remaining aten:", rest)
     assert "mi355x_sdpa" in mods and mods.count("mi355x_rope") == 2
+    assert "mi355x_dense_glu" in mods and "mi355x_silu_mul2" not in mods  # gate and up projections share one kernel
     assert not any(k in t for t in rest for k in ("clone", "aten.cat", "aten.neg")), rest  # no layout copies, no unfused rotary math
     heavy = [t for t in rest if any(k in t for k in ("aten.mm", "aten.bmm", "aten.addmm", "softmax", "aten.matmul"))]
     assert heavy == [], heavy  # every matmul and the softmax went to custom kernels

@@ -126,3 +126,45 @@ def test_batch_dense_compiled(device, form):
     assert [n.target for n in backend.compiled_graphs[-1].graph.nodes if n.op == "call_module"] == ["custom_batch_dense_layer_replacement"]
     want = fn(*[a.float() for a in args])
     close(got, want, K)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize(
+    "M,N,K",
+    [
+        (256, 128, 64),      # one tile, one slab
+        (8192, 1280, 256),   # 8 full tile columns + a 2-column tail computed as half-height tiles in the same launch
+        (1000, 200, 128),    # ragged rows and a last tile with 72 of 128 columns
+        (130, 8, 4096),      # a sliver of columns, deep K
+        (4096, 11008, 512),  # the Llama gate / up width
+    ],
+)
+def test_dense_glu_bit_identical_to_the_unfused_ops(device, dtype, M, N, K):
+    """silu(x Wg^T) * (x Wu^T) in one launch == two dense launches + the gate kernel, bit for bit, and within the
+    16-bit tolerance of the fp32 evaluation."""
+    g = torch.Generator().manual_seed(M + N + K)
+    x = torch.randn(M, K, generator=g).to(dtype).to(device)
+    wg = (torch.randn(N, K, generator=g) / K**0.5).to(dtype).to(device)
+    wu = (torch.randn(N, K, generator=g) / K**0.5).to(dtype).to(device)
+    ops = torch.ops.xpu_ops
+    got = ops.dense_glu(x, wg, wu)
+    two = ops.silu_mul2(ops.dense(x, wg, True, None, None, "none"), ops.dense(x, wu, True, None, None, "none"))
+    assert torch.equal(got, two)
+    ref = torch.nn.functional.silu(x.float() @ wg.float().t()) * (x.float() @ wu.float().t())
+    torch.testing.assert_close(got.float(), ref, rtol=1.6e-2, atol=2e-2)
+
+
+def test_dense_glu_strided_operands_and_rejects(device):
+    ops = torch.ops.xpu_ops
+    big = torch.randn(64, 512, device=device).bfloat16()
+    x = big[:, 128:384]  # row stride 512, K = 256
+    wbig = (torch.randn(2, 40, 256, device=device) / 16).bfloat16()
+    got = ops.dense_glu(x, wbig[0], wbig[1])
+    ref = torch.nn.functional.silu(x.float() @ wbig[0].float().t()) * (x.float() @ wbig[1].float().t())
+    torch.testing.assert_close(got.float(), ref, rtol=1.6e-2, atol=2e-2)
+    with pytest.raises(ValueError):
+        ops.dense_glu(x[:, :96], wbig[0][:, :96], wbig[1][:, :96])  # K not a multiple of 64
+    with pytest.raises(ValueError):
+        ops.dense_glu(x, wbig[0], wbig[1][:32])  # weights of different shape
+    with pytest.raises(ValueError):
+        ops.dense_glu(x.float(), wbig[0].float(), wbig[1].float())

@@ -404,8 +404,46 @@ def test_llama_block_graph_has_no_layout_copies(backend):
         gm = rewrite(mi355x_compiler(), fn, x, *[p[n] for n in names])
         mods = modules_called(gm)
         assert mods.count("mi355x_rope") == 2 and "mi355x_sdpa" in mods
+        assert mods.count("mi355x_dense_glu") == 1 and "mi355x_silu_mul2" not in mods
         left = aten_ops(gm)
         assert not any(k in t for t in left for k in ("clone", "cat", "neg", "cos", "sin", "arange", "softmax", "aten.mm", "aten.bmm")), left
+
+
+def test_gate_and_up_projections_become_one_gated_dense(caplog, backend):
+    def mlp(x, wg, wu):
+        return F.silu(F.linear(x, wg)) * F.linear(x, wu)
+
+    x = torch.randn(2, 8, 128).to(bf16)
+    wg, wu = torch.randn(96, 128).to(bf16), torch.randn(96, 128).to(bf16)
+    gm = rewrite(backend, mlp, x, wg, wu)
+    assert modules_called(gm) == ["mi355x_dense_glu"]
+    call = next(n for n in gm.graph.nodes if n.op == "call_module")
+    assert tuple(call.meta["val"].shape) == (16, 96)
+    out = next(n for n in gm.graph.nodes if n.op == "output").args[0][0]
+    assert tuple(out.meta["val"].shape) == (2, 8, 96)
+    assert "Pattern.FusedDenseGLU changed graph" in caplog.text
+
+
+def test_gated_dense_vetoes(caplog, backend):
+    def k_not_slab(x, wg, wu):  # K = 96 is not a multiple of 64: no gated kernel for it
+        return F.silu(F.linear(x, wg)) * F.linear(x, wu)
+
+    def different_inputs(x, y, wg, wu):
+        return F.silu(F.linear(x, wg)) * F.linear(y, wu)
+
+    def shared_gate(x, wg, wu):  # the gate projection has a second user
+        g = F.linear(x, wg)
+        return F.silu(g) * F.linear(x, wu), g
+
+    def kn_weights(x, wg, wu):  # [K, N] weights
+        return F.silu(x @ wg) * (x @ wu)
+
+    w = lambda *s: torch.randn(*s).to(bf16)  # noqa: E731
+    rewrite(backend, k_not_slab, w(16, 96), w(32, 96), w(32, 96))
+    rewrite(backend, different_inputs, w(16, 128), w(16, 128), w(32, 128), w(32, 128))
+    rewrite(backend, shared_gate, w(16, 128), w(32, 128), w(32, 128))
+    rewrite(backend, kn_weights, w(16, 128), w(128, 32), w(128, 32))
+    assert "Pattern.FusedDenseGLU changed graph" not in caplog.text
 
 
 def test_residual_add_moves_into_the_dense_epilogue(caplog, backend):

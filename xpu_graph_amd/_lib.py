@@ -51,6 +51,7 @@ _SIGNATURES = {
         [c_void_p, c_int64, c_int64, ctypes.POINTER(c_void_p), ctypes.POINTER(c_int64), c_int, c_void_p, c_int64, c_int, c_void_p],
     ),
     "xg_addn": (c_int, [ctypes.POINTER(c_void_p), c_int, c_void_p, c_int64, c_int, c_void_p]),
+    "xg_dense_glu": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64, c_int, c_void_p]),
     "xg_slice_sum_cat": (
         c_int,
         [c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64, ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(ctypes.c_int32), c_int, c_int, c_void_p],

@@ -4,6 +4,8 @@
 namespace xg {
 namespace gemm {
 int launch_f16(const GemmParams& p, bool b_trans, hipStream_t st);  // gemm_f16.hip
+int launch_glu_f16(const GemmParams& p, hipStream_t st);              // gemm_f16.hip
+int launch_glu_bf16(const GemmParams& p, hipStream_t st) { return launch_glu<bf16_t, bf16_t>(p, st); }
 int launch_bf16(const GemmParams& p, bool b_trans, hipStream_t st) {
   return b_trans ? launch_gemm<bf16_t, bf16_t, BLayout::KMajor>(p, st) : launch_gemm<bf16_t, bf16_t, BLayout::NMajor>(p, st);
 }
@@ -34,5 +36,26 @@ int xg_dense(const void* a, const void* b, const void* bias, const void* residua
   return dtype == XG_BF16 ? gemm::launch_bf16(p, b_trans != 0, st) : gemm::launch_f16(p, b_trans != 0, st);
 }
 
+int xg_dense_glu(const void* a, const void* w_gate, const void* w_up, void* out, int64_t M, int64_t N, int64_t K,
+                 int64_t lda, int64_t ldb, int dtype, xg_stream_t stream) {
+  using namespace xg;
+  using namespace xg::gemm;
+  if (a == nullptr || w_gate == nullptr || w_up == nullptr || out == nullptr) return XG_ERR_NULL_PTR;
+  if (M < 0 || N <= 0 || K <= 0 || lda < K || ldb < K) return XG_ERR_BAD_SHAPE;
+  if (M > 0x7fffffff || N > 0x7fffffff || K > 0x7fffffff) return XG_ERR_TOO_LARGE;
+  if (dtype != XG_BF16 && dtype != XG_F16) return XG_ERR_BAD_DTYPE;
+  if (K % 64 != 0) return XG_ERR_BAD_SHAPE;  // whole 128-byte K slabs: the gated kernel has no staged variant
+  if (N % 8 != 0 || lda % 8 != 0 || ldb % 8 != 0) return XG_ERR_BAD_ALIGN;
+  if (!aligned_to(a, 16) || !aligned_to(w_gate, 16) || !aligned_to(w_up, 16) || !aligned_to(out, 16)) return XG_ERR_BAD_ALIGN;
+  if (M == 0) return XG_OK;
+  GemmParams p = make_params(a, w_gate, nullptr, nullptr, out, M, N, K, lda, ldb, 0, XG_ACT_NONE, false);
+  p.B2 = w_up;
+  p.tiles_n = (int)((N + BN / 2 - 1) / (BN / 2));
+  // the direct-to-LDS loads address each operand with a 31-bit lane offset
+  const int64_t lim = 0x7fffffffLL;
+  if (M * lda * 2 >= lim || N * ldb * 2 >= lim) return XG_ERR_TOO_LARGE;
+  hipStream_t st = (hipStream_t)stream;
+  return dtype == XG_BF16 ? gemm::launch_glu_bf16(p, st) : gemm::launch_glu_f16(p, st);
+}
 
 }  // extern "C"

@@ -80,6 +80,7 @@ enum class BLayout { KMajor, NMajor };  // B stored [N, K] (K contiguous) or [K,
 struct GemmParams {
   const void* A;
   const void* B;
+  const void* B2;  // gated layer only: the second ("up") weight; B is then the gate weight
   const void* bias;
   const void* res;
   void* out;
@@ -371,6 +372,57 @@ __device__ __forceinline__ void epilogue(const GemmParams& p, const Lane& L, f32
   });
 }
 
+// Gated layer: waves (wm, 0) hold the gate and waves (wm, 1) the up projection of the same NI*32 rows x 128
+// columns.  Per half of 64 columns: all waves park (as above), a barrier, then each wave of the pair combines HALF of
+// the rows -- silu(gate) * up, one rounding, 16-byte stores -- reading the gate from its partner's or its own park.
+template <typename OT, int NI>
+__device__ __forceinline__ void epilogue_glu(const GemmParams& p, const Lane& L, f32x16 (&acc)[4][4], char* smem, int m0,
+                                             int n0) {
+  typedef OT O8 __attribute__((ext_vector_type(8)));
+  constexpr int PARK = 128 * 64 * 4;
+  char* park = smem + L.wave * PARK;
+  const char* gate = smem + (L.wm * 2) * PARK;
+  const char* up = smem + (L.wm * 2 + 1) * PARK;
+  const int m_base = m0 + L.wm * (NI * 32);
+  const int c = L.lane & 7, rr = L.lane >> 3;
+  static_for<2>([&](auto H) {
+    constexpr int h = decltype(H)::value;
+    static_for<2>([&](auto JJ) {
+      static_for<4>([&](auto G) {
+        static_for<NI>([&](auto I) {
+          constexpr int jj = decltype(JJ)::value, g = decltype(G)::value, i = decltype(I)::value;
+          const int row = i * 32 + L.l32;
+          const int chunk = (jj * 8 + g * 2 + L.half) ^ (row & 15);
+          const f32x16& a = acc[i][h * 2 + jj];
+          *reinterpret_cast<f32x4*>(park + row * 256 + (chunk << 4)) = f32x4{a[4 * g], a[4 * g + 1], a[4 * g + 2], a[4 * g + 3]};
+        });
+      });
+    });
+    __syncthreads();  // both parks of the pair are complete
+    const int n = n0 + h * 64 + c * 8;
+    const bool n_ok = n < p.N;  // N % 8 == 0: the 8 columns are in or out together
+    for (int it = 0; it < NI * 2; ++it) {
+      const int row = L.wn * (NI * 16) + it * 8 + rr;
+      const int m = m_base + row;
+      const int o0 = row * 256 + (((2 * c) ^ (row & 15)) << 4), o1 = row * 256 + (((2 * c + 1) ^ (row & 15)) << 4);
+      const f32x4 g0 = *reinterpret_cast<const f32x4*>(gate + o0), g1 = *reinterpret_cast<const f32x4*>(gate + o1);
+      const f32x4 u0 = *reinterpret_cast<const f32x4*>(up + o0), u1 = *reinterpret_cast<const f32x4*>(up + o1);
+      if (!(n_ok && m < p.M)) continue;
+      const float gv[8] = {g0[0], g0[1], g0[2], g0[3], g1[0], g1[1], g1[2], g1[3]};
+      const float uv[8] = {u0[0], u0[1], u0[2], u0[3], u1[0], u1[1], u1[2], u1[3]};
+      O8 o;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        // each projection is rounded to the storage type first, as the two separate layers would do
+        const float gr = to_f32(from_f32<OT>(gv[e])), ur = to_f32(from_f32<OT>(uv[e]));
+        o[e] = from_f32<OT>(gr / (1.f + __expf(-gr)) * ur);
+      }
+      *reinterpret_cast<O8*>(reinterpret_cast<OT*>(p.out) + (int64_t)m * p.ldc + n) = o;
+    }
+    __syncthreads();  // the parks are free for the next half
+  });
+}
+
 __device__ __forceinline__ void zero_acc(f32x16 (&acc)[4][4]) {
   const f32x16 zero = {};
 #pragma unroll
@@ -383,8 +435,13 @@ __device__ __forceinline__ void zero_acc(f32x16 (&acc)[4][4]) {
 // T: operand element type (bf16_t, f16_t, or uint8_t for OCP e4m3); OT: output / bias / residual type.
 // NI: 32-row A units per wave: 4 = 256 x 256 tile, 2 = 128 x 256 tile (used for the last, partial round of tiles).
 // bid / nb: this workgroup's index among the nb workgroups that share the tile grid of p.
-template <typename T, typename OT, BLayout BL, int NI>
+// GLU (gated layer, K-contiguous weights only): the 256 B rows of a tile are 128 rows of the gate weight followed by
+// the same 128 rows of the up weight, so waves with wn = 0 accumulate x Wg^T and waves with wn = 1 accumulate
+// x Wu^T for the SAME 128 output columns; the epilogue writes silu(gate) * up.  A slabs are shared, so the
+// operand traffic per output element is that of two separate layers minus one read of x.
+template <typename T, typename OT, BLayout BL, int NI, bool GLU = false>
 __device__ __forceinline__ void gemm_dma_tile(const GemmParams& p, int bid, int nb, char* smem) {
+  static_assert(!GLU || BL == BLayout::KMajor, "the gated layer is wired for K-contiguous weights");
   constexpr int EB = Elem<T>::BYTES;
   constexpr int KSTEPS = Elem<T>::KSTEPS;
   constexpr int SLAB_K = ROW_BYTES / EB;
@@ -392,7 +449,7 @@ __device__ __forceinline__ void gemm_dma_tile(const GemmParams& p, int bid, int 
 
   int tm, tn;
   tile_of_block(p, bid, nb, tm, tn);
-  const int m0 = tm * (NI * 64), n0 = tn * BN;
+  const int m0 = tm * (NI * 64), n0 = tn * (GLU ? BN / 2 : BN);
   const Lane L(NI);
 
   // Per-lane byte offsets of the 8 + 8 direct loads of a slab, relative to the slab's
@@ -408,7 +465,7 @@ __device__ __forceinline__ void gemm_dma_tile(const GemmParams& p, int bid, int 
       gr = gr < p.M ? gr : p.M - 1;  // rows past the edge re-read the last row; their results are never stored
       a_off[j] = (uint32_t)(((int64_t)gr * p.lda) * EB + lc * 16);
       if constexpr (BL == BLayout::KMajor) {
-        int gn = n0 + r;
+        int gn = n0 + (GLU ? (r & 127) : r);  // gated: tile rows 128..255 are rows 0..127 again, of the up weight
         gn = gn < p.N ? gn : p.N - 1;
         b_off[j] = (uint32_t)(((int64_t)gn * p.ldb) * EB + lc * 16);
       } else {
@@ -427,6 +484,7 @@ __device__ __forceinline__ void gemm_dma_tile(const GemmParams& p, int bid, int 
   const int wave_u = __builtin_amdgcn_readfirstlane(L.wave);  // LDS destinations of direct loads are wavefront-uniform
   const char* const a_base = reinterpret_cast<const char*>(p.A);
   const char* const b_base = reinterpret_cast<const char*>(p.B);
+  const char* const b2_base = reinterpret_cast<const char*>(GLU ? p.B2 : p.B);
 
   // load number Q (0..15) of slab kt into `stage`: uniform slab base + 32-bit lane offset
   auto issue = [&](auto Q, int kt, int stage) {
@@ -434,7 +492,8 @@ __device__ __forceinline__ void gemm_dma_tile(const GemmParams& p, int bid, int 
     if constexpr (q < 8 && q >= 2 * NI) return;  // a 128-row tile has only 4 A loads per wave
     char* dst = smem + stage * STAGE_BYTES + wave_u * 1024 + (q & 7) * 4096 + (q < 8 ? 0 : SLAB_BYTES);
     const uint32_t off = q < 8 ? a_off[q & 7] : b_off[q & 7];
-    const char* base = q < 8 ? a_base + kt * a_step : b_base + kt * b_step;
+    // B loads 8..11 fill tile rows 0..127, loads 12..15 rows 128..255 (the up weight of a gated layer)
+    const char* base = q < 8 ? a_base + kt * a_step : ((GLU && q >= 12) ? b2_base : b_base) + kt * b_step;
     load_to_lds16(base, off, (uint32_t)(size_t)(lvoid*)dst);
   };
 
@@ -449,9 +508,9 @@ __device__ __forceinline__ void gemm_dma_tile(const GemmParams& p, int bid, int 
     gr = gr < p.M ? gr : p.M - 1;
     pfa_ptr = reinterpret_cast<const char*>(p.A) + ((int64_t)gr * p.lda) * EB;
     if constexpr (BL == BLayout::KMajor) {
-      int gn = n0 + L.tid;
+      int gn = n0 + (GLU ? (L.tid & 127) : L.tid);
       gn = gn < p.N ? gn : p.N - 1;
-      pfb_ptr = reinterpret_cast<const char*>(p.B) + ((int64_t)gn * p.ldb) * EB;
+      pfb_ptr = reinterpret_cast<const char*>((GLU && L.tid >= 128) ? p.B2 : p.B) + ((int64_t)gn * p.ldb) * EB;
     } else {
       int gc = n0 + (L.tid & 3) * 64;
       gc = gc < p.N ? gc : (p.N - 8);
@@ -567,7 +626,8 @@ __device__ __forceinline__ void gemm_dma_tile(const GemmParams& p, int bid, int 
   __syncthreads();  // the slabs are dead: the epilogue reuses LDS
 
   asm volatile("s_waitcnt vmcnt(0)" : "+v"(pf_sink)::"memory");  // the last touches have landed: their register is free again
-  epilogue<OT, NI>(p, L, acc, smem, m0, n0);
+  if constexpr (GLU) epilogue_glu<OT, NI>(p, L, acc, smem, m0, n0);
+  else epilogue<OT, NI>(p, L, acc, smem, m0, n0);
 }
 
 template <typename T, typename OT, BLayout BL>
@@ -587,6 +647,25 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
     gemm_dma_tile<T, OT, BL, 4>(full, bid, n_full, smem);
   } else {
     gemm_dma_tile<T, OT, BL, 2>(rest, bid - n_full, (int)gridDim.x - n_full, smem);
+  }
+}
+
+// The gated layer: same two launch shapes as above.
+template <typename T, typename OT>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_glu_kernel(GemmParams p) {
+  extern __shared__ __align__(16) char smem[];
+  gemm_dma_tile<T, OT, BLayout::KMajor, 4, true>(p, blockIdx.x, gridDim.x, smem);
+}
+
+template <typename T, typename OT>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_glu_split_kernel(GemmParams full, GemmParams rest,
+                                                                                                               int n_full) {
+  extern __shared__ __align__(16) char smem[];
+  const int bid = blockIdx.x;  // uniform
+  if (bid < n_full) {
+    gemm_dma_tile<T, OT, BLayout::KMajor, 4, true>(full, bid, n_full, smem);
+  } else {
+    gemm_dma_tile<T, OT, BLayout::KMajor, 2, true>(rest, bid - n_full, (int)gridDim.x - n_full, smem);
   }
 }
 
@@ -783,11 +862,38 @@ int launch_gemm(const GemmParams& p, hipStream_t stream) {
   return status_from_hip(hipGetLastError());
 }
 
+// Gated layer: out[M, N] = silu(A Wg^T) * (A Wu^T), Wg = p.B and Wu = p.B2 both [N, K] with row stride ldb.
+// Output tiles are 256 x 128 (p.tiles_n counts 128-column tiles).  Needs whole K slabs: the caller checks dma_ok.
+template <typename T, typename OT>
+int launch_glu(const GemmParams& p, hipStream_t stream) {
+  constexpr int EB = Elem<T>::BYTES;
+  const int keep = full_tile_columns(p.tiles_m, p.tiles_n);
+  if (keep == p.tiles_n) return launch_kernel(gemm_glu_kernel<T, OT>, p, stream);
+  const int64_t n_split = (int64_t)keep * (BN / 2);
+  GemmParams full = p;
+  full.N = (int)n_split;
+  full.tiles_n = keep;
+  GemmParams rest = p;
+  rest.N = p.N - (int)n_split;
+  rest.tiles_n = p.tiles_n - keep;
+  rest.tiles_m = (p.M + 127) / 128;
+  rest.B = reinterpret_cast<const char*>(p.B) + n_split * p.ldb * EB;
+  rest.B2 = reinterpret_cast<const char*>(p.B2) + n_split * p.ldb * EB;
+  rest.out = reinterpret_cast<char*>(p.out) + n_split * (int64_t)sizeof(OT);
+  auto kernel = gemm_glu_split_kernel<T, OT>;
+  if (int st = set_smem_once(kernel)) return st;
+  const int64_t n_full = (int64_t)full.tiles_m * full.tiles_n, n_rest = (int64_t)rest.tiles_m * rest.tiles_n;
+  if (n_full + n_rest > 0x7fffffffLL) return XG_ERR_TOO_LARGE;
+  hipLaunchKernelGGL(kernel, dim3((unsigned)(n_full + n_rest)), dim3(kThreads), SMEM_BYTES, stream, full, rest, (int)n_full);
+  return status_from_hip(hipGetLastError());
+}
+
 inline GemmParams make_params(const void* a, const void* b, const void* bias, const void* residual, void* out, int64_t M,
                        int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldr, int act, bool bias_f32) {
   GemmParams p{};
   p.A = a;
   p.B = b;
+  p.B2 = nullptr;
   p.bias = bias;
   p.res = residual;
   p.out = out;

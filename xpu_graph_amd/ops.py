@@ -431,6 +431,7 @@ def build_slice_table(slice_lists, src_cols, elem_size, src_row_stride=None):
 # ------------------------------------------------------------- dense / SDPA
 _library.define("dense(Tensor x, Tensor weight, bool weight_trans, Tensor? bias, Tensor? residual, str act) -> Tensor")
 _library.define("dense_batched(Tensor x, Tensor weight, bool weight_trans, Tensor? bias, Tensor? residual, str act) -> Tensor")
+_library.define("dense_glu(Tensor x, Tensor w_gate, Tensor w_up) -> Tensor")
 _library.define(
     "dense_fp8(Tensor x_q, Tensor w_q, bool weight_trans, Tensor x_scale, Tensor w_scale, Tensor? bias, str act, ScalarType out_dtype) -> Tensor"
 )
@@ -651,7 +652,37 @@ def _rope_meta(x, cos, sin):
     return _empty_like_layout(_unit_last(x))
 
 
+def dense_glu_fits(x_shape, w_shape, dtype):
+    """What the gated kernel takes: 2-D x [M, K], two [N, K] weights, K a multiple of 64, N of 8, 16-bit floats."""
+    if len(x_shape) != 2 or len(w_shape) != 2 or dtype not in (torch.bfloat16, torch.float16):
+        return False
+    k, n = x_shape[1], w_shape[0]
+    ints = all(isinstance(d, int) for d in (*x_shape, *w_shape))
+    return ints and w_shape[1] == k and k % 64 == 0 and n % 8 == 0 and k > 0 and n > 0
+
+
+def _dense_glu(x, w_gate, w_up):
+    """silu(x @ w_gate.T) * (x @ w_up.T) in one launch; weights are [N, K] (torch.nn.Linear layout)."""
+    if w_gate.shape != w_up.shape or w_gate.dtype != x.dtype or w_up.dtype != x.dtype:
+        raise ValueError("dense_glu: the two weights must share shape and dtype with each other and with x")
+    if not dense_glu_fits(tuple(x.shape), tuple(w_gate.shape), x.dtype):
+        raise ValueError("dense_glu: needs x [M, K], weights [N, K], K % 64 == 0, N % 8 == 0, bf16 or f16")
+    x, w_gate, w_up = _row_major(x), _row_major(w_gate), _row_major(w_up)
+    if w_up.stride(0) != w_gate.stride(0):
+        w_gate, w_up = w_gate.contiguous(), w_up.contiguous()
+    m, k = x.shape
+    n = w_gate.shape[0]
+    out = torch.empty((m, n), dtype=x.dtype, device=x.device)
+    if out.numel() == 0:
+        return out
+    st = _lib.lib().xg_dense_glu(_ptr(x), _ptr(w_gate), _ptr(w_up), _ptr(out), m, n, k, x.stride(0), w_gate.stride(0), _code(x.dtype), _stream())
+    _lib.check(st, "xg_dense_glu")
+    return out
+
+
 _library.impl("dense", _dense, "CUDA")
+_library.impl("dense_glu", _dense_glu, "CUDA")
+_library.impl("dense_glu", lambda x, w_gate, w_up: torch.empty((x.shape[0], w_gate.shape[0]), dtype=x.dtype, device=x.device), "Meta")
 _library.impl("dense", _dense_meta, "Meta")
 _library.impl("dense_batched", _dense_batched, "CUDA")
 _library.impl("dense_batched", _dense_batched_meta, "Meta")

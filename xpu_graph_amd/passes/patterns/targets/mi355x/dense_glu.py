@@ -1,0 +1,84 @@
+"""silu(x Wg^T) * (x Wu^T): two dense calls and the SwiGLU gate -> one gated dense kernel.
+
+    silu_mul2(reshape?(dense(x, Wg, True, None, "none")), reshape?(dense(x, Wu, True, None, "none")))
+        ->  reshape?(dense_glu(x, Wg, Wu))
+
+Both projections read the same activations, both weights are [N, K] (torch.nn.Linear layout) of one shape, and each
+dense result (and its reshape) has no other user.  The kernel computes both projections in one workgroup -- the A
+operand is loaded once for the pair -- and applies the gate in its epilogue, so the two [M, N] intermediates are never
+written and the separate gate kernel disappears.  Results are bit-identical to the unfused sequence (each projection
+is rounded to the storage type before the gate).  No counterpart in the reference.
+"""
+import torch
+from torch import fx, nn
+
+from .....config import OptLevel
+from ...pattern import Pattern, PatternGroup
+from ...structure.dense import DENSE_NAME
+from ...utils.node_utils import VIEW_OPS, aten, is_call
+
+GLU_NAME = "mi355x_dense_glu"
+SILU_MUL2 = "mi355x_silu_mul2"
+
+
+class DenseGLUModule(nn.Module):
+    def forward(self, x, w_gate, w_up):
+        return torch.ops.xpu_ops.dense_glu(x, w_gate, w_up)
+
+
+def _plain_dense(node):
+    """(dense call, reshape or None) for `dense` or `reshape(dense)` with single users, no bias, no activation, [N, K] weight."""
+    view = None
+    if is_call(node, *VIEW_OPS) and len(node.users) == 1:
+        view, node = node, node.args[0]
+    if not (isinstance(node, fx.Node) and node.op == "call_module" and node.target == DENSE_NAME and len(node.users) == 1):
+        return None, None
+    if len(node.args) != 5 or node.kwargs:
+        return None, None
+    _, _, weight_trans, bias, act = node.args
+    if weight_trans is not True or bias is not None or act != "none":
+        return None, None
+    return node, view
+
+
+class FusedDenseGLU(Pattern):
+    _opt_level = OptLevel.level2
+    _pattern_group = PatternGroup.GROUP2
+
+    def process(self, gm):
+        from ..... import ops as _xops
+
+        g = gm.graph
+        changed = False
+        for node in list(g.nodes):
+            if not (node.op == "call_module" and node.target == SILU_MUL2 and len(node.args) == 2):
+                continue
+            (dg, vg), (du, vu) = _plain_dense(node.args[0]), _plain_dense(node.args[1])
+            if dg is None or du is None or dg is du or dg.args[0] is not du.args[0]:
+                continue
+            x, wg, wu = dg.args[0], dg.args[1], du.args[1]
+            vals = [n.meta.get("val") if isinstance(n, fx.Node) else None for n in (x, wg, wu)]
+            if not all(isinstance(v, torch.Tensor) for v in vals):
+                continue
+            xv, gv, uv = vals
+            if gv.shape != uv.shape or gv.dtype != xv.dtype or uv.dtype != xv.dtype:
+                continue
+            if not _xops.dense_glu_fits(tuple(xv.shape), tuple(gv.shape), xv.dtype):
+                continue
+            out_shape = node.meta["val"].shape if "val" in node.meta else None
+            if out_shape is None or not all(isinstance(d, int) for d in out_shape):
+                continue
+            if not hasattr(gm, GLU_NAME):
+                gm.add_submodule(GLU_NAME, DenseGLUModule())
+            with g.inserting_before(node):
+                fused = g.call_module(GLU_NAME, args=(x, wg, wu))
+                new = fused
+                if tuple(out_shape) != (xv.shape[0], gv.shape[0]):
+                    new = g.call_function(aten.reshape.default, (fused, list(out_shape)))
+            node.replace_all_uses_with(new)
+            g.erase_node(node)
+            for n in (vg, vu, dg, du):
+                if n is not None and len(n.users) == 0:
+                    g.erase_node(n)
+            changed = True
+        return changed
