@@ -369,6 +369,62 @@ class DenseFp8C4(DenseC4):
         return (lambda: eager.dense_fp8_silu_eager(x_q, W_q, s_x, s_w, b)), f"eager dequantise + fp32 matmul, first {self.cpu_rows} of 8192 rows"
 
 
+class DenseGluC5(Workload):
+    name = "C5 MLP gate+up: silu(x Wg^T) * (x Wu^T) bf16 M8192 K4096 N11008 (gated dense, one kernel)"
+    bound = "mfma"
+    dtype = "bf16"
+    unit = "TFLOP/s"
+    kernel = "gemm_glu_kernel<bf16> (256x128 output tiles: gate and up accumulators side by side, SwiGLU in the epilogue)"
+    work = 4 * 8192 * 4096 * 11008
+    traffic = None
+    n_sets = 3
+    cpu_rows = 256
+
+    def setup(self, torch, dev):
+        from xpu_graph_amd import _lib
+
+        self.torch = torch
+        g = torch.Generator().manual_seed(5)
+        self.sets = [
+            (
+                torch.randn(8192, 4096, generator=g).bfloat16().to(dev),
+                (0.02 * torch.randn(11008, 4096, generator=g)).bfloat16().to(dev),
+                (0.02 * torch.randn(11008, 4096, generator=g)).bfloat16().to(dev),
+            )
+            for _ in range(self.n_sets)
+        ]
+        self.outs = [torch.empty(8192, 11008, device=dev, dtype=torch.bfloat16) for _ in range(self.n_sets)]
+        self.lib = _lib.lib()
+        self.st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def op_call(self, i):
+        x, wg, wu = self.sets[i]
+        return self.torch.ops.xpu_ops.dense_glu(x, wg, wu)
+
+    def abi_call(self, i):
+        x, wg, wu = self.sets[i]
+        self.lib.xg_dense_glu(_p(x), _p(wg), _p(wu), _p(self.outs[i]), 8192, 11008, 4096, 4096, 4096, 2, self.st)
+
+    def check(self, torch):
+        x, wg, wu = self.sets[0]
+        rows = torch.arange(0, 8192, 97, device=x.device)
+        xf = x[rows].float()
+        want = torch.nn.functional.silu(xf @ wg.float().t()) * (xf @ wu.float().t())
+        torch.testing.assert_close(self.op_call(0)[rows].float(), want, rtol=1.6e-2, atol=2e-2)
+
+    def cpu_fn(self, torch):
+        from oracle import eager
+
+        x, wg, wu = (t.cpu() for t in self.sets[0])
+        x = x[: self.cpu_rows].contiguous()
+        fn, how = _default_path_compile(lambda x, wg, wu: torch.nn.functional.silu(torch.nn.functional.linear(x, wg)) * torch.nn.functional.linear(x, wu))
+        return (lambda: fn(x, wg, wu)), how + f", first {self.cpu_rows} of 8192 rows"
+
+    @property
+    def cpu_work(self):
+        return self.work * self.cpu_rows / 8192
+
+
 class SdpaC5(Workload):
     name = "C5 causal attention bf16 B4 H32 S2048 D128"
     bound = "mfma"
@@ -426,7 +482,7 @@ class LlamaBlockC5(Workload):
     bound = "mfma"
     dtype = "bf16"
     unit = "TFLOP/s"
-    kernel = "whole compiled block (7 dense, attention, 2 rotary, 3 norm / gate kernels)"
+    kernel = "whole compiled block (5 dense + 1 gated dense, attention, 2 rotary, 2 norm kernels)"
     traffic = None
     work = 2 * 8192 * (4 * 4096 * 4096 + 3 * 4096 * 11008) + 4 * 4 * 32 * 2048 * 2048 * 128 // 2
     n_sets = 1
@@ -480,7 +536,7 @@ class LlamaBlockC5(Workload):
 
 
 HEADLINE = AddLayerNormC2
-OTHERS = [RmsNormC1, SliceCatC3a, AddNC3b, DenseC4, DenseFp8C4, SdpaC5, LlamaBlockC5]
+OTHERS = [RmsNormC1, SliceCatC3a, AddNC3b, DenseC4, DenseFp8C4, DenseGluC5, SdpaC5, LlamaBlockC5]
 
 
 def run_workload(torch, dev, wl, steps, warmup, with_cpu=True):
