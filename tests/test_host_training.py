@@ -1,0 +1,146 @@
+"""Training path: the Dynamo graph is lowered to pre-dispatch Aten IR and rewritten in the `pregrad` stage before
+AOT differentiates it (reference tests/common/test_fuse_rmsnorm.py:66-157, test_fuse_layernorm.py training cases):
+the pattern fires, values and gradients agree with eager."""
+import pytest
+import torch
+import torch.nn.functional as F
+
+from xpu_graph_amd import OptLevel, Target, XpuGraph, XpuGraphConfig
+from xpu_graph_amd.fx_utils import dispatch_pregrad
+from xpu_graph_amd.test_utils import need_xpu_graph_logs
+
+
+def naive_rmsnorm(inputs, weight):
+    square = torch.square(inputs)
+    mean = torch.mean(square, dim=-1, keepdim=True)
+    root = torch.sqrt(mean + 1e-6)
+    return inputs / root * weight
+
+
+def naive_rmsnorm_variant(inputs, weight):
+    iroot = torch.rsqrt(torch.mean(inputs**2, dim=-1, keepdim=True) + 1e-6)
+    return weight * (inputs * iroot)
+
+
+def naive_rmsnorm_noweight(inputs, weight):
+    return inputs / (torch.mean(inputs * inputs, dim=-1, keepdim=True) + 1e-3) ** 0.5
+
+
+def naive_rmsnorm_liftdtype(inputs, weight):
+    return naive_rmsnorm(inputs.to(torch.float32), weight).to(inputs.dtype)
+
+
+def naive_layernorm(x, w, b):
+    mean = x.mean(-1, keepdim=True)
+    var = x.var(-1, keepdim=True, unbiased=False)
+    return (x - mean) * torch.rsqrt(var + 1e-5) * w + b
+
+
+def train_backend(**kw):
+    return XpuGraph(XpuGraphConfig(is_training=True, opt_level=OptLevel.level2, enable_cache=False, **kw))
+
+
+@pytest.mark.parametrize(
+    "fn,in_dtype,w_dtype",
+    [
+        (naive_rmsnorm, torch.float32, torch.float32),
+        (naive_rmsnorm_variant, torch.float32, torch.float32),
+        (naive_rmsnorm_noweight, torch.float32, torch.float32),
+        (naive_rmsnorm_liftdtype, torch.bfloat16, torch.float32),
+    ],
+)
+def test_rmsnorm_with_loss_and_grad(caplog, fn, in_dtype, w_dtype):
+    x = torch.randn(8, 1024, dtype=in_dtype, requires_grad=True)
+    w = torch.randn(1024, dtype=w_dtype, requires_grad=True)
+    dy = torch.randn(8, 1024, dtype=in_dtype)
+    backend = train_backend()  # before the log context: constructing a backend resets the logger's level
+    with need_xpu_graph_logs():
+        y0 = torch.compile(fn, backend=backend)(x, w)
+    gx0, gw0 = torch.autograd.grad((y0,), (x, w), (dy,), allow_unused=True)
+    y1 = fn(x, w)
+    gx1, gw1 = torch.autograd.grad((y1,), (x, w), (dy,), allow_unused=True)
+    tol = dict(rtol=1e-4, atol=1e-4) if in_dtype == torch.float32 else dict(rtol=1.6e-2, atol=1e-2)
+    torch.testing.assert_close(y0, y1, **tol)
+    torch.testing.assert_close(gx0, gx1, **tol)
+    if gw1 is None:
+        assert gw0 is None
+    else:
+        torch.testing.assert_close(gw0, gw1, rtol=1e-3, atol=1e-3 if in_dtype == torch.float32 else 0.5)
+    assert "xpu_graph passes start FxStage.pregrad" in caplog.text
+    assert "Pattern.FusedRMSNorm changed graph" in caplog.text
+
+
+def test_layernorm_with_loss_and_grad(caplog):
+    x = torch.randn(6, 256, requires_grad=True)
+    w, b = torch.randn(256, requires_grad=True), torch.randn(256, requires_grad=True)
+    dy = torch.randn(6, 256)
+    backend = train_backend()
+    with need_xpu_graph_logs():
+        y0 = torch.compile(naive_layernorm, backend=backend)(x, w, b)
+    g0 = torch.autograd.grad((y0,), (x, w, b), (dy,))
+    g1 = torch.autograd.grad((naive_layernorm(x, w, b),), (x, w, b), (dy,))
+    for a, c in zip(g0, g1):
+        torch.testing.assert_close(a, c, rtol=1e-4, atol=1e-4)
+    assert "Pattern.FusedLayerNorm changed graph" in caplog.text
+
+
+def test_pregrad_is_skipped_for_input_mutation(caplog):
+    def fn(x, buf):
+        buf.add_(1.0)
+        return (x * buf).sum(-1)
+
+    x = torch.randn(4, 8, requires_grad=True)
+    buf_c, buf_e = torch.zeros(4, 8), torch.zeros(4, 8)
+    backend = train_backend()
+    with need_xpu_graph_logs():
+        y0 = torch.compile(fn, backend=backend)(x, buf_c)
+    y1 = fn(x, buf_e)
+    torch.testing.assert_close(y0, y1)
+    torch.testing.assert_close(buf_c, buf_e)
+    (g0,) = torch.autograd.grad(y0.sum(), x)
+    torch.testing.assert_close(g0, torch.ones(4, 8))
+    assert "pregrad stage skipped" in caplog.text and "xpu_graph passes start FxStage.forward" in caplog.text
+
+
+def test_dispatch_pregrad_keeps_composites_and_signature():
+    def fn(x, w, b):
+        return (F.layer_norm(F.linear(x, w), (16,), None, b),)  # Dynamo graphs return tuples
+
+    gm = torch.fx.symbolic_trace(fn)
+    out = dispatch_pregrad(gm, [torch.randn(4, 8), torch.randn(16, 8), torch.randn(16)])
+    targets = [str(n.target) for n in out.graph.nodes if n.op == "call_function"]
+    assert targets == ["aten.linear.default", "aten.layer_norm.default"]
+    assert len([n for n in out.graph.nodes if n.op == "placeholder"]) == 3
+
+    class Holder(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.w = torch.nn.Parameter(torch.randn(3))
+
+        def forward(self, x):
+            return (x * self.w,)
+
+    with pytest.raises(NotImplementedError, match="parameters"):
+        dispatch_pregrad(torch.fx.symbolic_trace(Holder()), [torch.randn(3)])
+
+
+def test_mi355x_training_graphs_use_the_custom_ops(caplog):
+    """On the mi355x target the pregrad stage puts the HIP-backed norm and gate ops in; AOT differentiates through
+    their registered backward formulas (the forward graph below calls xpu_ops, which refuse CPU tensors)."""
+
+    def block(x, w, g, b, up):
+        h = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + 1e-6) * w
+        h = F.layer_norm(h, (64,), g, b, 1e-5)
+        return F.silu(h) * up
+
+    backend = XpuGraph(XpuGraphConfig(is_training=True, target=Target.mi355x, opt_level=OptLevel.level2, enable_cache=False))
+    args = [torch.randn(8, 64, requires_grad=True), torch.randn(64, requires_grad=True), torch.randn(64, requires_grad=True),
+            torch.randn(64, requires_grad=True), torch.randn(8, 64, requires_grad=True)]
+    with need_xpu_graph_logs(), pytest.raises(NotImplementedError):
+        torch.compile(block, backend=backend)(*args)
+    pregrad, forward = backend.compiled_graphs[-2:]
+    assert [n.target for n in pregrad.graph.nodes if n.op == "call_module"] == ["custom_rms_norm", "custom_layer_norm", "mi355x_silu_mul2"]
+    fwd_ops = [str(n.target) for n in forward.graph.nodes if n.op == "call_function"]
+    assert fwd_ops[:3] == ["xpu_ops.rms_norm.default", "xpu_ops.layer_norm.default", "xpu_ops.silu_mul2.default"]
+    for p in ("FusedRMSNorm", "CustomRMSNorm", "NativeNormToDefault", "CustomLayerNorm", "FusedSwiGLU"):
+        assert f"Pattern.{p} changed graph" in caplog.text, p

@@ -1,0 +1,101 @@
+"""Backward formulas for the custom ops that the `pregrad` stage may put into a training graph.
+
+The forward of each op is its HIP kernel; the backward is written in Aten ops (fp32 math on the saved inputs,
+statistics recomputed rather than saved), so AOT traces it into the backward graph like any other code and it runs
+on the device the tensors live on.  Registered once, when `xpu_graph_amd.ops` is imported.
+
+    rms_norm(x, w, eps)        y = x * r * w,            r = rsqrt(mean(x^2) + eps)
+    layer_norm(x, w, b, eps)   y = (x - m) * r * w + b,  r = rsqrt(var(x) + eps)
+    silu_mul2(g, u)            y = silu(g) * u
+    silu_mul(x)                y = silu(x[..., :d]) * x[..., d:]
+"""
+import torch
+
+_REGISTERED = False
+
+
+def _reduce_to(grad, shape):
+    """Sum `grad` over its leading dims down to `shape` (the shape of a weight that was broadcast over rows)."""
+    extra = grad.dim() - len(shape)
+    return grad.sum(dim=list(range(extra))) if extra > 0 else grad
+
+
+def _rms_setup(ctx, inputs, output):
+    x, w, eps = inputs
+    ctx.save_for_backward(x, w) if w is not None else ctx.save_for_backward(x)
+    ctx.has_w, ctx.eps = w is not None, eps
+
+
+def _rms_backward(ctx, gy):
+    saved = ctx.saved_tensors
+    x = saved[0]
+    w = saved[1] if ctx.has_w else None
+    xf, gf = x.float(), gy.float()
+    r = torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + ctx.eps)
+    xhat = xf * r
+    gxhat = gf * w.float() if w is not None else gf
+    gx = r * (gxhat - xhat * (gxhat * xhat).mean(-1, keepdim=True))
+    gw = _reduce_to(gf * xhat, w.shape).to(w.dtype) if w is not None and ctx.needs_input_grad[1] else None
+    return gx.to(x.dtype), gw, None
+
+
+def _ln_setup(ctx, inputs, output):
+    x, w, b, eps = inputs
+    ctx.save_for_backward(*(t for t in (x, w) if t is not None))
+    ctx.has_w, ctx.has_b, ctx.eps = w is not None, b is not None, eps
+    ctx.b_meta = (b.shape, b.dtype) if b is not None else None
+
+
+def _ln_backward(ctx, gy):
+    saved = ctx.saved_tensors
+    x = saved[0]
+    w = saved[1] if ctx.has_w else None
+    xf, gf = x.float(), gy.float()
+    mean = xf.mean(-1, keepdim=True)
+    xc = xf - mean
+    r = torch.rsqrt(xc.pow(2).mean(-1, keepdim=True) + ctx.eps)
+    xhat = xc * r
+    gxhat = gf * w.float() if w is not None else gf
+    gx = r * (gxhat - gxhat.mean(-1, keepdim=True) - xhat * (gxhat * xhat).mean(-1, keepdim=True))
+    gw = _reduce_to(gf * xhat, w.shape).to(w.dtype) if w is not None and ctx.needs_input_grad[1] else None
+    gb = _reduce_to(gf, ctx.b_meta[0]).to(ctx.b_meta[1]) if ctx.has_b and ctx.needs_input_grad[2] else None
+    return gx.to(x.dtype), gw, gb, None
+
+
+def _silu_grad(a):
+    s = torch.sigmoid(a)
+    return s * (1 + a * (1 - s))
+
+
+def _silu_mul2_setup(ctx, inputs, output):
+    ctx.save_for_backward(*inputs)
+
+
+def _silu_mul2_backward(ctx, gy):
+    g, u = ctx.saved_tensors
+    gf, uf, yf = g.float(), u.float(), gy.float()
+    return (yf * uf * _silu_grad(gf)).to(g.dtype), (yf * torch.nn.functional.silu(gf)).to(u.dtype)
+
+
+def _silu_mul_setup(ctx, inputs, output):
+    ctx.save_for_backward(inputs[0])
+
+
+def _silu_mul_backward(ctx, gy):
+    (x,) = ctx.saved_tensors
+    d = x.shape[-1] // 2
+    a, b = x[..., :d].float(), x[..., d:].float()
+    yf = gy.float()
+    return (torch.cat([yf * b * _silu_grad(a), yf * torch.nn.functional.silu(a)], dim=-1).to(x.dtype),)
+
+
+def register():
+    global _REGISTERED
+    if _REGISTERED:
+        return
+    reg = torch.library.register_autograd
+    reg("xpu_ops::rms_norm", _rms_backward, setup_context=_rms_setup)
+    reg("xpu_ops::layer_norm", _ln_backward, setup_context=_ln_setup)
+    reg("xpu_ops::silu_mul2", _silu_mul2_backward, setup_context=_silu_mul2_setup)
+    reg("xpu_ops::silu_mul", _silu_mul_backward, setup_context=_silu_mul_setup)
+    _REGISTERED = True

@@ -70,7 +70,10 @@ class XpuGraph:
         self._pass_manager.get_pattern_manager().insert_patterns(list(itertools.chain.from_iterable(plugins.values())))
 
     # -- compile one Aten graph ------------------------------------------------------
-    def _get_compiler(self, stage: FxStage):
+    def _get_compiler(self, stage: FxStage, boxed=True):
+        """The function AOT (or, for the pregrad stage, this class) calls with a graph and its sample inputs.
+        boxed: return the rewritten GraphModule wrapped for AOT's list calling convention, else the module itself."""
+
         def compile_stage(gm, sample_inputs):
             with local_logger(stage.name):
                 fake_mode, fake_inputs = fakify_tensors(sample_inputs)
@@ -82,7 +85,7 @@ class XpuGraph:
                         assert isinstance(cached, SerializableArtifact)
                         self.compiled_graphs.append(cached.artifact)
                         del self.compiled_graphs[:-8]
-                        return make_boxed_func(cached.artifact)
+                        return make_boxed_func(cached.artifact) if boxed else cached.artifact
                 with fake_mode:
                     with local_logger("before"):
                         logger.debug("before xpu_graph, graph like:\n %s", gm.print_readable(print_output=False))
@@ -104,7 +107,7 @@ class XpuGraph:
                 self.compiled_graphs.append(out)
                 del self.compiled_graphs[:-8]
                 # AOT's runtime wrappers call the compiled stage with one list of arguments
-                return make_boxed_func(out)
+                return make_boxed_func(out) if boxed else out
 
         return compile_stage
 
@@ -121,7 +124,12 @@ class XpuGraph:
             part = get_partition_fn(self._config.partition_fn)
             if part is not None:
                 aot_kwargs["partition_fn"] = part
-            compiled = aot_autograd(**aot_kwargs)(dynamo_gm, example_inputs)
+            # Patterns that replace a differentiable subgraph must run BEFORE autograd is traced: afterwards the
+            # forward graph hands the intermediates of that subgraph to the backward graph and nothing matches.
+            # So the Dynamo graph is first lowered to pre-dispatch Aten IR, rewritten in the `pregrad` stage, and
+            # AOT then differentiates the rewritten module (reference compiler.py:158-182).
+            pregrad_gm = self._pregrad(dynamo_gm, example_inputs)
+            compiled = aot_autograd(**aot_kwargs)(pregrad_gm if pregrad_gm is not None else dynamo_gm, example_inputs)
         else:
             aot_kwargs = {"fw_compiler": self._get_compiler(FxStage.inference), "keep_inference_input_mutations": True}
             # an inference compiler: trace without autograd whatever the caller's grad mode is
@@ -154,6 +162,20 @@ class XpuGraph:
             logger.info(f"Removed guards: {list(dropped)}")
             ctx.guards_context.dynamo_guards = guards - dropped
         return artifact
+
+    def _pregrad(self, dynamo_gm, example_inputs):
+        """The Dynamo graph as a rewritten pre-autograd Aten module, or None when it cannot be taken apart that way
+        (higher-order operators, tensor-subclass inputs, input mutation, parameters held by the module): the graph
+        then goes to AOT as it is and only the forward / backward stages see it."""
+        from .fx_utils import dispatch_pregrad
+
+        try:
+            dispatched = dispatch_pregrad(dynamo_gm, example_inputs)
+        except NotImplementedError as e:
+            logger.warning(f"pregrad stage skipped: {e}")
+            return None
+        logger.debug("after decompose, graph like:\n %s", dispatched.print_readable(print_output=False))
+        return self._get_compiler(FxStage.pregrad, boxed=False)(dispatched, example_inputs)
 
     def get_pattern_manager(self):
         return self._pass_manager.get_pattern_manager()

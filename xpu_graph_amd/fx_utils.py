@@ -47,3 +47,27 @@ def outside_fake_mode():
 
 def node_val(node):
     return node.meta.get("val") if isinstance(node, torch.fx.Node) else None
+
+
+def dispatch_pregrad(gm, example_inputs):
+    """Lower a Dynamo graph to functional PRE-DISPATCH Aten IR (composite ops such as linear or layer_norm stay
+    whole, autograd has not been traced) with the same inputs and outputs, ready for the `pregrad` pattern stage
+    (reference fx_utils.dispatch_graph(stage=FxStage.pregrad), src/xpu_graph/fx_utils.py:89-121).  Raises
+    NotImplementedError for graphs this cannot represent."""
+    from torch._functorch.aot_autograd import aot_export_module
+
+    if any(True for _ in gm.parameters()) or any(True for _ in gm.buffers()):
+        raise NotImplementedError("the graph owns parameters or buffers (Dynamo did not lift them to inputs)")
+    for n in gm.graph.nodes:
+        if n.op == "call_function" and isinstance(n.target, torch._ops.HigherOrderOperator):
+            raise NotImplementedError(f"higher-order operator {n.target}")
+    for t in example_inputs:
+        if isinstance(t, torch.Tensor) and type(t) not in (torch.Tensor, torch.nn.Parameter, FakeTensor):
+            raise NotImplementedError(f"tensor subclass input {type(t).__name__}")
+    try:
+        out, sig = aot_export_module(gm, list(example_inputs), trace_joint=False, pre_dispatch=True)
+    except Exception as e:  # export refuses some graphs (data-dependent control, unsupported mutation, ...)
+        raise NotImplementedError(f"pre-dispatch export failed: {type(e).__name__}: {e}") from e
+    if sig.user_inputs_to_mutate or sig.buffers_to_mutate or getattr(sig, "parameters_to_mutate", None) or sig.input_tokens:
+        raise NotImplementedError("the graph mutates its inputs")
+    return out

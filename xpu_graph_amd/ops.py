@@ -692,3 +692,9 @@ _library.impl("sdpa", _sdpa, "CUDA")
 _library.impl("sdpa", _sdpa_meta, "Meta")
 _library.impl("rope", _rope, "CUDA")
 _library.impl("rope", _rope_meta, "Meta")
+
+
+# ------------------------------------------------------------- training
+from . import autograd as _autograd  # noqa: E402
+
+_autograd.register()

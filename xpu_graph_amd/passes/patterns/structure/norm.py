@@ -27,7 +27,9 @@ def _swap(gm, default_cls, name, target_mod, needs):
 
 class CustomRMSNorm(Pattern):
     _opt_level = OptLevel.level2
-    _support_stages = [FxStage.inference]
+    # the reference keeps the custom norms out of training graphs (structure/custom_rmsnorm.py:12); here the
+    # target's norm ops carry backward formulas, so the swap may also happen before autograd is traced
+    _support_stages = [FxStage.inference, FxStage.pregrad]
 
     def __init__(self, target_mod: torch.nn.Module):
         super().__init__()
@@ -39,7 +41,7 @@ class CustomRMSNorm(Pattern):
 
 class CustomLayerNorm(Pattern):
     _opt_level = OptLevel.level2
-    _support_stages = [FxStage.inference]
+    _support_stages = [FxStage.inference, FxStage.pregrad]
 
     def __init__(self, target_mod: torch.nn.Module):
         super().__init__()

@@ -5,6 +5,8 @@ spelling; `aten.native_layer_norm` passes through it untouched.)
 
     native_layer_norm(x, [N], w, b, eps)[0]  -> fused_layer_norm(x, w, b, eps)
     _fused_rms_norm(x, [N], w, eps)[0]       -> fused_rms_norm(x, w, eps)
+    layer_norm(x, [N], w, b, eps, _)         -> fused_layer_norm(x, w, b, eps)     (pre-dispatch graphs: the
+    rms_norm(x, [N], w, eps)                 -> fused_rms_norm(x, w, eps)           composite ops are still whole)
 
 Only when the statistics outputs are unused and the norm is over the last axis.
 """
@@ -13,6 +15,7 @@ import operator
 import torch
 
 from .....config import OptLevel
+from .....fx_utils import FxStage
 from ...common.norms import LN_NAME, RMS_NAME
 from ...pattern import Pattern
 from ...utils.default_replacements import DefaultLayerNorm, DefaultRMSNorm
@@ -26,6 +29,7 @@ def _only_output0(node):
 
 class NativeNormToDefault(Pattern):
     _opt_level = OptLevel.level2
+    _support_stages = [FxStage.inference, FxStage.pregrad]
 
     def process(self, gm):
         if not hasattr(gm, LN_NAME):
@@ -44,17 +48,34 @@ class NativeNormToDefault(Pattern):
                 if eps is None:
                     eps = torch.finfo(x.meta["val"].dtype).eps
                 name, args = RMS_NAME, (x, w, eps)
+            elif is_call(node, aten.layer_norm.default):
+                x, nshape = node.args[:2]
+                w = node.args[2] if len(node.args) > 2 else None
+                b = node.args[3] if len(node.args) > 3 else None
+                eps = node.args[4] if len(node.args) > 4 else 1e-5
+                name, args = LN_NAME, (x, w, b, eps)
+            elif hasattr(aten, "rms_norm") and is_call(node, aten.rms_norm.default):
+                x, nshape = node.args[:2]
+                w = node.args[2] if len(node.args) > 2 else None
+                eps = node.args[3] if len(node.args) > 3 else None
+                if eps is None:
+                    eps = torch.finfo(x.meta["val"].dtype).eps
+                name, args = RMS_NAME, (x, w, eps)
             else:
                 continue
+            single = is_call(node, aten.layer_norm.default) or (hasattr(aten, "rms_norm") and is_call(node, aten.rms_norm.default))
             if len(nshape) != 1 or not same_shape(list(nshape), list(x.meta["val"].shape[-1:])):
                 continue
-            if not _only_output0(node) or not isinstance(eps, (int, float)):
+            if not isinstance(eps, (int, float)) or (not single and not _only_output0(node)):
                 continue
             with g.inserting_before(node):
                 new = g.call_module(name, args)
-            for u in list(node.users):
-                u.replace_all_uses_with(new)
-                g.erase_node(u)
+            if single:  # the composite ops return the normalised tensor itself
+                node.replace_all_uses_with(new)
+            else:
+                for u in list(node.users):
+                    u.replace_all_uses_with(new)
+                    g.erase_node(u)
             g.erase_node(node)
             changed = True
         return changed

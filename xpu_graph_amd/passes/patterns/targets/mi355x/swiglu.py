@@ -11,6 +11,7 @@ import torch
 from torch import fx, nn
 
 from .....config import OptLevel
+from .....fx_utils import FxStage
 from ...pattern import Pattern
 from ...utils.node_utils import aten, is_call, same_shape, sole_user_is
 
@@ -84,6 +85,7 @@ def match_swiglu(mul):
 
 class FusedSwiGLU(Pattern):
     _opt_level = OptLevel.level2
+    _support_stages = [FxStage.inference, FxStage.pregrad]  # silu_mul / silu_mul2 carry backward formulas
 
     def process(self, gm):
         if not hasattr(gm, "mi355x_silu_mul"):
