@@ -324,7 +324,7 @@ class DenseFp8C4(DenseC4):
     name = "C4 dense + bias + SiLU fp8 e4m3 (per-tensor x, per-channel W) M8192 K4096 N11008"
     dtype = "fp8"
     kernel = "gemm_dma_split_kernel<e4m3,[N,K] weight>"
-    traffic = None
+    traffic = 746.7e6  # FETCH_SIZE / WRITE_SIZE per launch (profiles/mfma_kernels_bench.md)
 
     def setup(self, torch, dev):
         from oracle import eager, inputs
@@ -376,7 +376,7 @@ class DenseGluC5(Workload):
     unit = "TFLOP/s"
     kernel = "gemm_glu_kernel<bf16> (256x128 output tiles: gate and up accumulators side by side, SwiGLU in the epilogue)"
     work = 4 * 8192 * 4096 * 11008
-    traffic = None
+    traffic = 2382.0e6  # FETCH_SIZE / WRITE_SIZE per launch (profiles/mfma_kernels_bench.md)
     n_sets = 3
     cpu_rows = 256
 
