@@ -144,3 +144,24 @@ def test_mi355x_training_graphs_use_the_custom_ops(caplog):
     assert fwd_ops[:3] == ["xpu_ops.rms_norm.default", "xpu_ops.layer_norm.default", "xpu_ops.silu_mul2.default"]
     for p in ("FusedRMSNorm", "CustomRMSNorm", "NativeNormToDefault", "CustomLayerNorm", "FusedSwiGLU"):
         assert f"Pattern.{p} changed graph" in caplog.text, p
+
+
+def test_linear_is_decomposed_for_the_dense_pattern_in_pregrad(caplog):
+    """Pre-dispatch graphs keep aten.linear whole; DecomposeLinear turns it into (add)mm so that the dense
+    pattern fires before autograd is traced (the dense op has a backward formula)."""
+
+    def mlp(x, w1, b1, w2):
+        return F.linear(F.relu(F.linear(x, w1, b1)), w2)
+
+    bf = torch.bfloat16
+    backend = XpuGraph(XpuGraphConfig(is_training=True, target=Target.mi355x, opt_level=OptLevel.level2, enable_cache=False))
+    args = [torch.randn(2, 8, 64).to(bf).requires_grad_(True), torch.randn(128, 64).to(bf).requires_grad_(True),
+            torch.randn(128).to(bf).requires_grad_(True), torch.randn(64, 128).to(bf).requires_grad_(True)]
+    with need_xpu_graph_logs(), pytest.raises(NotImplementedError):
+        torch.compile(mlp, backend=backend)(*args)
+    pregrad = backend.compiled_graphs[-2]
+    calls = [n for n in pregrad.graph.nodes if n.op == "call_module"]
+    assert [n.target for n in calls] == ["custom_dense_layer_replacement"] * 2
+    assert calls[0].args[2] is True and calls[0].args[3] is not None  # [N, K] weight, bias kept
+    assert not any("linear" in str(n.target) or "aten.mm" in str(n.target) for n in pregrad.graph.nodes)
+    assert "Pattern.DecomposeLinear changed graph" in caplog.text and "Pattern.CustomDenseLayer changed graph" in caplog.text

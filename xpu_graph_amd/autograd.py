@@ -8,6 +8,12 @@ on the device the tensors live on.  Registered once, when `xpu_graph_amd.ops` is
     layer_norm(x, w, b, eps)   y = (x - m) * r * w + b,  r = rsqrt(var(x) + eps)
     silu_mul2(g, u)            y = silu(g) * u
     silu_mul(x)                y = silu(x[..., :d]) * x[..., d:]
+    dense(x, W, trans, bias, residual, act)   y = act(x W(^T) + bias + residual)
+
+The input gradient of the dense layer is itself a dense layer over the same weight read the other way, so it runs on
+the HIP kernel; the weight gradient needs a transposed left operand, which that kernel does not take, and is an Aten
+matmul.  For activations whose derivative cannot be told from the output (silu, gelu) the pre-activation is
+recomputed with one more dense call.
 """
 import torch
 
@@ -89,6 +95,48 @@ def _silu_mul_backward(ctx, gy):
     return (torch.cat([yf * b * _silu_grad(a), yf * torch.nn.functional.silu(a)], dim=-1).to(x.dtype),)
 
 
+def _dense_setup(ctx, inputs, output):
+    x, weight, weight_trans, bias, residual, act = inputs
+    ctx.save_for_backward(x, weight, output, *(t for t in (bias, residual) if t is not None))
+    ctx.trans, ctx.act = weight_trans, act
+    ctx.has_bias, ctx.has_res = bias is not None, residual is not None
+
+
+def _dense_backward(ctx, gy):
+    saved = ctx.saved_tensors
+    x, weight, y = saved[:3]
+    rest = list(saved[3:])
+    bias = rest.pop(0) if ctx.has_bias else None
+    residual = rest.pop(0) if ctx.has_res else None
+    act = ctx.act
+    gf = gy.float()
+    if act == "none":
+        gz = gf
+    elif act == "relu":
+        gz = gf * (y > 0)
+    elif act == "sigmoid":
+        yf = y.float()
+        gz = gf * yf * (1 - yf)
+    else:
+        z = torch.ops.xpu_ops.dense(x, weight, ctx.trans, bias, residual, "none").float()
+        if act == "silu":
+            gz = gf * _silu_grad(z)
+        elif act == "gelu":
+            cdf = 0.5 * (1 + torch.erf(z * 0.7071067811865476))
+            gz = gf * (cdf + z * torch.exp(-0.5 * z * z) * 0.3989422804014327)
+        else:
+            raise NotImplementedError(f"dense backward: activation {act!r}")
+    gz = gz.to(x.dtype)
+    need = ctx.needs_input_grad
+    gx = torch.ops.xpu_ops.dense(gz, weight, not ctx.trans, None, None, "none") if need[0] else None
+    gw = None
+    if need[1]:
+        gw = (gz.t() @ x) if ctx.trans else (x.t() @ gz)
+    gb = gz.float().sum(0).to(bias.dtype) if ctx.has_bias and need[3] else None
+    gr = gz if ctx.has_res and need[4] else None
+    return gx, gw, None, gb, gr, None
+
+
 def register():
     global _REGISTERED
     if _REGISTERED:
@@ -98,4 +146,5 @@ def register():
     reg("xpu_ops::layer_norm", _ln_backward, setup_context=_ln_setup)
     reg("xpu_ops::silu_mul2", _silu_mul2_backward, setup_context=_silu_mul2_setup)
     reg("xpu_ops::silu_mul", _silu_mul_backward, setup_context=_silu_mul_setup)
+    reg("xpu_ops::dense", _dense_backward, setup_context=_dense_setup)
     _REGISTERED = True

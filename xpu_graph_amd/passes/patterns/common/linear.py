@@ -55,3 +55,39 @@ class FusedAddMM(Pattern):
             g.erase_node(node)
             changed = True
         return changed
+
+
+class DecomposeLinear(Pattern):
+    """Pre-dispatch graphs keep `aten.linear(x, W, b)` whole; the dense patterns speak mm / addmm:
+
+        linear(x, W, b)  ->  reshape(addmm(b, reshape(x, [-1, K]), t(W)), [..., N])      (mm without b)
+
+    Only in the pregrad stage (after autograd is traced, linear is already decomposed this way)."""
+
+    _opt_level = OptLevel.level2
+    _support_stages = [FxStage.pregrad]
+
+    def process(self, gm):
+        g = gm.graph
+        changed = False
+        for node in list(g.nodes):
+            if not is_call(node, aten.linear.default):
+                continue
+            x, w = node.args[0], node.args[1]
+            bias = node.args[2] if len(node.args) > 2 else node.kwargs.get("bias")
+            xv, wv = x.meta.get("val"), w.meta.get("val")
+            if not isinstance(xv, torch.Tensor) or not isinstance(wv, torch.Tensor) or wv.dim() != 2 or xv.dim() < 1:
+                continue
+            if bias is not None and bias.meta["val"].dim() != 1:
+                continue
+            k, n = wv.shape[1], wv.shape[0]
+            with g.inserting_before(node):
+                x2 = x if xv.dim() == 2 else g.call_function(aten.reshape.default, (x, [-1, k]))
+                wt = g.call_function(aten.t.default, (w,))
+                y = g.call_function(aten.mm.default, (x2, wt)) if bias is None else g.call_function(aten.addmm.default, (bias, x2, wt))
+                if xv.dim() != 2:
+                    y = g.call_function(aten.reshape.default, (y, list(xv.shape[:-1]) + [n]))
+            node.replace_all_uses_with(y)
+            g.erase_node(node)
+            changed = True
+        return changed

@@ -7,6 +7,7 @@ arguments and may veto the rewrite, which leaves the Aten subgraph in place."""
 from torch import fx
 
 from ....config import OptLevel
+from ....fx_utils import FxStage
 from ..pattern import Pattern
 from ..utils.node_utils import activation_name, arg, aten, is_call, mm_operands, sole_user_is, strip_transpose
 
@@ -36,6 +37,8 @@ def match_dense(node):
 
 class CustomDenseLayer(Pattern):
     _opt_level = OptLevel.level2
+    # pregrad as well: the target's dense op carries a backward formula (the reference keeps it to inference)
+    _support_stages = [FxStage.inference, FxStage.pregrad]
 
     def __init__(self, target_mod, constraint_fn=None):
         super().__init__()
