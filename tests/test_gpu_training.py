@@ -75,6 +75,9 @@ def test_swiglu_halves_gradient(device):
 def test_dense_backward_formula(device, act, weight_trans):
     """Gradients of xpu_ops.dense (input gradient on the HIP kernel, weight gradient an Aten matmul) against
     autograd of the same layer evaluated in fp32."""
+    import xpu_graph_amd.ops as xops
+
+    xops.enable_autograd()
     torch.manual_seed(1)
     M, K, N = 384, 256, 192
     bf = torch.bfloat16

@@ -2,7 +2,9 @@
 
 The forward of each op is its HIP kernel; the backward is written in Aten ops (fp32 math on the saved inputs,
 statistics recomputed rather than saved), so AOT traces it into the backward graph like any other code and it runs
-on the device the tensors live on.  Registered once, when `xpu_graph_amd.ops` is imported.
+on the device the tensors live on.  Registered once per process, on demand (`ops.enable_autograd()`, called by a
+backend constructed with is_training=True on the mi355x target): a Python autograd formula costs every call of the op
+a few microseconds of dispatch, which inference-only processes should not pay.
 
     rms_norm(x, w, eps)        y = x * r * w,            r = rsqrt(mean(x^2) + eps)
     layer_norm(x, w, b, eps)   y = (x - m) * r * w + b,  r = rsqrt(var(x) + eps)

@@ -64,6 +64,10 @@ class XpuGraph:
         self._orig_ctx = {}
         self.compiled_graphs = []  # the last few rewritten GraphModules, newest last (inspection / tests)
         self._set_context()
+        if config.is_training and config.target == Target.mi355x:
+            from . import ops as _xops
+
+            _xops.enable_autograd()  # the target's norm / gate / dense ops may enter training graphs
         self._pass_manager = PassManager(config)
         # plugin patterns run before the built-in ones of their group
         plugins = __PLUGIN_PATTERN_GROUP__.get(config.target, {})

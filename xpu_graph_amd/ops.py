@@ -695,6 +695,10 @@ _library.impl("rope", _rope_meta, "Meta")
 
 
 # ------------------------------------------------------------- training
-from . import autograd as _autograd  # noqa: E402
+def enable_autograd():
+    """Register the backward formulas of the ops that may appear in training graphs (xpu_graph_amd/autograd.py).
+    Done on demand -- by a backend constructed with is_training=True -- because an op with a Python autograd
+    formula pays a few microseconds of dispatch on every call, which inference-only processes need not."""
+    from . import autograd as _autograd
 
-_autograd.register()
+    _autograd.register()
