@@ -219,3 +219,42 @@ def test_interceptor_on_the_mi355x_target(device, caplog, tmp_path, monkeypatch)
         torch.testing.assert_close(out, eager.dense_silu_eager(x, W, b), rtol=1.6e-2, atol=2e-2)
         run_with("rtol=0,atol=1e-7")  # the fused epilogue rounds once, eager three times: not bit-identical
     assert "The inference pass diverges" in caplog.text
+
+
+def test_dynamic_batch_one_compile_many_sizes(device):
+    """The batch dimension marked dynamic: one compile serves several batch sizes, every fused kernel takes the row
+    count at run time, results follow eager (reference tests compile most patterns with dynamic=True as well)."""
+    import torch.nn.functional as F
+
+    torch._dynamo.reset()
+    offs = [7, 100, 40, 200]
+    g = torch.Generator().manual_seed(3)
+    w_norm = torch.randn(256, generator=g).to(device)
+    W = (torch.randn(256, 128, generator=g) / 16).bfloat16().to(device)
+    b = torch.randn(128, generator=g).bfloat16().to(device)
+
+    def fn(src, x):
+        cat = torch.cat([src[:, o : o + 8] for o in offs], dim=1)
+        h = eager.rmsnorm_eager(x, w_norm, 1e-6)
+        y = F.silu(h.bfloat16() @ W + b)
+        return cat, h, y
+
+    backend = mi355x_compiler()
+    compiled = torch.compile(fn, backend=backend, dynamic=None)
+    n_graphs = 0
+    for rows in (48, 200, 7):
+        src = torch.randn(rows, 512, generator=g).to(device)
+        x = torch.randn(rows, 256, generator=g).to(device)
+        torch._dynamo.mark_dynamic(src, 0)
+        torch._dynamo.mark_dynamic(x, 0)
+        with torch.no_grad():
+            cat, h, y = compiled(src, x)
+            cat_e, h_e, y_e = fn(src, x)
+        if n_graphs == 0:
+            n_graphs = len(backend.compiled_graphs)
+            mods = sorted(n.target for n in backend.compiled_graphs[-1].graph.nodes if n.op == "call_module")
+            assert mods == ["custom_dense_layer_replacement", "custom_rms_norm", "fuse_slice_cat"]
+        assert torch.equal(cat, cat_e)
+        torch.testing.assert_close(h, h_e, rtol=1e-5, atol=1e-5)
+        torch.testing.assert_close(y, y_e, rtol=1.6e-2, atol=2e-2)
+    assert len(backend.compiled_graphs) == n_graphs  # no recompilation for the other batch sizes

@@ -657,7 +657,7 @@ def dense_glu_fits(x_shape, w_shape, dtype):
     if len(x_shape) != 2 or len(w_shape) != 2 or dtype not in (torch.bfloat16, torch.float16):
         return False
     k, n = x_shape[1], w_shape[0]
-    ints = all(isinstance(d, int) for d in (*x_shape, *w_shape))
+    ints = all(isinstance(d, int) for d in (k, *w_shape))  # the row count may be symbolic
     return ints and w_shape[1] == k and k % 64 == 0 and n % 8 == 0 and k > 0 and n > 0
 
 

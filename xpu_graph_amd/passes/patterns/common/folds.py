@@ -27,6 +27,11 @@ def _storage_key(node):
     return None
 
 
+def _same_storage(a, b):
+    """Keys of _storage_key; a node without storage (a size-valued placeholder of a dynamic graph) shares none."""
+    return a is not None and b is not None and a == b
+
+
 def _output_storages(gm):
     out = list(gm.graph.nodes)[-1]
     assert out.op == "output"
@@ -183,9 +188,9 @@ class FoldClone(Pattern):
         if key is None or src.op not in ("call_module", "call_function"):
             return False
         for n in gm.graph.nodes:
-            if n.op in ("placeholder", "get_attr") and _storage_key(n) == key:
+            if n.op in ("placeholder", "get_attr") and _same_storage(_storage_key(n), key):
                 return False
-        if any(o is not clone and _storage_key(o) == key for o in out_nodes):
+        if any(o is not clone and _same_storage(_storage_key(o), key) for o in out_nodes):
             return False
         fmt = clone.kwargs.get("memory_format", torch.preserve_format)
         return fmt in (torch.preserve_format, torch.contiguous_format) and src.meta["val"].is_contiguous()

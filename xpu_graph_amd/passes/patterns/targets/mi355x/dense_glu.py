@@ -15,7 +15,7 @@ from torch import fx, nn
 from .....config import OptLevel
 from ...pattern import Pattern, PatternGroup
 from ...structure.dense import DENSE_NAME
-from ...utils.node_utils import VIEW_OPS, aten, is_call
+from ...utils.node_utils import VIEW_OPS, aten, is_call, same_shape
 
 GLU_NAME = "mi355x_dense_glu"
 SILU_MUL2 = "mi355x_silu_mul2"
@@ -65,16 +65,20 @@ class FusedDenseGLU(Pattern):
                 continue
             if not _xops.dense_glu_fits(tuple(xv.shape), tuple(gv.shape), xv.dtype):
                 continue
-            out_shape = node.meta["val"].shape if "val" in node.meta else None
-            if out_shape is None or not all(isinstance(d, int) for d in out_shape):
+            out_shape = list(node.meta["val"].shape) if "val" in node.meta else None
+            if out_shape is None:
                 continue
+            symbolic = [i for i, d in enumerate(out_shape) if not isinstance(d, int)]
+            if len(symbolic) > 1:  # the reshape back can leave one dim (the batch) to be inferred
+                continue
+            back_shape = [(-1 if i in symbolic else d) for i, d in enumerate(out_shape)]
             if not hasattr(gm, GLU_NAME):
                 gm.add_submodule(GLU_NAME, DenseGLUModule())
             with g.inserting_before(node):
                 fused = g.call_module(GLU_NAME, args=(x, wg, wu))
                 new = fused
-                if tuple(out_shape) != (xv.shape[0], gv.shape[0]):
-                    new = g.call_function(aten.reshape.default, (fused, list(out_shape)))
+                if not same_shape(out_shape, [xv.shape[0], gv.shape[0]]):
+                    new = g.call_function(aten.reshape.default, (fused, back_shape))
             node.replace_all_uses_with(new)
             g.erase_node(node)
             for n in (vg, vu, dg, du):

@@ -88,15 +88,23 @@ def is_causal_constant(mask, sq, skv):
         return bool((m[~upper] == 0).all()) and bool(((masked == float("-inf")) | (masked <= lowest)).all())
 
 
+def _static(*dims):
+    return all(isinstance(d, int) for d in dims)
+
+
 def _same_attention_problem(src, dims):
     """src is 4-D [B', H', S, D] with B'*H' == B*H and the same S, D: every (batch, head) pair is an
-    independent attention problem, so how the leading two axes are split does not matter."""
+    independent attention problem, so how the leading two axes are split does not matter.  S, D and the head
+    counts must be static; the batch may be symbolic."""
     if not (isinstance(src, fx.Node) and "val" in src.meta and isinstance(src.meta["val"], torch.Tensor)):
         return False
     shp = list(src.meta["val"].shape)
-    if len(shp) != 4 or not all(isinstance(d, int) for d in shp + list(dims)):
+    dims = list(dims)
+    if len(shp) != 4 or len(dims) != 4 or not _static(*shp[2:], *dims[2:]):
         return False
-    return shp[2:] == list(dims[2:]) and shp[0] * shp[1] == dims[0] * dims[1]
+    if shp[2:] != dims[2:]:
+        return False
+    return same_shape([shp[0] * shp[1]], [dims[0] * dims[1]])
 
 
 def _through_clone(node):
@@ -134,17 +142,21 @@ def _peel_k(node, dims):
 
 
 def _supported(q, k, v):
+    """bf16 / f16 4-D operands, head dim 64 or 128, static head counts and sequence lengths (the batch may be
+    symbolic), kv heads dividing the query heads."""
     vq, vk, vv = (n.meta.get("val") for n in (q, k, v))
     if not all(isinstance(t, torch.Tensor) and t.dim() == 4 for t in (vq, vk, vv)):
         return False
     if vq.dtype not in _DTYPES or vk.dtype != vq.dtype or vv.dtype != vq.dtype:
         return False
     B, H, Sq, D = vq.shape
-    if not all(isinstance(d, int) for d in (B, H, Sq, D, *vk.shape, *vv.shape)):
+    if not _static(H, Sq, D, *vk.shape[1:], *vv.shape[1:]):
         return False
     if D not in _HEAD_DIMS or vk.shape[-1] != D or vv.shape[-1] != D:
         return False
-    if vk.shape[0] != B or vv.shape != vk.shape or vk.shape[1] == 0 or H % vk.shape[1] != 0:
+    if not (same_shape([vk.shape[0]], [B]) and same_shape([vv.shape[0]], [B])):
+        return False
+    if list(vv.shape[1:]) != list(vk.shape[1:]) or vk.shape[1] == 0 or H % vk.shape[1] != 0:
         return False
     return True
 
@@ -186,7 +198,9 @@ class FusedCausalSDPA(Pattern):
                 dropout = node.args[4] if len(node.args) > 4 else node.kwargs.get("dropout_p", 0.0)
                 causal = node.args[5] if len(node.args) > 5 else node.kwargs.get("is_causal", False)
                 scale = node.kwargs.get("scale")
-                if node.kwargs.get("enable_gqa", False) or dropout != 0.0 or not _supported(q, k, v):
+                if node.kwargs.get("enable_gqa", False) or dropout != 0.0:
+                    continue
+                if not all(isinstance(n, fx.Node) and isinstance(n.meta.get("val"), torch.Tensor) and n.meta["val"].dim() == 4 for n in (q, k, v)):
                     continue
                 sq, skv = q.meta["val"].shape[2], k.meta["val"].shape[2]
                 if mask is not None:
@@ -196,13 +210,25 @@ class FusedCausalSDPA(Pattern):
                 q2 = _peel_qv(q, q.meta["val"].shape)
                 k2 = _peel_k(k, k.meta["val"].shape)
                 v2 = _peel_qv(v, v.meta["val"].shape)
-                lead = {tuple(n.meta["val"].shape[:2]) for n in (q2, k2, v2)}
-                peeled = q2 is not q and k2 is not k and v2 is not v and len(lead) == 1
+                lead_q = list(q2.meta["val"].shape[:2])
+                same_lead = all(same_shape(list(n.meta["val"].shape[:2]), lead_q) for n in (k2, v2))
+                peeled = q2 is not q and k2 is not k and v2 is not v and same_lead
+                out_shape = list(node.meta["val"].shape)
+                # shape argument of the reshape back: ints, with -1 for the one dim that may be symbolic (the batch)
+                symbolic = [i for i, d in enumerate(out_shape) if not isinstance(d, int)]
+                back_shape = [(-1 if i in symbolic else d) for i, d in enumerate(out_shape)]
+                needs_back = peeled and not same_shape(list(q2.meta["val"].shape), out_shape)
+                if needs_back and len(symbolic) > 1:
+                    peeled = needs_back = False
+                if peeled and not _supported(q2, k2, v2):
+                    peeled = needs_back = False
                 if not peeled:
                     q2, k2, v2 = q, k, v
-                out_shape = tuple(node.meta["val"].shape)
+                    # (with a symbolic batch FusedSDPA folds it into the head axis: only the peeled views qualify)
+                    if not _supported(q, k, v):
+                        continue
 
-                def replace(new, old=node, reshape_back=peeled and tuple(q2.meta["val"].shape) != out_shape, shp=out_shape):
+                def replace(new, old=node, reshape_back=needs_back, shp=back_shape):
                     if reshape_back:
                         with gm.graph.inserting_after(new):
                             new = gm.graph.call_function(aten.reshape.default, (new, shp))

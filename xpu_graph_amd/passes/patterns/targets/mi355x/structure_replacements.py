@@ -28,13 +28,15 @@ class _SliceTables:
         self._cache = {}
 
     def get(self, src, slice_lists):
+        if isinstance(src, FakeTensor):
+            # shape propagation only (sizes and strides may be symbolic): the op's output shape depends on the
+            # slice widths alone, so any table stands in
+            out_cols = [sum(e - s for s, e in sl) for sl in slice_lists]
+            return torch.empty((1, 4), dtype=torch.int32, device=src.device), 4, out_cols
         key = (tuple(tuple(map(tuple, sl)) for sl in slice_lists), src.shape[1], src.stride(0), src.element_size(), str(src.device))
         hit = self._cache.get(key)
         if hit is None:
             table, chunk, out_cols = _xops.build_slice_table(slice_lists, src.shape[1], src.element_size(), src.stride(0))
-            if isinstance(src, FakeTensor):
-                # shape propagation only: a table of the right shape, nothing cached
-                return torch.empty(table.shape, dtype=torch.int32, device=src.device), chunk, out_cols
             hit = (table.to(src.device), chunk, out_cols)
             self._cache[key] = hit
         return hit

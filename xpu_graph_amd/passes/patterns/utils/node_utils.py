@@ -76,9 +76,19 @@ def rank(node):
     return len(node.meta["val"].shape)
 
 
+def _dim_value(d):
+    """A graph node that stands for a size (sym_size of a dynamic dim) compares by the symbol it carries."""
+    if isinstance(d, fx.Node):
+        return d.meta.get("val")
+    return d
+
+
 def same_shape(a, b):
-    a = list(a) if isinstance(a, (torch.Size, tuple)) else a
-    b = list(b) if isinstance(b, (torch.Size, tuple)) else b
+    """Provably equal shapes; entries may be ints, SymInts or size-valued graph nodes.  Unknown -> False."""
+    a = [_dim_value(d) for d in (a if isinstance(a, (list, tuple, torch.Size)) else [a])]
+    b = [_dim_value(d) for d in (b if isinstance(b, (list, tuple, torch.Size)) else [b])]
+    if len(a) != len(b) or any(d is None or isinstance(d, torch.Tensor) for d in a + b):
+        return False
     return statically_known_true(sym_eq(a, b))
 
 
