@@ -5,7 +5,6 @@
 namespace xg {
 namespace {
 
-__device__ __forceinline__ float silu_f32(float v) { return v / (1.0f + __expf(-v)); }
 
 // gate/up are [rows, d] views with row strides in elements; nvec = d / VW.
 template <typename T, int VW>

@@ -300,8 +300,8 @@ __device__ __forceinline__ void epilogue_rows(const GemmParams& p, const char* p
       float t = v[e];
       if constexpr (ACT == XG_ACT_RELU) t = fmaxf(t, 0.f);
       if constexpr (ACT == XG_ACT_GELU) t = 0.5f * t * (1.f + erff(t * 0.70710678118654752f));
-      if constexpr (ACT == XG_ACT_SILU) t = t / (1.f + __expf(-t));
-      if constexpr (ACT == XG_ACT_SIGMOID) t = 1.f / (1.f + __expf(-t));
+      if constexpr (ACT == XG_ACT_SILU) t = silu_f32(t);
+      if constexpr (ACT == XG_ACT_SIGMOID) t = sigmoid_f32(t);
       o[e] = from_f32<OT>(t);
     }
     *reinterpret_cast<O8*>(reinterpret_cast<OT*>(p.out) + (int64_t)m * p.ldc + n) = o;
@@ -415,7 +415,7 @@ __device__ __forceinline__ void epilogue_glu(const GemmParams& p, const Lane& L,
       for (int e = 0; e < 8; ++e) {
         // each projection is rounded to the storage type first, as the two separate layers would do
         const float gr = to_f32(from_f32<OT>(gv[e])), ur = to_f32(from_f32<OT>(uv[e]));
-        o[e] = from_f32<OT>(gr / (1.f + __expf(-gr)) * ur);
+        o[e] = from_f32<OT>(silu_f32(gr) * ur);
       }
       *reinterpret_cast<O8*>(reinterpret_cast<OT*>(p.out) + (int64_t)m * p.ldc + n) = o;
     }

@@ -51,6 +51,14 @@ __device__ __forceinline__ T from_f32(float v) {
   return (T)v;  // round-to-nearest-even; gfx950 has native f32->bf16 conversion
 }
 
+// sigmoid and SiLU in fp32 from the hardware's exp2 and reciprocal (each within 1 ulp): four instructions instead of
+// the dozen of an IEEE division.  Every kernel that applies them uses these two, so fused and unfused paths round
+// identically.  t = -inf gives NaN for SiLU, as x * sigmoid(x) does in eager.
+__device__ __forceinline__ float sigmoid_f32(float t) {
+  return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(t * -1.44269504088896340736f));
+}
+__device__ __forceinline__ float silu_f32(float t) { return t * sigmoid_f32(t); }
+
 // 16-byte global load / store.  The NT variants mark the access as streaming
 // (data that is touched once), which keeps it from displacing reused lines.
 template <typename V>
