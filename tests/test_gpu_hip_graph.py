@@ -62,3 +62,70 @@ def test_runner_rejects_other_shapes_and_resets(device):
     assert again.mempool is None
     again.capture(a, clone_args=True)
     torch.testing.assert_close(again(a).float(), F.layer_norm(a + a, (64,)).float(), rtol=1.6e-2, atol=1e-2)
+
+
+def test_partitioned_mixed_graph_records_the_device_parts(device):
+    """The reference's mixed-device case (tests/mlu/test_mlu_graph.py:62-120): device → host → device; the host
+    part stays in the outer module, each device part is recorded and replayed with new inputs."""
+    from torch.fx.experimental.proxy_tensor import make_fx
+
+    from xpu_graph_amd.backends.device_graph import device_graph_compiler
+
+    class Mixed(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.l1 = torch.nn.Linear(32, 32)
+            self.l2 = torch.nn.Linear(32, 32)
+
+        def forward(self, x):
+            x = self.l1(x)
+            x = x.cpu()
+            x = x + 1.0
+            x = x.to(device)
+            return self.l2(x)
+
+    model = Mixed().to(device)
+    x1 = torch.randn(16, 32, device=device)
+    with torch.no_grad():
+        gm = make_fx(model)(x1)
+        out = device_graph_compiler(gm, [x1], "cuda")
+        regions = [m for _, m in out.named_children() if m.__class__.__name__ == "_LazyXPUGraph"]
+        assert len(regions) == 2
+        for step in range(3):
+            x = torch.randn(16, 32, device=device) * (step + 1)
+            torch.testing.assert_close(out(x).clone(), model(x), rtol=1e-3, atol=1e-3)
+            (x @ x.t()).sum().item()
+        assert all(r.recorded == 1 for r in regions)
+
+
+def test_backend_with_device_graph_vendor_config(device):
+    """XpuGraphConfig(vendor_compiler_config={"compiler": "device_graph"}) as in the reference
+    (tests/mlu/test_mlu_graph.py:31-60): the compiled function records on its first call and replays afterwards;
+    the recorded region holds the target's kernels."""
+    from xpu_graph_amd import OptLevel, Target, XpuGraph, XpuGraphConfig
+
+    bf = torch.bfloat16
+    g = torch.Generator().manual_seed(1)
+    gam = (1 + 0.1 * torch.randn(512, generator=g)).to(bf).to(device)
+    w1 = (0.05 * torch.randn(512, 1024, generator=g)).to(bf).to(device)
+    b1 = (0.05 * torch.randn(1024, generator=g)).to(bf).to(device)
+    w2 = (0.05 * torch.randn(512, 1024, generator=g)).to(bf).to(device)
+    backend = XpuGraph(
+        XpuGraphConfig(False, target=Target.mi355x, opt_level=OptLevel.level2, enable_cache=False, vendor_compiler_config={"compiler": "device_graph"})
+    )
+    compiled = torch.compile(mlp_block, backend=backend, dynamic=False)
+    for step in range(4):
+        xs = torch.randn(256, 512, device=device).to(bf) * (step + 1)
+        rs = torch.randn(256, 512, device=device).to(bf)
+        with torch.no_grad():
+            y, h = compiled(xs, rs, gam, w1, b1, w2)
+            y, h = y.clone(), h.clone()
+            y_ref, h_ref = mlp_block(xs, rs, gam, w1, b1, w2)
+        (xs.float() @ xs.float().t()).sum().item()  # eager work and a synchronisation between replays
+        assert torch.equal(h, h_ref)
+        torch.testing.assert_close(y.float(), y_ref.float(), rtol=1.6e-2, atol=3e-2)
+    outer = backend.compiled_graphs[-1]  # the partitioner rewrites the module in place: one region holds everything
+    (region,) = [m for _, m in outer.named_children() if m.__class__.__name__ == "_LazyXPUGraph"]
+    assert region.recorded == 1
+    mods = [n.target for n in region.region.graph.nodes if n.op == "call_module"]
+    assert len(mods) >= 3, mods  # add+norm, dense+silu, dense

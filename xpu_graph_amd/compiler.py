@@ -89,7 +89,8 @@ class XpuGraph:
                         assert isinstance(cached, SerializableArtifact)
                         self.compiled_graphs.append(cached.artifact)
                         del self.compiled_graphs[:-8]
-                        return make_boxed_func(cached.artifact) if boxed else cached.artifact
+                        runnable = self._vendor_compile(cached.artifact, fake_inputs, stage)
+                        return make_boxed_func(runnable) if boxed else runnable
                 with fake_mode:
                     with local_logger("before"):
                         logger.debug("before xpu_graph, graph like:\n %s", gm.print_readable(print_output=False))
@@ -100,8 +101,6 @@ class XpuGraph:
                         logger.info("xpu_graph passes complete")
                         logger.debug("after xpu_graph, graph like:\n %s", out.print_readable(print_output=False))
                     logger.info(f"node statistic: before {before} after {_node_census(out)}")
-                    if self._config.vendor_compiler_config is not None:
-                        logger.warning("vendor_compiler_config is ignored: this backend runs the rewritten graph directly")
                 if hashkey is not None:
                     try:
                         # what runs is the re-loaded artifact, i.e. what a later process would get
@@ -110,8 +109,11 @@ class XpuGraph:
                         logger.warning(f"Artifact is not serializable ({e}), skip cache.")
                 self.compiled_graphs.append(out)
                 del self.compiled_graphs[:-8]
+                # the cache holds the rewritten graph; what the post-pass hook builds around it (recordings of
+                # device graphs) is made again, cheaply, in every process
+                runnable = self._vendor_compile(out, fake_inputs, stage)
                 # AOT's runtime wrappers call the compiled stage with one list of arguments
-                return make_boxed_func(out) if boxed else out
+                return make_boxed_func(runnable) if boxed else runnable
 
         return compile_stage
 
@@ -166,6 +168,18 @@ class XpuGraph:
             logger.info(f"Removed guards: {list(dropped)}")
             ctx.guards_context.dynamo_guards = guards - dropped
         return artifact
+
+    def _vendor_compile(self, gm, fake_inputs, stage: FxStage):
+        """The post-pass hook (reference compiler.py:90-103): with `vendor_compiler_config` set, every stage but
+        pregrad goes through `backends.vendor_compiler`."""
+        cfg = self._config.vendor_compiler_config
+        if cfg is None or stage == FxStage.pregrad:
+            return gm
+        from .backends import vendor_compiler
+
+        return vendor_compiler(
+            gm, fake_inputs, self._config.target, is_inference=stage == FxStage.inference, is_backward=stage == FxStage.backward, **cfg
+        )
 
     def _pregrad(self, dynamo_gm, example_inputs):
         """The Dynamo graph as a rewritten pre-autograd Aten module, or None when it cannot be taken apart that way

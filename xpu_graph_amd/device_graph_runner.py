@@ -14,6 +14,9 @@ import torch
 import torch.utils._pytree as pytree
 
 
+_RUNNERS = {}  # target name -> runner class
+
+
 class GraphRunner(torch.nn.Module):
     def __init__(
         self,
@@ -34,6 +37,11 @@ class GraphRunner(torch.nn.Module):
     @property
     def mempool(self):
         return self._mempool
+
+    def __class_getitem__(cls, target):
+        """`GraphRunner[Target.mi355x]` is the runner class of that target (reference utils.py:252-256); a target
+        with no runner of its own gets the class itself."""
+        return _RUNNERS.get(getattr(target, "value", target), cls)
 
     def clone(self):
         return type(self)(self._callable_target, self._init_param_callback, self._copy_param_callback)
@@ -88,3 +96,6 @@ class HIPGraphRunner(GraphRunner):
         assert self._copy_param_callback(self._input_buffers, *args, **kwargs), "arguments do not fit the recorded buffers"
         self._graph.replay()
         return self._output
+
+
+_RUNNERS["mi355x"] = HIPGraphRunner
