@@ -48,6 +48,29 @@ def test_dense_shapes(device, dtype, weight_trans, M, N, K):
     close(got, ref32(x, W, weight_trans, None, None, "none"), K)
 
 
+@pytest.mark.parametrize("weight_trans", [False, True])
+@pytest.mark.parametrize("M,N,K", [(1, 8, 64), (70, 72, 128), (300, 264, 192), (33, 4096, 4096), (256, 11008, 4096), (2048, 4096, 1024)])
+def test_dense_small_problems_take_the_64x64_kernel(device, weight_trans, M, N, K):
+    """Whole K slabs and at most half a machine of 256 x 256 tiles: the split-K 64 x 64 kernel.  Ragged M and N,
+    one slab and many, bias + residual + activation, and bit-identity with the large-tile kernel's rounding rule
+    (one rounding of the fp32 result) through the fp32 reference."""
+    g = torch.Generator().manual_seed(M * 7 + N + K)
+    x = torch.randn(M, K, generator=g).bfloat16().to(device)
+    W = (torch.randn(N, K, generator=g) / K**0.5).bfloat16().to(device)
+    if not weight_trans:
+        W = W.t().contiguous()
+    b = torch.randn(N, generator=g).bfloat16().to(device)
+    res = torch.randn(M, N, generator=g).bfloat16().to(device)
+    close(_ops().dense(x, W, weight_trans, None, None, "none"), ref32(x, W, weight_trans, None, None, "none"), K)
+    close(_ops().dense(x, W, weight_trans, b, res, "gelu"), ref32(x, W, weight_trans, b, res, "gelu"), K)
+    # exact products: small integers, so every partial sum is exact in fp32 and the result must be bit-exact
+    xi = torch.randint(-2, 3, (M, K), generator=g).bfloat16().to(device)
+    Wi = torch.randint(-2, 3, (N, K), generator=g).bfloat16().to(device)
+    Wi = Wi if weight_trans else Wi.t().contiguous()
+    want = (xi.float() @ (Wi.float().t() if weight_trans else Wi.float())).bfloat16()
+    assert torch.equal(_ops().dense(xi, Wi, weight_trans, None, None, "none"), want)
+
+
 @pytest.mark.parametrize("act", ["none", "relu", "gelu", "silu", "sigmoid"])
 def test_dense_bias_residual_activation(device, act):
     M, N, K = 320, 520, 136
