@@ -67,10 +67,11 @@ def test_writes_into_arguments_stay_outside():
     out = device_graph_compiler(gm, [], "cpu", runner_cls=ReplayOnBuffers)
     top = [str(n.target) for n in out.graph.nodes if n.op == "call_function"]
     assert "aten.copy_.default" in top
-    x, buf = torch.randn(4), torch.zeros(4)
-    res = out(x, buf)
-    torch.testing.assert_close(buf, x * 2.0)  # the caller's tensor was written, not a private copy
-    torch.testing.assert_close(res, x * 2.0 + 1.0)
+    for _ in range(3):  # unrecorded first call, then recorded ones
+        x, buf = torch.randn(4), torch.zeros(4)
+        res = out(x, buf)
+        torch.testing.assert_close(buf, x * 2.0)  # the caller's tensor was written, not a private copy
+        torch.testing.assert_close(res, x * 2.0 + 1.0)
 
 
 def test_mixed_graph_splits_around_the_unrecordable_node_and_replays_with_new_inputs():
@@ -93,16 +94,18 @@ def test_mixed_graph_splits_around_the_unrecordable_node_and_replays_with_new_in
     out = device_graph_compiler(gm, [x1], "cpu", runner_cls=ReplayOnBuffers)
     regions = _regions(out)
     assert len(regions) >= 2
-    torch.testing.assert_close(out(x1), model(x1))
-    x2 = torch.randn(16, 32)
+    torch.testing.assert_close(out(x1), model(x1))  # the first call runs unrecorded
+    assert ReplayOnBuffers.captures == before
+    x2, x3 = torch.randn(16, 32), torch.randn(16, 32)
     torch.testing.assert_close(out(x2), model(x2))
+    torch.testing.assert_close(out(x3), model(x3))
     torch.testing.assert_close(out(x1), model(x1))
-    assert ReplayOnBuffers.captures - before == len(regions)  # recorded once each, replayed afterwards
-    # parameters are owned by the outer module: recorded in place, not among the per-call buffers
     first = regions[0]
+    assert first.recorded == 1  # recorded once, replayed afterwards
+    # parameters are owned by the outer module: recorded in place, not among the per-call buffers
     runner = next(iter(first._runners.values()))
     assert len(first._owned) == 2 and len(runner._input_buffers) == 1
-    assert runner._input_buffers[0].data_ptr() != x1.data_ptr()  # clone_args: a private buffer
+    assert runner._input_buffers[0].data_ptr() not in (x1.data_ptr(), x2.data_ptr())  # clone_args: a private buffer
 
 
 def test_one_recording_per_signature_with_eviction():
@@ -129,15 +132,39 @@ def test_clone_outputs_and_caller_buffers():
     gm = make_fx(f)(torch.randn(4))
     shared = device_graph_compiler(gm, [], "cpu", runner_cls=ReplayOnBuffers, clone_args=False)
     (region,) = _regions(shared)
-    x = torch.randn(4)
+    x, y = torch.randn(4), torch.randn(4)
     shared(x)
-    assert next(iter(region._runners.values()))._input_buffers[0].data_ptr() == x.data_ptr()
+    shared(y)
+    assert next(iter(region._runners.values()))._input_buffers[0].data_ptr() == y.data_ptr()  # the caller's own tensor
     gm2 = make_fx(f)(torch.randn(4))
     cloned = device_graph_compiler(gm2, [], "cpu", runner_cls=ReplayOnBuffers, clone_outputs=True)
-    a = cloned(torch.ones(4))
-    b = cloned(torch.full((4,), 2.0))
-    torch.testing.assert_close(a, torch.full((4,), 3.0))
-    torch.testing.assert_close(b, torch.full((4,), 6.0))
+    ins = [torch.full((4,), float(v)) for v in (1, 2, 3)]
+    a, b, c = (cloned(t) for t in ins)
+    for got, v in zip((a, b, c), (3.0, 6.0, 9.0)):
+        torch.testing.assert_close(got, torch.full((4,), v))  # a later replay did not overwrite an earlier result
+
+
+def test_tensors_that_keep_their_address_are_recorded_in_place():
+    """Weights handed in as graph inputs (no get_attr) are not copied per call; one that moves later is."""
+
+    def f(x, w):
+        return x @ w
+
+    gm = make_fx(f)(torch.randn(4, 8), torch.randn(8, 8))
+    out = device_graph_compiler(gm, [], "cpu", runner_cls=ReplayOnBuffers)
+    (region,) = _regions(out)
+    w = torch.randn(8, 8)
+    xs = [torch.randn(4, 8) for _ in range(5)]
+    for x in xs[:3]:
+        torch.testing.assert_close(out(x, w), f(x, w))
+    runner = next(iter(region._runners.values()))
+    assert region.recorded == 1 and len(runner._input_buffers) == 1  # x only: w is read where it lives
+    w2 = torch.randn(8, 8)
+    torch.testing.assert_close(out(xs[3], w2), f(xs[3], w2))  # w moved: recorded again, refreshed per call from now on
+    w3 = torch.randn(8, 8)
+    torch.testing.assert_close(out(xs[4], w3), f(xs[4], w3))
+    runner = next(iter(region._runners.values()))
+    assert region.recorded == 1 and len(runner._input_buffers) == 2
 
 
 def test_vendor_compiler_hook_dispatches_by_target():

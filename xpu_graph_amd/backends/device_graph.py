@@ -11,10 +11,12 @@ does), minus the nodes a recording cannot hold -- results whose shape or value d
 synchronise), host arithmetic on sizes, and operators that write into one of their arguments (a recording
 runs on private copies of its inputs, so the write would miss the caller's tensor).
 
-How a region runs: its inputs are split once, from the graph itself, into tensors the outer module owns
-(parameters and constants reached by get_attr: recorded in place, never copied) and per-call tensors (copied
-into buffers the recording reads).  One recording is kept per input signature (shapes, strides, dtypes, integer
-arguments, addresses of the owned tensors), so a region reached with several batch sizes records once per size.
+How a region runs: the first call runs it unrecorded.  From the second call on its inputs are split into
+tensors recorded in place -- those the outer module owns (parameters and constants reached by get_attr) and those
+that kept their address since the first call (weights passed as graph inputs, a fixed input buffer) -- and
+per-call tensors, copied into buffers the recording reads.  One recording is kept per input signature (shapes,
+strides, dtypes, integer arguments, addresses of the tensors recorded in place), so a region reached with several
+batch sizes records once per size.
 The tensors a region returns live in the recording's memory pool and are overwritten by its next replay unless
 `clone_outputs` is set.
 """
@@ -88,8 +90,13 @@ def _signature(args, owned):
 
 
 class _LazyXPUGraph(torch.nn.Module):
-    """One recordable region.  Recording waits for the first call: operators before the region may change state
-    it reads, and only real arguments say which addresses the owned tensors have."""
+    """One recordable region.
+
+    The first call runs the region as it is: operators before the region may change state it reads, modules inside
+    it may build tables on first use, and only a later call can tell which arguments keep their address from call
+    to call (weights handed in as graph inputs, a caller's fixed input buffer).  Such tensors are recorded where
+    they are, like the owned ones; the others get buffers that every call refreshes.  A tensor that was taken for
+    fixed and then moves is refreshed like the others from then on (all recordings are made again, once)."""
 
     def __init__(self, region: torch.nn.Module, runner_cls, owned_positions=(), memory_pool=None, clone_args=True,
                  clone_outputs=False, max_graphs=8):
@@ -102,13 +109,44 @@ class _LazyXPUGraph(torch.nn.Module):
         self._clone_outputs = bool(clone_outputs)
         self._max_graphs = max(1, int(max_graphs))
         self._runners = OrderedDict()  # signature -> runner, least recently used first
+        self._first_ptrs = None  # addresses of the tensor arguments of the first call
+        self._fixed = None  # positions recorded in place (owned + those that kept their address) -> address
 
     @property
     def recorded(self):
         return len(self._runners)
 
+    @staticmethod
+    def _ptrs(args):
+        return [a.data_ptr() if isinstance(a, torch.Tensor) else None for a in args]
+
     def _per_call(self, args):
-        return [a for i, a in enumerate(args) if isinstance(a, torch.Tensor) and i not in self._owned]
+        return [a for i, a in enumerate(args) if isinstance(a, torch.Tensor) and i not in self._fixed]
+
+    def _settle_fixed(self, args):
+        now = self._ptrs(args)
+        if self._fixed is None:
+            keep = [
+                i
+                for i, (was, is_) in enumerate(zip(self._first_ptrs, now))
+                if is_ is not None and (i in self._owned or was == is_ or isinstance(args[i], torch.nn.Parameter))
+            ]
+            self._fixed = {i: now[i] for i in keep}
+            return
+        moved = [i for i, ptr in self._fixed.items() if i not in self._owned and now[i] != ptr]
+        if moved:
+            logger.debug(f"device graph: arguments {moved} moved, they are refreshed per call from now on")
+            for i in moved:
+                del self._fixed[i]
+            self._drop_recordings()
+        for i in self._owned:  # a replaced parameter: its address is part of the signature
+            if i in self._fixed:
+                self._fixed[i] = now[i]
+
+    def _drop_recordings(self):
+        for runner in self._runners.values():
+            runner.reset()
+        self._runners.clear()
 
     def _new_runner(self, args):
         def init_param_callback(*a):
@@ -125,14 +163,17 @@ class _LazyXPUGraph(torch.nn.Module):
 
         runner = self._runner_cls(self.region, init_param_callback=init_param_callback, copy_param_callback=copy_param_callback)
         if self._clone_args:
-            # private buffers for the per-call tensors (the caller may free or overwrite its own between calls);
-            # owned tensors are recorded where they are
-            args = [a.detach().clone() if isinstance(a, torch.Tensor) and i not in self._owned else a for i, a in enumerate(args)]
+            # private buffers for the per-call tensors (the caller may free or overwrite its own between calls)
+            args = [a.detach().clone() if isinstance(a, torch.Tensor) and i not in self._fixed else a for i, a in enumerate(args)]
         runner.capture(*args, memory_pool=self._memory_pool, clone_args=False)
         return runner
 
     def forward(self, *args):
-        key = _signature(args, self._owned)
+        if self._first_ptrs is None:
+            self._first_ptrs = self._ptrs(args)
+            return self.region(*args)
+        self._settle_fixed(args)
+        key = _signature(args, self._fixed)
         runner = self._runners.get(key)
         if runner is None:
             if len(self._runners) >= self._max_graphs:
