@@ -165,3 +165,43 @@ def test_linear_is_decomposed_for_the_dense_pattern_in_pregrad(caplog):
     assert calls[0].args[2] is True and calls[0].args[3] is not None  # [N, K] weight, bias kept
     assert not any("linear" in str(n.target) or "aten.mm" in str(n.target) for n in pregrad.graph.nodes)
     assert "Pattern.DecomposeLinear changed graph" in caplog.text and "Pattern.CustomDenseLayer changed graph" in caplog.text
+
+
+def test_backward_formulas_reach_ops_that_were_traced_before_registration():
+    """An inference compile that traces xpu_ops::dense BEFORE any training backend exists must not hide the
+    backward formula registered later: the joint graph then saves the dense operands for the backward pass (in a
+    fresh process: registration happens once per process)."""
+    import subprocess
+    import sys
+
+    code = r'''
+import warnings, torch, torch.nn.functional as F
+from xpu_graph_amd import OptLevel, Target, XpuGraph, XpuGraphConfig
+def mlp(x, w1, b1, w2):
+    return F.linear(F.silu(F.linear(x, w1, b1)), w2)
+bf = torch.bfloat16
+args = [torch.randn(16, 64).to(bf), torch.randn(128, 64).to(bf), torch.randn(128).to(bf), torch.randn(64, 128).to(bf)]
+first = XpuGraph(XpuGraphConfig(False, target=Target.mi355x, opt_level=OptLevel.level2, enable_cache=False))
+try:
+    with torch.no_grad():
+        torch.compile(mlp, backend=first, dynamic=False)(*args)
+except NotImplementedError:
+    pass  # the kernels refuse CPU tensors; the trace is what matters
+assert any("dense" in str(n.target) for n in first.compiled_graphs[-1].graph.nodes)
+torch._dynamo.reset()
+train = XpuGraph(XpuGraphConfig(True, target=Target.mi355x, opt_level=OptLevel.level2, enable_cache=False))
+with warnings.catch_warnings(record=True) as seen:
+    warnings.simplefilter("always")
+    try:
+        torch.compile(mlp, backend=train, dynamic=False)(*[a.clone().requires_grad_(True) for a in args])
+    except NotImplementedError:
+        pass
+assert not [w for w in seen if "autograd kernel was not registered" in str(w.message)], [str(w.message)[:80] for w in seen]
+forward = train.compiled_graphs[-1]
+outs = list(forward.graph.nodes)[-1].args[0]
+print("FORWARD_OUTPUTS", len(outs))
+'''
+    proc = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    n_out = int(proc.stdout.split("FORWARD_OUTPUTS")[1].split()[0])
+    assert n_out >= 5, n_out  # y + the operands both dense backward formulas keep (x, weights, outputs, bias)

@@ -149,4 +149,10 @@ def register():
     reg("xpu_ops::silu_mul2", _silu_mul2_backward, setup_context=_silu_mul2_setup)
     reg("xpu_ops::silu_mul", _silu_mul_backward, setup_context=_silu_mul_setup)
     reg("xpu_ops::dense", _dense_backward, setup_context=_dense_setup)
+    # An op that was traced before (an inference compile earlier in the process) has its dispatch decisions cached
+    # on the Python side; a stale entry for the Autograd key would keep sending traces to the "no formula" fallback.
+    for name in ("rms_norm", "layer_norm", "silu_mul2", "silu_mul", "dense"):
+        packet = getattr(torch.ops.xpu_ops, name)
+        for overload in packet.overloads():
+            getattr(packet, overload)._dispatch_cache.clear()
     _REGISTERED = True
