@@ -309,7 +309,7 @@ __device__ __forceinline__ void epilogue_rows(const GemmParams& p, const char* p
       if constexpr (ACT == XG_ACT_SIGMOID) t = sigmoid_f32(t);
       o[e] = from_f32<OT>(t);
     }
-    *reinterpret_cast<O8*>(reinterpret_cast<OT*>(p.out) + (int64_t)m * p.ldc + n) = o;
+    store_vec_nt(reinterpret_cast<O8*>(reinterpret_cast<OT*>(p.out) + (int64_t)m * p.ldc + n), o);  // written once, read by another kernel
   }
 }
 
@@ -436,7 +436,7 @@ __device__ __forceinline__ void epilogue_glu(const GemmParams& p, const Lane& L,
         const float gr = to_f32(from_f32<OT>(gv[e])), ur = to_f32(from_f32<OT>(uv[e]));
         o[e] = from_f32<OT>(silu_f32(gr) * ur);
       }
-      *reinterpret_cast<O8*>(reinterpret_cast<OT*>(p.out) + (int64_t)m * p.ldc + n) = o;
+      store_vec_nt(reinterpret_cast<O8*>(reinterpret_cast<OT*>(p.out) + (int64_t)m * p.ldc + n), o);  // written once, read by another kernel
     }
     __syncthreads();  // the parks are free for the next half
   });
@@ -979,7 +979,7 @@ __global__ __launch_bounds__(kThreads) void gemm_small_kernel(GemmParams p) {
         const float gr = to_f32(from_f32<OT>(gv[e])), ur = to_f32(from_f32<OT>(uv[e]));
         o[e] = from_f32<OT>(silu_f32(gr) * ur);
       }
-      *reinterpret_cast<O8*>(reinterpret_cast<OT*>(p.out) + (int64_t)m * p.ldc + n) = o;
+      store_vec_nt(reinterpret_cast<O8*>(reinterpret_cast<OT*>(p.out) + (int64_t)m * p.ldc + n), o);  // written once, read by another kernel
     }
   }
 }
