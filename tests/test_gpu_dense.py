@@ -49,11 +49,13 @@ def test_dense_shapes(device, dtype, weight_trans, M, N, K):
 
 
 @pytest.mark.parametrize("weight_trans", [False, True])
-@pytest.mark.parametrize("M,N,K", [(1, 8, 64), (70, 72, 128), (300, 264, 192), (33, 4096, 4096), (256, 11008, 4096), (2048, 4096, 1024)])
-def test_dense_small_problems_take_the_64x64_kernel(device, weight_trans, M, N, K):
-    """Whole K slabs and at most half a machine of 256 x 256 tiles: the split-K 64 x 64 kernel.  Ragged M and N,
-    one slab and many, bias + residual + activation, and bit-identity with the large-tile kernel's rounding rule
-    (one rounding of the fp32 result) through the fp32 reference."""
+@pytest.mark.parametrize(
+    "M,N,K", [(1, 8, 64), (70, 72, 128), (300, 264, 192), (33, 4096, 4096), (256, 11008, 4096), (1024, 4096, 512), (2048, 4096, 1024), (1300, 4104, 256)]
+)
+def test_dense_small_and_underfilled_grids(device, weight_trans, M, N, K):
+    """Whole K slabs and at most a quarter of a machine of 256 x 256 tiles: the split-K 64 x 64 kernel; grids
+    between that and one full round: 128 x 256 tiles throughout (the last two shapes).  Ragged M and N, one slab
+    and many, bias + residual + activation, and exact integer products."""
     g = torch.Generator().manual_seed(M * 7 + N + K)
     x = torch.randn(M, K, generator=g).bfloat16().to(device)
     W = (torch.randn(N, K, generator=g) / K**0.5).bfloat16().to(device)
@@ -175,6 +177,23 @@ def test_dense_glu_bit_identical_to_the_unfused_ops(device, dtype, M, N, K):
     assert torch.equal(got, two)
     ref = torch.nn.functional.silu(x.float() @ wg.float().t()) * (x.float() @ wu.float().t())
     torch.testing.assert_close(got.float(), ref, rtol=1.6e-2, atol=2e-2)
+
+
+@pytest.mark.parametrize("M,N,K", [(1024, 4096, 256), (900, 2056, 128)])
+def test_dense_glu_half_height_grid(device, M, N, K):
+    """A gated layer whose full-size grid would leave most of a round empty runs as 128-row tiles throughout."""
+    g = torch.Generator().manual_seed(M + N)
+    x = torch.randn(M, K, generator=g).bfloat16().to(device)
+    wg = (torch.randn(N, K, generator=g) / K**0.5).bfloat16().to(device)
+    wu = (torch.randn(N, K, generator=g) / K**0.5).bfloat16().to(device)
+    got = torch.ops.xpu_ops.dense_glu(x, wg, wu)
+    ref = torch.nn.functional.silu(x.float() @ wg.float().t()) * (x.float() @ wu.float().t())
+    torch.testing.assert_close(got.float(), ref, rtol=1.6e-2, atol=2e-2)
+    xi = torch.randint(-2, 3, (M, K), generator=g).bfloat16().to(device)
+    wi = torch.randint(-2, 3, (N, K), generator=g).bfloat16().to(device)
+    gate = (xi.float() @ wi.float().t()).bfloat16().float()
+    want = (torch.nn.functional.silu(gate) * gate).bfloat16()
+    torch.testing.assert_close(torch.ops.xpu_ops.dense_glu(xi, wi, wi).float(), want.float(), rtol=8e-3, atol=1e-2)
 
 
 def test_dense_glu_strided_operands_and_rejects(device):

@@ -10,10 +10,11 @@
 // per SIMD.  K advances in slabs of 128 BYTES per row (64 bf16/f16 or 128 fp8
 // elements), double-buffered in 128 KiB of LDS.
 //
-// Problems whose 256 x 256 tiles would fill less than 3/8 of the compute units
+// Problems whose 256 x 256 tiles would fill at most a quarter of the compute units
 // (small batches: a decode step, a short prefill) go to gemm_small_kernel instead:
 // 64 x 64 tiles with K split between the four wavefronts of a workgroup; its
-// description sits with its code below.
+// description sits with its code below.  Grids in between that would leave much
+// of a round empty run as 128 x 256 tiles throughout (half_height_wins).
 //
 // Two large-tile kernels share everything but the way a slab reaches LDS:
 //  * gemm_dma_kernel (K a multiple of the slab): `global_load_lds_dwordx4` moves
@@ -669,7 +670,14 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
   }
 }
 
-// The gated layer: same two launch shapes as above.
+// Every tile half height: for grids whose full-size tiles would leave a large part of a round empty.
+template <typename T, typename OT, BLayout BL>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_dma_half_kernel(GemmParams p) {
+  extern __shared__ __align__(16) char smem[];
+  gemm_dma_tile<T, OT, BL, 2>(p, blockIdx.x, gridDim.x, smem);
+}
+
+// The gated layer: same launch shapes as above.
 template <typename T, typename OT>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_glu_kernel(GemmParams p) {
   extern __shared__ __align__(16) char smem[];
@@ -689,6 +697,12 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
 }
 
 // ---- kernel 2: slabs staged through registers (any K) --------------------------------------
+template <typename T, typename OT>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_glu_half_kernel(GemmParams p) {
+  extern __shared__ __align__(16) char smem[];
+  gemm_dma_tile<T, OT, BLayout::KMajor, 2, true>(p, blockIdx.x, gridDim.x, smem);
+}
+
 template <typename T, typename OT, BLayout BL>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_staged_kernel(GemmParams p) {
   extern __shared__ __align__(16) char smem[];
@@ -1044,11 +1058,12 @@ inline int full_tile_columns(int tm, int tn) {
 }
 
 // Large tiles that would leave most compute units idle give way to the 64 x 64 kernel.  Measured crossover on
-// 256 compute units (N = K = 4096): 64 large tiles take 84 us against 48 us, 128 large tiles 88 us against 96 us.
+// 256 compute units (N = K = 4096, us, 64 x 64 kernel / half-height tiles / full tiles): 64 tiles 54 / 58 / 83,
+// 80 tiles 71 / 62 / 86, 128 tiles 98 / 66 / 88.
 inline int small_tile_limit() {
   static const int n = [] {
     const char* e = getenv("XG_GEMM_SMALL_MAX");
-    return e ? atoi(e) : cu_count() * 3 / 8;
+    return e ? atoi(e) : cu_count() / 4;
   }();
   return n;
 }
@@ -1067,6 +1082,17 @@ int launch_small(GemmParams p, hipStream_t stream) {
   return status_from_hip(hipGetLastError());
 }
 
+// A half-height (128-row) tile takes 0.55 of a full tile's time for half of its work, so a grid of them pays when
+// the full-size grid leaves much of its last round empty (128 full tiles on 256 units: one round of 256 half tiles,
+// 0.55 instead of 1).  tn: tile columns; the tile rows follow from M.
+inline bool half_height_wins(int M, int tn) {
+  static const bool off = getenv("XG_GEMM_NO_HALF") != nullptr;
+  const int64_t cus = cu_count();
+  const int64_t full = (int64_t)((M + BM - 1) / BM) * tn, half = (int64_t)((M + 127) / 128) * tn;
+  const double t_full = (double)((full + cus - 1) / cus), t_half = 0.55 * (double)((half + cus - 1) / cus);
+  return !off && t_half < 0.95 * t_full;
+}
+
 template <typename T, typename OT, BLayout BL>
 int launch_gemm(const GemmParams& p, hipStream_t stream) {
   if (!dma_ok<T>(p, BL)) return launch_kernel(gemm_staged_kernel<T, OT, BL>, p, stream);
@@ -1074,7 +1100,14 @@ int launch_gemm(const GemmParams& p, hipStream_t stream) {
     if ((int64_t)p.tiles_m * p.tiles_n <= small_tile_limit()) return launch_small<T, OT, BL>(p, stream);
   }
   const int keep = full_tile_columns(p.tiles_m, p.tiles_n);
-  if (keep == p.tiles_n) return launch_kernel(gemm_dma_kernel<T, OT, BL>, p, stream);
+  if (keep == p.tiles_n) {
+    if (half_height_wins(p.M, p.tiles_n)) {
+      GemmParams h = p;
+      h.tiles_m = (p.M + 127) / 128;
+      return launch_kernel(gemm_dma_half_kernel<T, OT, BL>, h, stream);
+    }
+    return launch_kernel(gemm_dma_kernel<T, OT, BL>, p, stream);
+  }
   // columns [0, keep * BN): full tiles; the rest: 128-row tiles on operand pointers moved to the split column
   constexpr int EB = Elem<T>::BYTES;
   const int64_t n_split = (int64_t)keep * BN;
@@ -1105,7 +1138,14 @@ int launch_glu(const GemmParams& p, hipStream_t stream) {
   constexpr int EB = Elem<T>::BYTES;
   if ((int64_t)p.tiles_m * p.tiles_n <= small_tile_limit()) return launch_small<T, OT, BLayout::KMajor, true>(p, stream);
   const int keep = full_tile_columns(p.tiles_m, p.tiles_n);
-  if (keep == p.tiles_n) return launch_kernel(gemm_glu_kernel<T, OT>, p, stream);
+  if (keep == p.tiles_n) {
+    if (half_height_wins(p.M, p.tiles_n)) {
+      GemmParams h = p;
+      h.tiles_m = (p.M + 127) / 128;
+      return launch_kernel(gemm_glu_half_kernel<T, OT>, h, stream);
+    }
+    return launch_kernel(gemm_glu_kernel<T, OT>, p, stream);
+  }
   const int64_t n_split = (int64_t)keep * (BN / 2);
   GemmParams full = p;
   full.N = (int)n_split;
