@@ -15,7 +15,6 @@ replacement modules pickle by class reference).  Cache files are written and rea
 import hashlib
 import importlib
 import io
-import operator
 import os
 import pickle
 from abc import ABC, abstractmethod

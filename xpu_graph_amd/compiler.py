@@ -20,7 +20,7 @@ import torch
 from torch._dynamo.backends.common import aot_autograd
 from torch._functorch.aot_autograd import make_boxed_func
 
-from .cache import SerializableArtifact, SerializableGraphModule, XpuGraphCache, default_cache
+from .cache import SerializableArtifact, SerializableGraphModule, default_cache
 from .config import Target, XpuGraphConfig, get_partition_fn
 from .fx_utils import FxStage, fakify_tensors
 from .passes.pass_manager import PassManager

@@ -12,7 +12,7 @@ from torch import fx
 from ....config import OptLevel
 from ....fx_utils import FxStage
 from ..pattern import Pattern
-from ..utils.node_utils import aten, is_call, same_shape, shape
+from ..utils.node_utils import aten, is_call, same_shape
 
 FUSED_ADDN_LIMIT = 4
 

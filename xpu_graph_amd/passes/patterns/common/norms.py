@@ -11,7 +11,6 @@ square as pow 2, x*x or aten.square; eps on either side of the add; mean over
 LayerNorm the variance may be aten.var.dim or aten.var.correction with
 correction 0 (what `unbiased=False` traces to on current torch).
 """
-import torch
 from torch import fx
 
 from ....config import OptLevel

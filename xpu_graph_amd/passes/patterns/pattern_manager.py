@@ -1,6 +1,6 @@
 """Owns every pattern and runs them: groups in order, five sweeps per group
 (reference src/xpu_graph/passes/patterns/pattern_manager.py:14-139)."""
-from typing import Callable, List
+from typing import List
 
 import torch.fx as fx
 

@@ -7,9 +7,8 @@ and can carry extra checks over the FakeTensors bound to the pattern's inputs.
 The registry is process-global and not thread safe.
 """
 import contextlib
-import functools
 import inspect
-from typing import Callable, List, Union
+from typing import Callable, Union
 
 import torch
 from torch import fx

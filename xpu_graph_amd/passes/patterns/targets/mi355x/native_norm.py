@@ -10,7 +10,6 @@ spelling; `aten.native_layer_norm` passes through it untouched.)
 
 Only when the statistics outputs are unused and the norm is over the last axis.
 """
-import operator
 
 import torch
 

@@ -13,7 +13,6 @@ puts in front of q, k, v: the kernel takes strides, so the [B, H, S, D] views
 are passed as they are.
 """
 import math
-import operator
 
 import torch
 from torch import fx, nn
