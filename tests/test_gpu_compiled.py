@@ -258,3 +258,30 @@ def test_dynamic_batch_one_compile_many_sizes(device):
         torch.testing.assert_close(h, h_e, rtol=1e-5, atol=1e-5)
         torch.testing.assert_close(y, y_e, rtol=1.6e-2, atol=2e-2)
     assert len(backend.compiled_graphs) == n_graphs  # no recompilation for the other batch sizes
+
+
+@pytest.mark.parametrize("freeze", [False, True])
+@pytest.mark.parametrize("name", ["Linear1", "RotateHalves", "InplaceAfterClone", "DataDependentScatter", "WithDropout"])
+def test_model_zoo_on_the_mi355x_target(device, name, freeze):
+    """The small-module zoo of tests/test_host_models.py (reference tests/common/test_models.py) on the GPU with the
+    mi355x target, dynamic shapes, fp16: in-place updates, data-dependent shapes and dropout survive the rewrite;
+    the linear layers run on the dense kernel."""
+    import test_host_models as zoo
+
+    from xpu_graph_amd import OptLevel, Target, XpuGraph, XpuGraphConfig
+
+    cls = getattr(zoo, name)
+    golden, compiled = cls().to(device).half().eval(), cls().to(device).half().eval()
+    compiled.load_state_dict(golden.state_dict())
+    backend = XpuGraph(XpuGraphConfig(is_training=False, target=Target.mi355x, opt_level=OptLevel.level2, freeze=freeze, enable_cache=False))
+    compiled.forward = torch.compile(compiled.forward, backend=backend, dynamic=True)
+    x = torch.randn(80, zoo.DIM, device=device).half()
+    keep = x.clone()
+    with torch.inference_mode():
+        with torch.random.fork_rng(device_type="cuda"):
+            want = golden(keep)
+        got = compiled(x)
+    assert torch.equal(x, keep)
+    assert got.shape == want.shape
+    torch.testing.assert_close(got.float(), want.float(), rtol=1.6e-2, atol=2e-2)
+    torch._dynamo.reset()
