@@ -15,6 +15,7 @@ from .cache import XpuGraphCache, XpuGraphLocalCache, default_cache, no_cache
 from .compiler import XpuGraph, XpuGraphCompiler, XpuGraphRuntimeArtifact
 from .config import OptLevel, Target, XpuGraphConfig
 from .device_graph_runner import GraphRunner, HIPGraphRunner
+from .guard_filters import skip_all_guards_unsafe
 from .passes.patterns.plugin_pattern import (
     deregister_plugin_patterns,
     enable_plugin_patterns,
@@ -44,6 +45,7 @@ __all__ = [
     "register_this_as_pattern_constraint",
     "deregister_plugin_patterns",
     "enable_plugin_patterns",
+    "skip_all_guards_unsafe",
 ]
 
 

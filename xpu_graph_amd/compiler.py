@@ -80,6 +80,8 @@ class XpuGraph:
 
         def compile_stage(gm, sample_inputs):
             with local_logger(stage.name):
+                if stage == FxStage.inference:
+                    logger.info("decompose graph complete")
                 fake_mode, fake_inputs = fakify_tensors(sample_inputs)
                 hashkey = None
                 if self._cache is not None:
@@ -134,10 +136,12 @@ class XpuGraph:
             # forward graph hands the intermediates of that subgraph to the backward graph and nothing matches.
             # So the Dynamo graph is first lowered to pre-dispatch Aten IR, rewritten in the `pregrad` stage, and
             # AOT then differentiates the rewritten module (reference compiler.py:158-182).
-            pregrad_gm = self._pregrad(dynamo_gm, example_inputs)
+            pregrad_gm = None if self._needs_plain_dispatch(dynamo_gm, example_inputs) else self._pregrad(dynamo_gm, example_inputs)
             compiled = aot_autograd(**aot_kwargs)(pregrad_gm if pregrad_gm is not None else dynamo_gm, example_inputs)
         else:
             aot_kwargs = {"fw_compiler": self._get_compiler(FxStage.inference), "keep_inference_input_mutations": True}
+            self._needs_plain_dispatch(dynamo_gm, example_inputs)  # for its warnings: AOT handles both cases
+            logger.info("decompose graph start...")  # "complete" is logged by the stage that receives the Aten graph
             # an inference compiler: trace without autograd whatever the caller's grad mode is
             with torch.no_grad():
                 compiled = aot_autograd(**aot_kwargs)(dynamo_gm, example_inputs)
@@ -169,6 +173,24 @@ class XpuGraph:
             ctx.guards_context.dynamo_guards = guards - dropped
         return artifact
 
+    def _needs_plain_dispatch(self, dynamo_gm, example_inputs):
+        """True when the Dynamo graph must go to AOT as it is (reference compiler.py:125-138): in training, bodies
+        of higher-order operators would be lost to a pre-autograd rewrite; tensor-subclass inputs need AOT's own
+        unwrapping.  Says which of the two it found."""
+        from .fx_utils import find_hop_nodes, find_subclass_inputs
+
+        plain = False
+        if self._config.is_training:
+            hops = find_hop_nodes(dynamo_gm)
+            if hops:
+                logger.warning(f"Higher order operators detected: {', '.join(str(op) for op in hops)}.")
+                plain = True
+        subclasses = find_subclass_inputs(example_inputs)
+        if subclasses:
+            logger.warning(f"Subclass inputs detected: {', '.join(str(cls) for cls in subclasses)}.")
+            plain = True
+        return plain
+
     def _vendor_compile(self, gm, fake_inputs, stage: FxStage):
         """The post-pass hook (reference compiler.py:90-103): with `vendor_compiler_config` set, every stage but
         pregrad goes through `backends.vendor_compiler`."""
@@ -187,11 +209,13 @@ class XpuGraph:
         then goes to AOT as it is and only the forward / backward stages see it."""
         from .fx_utils import dispatch_pregrad
 
+        logger.info("decompose graph start...")
         try:
             dispatched = dispatch_pregrad(dynamo_gm, example_inputs)
         except NotImplementedError as e:
             logger.warning(f"pregrad stage skipped: {e}")
             return None
+        logger.info("decompose graph complete")
         logger.debug("after decompose, graph like:\n %s", dispatched.print_readable(print_output=False))
         return self._get_compiler(FxStage.pregrad, boxed=False)(dispatched, example_inputs)
 

@@ -49,6 +49,28 @@ def node_val(node):
     return node.meta.get("val") if isinstance(node, torch.fx.Node) else None
 
 
+def find_hop_nodes(gm):
+    """{operator: [nodes]} for the higher-order operators of a Dynamo graph (autograd.Function applications,
+    activation checkpoints, control flow): their bodies are sub-graphs a flat Aten rewrite cannot see
+    (reference fx_utils.py:410-420)."""
+    hops = {}
+    for n in gm.graph.nodes:
+        if n.op == "call_function" and isinstance(n.target, torch._ops.HigherOrderOperator):
+            hops.setdefault(n.target, []).append(n)
+    return hops
+
+
+def find_subclass_inputs(inputs):
+    """{type: [tensors]} for inputs that are traceable tensor subclasses (reference fx_utils.py:423-436)."""
+    from torch.utils._python_dispatch import is_traceable_wrapper_subclass_type
+
+    found = {}
+    for t in inputs:
+        if isinstance(t, torch.Tensor) and is_traceable_wrapper_subclass_type(type(t)):
+            found.setdefault(type(t), []).append(t)
+    return found
+
+
 def dispatch_pregrad(gm, example_inputs):
     """Lower a Dynamo graph to functional PRE-DISPATCH Aten IR (composite ops such as linear or layer_norm stay
     whole, autograd has not been traced) with the same inputs and outputs, ready for the `pregrad` pattern stage
