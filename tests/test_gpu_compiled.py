@@ -285,3 +285,66 @@ def test_model_zoo_on_the_mi355x_target(device, name, freeze):
     assert got.shape == want.shape
     torch.testing.assert_close(got.float(), want.float(), rtol=1.6e-2, atol=2e-2)
     torch._dynamo.reset()
+
+
+def _naive_layer_norm(x, w, b):
+    dt = x.dtype
+    x = x.to(torch.float32)
+    mean = torch.mean(x, dim=-1, keepdim=True)
+    var = torch.var(x, dim=-1, keepdim=True, unbiased=False)
+    return (w * ((x - mean) / ((var + 1e-6) ** 0.5)) + b).to(dt)
+
+
+def _layer_norm_between_pointwise(x, w, b):
+    a = x * torch.sigmoid(x) * 0.1
+    n = _naive_layer_norm(a, w, b)
+    return n * n + 1e-6
+
+
+@pytest.mark.parametrize("act_dtype,param_dtype", [(torch.float32, torch.float32), (torch.float32, torch.float16),
+                                                   (torch.float16, torch.float16), (torch.float32, torch.bfloat16)])
+@pytest.mark.parametrize("fn", [_naive_layer_norm, _layer_norm_between_pointwise])
+def test_layer_norm_with_mixed_activation_and_parameter_types(device, caplog, fn, act_dtype, param_dtype):
+    """Activations and affine parameters of different types (reference tests/mlu/test_mixedtype_layernorm.py:19-92):
+    the matcher fires and the kernel takes the mix."""
+    from xpu_graph_amd.test_utils import need_xpu_graph_logs
+
+    backend = mi355x_compiler()
+    x = torch.randn(8, 1024, device=device, dtype=act_dtype)
+    w = torch.randn(1024, device=device, dtype=param_dtype)
+    b = torch.randn(1024, device=device, dtype=param_dtype)
+    with need_xpu_graph_logs(), torch.no_grad():
+        got = torch.compile(fn, backend=backend, dynamic=False)(x, w, b)
+    assert "Pattern.FusedLayerNorm changed graph" in caplog.text
+    mods = [str(n.target) for n in backend.compiled_graphs[-1].graph.nodes if n.op == "call_module"]
+    assert any("norm" in m for m in mods), mods
+    want = fn(x, w, b)
+    assert got.dtype == want.dtype
+    torch.testing.assert_close(got.float(), want.float(), rtol=1e-2, atol=1e-2)
+    torch._dynamo.reset()
+
+
+@pytest.mark.parametrize("param_dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("fn", [_naive_layer_norm, _layer_norm_between_pointwise])
+def test_layer_norm_mixed_types_loss_and_grad(device, caplog, fn, param_dtype):
+    from xpu_graph_amd import OptLevel, Target, XpuGraph, XpuGraphConfig
+    from xpu_graph_amd.test_utils import need_xpu_graph_logs
+
+    backend = XpuGraph(XpuGraphConfig(is_training=True, target=Target.mi355x, opt_level=OptLevel.level2, enable_cache=False))
+    x = torch.randn(8, 1024, device=device, requires_grad=True)
+    w = torch.randn(1024, device=device, dtype=param_dtype, requires_grad=True)
+    b = torch.randn(1024, device=device, dtype=param_dtype, requires_grad=True)
+    dy = torch.randn(8, 1024, device=device)
+    with need_xpu_graph_logs():
+        y0 = torch.compile(fn, backend=backend, dynamic=False)(x, w, b)
+        g0 = torch.autograd.grad((y0,), (x, w, b), (dy,), allow_unused=True)
+    assert "Pattern.FusedLayerNorm changed graph" in caplog.text
+    y1 = fn(x, w, b)
+    g1 = torch.autograd.grad((y1,), (x, w, b), (dy,), allow_unused=True)
+    torch.testing.assert_close(y0.float(), y1.float(), rtol=1e-2, atol=1e-2)
+    for a, c in zip(g0, g1):
+        assert (a is None) == (c is None)
+        if a is not None:
+            assert a.dtype == c.dtype
+            torch.testing.assert_close(a.float(), c.float(), rtol=2e-2, atol=2e-2 * max(1.0, c.float().abs().mean().item()))
+    torch._dynamo.reset()
