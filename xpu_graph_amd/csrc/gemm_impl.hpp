@@ -1000,8 +1000,7 @@ __global__ __launch_bounds__(kThreads) void gemm_small_kernel(GemmParams p) {
 
 template <typename K>
 int set_smem_once(K kernel) {
-  static hipError_t st = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES);
-  return st == hipSuccess ? XG_OK : XG_ERR_LAUNCH;
+  return allow_dynamic_lds(reinterpret_cast<const void*>(kernel), SMEM_BYTES);
 }
 
 template <typename K>
@@ -1071,8 +1070,7 @@ inline int small_tile_limit() {
 template <typename T, typename OT, BLayout BL, bool GLU = false>
 int launch_small(GemmParams p, hipStream_t stream) {
   auto kernel = gemm_small_kernel<T, OT, BL, GLU>;
-  static hipError_t st = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, S_SMEM_BYTES);
-  if (st != hipSuccess) return XG_ERR_LAUNCH;
+  if (int st = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), S_SMEM_BYTES)) return st;
   constexpr int cols = GLU ? S_TILE / 2 : S_TILE;
   p.tiles_m = (p.M + S_TILE - 1) / S_TILE;
   p.tiles_n = (p.N + cols - 1) / cols;

@@ -349,8 +349,7 @@ template <typename T, int D>
 int launch(const Params& p, hipStream_t stream) {
   constexpr int SMEM = 2 * 2 * BKV * D * 2;
   auto kernel = sdpa_fwd_kernel<T, D>;
-  static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, SMEM);
-  if (attr != hipSuccess) return XG_ERR_LAUNCH;
+  if (int st = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), SMEM)) return st;
   const int64_t blocks = (int64_t)p.B * p.H * p.n_qb;
   hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(kThreads), SMEM, stream, p);
   return status_from_hip(hipGetLastError());

@@ -4,7 +4,10 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <mutex>
+#include <set>
 #include <type_traits>
+#include <utility>
 
 #include "../../include/xpu_graph_amd.h"
 
@@ -141,6 +144,20 @@ __device__ __forceinline__ void load_to_lds16(const void* base, uint32_t lane_of
 }
 
 inline int status_from_hip(hipError_t e) { return e == hipSuccess ? XG_OK : XG_ERR_LAUNCH; }
+
+// Raise the dynamic-LDS limit of `kernel` to `bytes` on the current device, once per (kernel, device).  Keyed by the
+// kernel's address, not by its type: many kernels here share one signature.
+inline int allow_dynamic_lds(const void* kernel, int bytes) {
+  static std::mutex mu;
+  static std::set<std::pair<const void*, int>> done;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return XG_ERR_LAUNCH;
+  std::lock_guard<std::mutex> lock(mu);
+  if (done.count({kernel, dev})) return XG_OK;
+  if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) return XG_ERR_LAUNCH;
+  done.insert({kernel, dev});
+  return XG_OK;
+}
 
 inline bool aligned_to(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
 
