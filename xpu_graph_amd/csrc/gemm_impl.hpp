@@ -831,9 +831,14 @@ template <typename T, typename OT, BLayout BL, bool GLU = false>
 __global__ __launch_bounds__(kThreads) void gemm_small_kernel(GemmParams p) {
   extern __shared__ __align__(16) char smem[];
   constexpr int EB = Elem<T>::BYTES;
-  static_assert(EB == 2, "16-bit operands only");
+  constexpr bool F8 = EB == 1;
+  static_assert(!F8 || (BL == BLayout::KMajor && !GLU), "fp8: K-contiguous weights, plain layer");
   static_assert(!GLU || BL == BLayout::KMajor, "the gated layer is wired for K-contiguous weights");
   constexpr int SLAB_K = ROW_BYTES / EB;
+  // fp8 slabs have two k-steps (of 64 elements): wavefront w takes k-step w & 1 and the 32 output columns w >> 1,
+  // so two partial tiles are summed instead of four.  NJ: 32-column units a wavefront accumulates.
+  constexpr int NJ = F8 ? 1 : 2;
+  constexpr int PARTS = F8 ? 2 : 4;
 
   int tm, tn;
   tile_of_block(p, blockIdx.x, gridDim.x, tm, tn);
@@ -874,13 +879,19 @@ __global__ __launch_bounds__(kThreads) void gemm_small_kernel(GemmParams p) {
       load_to_lds16((q == 0 ? b_base : b2_base) + kt * b_step, b_off[q], (uint32_t)(size_t)(lvoid*)(dst + S_SLAB_BYTES + q * 4096));
   };
 
-  // fragment addresses of this wavefront's k-step (= wave) inside a stage
+  // fragment addresses of this wavefront's k-step inside a stage
+  const int ks = F8 ? (wave & 1) : wave;
+  const int jbase = F8 ? (wave >> 1) : 0;  // first 32-column unit of this wavefront
   int a_frag[2], b_frag[2];
 #pragma unroll
   for (int u = 0; u < 2; ++u) {
     const int row = u * 32 + l32;
-    a_frag[u] = row * ROW_BYTES + (((wave * 2 + half) ^ swz(row)) << 4);
-    if constexpr (BL == BLayout::KMajor) {
+    // 16-bit: chunk 2 ks + half; fp8: chunks 4 ks + 2 half and the next one (read as frag + 16 ^ ... below)
+    a_frag[u] = row * ROW_BYTES + (((F8 ? ks * 4 + half * 2 : ks * 2 + half) ^ swz(row)) << 4);
+    if constexpr (F8) {
+      const int brow = (jbase + u) * 32 + l32;  // only u = 0 is used
+      b_frag[u] = S_SLAB_BYTES + brow * ROW_BYTES + (((ks * 4 + half * 2) ^ swz(brow)) << 4);
+    } else if constexpr (BL == BLayout::KMajor) {
       b_frag[u] = S_SLAB_BYTES + a_frag[u];
     } else {
       const int kr = wave * 16 + half * 8 + (p16 >> 2);
@@ -915,10 +926,20 @@ __global__ __launch_bounds__(kThreads) void gemm_small_kernel(GemmParams p) {
     Frag<T> fa[2], fb[2];
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
-      fa[u].v = *reinterpret_cast<const u32x4*>(st + a_frag[u]);
-      if constexpr (BL == BLayout::KMajor) {
+      if constexpr (F8) {
+        // the second 16-byte chunk of a lane's 32 bytes is the neighbour chunk: slot ^ 1 (the xor of the layout
+        // only touches the chunk index, and chunk + 1 == chunk ^ 1 for the even chunk the lane starts at)
+        fa[u].lo = *reinterpret_cast<const u32x4*>(st + a_frag[u]);
+        fa[u].hi = *reinterpret_cast<const u32x4*>(st + (a_frag[u] ^ 16));
+        if (u < NJ) {
+          fb[u].lo = *reinterpret_cast<const u32x4*>(st + b_frag[u]);
+          fb[u].hi = *reinterpret_cast<const u32x4*>(st + (b_frag[u] ^ 16));
+        }
+      } else if constexpr (BL == BLayout::KMajor) {
+        fa[u].v = *reinterpret_cast<const u32x4*>(st + a_frag[u]);
         fb[u].v = *reinterpret_cast<const u32x4*>(st + b_frag[u]);
       } else {
+        fa[u].v = *reinterpret_cast<const u32x4*>(st + a_frag[u]);
         const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(st + b_frag[u]));
         const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(st + b_frag[u] + 4 * ROW_BYTES));
         const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
@@ -928,25 +949,26 @@ __global__ __launch_bounds__(kThreads) void gemm_small_kernel(GemmParams p) {
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
-      for (int j = 0; j < 2; ++j) acc[i][j] = mma(fb[j], fa[i], acc[i][j]);
+      for (int j = 0; j < NJ; ++j) acc[i][j] = mma(fb[j], fa[i], acc[i][j]);
   }
   __syncthreads();  // the slabs are dead: the partial tiles take their place
 
-  // park this wavefront's partial tile: row r at r * 256, 16-byte chunk (4 columns) c at slot c ^ (r & 15)
-  char* park = smem + wave * (S_TILE * S_TILE * 4);
+  // park this wavefront's partial tile (fp8: its 32 columns of partial tile ks): row r at r * 256, 16-byte chunk
+  // (4 columns) c at slot c ^ (r & 15)
+  char* park = smem + (F8 ? ks : wave) * (S_TILE * S_TILE * 4);
 #pragma unroll
   for (int i = 0; i < 2; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < NJ; ++j)
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
         const int row = i * 32 + l32;
-        const int chunk = (j * 8 + g * 2 + half) ^ (row & 15);
+        const int chunk = ((jbase + j) * 8 + g * 2 + half) ^ (row & 15);
         const f32x16& a = acc[i][j];
         *reinterpret_cast<f32x4*>(park + row * 256 + (chunk << 4)) = f32x4{a[4 * g], a[4 * g + 1], a[4 * g + 2], a[4 * g + 3]};
       }
   __syncthreads();
-  // Sum the four partial tiles into the first one.  A thread sums exactly the (row, 8 columns) pieces it finishes
+  // Sum the partial tiles (four; fp8: two) into the first one.  A thread sums exactly the (row, 8 columns) pieces it finishes
   // below -- rows wave * 16 + pass * 8 + lane / 8, columns (lane & 7) * 8 -- so no barrier is needed in between.
 #pragma unroll
   for (int it = 0; it < 2; ++it) {
@@ -957,7 +979,7 @@ __global__ __launch_bounds__(kThreads) void gemm_small_kernel(GemmParams p) {
       char* at = smem + row * 256 + (((2 * c + hh) ^ (row & 15)) << 4);
       f32x4 v = *reinterpret_cast<const f32x4*>(at);
 #pragma unroll
-      for (int w = 1; w < 4; ++w) v += *reinterpret_cast<const f32x4*>(at + w * (S_TILE * S_TILE * 4));
+      for (int w = 1; w < PARTS; ++w) v += *reinterpret_cast<const f32x4*>(at + w * (S_TILE * S_TILE * 4));
       *reinterpret_cast<f32x4*>(at) = v;
     }
   }
@@ -1094,9 +1116,7 @@ inline bool half_height_wins(int M, int tn) {
 template <typename T, typename OT, BLayout BL>
 int launch_gemm(const GemmParams& p, hipStream_t stream) {
   if (!dma_ok<T>(p, BL)) return launch_kernel(gemm_staged_kernel<T, OT, BL>, p, stream);
-  if constexpr (Elem<T>::BYTES == 2) {
-    if ((int64_t)p.tiles_m * p.tiles_n <= small_tile_limit()) return launch_small<T, OT, BL>(p, stream);
-  }
+  if ((int64_t)p.tiles_m * p.tiles_n <= small_tile_limit()) return launch_small<T, OT, BL>(p, stream);
   const int keep = full_tile_columns(p.tiles_m, p.tiles_n);
   if (keep == p.tiles_n) {
     if (half_height_wins(p.M, p.tiles_n)) {
