@@ -365,7 +365,6 @@ __device__ __forceinline__ void epilogue_rows_act(const GemmParams& p, const cha
 template <typename OT, int NI = 4>
 __device__ __forceinline__ void epilogue(const GemmParams& p, const Lane& L, f32x16 (&acc)[4][4], char* smem, int m0,
                                          int n0) {
-  typedef OT O8 __attribute__((ext_vector_type(8)));
   char* park = smem + L.wave * (128 * 64 * 4);
   const float a_sc = p.a_scale ? *p.a_scale : 1.f;
   const int m_base = m0 + L.wm * (NI * 32);

@@ -215,8 +215,8 @@ struct SliceSumTable {
 
 template <typename T, int VEC>
 __global__ __launch_bounds__(256) void slice_sum_cat_kernel(const T* __restrict__ x, T* __restrict__ out, SliceSumTable tbl,
-                                                             int n_slices, int64_t batch, int cvecs, int64_t x_bs,
-                                                             int64_t x_rs, int64_t total) {
+                                                             int n_slices, int cvecs, int64_t x_bs, int64_t x_rs,
+                                                             int64_t total) {
   typedef T VT __attribute__((ext_vector_type(VEC)));
   const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (idx >= total) return;
@@ -267,10 +267,10 @@ int slice_sum_typed(const void* x, void* out, int64_t batch, int64_t rows, int64
   if (cvecs > 0x7fffffffLL || blocks > 0x7fffffffLL) return XG_ERR_TOO_LARGE;
   if (vec)
     hipLaunchKernelGGL((slice_sum_cat_kernel<T, V>), dim3((unsigned)blocks), dim3(256), 0, stream, (const T*)x, (T*)out, tbl, n,
-                       batch, (int)cvecs, x_bs, x_rs, total);
+                       (int)cvecs, x_bs, x_rs, total);
   else
     hipLaunchKernelGGL((slice_sum_cat_kernel<T, 1>), dim3((unsigned)blocks), dim3(256), 0, stream, (const T*)x, (T*)out, tbl, n,
-                       batch, (int)cvecs, x_bs, x_rs, total);
+                       (int)cvecs, x_bs, x_rs, total);
   return status_from_hip(hipGetLastError());
 }
 
