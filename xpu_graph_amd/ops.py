@@ -43,7 +43,21 @@ for _s in _SCHEMAS:
 
 
 def _stream():
-    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    """The current stream of the current device as a raw handle.  The private accessors are what
+    torch.cuda.current_stream() ends in; going through the Stream object costs about 4 us per call, a third of an
+    op's host time."""
+    return _raw_stream(_current_device())
+
+
+try:
+    _raw_stream = torch._C._cuda_getCurrentRawStream
+    _current_device = torch._C._cuda_getDevice
+except AttributeError:  # a torch build without these accessors
+
+    def _raw_stream(index):
+        return torch.cuda.current_stream(index).cuda_stream
+
+    _current_device = torch.cuda.current_device
 
 
 def _code(dtype):
@@ -54,7 +68,7 @@ def _code(dtype):
 
 
 def _ptr(t: Optional[torch.Tensor]):
-    return None if t is None else ctypes.c_void_p(t.data_ptr())
+    return None if t is None else t.data_ptr()  # ctypes turns the integer into the declared pointer type
 
 
 def _rows_2d(x: torch.Tensor):
