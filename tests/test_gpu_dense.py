@@ -112,6 +112,29 @@ def test_dense_c4_full_size(device):
     assert torch.equal(got_t, got)  # both weight layouts run the same arithmetic in the same order
 
 
+def test_dense_c4_full_size_permutation_properties(device):
+    """Size-independent properties at the full C4 shape: an output element is one dot product accumulated in a fixed
+    order over K, so permuting weight columns (with the bias) or activation rows must permute the result BIT FOR BIT
+    -- whichever tile, tile height or launch half an element lands in -- and the gated layer with equal gate and up
+    weights must equal silu(z) * z of the plain layer's rounded z."""
+    x, W, b = inputs.c4_dense(device=device)
+    ops = _ops()
+    base = ops.dense(x, W, False, b, None, "silu")
+    g = torch.Generator().manual_seed(11)
+    pc = torch.randperm(W.shape[1], generator=g).to(device)
+    assert torch.equal(ops.dense(x, W[:, pc].contiguous(), False, b[pc].contiguous(), None, "silu"), base[:, pc])
+    pr = torch.randperm(x.shape[0], generator=g).to(device)
+    assert torch.equal(ops.dense(x[pr].contiguous(), W, False, b, None, "silu"), base[pr])
+    # the [N, K] layout and a row-strided activation view go through other load paths, same arithmetic
+    Wt = W.t().contiguous()
+    wide = torch.empty(x.shape[0], x.shape[1] + 64, dtype=x.dtype, device=device)
+    wide[:, : x.shape[1]] = x
+    assert torch.equal(ops.dense(wide[:, : x.shape[1]], Wt, True, b, None, "silu"), base)
+    z = ops.dense(x, Wt, True, None, None, "none")
+    glu = ops.dense_glu(x, Wt, Wt)
+    assert torch.equal(glu, ops.silu_mul2(z, z))
+
+
 def test_dense_rejects_what_the_kernel_cannot_take(device):
     from xpu_graph_amd._lib import XgError
 

@@ -111,3 +111,25 @@ def test_norm_empty_and_errors(device):
         _ops().rms_norm(torch.randn(4, 8), None, 1e-6)  # CPU tensors: there is no fallback
     with pytest.raises(TypeError):
         _ops().rms_norm(torch.randn(4, 8, device=device, dtype=torch.float64), None, 1e-6)
+
+
+def test_add_layer_norm_c2_full_size_properties(device):
+    """Size-independent properties at the full C2 shape: unit-affine rows come out with mean 0 and variance 1; a shift
+    of the input by a per-row constant does not change the result (up to the rounding of the shifted input); the
+    second output is the rounded sum, bit for bit; repeated launches agree bit for bit."""
+    x, r, g, b = inputs.c2_add_layernorm(device=device)
+    ops = _ops()
+    one, zero = torch.ones_like(g), torch.zeros_like(b)
+    y, h = ops.add_layer_norm(x, r, one, zero, 1e-5)
+    assert torch.equal(h, x + r)
+    yf = y.float()
+    torch.testing.assert_close(yf.mean(-1), torch.zeros(x.shape[0], device=device), rtol=0, atol=2e-3)
+    torch.testing.assert_close(yf.var(-1, unbiased=False), torch.ones(x.shape[0], device=device), rtol=1e-2, atol=1e-2)
+    y2, h2 = ops.add_layer_norm(x, r, one, zero, 1e-5)
+    assert torch.equal(y, y2) and torch.equal(h, h2)
+    # fp32 inputs for the shift property (a bf16 shift would round the data itself)
+    xf = x.float()
+    shift = torch.randn(x.shape[0], 1, device=device) * 4
+    a = ops.layer_norm(xf, g.float(), b.float(), 1e-5)
+    c = ops.layer_norm(xf + shift, g.float(), b.float(), 1e-5)
+    torch.testing.assert_close(a, c, rtol=1e-4, atol=1e-4)

@@ -124,6 +124,28 @@ def test_sdpa_c5_full_size(device):
     assert torch.equal(_ops().sdpa(q, k, ones, True, scale), ones)
 
 
+def test_sdpa_c5_full_size_permutation_and_prefix_properties(device):
+    """At the full C5 shape: heads and batches are independent problems, so permuting them permutes the output bit
+    for bit (whatever workgroup order or XCD a head lands on); under the causal mask the first n query rows do not
+    depend on later keys, so a prefix of the sequence gives the same first rows bit for bit; the same holds through
+    strided [B, S, H, D] storage."""
+    B, H, S, D = 4, 32, 2048, 128
+    q, k, v = make(B, H, H, S, S, D, torch.bfloat16, device, seed=5)
+    scale = 1.0 / math.sqrt(D)
+    ops = _ops()
+    base = ops.sdpa(q, k, v, True, scale)
+    g = torch.Generator().manual_seed(3)
+    ph = torch.randperm(H, generator=g).to(device)
+    pb = torch.randperm(B, generator=g).to(device)
+    got = ops.sdpa(q[pb][:, ph].contiguous(), k[pb][:, ph].contiguous(), v[pb][:, ph].contiguous(), True, scale)
+    assert torch.equal(got, base[pb][:, ph])
+    n = 1280  # ten query blocks; keys 1280.. are never visible to them
+    pre = ops.sdpa(q[:, :, :n].contiguous(), k[:, :, :n].contiguous(), v[:, :, :n].contiguous(), True, scale)
+    assert torch.equal(pre, base[:, :, :n])
+    qs, ks, vs = (t.transpose(1, 2).contiguous().transpose(1, 2) for t in (q, k, v))  # [B, S, H, D] storage
+    assert torch.equal(ops.sdpa(qs, ks, vs, True, scale), base)
+
+
 def test_sdpa_rejects_what_the_kernel_cannot_take(device):
     q, k, v = make(1, 2, 2, 64, 64, 128, torch.bfloat16, device)
     with pytest.raises(Exception):
