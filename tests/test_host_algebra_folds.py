@@ -269,3 +269,62 @@ def test_detach_disappears_in_inference(caplog, infer_backend):
     with need_xpu_graph_logs(), torch.no_grad():
         run(infer_backend, lambda a: a.detach() * 2 + a.detach(), torch.randn(8, 8), exact=True)
     assert "Pattern.FoldDetach changed graph" in caplog.text
+
+
+# ---- hand-written GELU ---------------------------------------------------------------------------------------------
+import math  # noqa: E402
+
+GELUS = [
+    ("none", lambda x: 0.5 * (1 + torch.erf(x / math.sqrt(2))) * x),
+    ("none", lambda x: x * 0.5 * (torch.erf(x * (1 / math.sqrt(2))) + 1.0)),
+    ("tanh", lambda x: 0.5 * x * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (x + 0.044715 * torch.pow(x, 3.0))))),
+    ("tanh", lambda x: x * (1.0 + torch.tanh((x + x * x * x * 0.044715) * math.sqrt(2.0 / math.pi))) * 0.5),
+]
+
+
+@pytest.mark.parametrize("idx", range(len(GELUS)))
+def test_hand_written_gelu_becomes_aten_gelu(caplog, infer_backend, idx):
+    kind, fn = GELUS[idx]
+    x = torch.randn(64, 32)
+    with need_xpu_graph_logs():
+        got = torch.compile(fn, backend=infer_backend)(x)
+    torch.testing.assert_close(got, fn(x), rtol=1e-5, atol=1e-6)
+    torch.testing.assert_close(got, torch.nn.functional.gelu(x, approximate=kind), rtol=1e-5, atol=1e-6)
+    assert "Pattern.Gelu changed graph" in caplog.text
+    final = infer_backend.compiled_graphs[-1]
+    calls = [n for n in final.graph.nodes if n.op == "call_function"]
+    assert [str(n.target) for n in calls] == ["aten.gelu.default"]
+    assert calls[0].kwargs.get("approximate", "none") == kind
+    torch._dynamo.reset()
+
+
+def test_near_gelu_is_left_alone(caplog, infer_backend):
+    fns = [
+        lambda x: 0.5 * (1 + torch.erf(x / 1.5)) * x,  # another divisor
+        lambda x: 0.5 * (1 + torch.erf(x / math.sqrt(2))) * (x + 1),  # the gate multiplies something else
+        lambda x: 0.5 * x * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (x + 0.05 * torch.pow(x, 3.0)))),  # another cubic weight
+    ]
+    with need_xpu_graph_logs():
+        for fn in fns:
+            run(infer_backend, fn, torch.randn(16, 8))
+    assert "Pattern.Gelu changed graph" not in caplog.text
+
+
+def test_recognised_gelu_becomes_the_dense_layers_activation():
+    """On the mi355x target the dense pattern takes aten.gelu as its activation: a hand-written erf GELU behind a
+    matmul + bias therefore ends in ONE dense call (the kernels refuse CPU tensors, so only the rewrite is checked)."""
+    from xpu_graph_amd import OptLevel, Target
+
+    def fn(x, w, b):
+        z = torch.addmm(b, x, w)
+        return 0.5 * z * (1 + torch.erf(z / math.sqrt(2)))
+
+    bf = torch.bfloat16
+    backend = XpuGraph(XpuGraphConfig(is_training=False, target=Target.mi355x, opt_level=OptLevel.level2, enable_cache=False))
+    args = [torch.randn(16, 64).to(bf), torch.randn(64, 128).to(bf), torch.randn(128).to(bf)]
+    with pytest.raises(NotImplementedError), torch.no_grad():
+        torch.compile(fn, backend=backend, dynamic=False)(*args)
+    calls = [n for n in backend.compiled_graphs[-1].graph.nodes if n.op in ("call_module", "call_function")]
+    assert [str(n.target) for n in calls] == ["custom_dense_layer_replacement"]
+    assert calls[0].args[-1] == "gelu"
+    torch._dynamo.reset()

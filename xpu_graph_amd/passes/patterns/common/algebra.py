@@ -392,3 +392,116 @@ class ChangeTensorLike(Pattern):
             gm.graph.erase_node(n)
             changed = True
         return changed
+
+
+def _close(a, b):
+    return type(a) in (int, float) and abs(a - b) <= 1e-6 * max(1.0, abs(b))
+
+
+def _factors(node, root=True):
+    """Leaves of the product tree under `node` (a mul.Tensor): inner muls are opened when nothing else reads them."""
+    if is_call(node, aten.mul.Tensor, aten.mul.Scalar) and (root or len(node.users) == 1):
+        return _factors(node.args[0], False) + _factors(node.args[1], False)
+    return [node]
+
+
+def _split(factors, n_nodes):
+    """(scalar product, node factors) when there are exactly n_nodes node factors, else None."""
+    scalar, nodes = 1.0, []
+    for f in factors:
+        if isinstance(f, fx.Node):
+            nodes.append(f)
+        elif type(f) in (int, float):
+            scalar *= f
+        else:
+            return None
+    return (scalar, nodes) if len(nodes) == n_nodes else None
+
+
+def _one_plus(node, inner_target):
+    """node == 1 + inner_target(arg): returns the inner call, else None."""
+    if not is_call(node, aten.add.Tensor, aten.add.Scalar) or kwarg(node, "alpha") not in (None, 1):
+        return None
+    a, b = node.args[0], node.args[1]
+    inner = a if _close(b, 1.0) else (b if _close(a, 1.0) else None)
+    return inner if is_call(inner, inner_target) else None
+
+
+class Gelu(Pattern):
+    """Hand-written GELU becomes aten.gelu, which the dense-layer pattern can then take as its activation:
+    0.5 * x * (1 + erf(x / sqrt 2)) -> gelu(x);  0.5 * x * (1 + tanh(sqrt(2 / pi) * (x + 0.044715 x^3))) ->
+    gelu(x, approximate="tanh").  Factors may come in any order and association (reference common/gelu.py:9-56,
+    which maps the tanh form to the exact gelu; the approximation is kept here)."""
+
+    _support_stages = [FxStage.inference, FxStage.pregrad]
+
+    @staticmethod
+    def _erf_form(x, plus):
+        erf = _one_plus(plus, aten.erf.default)
+        if erf is None:
+            return False
+        inner = erf.args[0]
+        if is_call(inner, aten.div.Tensor, aten.div.Scalar):
+            return inner.args[0] is x and _close(inner.args[1], 2**0.5) and not inner.kwargs.get("rounding_mode")
+        if is_call(inner, aten.mul.Tensor, aten.mul.Scalar):
+            got = _split(_factors(inner), 1)
+            return got is not None and got[1][0] is x and _close(got[0], 0.5**0.5)
+        return False
+
+    @staticmethod
+    def _cube_of(node, x):
+        if is_call(node, aten.pow.Tensor_Scalar):
+            return node.args[0] is x and _close(node.args[1], 3.0)
+        got = _split(_factors(node), 3) if is_call(node, aten.mul.Tensor) else None
+        return got is not None and _close(got[0], 1.0) and all(f is x for f in got[1])
+
+    @classmethod
+    def _tanh_form(cls, x, plus):
+        tanh = _one_plus(plus, aten.tanh.default)
+        if tanh is None or not is_call(tanh.args[0], aten.mul.Tensor, aten.mul.Scalar):
+            return False
+        got = _split(_factors(tanh.args[0]), 1)
+        if got is None or not _close(got[0], (2.0 / 3.141592653589793) ** 0.5):
+            return False
+        poly = got[1][0]  # x + 0.044715 x^3
+        if not is_call(poly, aten.add.Tensor) or kwarg(poly, "alpha") not in (None, 1):
+            return False
+        for lin, cub in ((poly.args[0], poly.args[1]), (poly.args[1], poly.args[0])):
+            if lin is not x or not is_call(cub, aten.mul.Tensor, aten.mul.Scalar):
+                continue
+            parts = _factors(cub)
+            scalar = 1.0
+            rest = []
+            for f in parts:
+                if type(f) in (int, float):
+                    scalar *= f
+                else:
+                    rest.append(f)
+            if not _close(scalar, 0.044715):
+                continue
+            if len(rest) == 1 and cls._cube_of(rest[0], x):
+                return True
+            if len(rest) == 3 and all(f is x for f in rest):
+                return True
+        return False
+
+    def process(self, gm):
+        changed = False
+        for n in reversed(list(gm.graph.nodes)):
+            if not is_call(n, aten.mul.Tensor, aten.mul.Scalar) or "val" not in n.meta or not n.users:
+                continue
+            got = _split(_factors(n), 2)
+            if got is None or not _close(got[0], 0.5):
+                continue
+            for x, plus in (got[1], got[1][::-1]):
+                if "val" not in x.meta or x.meta["val"].shape != n.meta["val"].shape or x.meta["val"].dtype != n.meta["val"].dtype:
+                    continue
+                kind = "none" if self._erf_form(x, plus) else ("tanh" if self._tanh_form(x, plus) else None)
+                if kind is None:
+                    continue
+                with gm.graph.inserting_before(n):
+                    res = gm.graph.call_function(aten.gelu.default, (x,), {} if kind == "none" else {"approximate": "tanh"})
+                n.replace_all_uses_with(res)
+                changed = True
+                break
+        return changed
