@@ -348,3 +348,33 @@ def test_layer_norm_mixed_types_loss_and_grad(device, caplog, fn, param_dtype):
             assert a.dtype == c.dtype
             torch.testing.assert_close(a.float(), c.float(), rtol=2e-2, atol=2e-2 * max(1.0, c.float().abs().mean().item()))
     torch._dynamo.reset()
+
+
+@pytest.mark.parametrize("form", ["erf", "tanh"])
+def test_hand_written_gelu_runs_in_the_dense_epilogue_or_as_aten_gelu(device, form):
+    """A GELU written out in elementary ops behind matmul + bias: the erf form becomes the dense kernel's activation
+    (one launch); the tanh form becomes aten.gelu(approximate="tanh") behind a plain dense launch."""
+    import math
+
+    def fn(x, w, b):
+        z = torch.addmm(b, x, w)
+        if form == "erf":
+            return 0.5 * z * (1 + torch.erf(z / math.sqrt(2)))
+        return 0.5 * z * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (z + 0.044715 * torch.pow(z, 3.0))))
+
+    g = torch.Generator().manual_seed(4)
+    bf = torch.bfloat16
+    x = torch.randn(384, 256, generator=g).to(bf).to(device)
+    w = (torch.randn(256, 512, generator=g) / 16).to(bf).to(device)
+    b = torch.randn(512, generator=g).to(bf).to(device)
+    backend = mi355x_compiler()
+    with torch.no_grad():
+        got = torch.compile(fn, backend=backend, dynamic=False)(x, w, b)
+    want = torch.nn.functional.gelu(torch.addmm(b.float(), x.float(), w.float()), approximate="none" if form == "erf" else "tanh")
+    torch.testing.assert_close(got.float(), want, rtol=1.6e-2, atol=2e-2)
+    calls = [str(n.target) for n in backend.compiled_graphs[-1].graph.nodes if n.op in ("call_module", "call_function")]
+    if form == "erf":
+        assert calls == ["custom_dense_layer_replacement"], calls
+    else:
+        assert calls == ["custom_dense_layer_replacement", "aten.gelu.default"], calls
+    torch._dynamo.reset()

@@ -509,3 +509,24 @@ def test_batch_dense_layer_vetoes(backend):
     x, w = torch.randn(2, 8, 12).to(bf16), torch.randn(2, 12, 8).to(bf16)  # K not a multiple of 8
     gm = rewrite(mi355x_compiler(), lambda x, w: torch.bmm(x, w), x, w, must_fail=False)
     assert modules_called(gm) == []
+
+
+def test_tanh_gelu_is_not_taken_for_the_erf_gelu_of_the_dense_kernel():
+    """aten.gelu(approximate="tanh") behind a matmul stays an Aten op: the dense epilogue evaluates the erf form."""
+    import torch.nn.functional as F
+
+    from xpu_graph_amd import OptLevel, Target, XpuGraph, XpuGraphConfig
+
+    def fn(x, w, w2, b):
+        return F.gelu(torch.addmm(b, x, w), approximate="tanh"), F.gelu(torch.addmm(b, x, w2))
+
+    bf = torch.bfloat16
+    backend = XpuGraph(XpuGraphConfig(is_training=False, target=Target.mi355x, opt_level=OptLevel.level2, enable_cache=False))
+    args = [torch.randn(16, 64).to(bf), torch.randn(64, 128).to(bf), torch.randn(64, 128).to(bf), torch.randn(128).to(bf)]
+    with pytest.raises(NotImplementedError), torch.no_grad():
+        torch.compile(fn, backend=backend, dynamic=False)(*args)
+    calls = [n for n in backend.compiled_graphs[-1].graph.nodes if n.op in ("call_module", "call_function")]
+    acts = sorted(n.args[-1] for n in calls if n.op == "call_module")
+    assert acts == ["gelu", "none"]
+    assert sum(1 for n in calls if "aten.gelu" in str(n.target)) == 1
+    torch._dynamo.reset()

@@ -116,8 +116,13 @@ def skip_layout_ops(node):
 
 
 def activation_name(node):
+    """Name of the activation a node applies, for the ops a dense epilogue can evaluate; a gelu that asks for the
+    tanh approximation is not the erf gelu of the kernels."""
     if isinstance(node, fx.Node) and node.op == "call_function":
-        return ACTIVATIONS.get(node.target)
+        name = ACTIVATIONS.get(node.target)
+        if name == "gelu" and node.kwargs.get("approximate", "none") != "none":
+            return None
+        return name
     return None
 
 
