@@ -247,3 +247,32 @@ def test_output_clone_of_private_intermediate_is_dropped():
     for a, b in zip(got, aliased(x)):
         assert torch.equal(a, b)
     assert got[0].data_ptr() != got[1].data_ptr() and got[2].data_ptr() != x.data_ptr() and got[3].data_ptr() != x.data_ptr()
+
+
+def test_matchers_respect_arguments_that_change_the_meaning(caplog):
+    """add(mm, bias, alpha=2) is not addmm(bias); a softmax over the QUERY axis, or one that leaves in fp32, is not
+    attention; a masked sum with alpha != 1 is not an additive mask."""
+    import xpu_graph_amd
+    from xpu_graph_amd.test_utils import need_xpu_graph_logs
+
+    backend = xpu_graph_amd.XpuGraph(xpu_graph_amd.XpuGraphConfig(is_training=False, opt_level=xpu_graph_amd.OptLevel.level2, enable_cache=False))
+
+    def scaled_bias(x, w, b):
+        return torch.add(torch.mm(x, w), b, alpha=2.0)
+
+    def softmax_over_queries(q, k, v):
+        return torch.bmm(torch.softmax(torch.bmm(q, k.transpose(1, 2)) * 0.125, dim=1), v)
+
+    def scaled_mask(q, k, v, m):
+        return torch.bmm(torch.softmax(torch.add(torch.bmm(q, k.transpose(1, 2)) * 0.125, m, alpha=3.0), dim=-1), v)
+
+    q, k, v = (torch.randn(4, 16, 64) for _ in range(3))
+    m = torch.randn(4, 16, 16)
+    with need_xpu_graph_logs():
+        for fn, args in ((scaled_bias, (torch.randn(8, 16), torch.randn(16, 4), torch.randn(4))),
+                         (softmax_over_queries, (q, k, v)), (scaled_mask, (q, k, v, m))):
+            got = torch.compile(fn, backend=backend, dynamic=False)(*args)
+            torch.testing.assert_close(got, fn(*args), rtol=1e-4, atol=1e-5)
+            torch._dynamo.reset()
+    assert "Pattern.FusedAddMM changed graph" not in caplog.text
+    assert "Pattern.FusedSDPA changed graph" not in caplog.text

@@ -530,3 +530,16 @@ def test_tanh_gelu_is_not_taken_for_the_erf_gelu_of_the_dense_kernel():
     assert acts == ["gelu", "none"]
     assert sum(1 for n in calls if "aten.gelu" in str(n.target)) == 1
     torch._dynamo.reset()
+
+
+def test_slice_bounds_past_the_source_are_clamped_like_eager():
+    """x[:, 5:10000] and x[:, -10000:3] are legal eager slices; the fused slice/cat must see the clamped ranges."""
+    from xpu_graph_amd.passes.patterns.structure.slice_cat import slice_run_params
+
+    def fn(x):
+        return torch.cat([x[:, 5:10000], x[:, -10000:3], x[:, 7:7], x[:, 2:6]], dim=1)
+
+    gm = torch.fx.experimental.proxy_tensor.make_fx(fn)(torch.randn(4, 16))
+    slices = [n for n in gm.graph.nodes if n.op == "call_function" and n.target == torch.ops.aten.slice.Tensor and n.args[1] == 1]
+    src, params = slice_run_params(slices)
+    assert params == [(5, 16), (0, 3), (7, 7), (2, 6)]

@@ -20,7 +20,7 @@ from ....utils import logger
 from ...general import is_constant
 from ..pattern import Pattern
 from ..utils.default_replacements import SDPAWrappedScale
-from ..utils.node_utils import SymShapes, arg, aten, is_call, same_shape, skip_layout_ops
+from ..utils.node_utils import SymShapes, arg, aten, is_call, kwarg, same_shape, skip_layout_ops
 
 
 def attention_dims(q_shape, k_shape, v_shape, mask_shape):
@@ -71,10 +71,16 @@ def match_attention(node):
     softmax = skip_layout_ops(probs)
     if not is_call(softmax, aten._softmax.default, aten._safe_softmax.default):
         return None
+    sm_rank = len(softmax.meta["val"].shape)
+    sm_dim = arg(softmax, 1)
+    if not isinstance(sm_dim, int) or sm_dim % sm_rank != sm_rank - 1:
+        return None  # attention normalises over the keys, the last dim of the scores
+    if is_call(softmax, aten._softmax.default) and arg(softmax, 2):
+        return None  # half_to_float: probabilities leave in fp32, which the fused op does not return
     cur = skip_layout_ops(softmax.args[0])
 
     mask, mask_added, has_mask = None, False, False
-    if is_call(cur, aten.add.Tensor, aten.sub.Tensor):
+    if is_call(cur, aten.add.Tensor, aten.sub.Tensor) and kwarg(cur, "alpha") in (None, 1):
         mask, mask_added, has_mask = arg(cur, 1), cur.target == aten.add.Tensor, True
         cur = skip_layout_ops(cur.args[0])
 
@@ -90,7 +96,7 @@ def match_attention(node):
 
     if is_call(cur, aten.bmm.default):
         q, k = arg(cur, 0), arg(cur, 1)
-    elif is_call(cur, aten.baddbmm.default) and not has_mask and not has_scale:
+    elif is_call(cur, aten.baddbmm.default) and not has_mask and not has_scale and kwarg(cur, "beta") in (None, 1) and kwarg(cur, "alpha") in (None, 1):
         mask, q, k = arg(cur, 0), arg(cur, 1), arg(cur, 2)
         has_mask, mask_added = True, True
     else:

@@ -15,8 +15,8 @@ from ..utils.node_utils import aten, is_call, mm_operands, same_shape
 
 
 def match_mm_plus_bias(node):
-    if not is_call(node, aten.add.Tensor):
-        return None
+    if not is_call(node, aten.add.Tensor) or len(node.args) != 2 or node.kwargs.get("alpha", 1) != 1:
+        return None  # add(mm, bias, alpha=a) scales the bias: not an addmm with beta = 1
     for mm, bias in ((node.args[0], node.args[1]), (node.args[1], node.args[0])):
         ops = mm_operands(mm) if isinstance(mm, fx.Node) else None
         if ops is None:

@@ -35,6 +35,8 @@ def slice_run_params(nodes):
         return None
     src = nodes[0].args[0]
     width = src.meta["val"].shape[-1]
+    if not isinstance(width, int):
+        return None  # a symbolic width: the column table cannot be built at compile time
     params = []
     for n in nodes:
         if n.args[0] is not src or len(n.args) < 4 or n.args[1] != 1:
@@ -51,6 +53,9 @@ def slice_run_params(nodes):
             end = width + end
         if start < 0:
             start = width + start
+        # eager slicing clamps bounds to the source (x[:, 5:10000] is x[:, 5:]; an empty range stays empty)
+        start = max(0, min(start, width))
+        end = max(start, min(end, width))
         params.append((start, end))
     return src, params
 
