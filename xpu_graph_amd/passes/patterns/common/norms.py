@@ -46,7 +46,7 @@ def _inverse_root_operand(node, is_div):
 
 def _split_eps_add(node):
     """add.Tensor(t, eps) or add.Tensor(eps, t) with a python-number eps -> (t, eps)."""
-    if not is_call(node, aten.add.Tensor, aten.add.Scalar):
+    if not is_call(node, aten.add.Tensor, aten.add.Scalar) or kwarg(node, "alpha") not in (None, 1):
         return None
     a, b = arg(node, 0), arg(node, 1)
     if isinstance(b, _NUM) and isinstance(a, fx.Node):
@@ -89,6 +89,8 @@ def match_unweighted_rmsnorm(node):
         return None
     if not is_call(mean, aten.mean.dim) or not _last_dim_only(arg(mean, 1), arg(mean, 0)) or kwarg(mean, "keepdim") is not True:
         return None
+    if kwarg(mean, "dtype") not in (None, mean.meta["val"].dtype if "val" in mean.meta else None, arg(mean, 0).meta["val"].dtype):
+        return None  # a mean that also converts its input
     sq = arg(mean, 0)
     if not isinstance(sq, fx.Node) or not sole_user_is(sq, mean):
         return None
