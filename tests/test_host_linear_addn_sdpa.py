@@ -276,3 +276,40 @@ def test_matchers_respect_arguments_that_change_the_meaning(caplog):
             torch._dynamo.reset()
     assert "Pattern.FusedAddMM changed graph" not in caplog.text
     assert "Pattern.FusedSDPA changed graph" not in caplog.text
+
+
+@pytest.mark.parametrize("is_training", [False, True])
+@pytest.mark.parametrize(
+    "in_dtype,bias_kind",
+    [(torch.float32, torch.float32), (torch.float32, float), (torch.float32, None), (torch.bfloat16, torch.bfloat16),
+     (torch.float16, torch.float16), (torch.bfloat16, torch.float32), (torch.float16, torch.bfloat16)],
+)
+def test_bmm_plus_bias_becomes_baddbmm(caplog, is_training, in_dtype, bias_kind):
+    """The batched twin of mm + bias (reference tests/common/test_fuse_baddbmm.py:15-90): tensor, python-number and
+    absent biases, biases of another type than the product."""
+    import torch.nn.functional as F
+
+    import xpu_graph_amd
+    from xpu_graph_amd.test_utils import is_similar, need_xpu_graph_logs
+
+    def fn(x, w, bias=None):
+        out = torch.bmm(x, w)
+        out = out + bias if bias is not None else out
+        return F.gelu(out)
+
+    backend = xpu_graph_amd.XpuGraph(xpu_graph_amd.XpuGraphConfig(is_training=is_training, opt_level=xpu_graph_amd.OptLevel.level2, enable_cache=False))
+    x = torch.randn(64, 37, 16, dtype=in_dtype)
+    w = torch.randn(64, 16, 16, dtype=in_dtype, requires_grad=is_training)
+    if bias_kind is float:
+        bias = 3.0
+    elif bias_kind is None:
+        bias = None
+    else:
+        bias = torch.randn(16, dtype=bias_kind, requires_grad=is_training)
+    want = fn(x, w, bias)
+    with need_xpu_graph_logs():
+        got = torch.compile(fn, backend=backend, dynamic=is_training)(x, w, bias)
+    assert got.dtype == want.dtype
+    assert is_similar(got.float(), want.float(), rtol=2e-2, atol=2e-2)
+    assert ("Pattern.FusedBAddBMM changed graph" in caplog.text) == (bias is not None)
+    torch._dynamo.reset()

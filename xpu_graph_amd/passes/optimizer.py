@@ -47,7 +47,8 @@ class Optimizer(abc.ABC):
             return False
         gm.graph.lint()
         gm.recompile()
-        base = type(self).__bases__[0].__name__
+        # the family a pass belongs to ("Pattern", "Optimizer"), however many helper classes sit in between
+        base = next((c.__name__ for c in type(self).__mro__[1:] if c.__name__ in ("Pattern", "Optimizer")), type(self).__bases__[0].__name__)
         logger.debug(f"{base}.{self} changed graph, before: {before} nodes, after: {len(gm.graph.nodes)} nodes.")
         if self._dump_graph:
             self._dump(gm)

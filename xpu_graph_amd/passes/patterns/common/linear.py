@@ -14,11 +14,20 @@ from ..pattern import Pattern
 from ..utils.node_utils import aten, is_call, mm_operands, same_shape
 
 
-def match_mm_plus_bias(node):
+def bmm_operands(node):
+    """(lhs, rhs) of a bmm, or of a matmul of two 3-D tensors; None otherwise."""
+    if is_call(node, aten.bmm.default):
+        return node.args[0], node.args[1]
+    if is_call(node, aten.matmul.default) and all(isinstance(a, fx.Node) and "val" in a.meta and a.meta["val"].dim() == 3 for a in node.args[:2]):
+        return node.args[0], node.args[1]
+    return None
+
+
+def match_mm_plus_bias(node, operands=mm_operands):
     if not is_call(node, aten.add.Tensor) or len(node.args) != 2 or node.kwargs.get("alpha", 1) != 1:
         return None  # add(mm, bias, alpha=a) scales the bias: not an addmm with beta = 1
     for mm, bias in ((node.args[0], node.args[1]), (node.args[1], node.args[0])):
-        ops = mm_operands(mm) if isinstance(mm, fx.Node) else None
+        ops = operands(mm) if isinstance(mm, fx.Node) else None
         if ops is None:
             continue
         if len(mm.users) != 1 or not same_shape(node.meta["val"].shape, mm.meta["val"].shape):
@@ -30,13 +39,16 @@ def match_mm_plus_bias(node):
 class FusedAddMM(Pattern):
     _opt_level = OptLevel.level2
     _support_stages = [FxStage.inference, FxStage.forward, FxStage.pregrad]
+    _operands = staticmethod(mm_operands)
+    _fused = aten.addmm.default
+    _name = "addmm_replacement"
 
     def process(self, gm):
         g = gm.graph
         cast = aten.to.dtype if self._current_stage == FxStage.pregrad else aten._to_copy.default
         changed = False
         for node in reversed(g.nodes):
-            m = match_mm_plus_bias(node)
+            m = match_mm_plus_bias(node, self._operands)
             if m is None:
                 continue
             bias, x, w = m
@@ -48,13 +60,21 @@ class FusedAddMM(Pattern):
                     )
                 elif bias.meta["val"].dtype != x_val.dtype:
                     bias = g.create_node("call_function", cast, (bias,), {"dtype": x_val.dtype}, name="bias_cast")
-                new = g.create_node("call_function", aten.addmm.default, (bias, x, w), name="addmm_replacement")
+                new = g.create_node("call_function", self._fused, (bias, x, w), name=self._name)
                 if x_val.dtype != node.meta["val"].dtype:
                     new = g.create_node("call_function", cast, (new,), {"dtype": node.meta["val"].dtype}, name="input_cast")
             node.replace_all_uses_with(new)
             g.erase_node(node)
             changed = True
         return changed
+
+
+class FusedBAddBMM(FusedAddMM):
+    """bmm + bias -> baddbmm, the batched twin of FusedAddMM (reference common/fuse_baddbmm.py:11-89)."""
+
+    _operands = staticmethod(bmm_operands)
+    _fused = aten.baddbmm.default
+    _name = "baddbmm_replacement"
 
 
 class DecomposeLinear(Pattern):
