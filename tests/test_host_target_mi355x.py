@@ -543,3 +543,31 @@ def test_slice_bounds_past_the_source_are_clamped_like_eager():
     slices = [n for n in gm.graph.nodes if n.op == "call_function" and n.target == torch.ops.aten.slice.Tensor and n.args[1] == 1]
     src, params = slice_run_params(slices)
     assert params == [(5, 16), (0, 3), (7, 7), (2, 6)]
+
+
+def test_repeated_gather_index_becomes_a_broadcast_view(caplog):
+    """reference tests/mlu/test_repeat_to_expand.py:8-38: arange -> expand -> unsqueeze -> repeat -> gather."""
+
+    def fn(x, n):
+        idx = torch.arange(n).reshape(1, -1).expand(x.shape[0], -1)
+        idx = idx.unsqueeze(-1).repeat(1, 1, x.shape[2])
+        return x.gather(index=idx, dim=1)
+
+    def real_repeat(x, idx):
+        return x.gather(index=idx.repeat(2, 1, 1), dim=1)  # copies along a real axis: must stay
+
+    backend = XpuGraph(XpuGraphConfig(is_training=False, target=Target.mi355x, opt_level=OptLevel.level1, enable_cache=False))
+    x = torch.randn(12, 40, 16)
+    with need_xpu_graph_logs():
+        got = torch.compile(fn, backend=backend, dynamic=True)(x, 9)
+    assert torch.equal(got, fn(x, 9))
+    assert "Pattern.FusedGatherToCopy changed graph" in caplog.text
+    assert not any("repeat" in str(n.target) for n in backend.compiled_graphs[-1].graph.nodes)
+    caplog.clear()
+    torch._dynamo.reset()
+    idx = torch.randint(0, 40, (6, 5, 16))
+    with need_xpu_graph_logs():
+        got = torch.compile(real_repeat, backend=backend, dynamic=False)(x, idx)
+    assert torch.equal(got, real_repeat(x, idx))
+    assert "Pattern.FusedGatherToCopy changed graph" not in caplog.text
+    torch._dynamo.reset()
