@@ -328,3 +328,4 @@ def test_recognised_gelu_becomes_the_dense_layers_activation():
     assert [str(n.target) for n in calls] == ["custom_dense_layer_replacement"]
     assert calls[0].args[-1] == "gelu"
     torch._dynamo.reset()
+

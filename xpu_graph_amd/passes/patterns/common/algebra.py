@@ -505,3 +505,4 @@ class Gelu(Pattern):
                 changed = True
                 break
         return changed
+
