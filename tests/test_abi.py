@@ -65,3 +65,22 @@ def test_argument_validation_needs_no_gpu():
     assert lib.xg_slice_sum_cat(p, p, 2, 4, 8, 32, 8, i32(0, 0, 0), i32(1, 2, 3), 3, 9, None) == -1  # unknown dtype
     assert lib.xg_slice_sum_cat(p, p, 0, 4, 8, 32, 8, i32(0, 0, 0), i32(1, 2, 3), 3, 0, None) == 0  # empty batch
     assert lib.xg_silu_mul(p, p, 2, 8, 8, 0, None) == -2  # row stride < 2*d
+
+
+def test_a_missing_library_is_an_error_not_a_fallback(monkeypatch, tmp_path):
+    from xpu_graph_amd import _lib
+
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "libxpu_graph_amd.so"))
+    with pytest.raises(ImportError, match="no fallback"):
+        _lib.lib()
+
+
+def test_the_ops_have_no_cpu_kernel():
+    import torch
+
+    import xpu_graph_amd.ops  # noqa: F401  registers torch.ops.xpu_ops.*
+
+    x = torch.randn(4, 8)
+    with pytest.raises((NotImplementedError, RuntimeError)):
+        torch.ops.xpu_ops.rms_norm(x, torch.ones(8), 1e-6)
