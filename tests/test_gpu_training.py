@@ -126,3 +126,57 @@ def test_mlp_training_step(device):
     err = lambda a, c: (a.float() - c).abs().mean().item()  # noqa: E731
     for a, c, e in zip(g0, g1, g2):
         assert err(a, c) <= 2 * err(e, c) + 1e-2 * c.abs().mean().item(), (err(a, c), err(e, c), c.abs().mean().item())
+
+
+def test_gated_dense_backward_formula(device):
+    """Gradients of xpu_ops.dense_glu (projections recomputed and input gradient on the HIP dense kernel, weight
+    gradients Aten matmuls) against autograd of silu(x Wg^T) * (x Wu^T) evaluated in fp32."""
+    import xpu_graph_amd.ops as xops
+
+    xops.enable_autograd()
+    torch.manual_seed(3)
+    M, K, N = 384, 256, 192
+    bf = torch.bfloat16
+    x = torch.randn(M, K, device=device).to(bf).requires_grad_(True)
+    wg = (torch.randn(N, K, device=device) / 16).to(bf).requires_grad_(True)
+    wu = (torch.randn(N, K, device=device) / 16).to(bf).requires_grad_(True)
+    dy = torch.randn(M, N, device=device).to(bf)
+    y = torch.ops.xpu_ops.dense_glu(x, wg, wu)
+    g = torch.autograd.grad((y,), (x, wg, wu), (dy,))
+    fx, fg, fu = (t.detach().float().requires_grad_(True) for t in (x, wg, wu))
+    ref = F.silu(fx @ fg.t()) * (fx @ fu.t())
+    gref = torch.autograd.grad((ref,), (fx, fg, fu), (dy.float(),))
+    torch.testing.assert_close(y.float(), ref, rtol=1.6e-2, atol=3e-2)
+    for name, a, c in zip("x wg wu".split(), g, gref):
+        scale = c.abs().mean().item()
+        assert (a.float() - c).abs().mean().item() <= 2e-2 * scale + 1e-3, (name, (a.float() - c).abs().mean().item(), scale)
+
+
+def test_gated_mlp_training_step(device):
+    """RMSNorm -> SwiGLU MLP (gate, up, down projections), compiled for training on the mi355x target: the forward
+    graph calls the gated dense kernel once and the dense kernel once, loss and gradients follow eager."""
+
+    def mlp(x, nw, wg, wu, wd):
+        h = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + 1e-6) * nw
+        return x + F.linear(F.silu(F.linear(h, wg)) * F.linear(h, wu), wd)
+
+    torch.manual_seed(4)
+    bf = torch.bfloat16
+    mk = lambda *s, k=1.0: (torch.randn(*s, device=device) * k).to(bf).requires_grad_(True)  # noqa: E731
+    args = [mk(4, 128, 512), mk(512), mk(1024, 512, k=0.05), mk(1024, 512, k=0.05), mk(512, 1024, k=0.05)]
+    be = backend()
+    y0 = torch.compile(mlp, backend=be, dynamic=False)(*args)
+    loss0 = y0.float().pow(2).mean()
+    g0 = torch.autograd.grad(loss0, args)
+    fwd_ops = [str(n.target) for n in be.compiled_graphs[1].graph.nodes if n.op == "call_function"]
+    assert fwd_ops.count("xpu_ops.dense_glu.default") == 1 and fwd_ops.count("xpu_ops.dense.default") == 1, fwd_ops
+    assert not any("aten.mm" in t or "aten.addmm" in t for t in fwd_ops)
+    ref_args = [a.detach().float().requires_grad_(True) for a in args]
+    loss1 = mlp(*ref_args).pow(2).mean()
+    g1 = torch.autograd.grad(loss1, ref_args)
+    assert abs(loss0.item() - loss1.item()) <= 2e-2 * abs(loss1.item())
+    eag_args = [a.detach().clone().requires_grad_(True) for a in args]
+    g2 = torch.autograd.grad(mlp(*eag_args).float().pow(2).mean(), eag_args)
+    err = lambda a, c: (a.float() - c).abs().mean().item()  # noqa: E731
+    for a, c, e in zip(g0, g1, g2):
+        assert err(a, c) <= 2 * err(e, c) + 1e-2 * c.abs().mean().item(), (err(a, c), err(e, c), c.abs().mean().item())

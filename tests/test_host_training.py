@@ -167,6 +167,24 @@ def test_linear_is_decomposed_for_the_dense_pattern_in_pregrad(caplog):
     assert "Pattern.DecomposeLinear changed graph" in caplog.text and "Pattern.CustomDenseLayer changed graph" in caplog.text
 
 
+def test_gated_mlp_becomes_one_gated_dense_call_in_pregrad(caplog):
+    """silu(linear(x, Wg)) * linear(x, Wu) -> linear: the gate and up projections leave the pregrad stage as ONE
+    gated dense module (it has a backward formula), the down projection as a dense module."""
+
+    def mlp(x, wg, wu, wd):
+        return F.linear(F.silu(F.linear(x, wg)) * F.linear(x, wu), wd)
+
+    bf = torch.bfloat16
+    backend = XpuGraph(XpuGraphConfig(is_training=True, target=Target.mi355x, opt_level=OptLevel.level2, enable_cache=False))
+    args = [torch.randn(2, 8, 64).to(bf).requires_grad_(True), torch.randn(128, 64).to(bf).requires_grad_(True),
+            torch.randn(128, 64).to(bf).requires_grad_(True), torch.randn(64, 128).to(bf).requires_grad_(True)]
+    with need_xpu_graph_logs(), pytest.raises(NotImplementedError):
+        torch.compile(mlp, backend=backend)(*args)
+    pregrad = backend.compiled_graphs[-2]
+    assert [n.target for n in pregrad.graph.nodes if n.op == "call_module"] == ["mi355x_dense_glu", "custom_dense_layer_replacement"]
+    assert "Pattern.FusedDenseGLU changed graph" in caplog.text
+
+
 def test_backward_formulas_reach_ops_that_were_traced_before_registration():
     """An inference compile that traces xpu_ops::dense BEFORE any training backend exists must not hide the
     backward formula registered later: the joint graph then saves the dense operands for the backward pass (in a

@@ -11,11 +11,13 @@ a few microseconds of dispatch, which inference-only processes should not pay.
     silu_mul2(g, u)            y = silu(g) * u
     silu_mul(x)                y = silu(x[..., :d]) * x[..., d:]
     dense(x, W, trans, bias, residual, act)   y = act(x W(^T) + bias + residual)
+    dense_glu(x, Wg, Wu)       y = silu(x Wg^T) * (x Wu^T)
 
 The input gradient of the dense layer is itself a dense layer over the same weight read the other way, so it runs on
 the HIP kernel; the weight gradient needs a transposed left operand, which that kernel does not take, and is an Aten
 matmul.  For activations whose derivative cannot be told from the output (silu, gelu) the pre-activation is
-recomputed with one more dense call.
+recomputed with one more dense call.  The gated layer saves only its inputs: both projections are recomputed on the
+dense kernel, the two input-gradient products run as one chain (the second takes the first as its residual).
 """
 import torch
 
@@ -139,6 +141,27 @@ def _dense_backward(ctx, gy):
     return gx, gw, None, gb, gr, None
 
 
+def _dense_glu_setup(ctx, inputs, output):
+    ctx.save_for_backward(*inputs)
+
+
+def _dense_glu_backward(ctx, gy):
+    x, w_gate, w_up = ctx.saved_tensors
+    dense = torch.ops.xpu_ops.dense
+    gate = dense(x, w_gate, True, None, None, "none").float()
+    up = dense(x, w_up, True, None, None, "none").float()
+    gf = gy.float()
+    d_gate = (gf * up * _silu_grad(gate)).to(x.dtype)
+    d_up = (gf * torch.nn.functional.silu(gate)).to(x.dtype)
+    need = ctx.needs_input_grad
+    gx = None
+    if need[0]:
+        gx = dense(d_up, w_up, False, None, dense(d_gate, w_gate, False, None, None, "none"), "none")
+    gwg = d_gate.t() @ x if need[1] else None
+    gwu = d_up.t() @ x if need[2] else None
+    return gx, gwg, gwu
+
+
 def register():
     global _REGISTERED
     if _REGISTERED:
@@ -149,9 +172,10 @@ def register():
     reg("xpu_ops::silu_mul2", _silu_mul2_backward, setup_context=_silu_mul2_setup)
     reg("xpu_ops::silu_mul", _silu_mul_backward, setup_context=_silu_mul_setup)
     reg("xpu_ops::dense", _dense_backward, setup_context=_dense_setup)
+    reg("xpu_ops::dense_glu", _dense_glu_backward, setup_context=_dense_glu_setup)
     # An op that was traced before (an inference compile earlier in the process) has its dispatch decisions cached
     # on the Python side; a stale entry for the Autograd key would keep sending traces to the "no formula" fallback.
-    for name in ("rms_norm", "layer_norm", "silu_mul2", "silu_mul", "dense"):
+    for name in ("rms_norm", "layer_norm", "silu_mul2", "silu_mul", "dense", "dense_glu"):
         packet = getattr(torch.ops.xpu_ops, name)
         for overload in packet.overloads():
             getattr(packet, overload)._dispatch_cache.clear()

@@ -13,6 +13,7 @@ import torch
 from torch import fx, nn
 
 from .....config import OptLevel
+from .....fx_utils import FxStage
 from ...pattern import Pattern, PatternGroup
 from ...structure.dense import DENSE_NAME
 from ...utils.node_utils import VIEW_OPS, aten, is_call, same_shape
@@ -44,6 +45,7 @@ def _plain_dense(node):
 class FusedDenseGLU(Pattern):
     _opt_level = OptLevel.level2
     _pattern_group = PatternGroup.GROUP2
+    _support_stages = [FxStage.inference, FxStage.pregrad]  # dense_glu carries a backward formula
 
     def process(self, gm):
         from ..... import ops as _xops
