@@ -180,3 +180,29 @@ def test_gated_mlp_training_step(device):
     err = lambda a, c: (a.float() - c).abs().mean().item()  # noqa: E731
     for a, c, e in zip(g0, g1, g2):
         assert err(a, c) <= 2 * err(e, c) + 1e-2 * c.abs().mean().item(), (err(a, c), err(e, c), c.abs().mean().item())
+
+
+@pytest.mark.parametrize("table_grads", [False, True])
+def test_rotary_backward_formula(device, table_grads):
+    """The input gradient of xpu_ops.rope is the rotary kernel on a rewritten sine table (halves swapped, negated);
+    the table gradients are Aten sums.  Against autograd of the written-out formula in fp32; the sine table has
+    different halves so that the swap matters."""
+    import xpu_graph_amd.ops as xops
+
+    xops.enable_autograd()
+    torch.manual_seed(5)
+    B, H, S, D = 2, 4, 96, 64
+    bf = torch.bfloat16
+    x = torch.randn(B, S, H, D, device=device).to(bf).transpose(1, 2).requires_grad_(True)  # [B, H, S, D] view
+    cos = torch.randn(S, D, device=device).to(bf).requires_grad_(table_grads)
+    sin = torch.randn(S, D, device=device).to(bf).requires_grad_(table_grads)
+    dy = torch.randn(B, H, S, D, device=device).to(bf)
+    wrt = (x, cos, sin) if table_grads else (x,)
+    g = torch.autograd.grad((torch.ops.xpu_ops.rope(x, cos, sin),), wrt, (dy,))
+    fx, fc, fs = (t.detach().float().requires_grad_(True) for t in (x, cos, sin))
+    ref = fx * fc + torch.cat([-fx[..., D // 2:], fx[..., : D // 2]], dim=-1) * fs
+    gref = torch.autograd.grad((ref,), (fx, fc, fs) if table_grads else (fx,), (dy.float(),))
+    for name, a, c in zip("x cos sin".split(), g, gref):
+        scale = c.abs().mean().item()
+        assert a.shape == c.shape
+        assert (a.float() - c).abs().mean().item() <= 1e-2 * scale + 1e-3, (name, (a.float() - c).abs().mean().item(), scale)

@@ -185,6 +185,23 @@ def test_gated_mlp_becomes_one_gated_dense_call_in_pregrad(caplog):
     assert "Pattern.FusedDenseGLU changed graph" in caplog.text
 
 
+def test_rotary_embedding_is_one_module_in_pregrad(caplog):
+    """x * cos + rotate_half(x) * sin on a [B, H, S, D] tensor leaves the pregrad stage as the rotary module."""
+
+    def rot(x, cos, sin):
+        d = x.shape[-1] // 2
+        return (x * cos + torch.cat([-x[..., d:], x[..., :d]], dim=-1) * sin) * 2.0
+
+    bf = torch.bfloat16
+    backend = XpuGraph(XpuGraphConfig(is_training=True, target=Target.mi355x, opt_level=OptLevel.level2, enable_cache=False))
+    args = [torch.randn(2, 4, 16, 64).to(bf).requires_grad_(True), torch.randn(16, 64).to(bf), torch.randn(16, 64).to(bf)]
+    with need_xpu_graph_logs(), pytest.raises(NotImplementedError):
+        torch.compile(rot, backend=backend)(*args)
+    pregrad = backend.compiled_graphs[-2]
+    assert [n.target for n in pregrad.graph.nodes if n.op == "call_module"] == ["mi355x_rope"]
+    assert "Pattern.FusedRoPE changed graph" in caplog.text
+
+
 def test_backward_formulas_reach_ops_that_were_traced_before_registration():
     """An inference compile that traces xpu_ops::dense BEFORE any training backend exists must not hide the
     backward formula registered later: the joint graph then saves the dense operands for the backward pass (in a

@@ -12,6 +12,7 @@ a few microseconds of dispatch, which inference-only processes should not pay.
     silu_mul(x)                y = silu(x[..., :d]) * x[..., d:]
     dense(x, W, trans, bias, residual, act)   y = act(x W(^T) + bias + residual)
     dense_glu(x, Wg, Wu)       y = silu(x Wg^T) * (x Wu^T)
+    rope(x, cos, sin)          y = x * cos + rotate_half(x) * sin,  rotate_half(x) = cat(-x[D/2:], x[:D/2])
 
 The input gradient of the dense layer is itself a dense layer over the same weight read the other way, so it runs on
 the HIP kernel; the weight gradient needs a transposed left operand, which that kernel does not take, and is an Aten
@@ -162,6 +163,35 @@ def _dense_glu_backward(ctx, gy):
     return gx, gwg, gwu
 
 
+def _rotate_half(t):
+    d = t.shape[-1] // 2
+    return torch.cat([-t[..., d:], t[..., :d]], dim=-1)
+
+
+def _rope_setup(ctx, inputs, output):
+    ctx.save_for_backward(*inputs)
+
+
+def _rope_backward(ctx, gy):
+    # rotate_half is a signed permutation R with R^T = -R, so gx = gy * cos - R(gy * sin) = gy * cos + R(gy) * sin'
+    # with sin' = -swap_halves(sin): the rotary kernel itself, on a rewritten [S, D] sine table.
+    x, cos, sin = ctx.saved_tensors
+    need = ctx.needs_input_grad
+    gx = None
+    if need[0]:
+        d = sin.shape[-1] // 2
+        sin_t = -torch.cat([sin[..., d:], sin[..., :d]], dim=-1)
+        gx = torch.ops.xpu_ops.rope(gy, cos, sin_t)
+    gcos = gsin = None
+    if need[1] or need[2]:
+        gf, xf = gy.float(), x.float()
+        if need[1]:
+            gcos = (gf * xf).sum(dim=(0, 1)).reshape(cos.shape).to(cos.dtype)
+        if need[2]:
+            gsin = (gf * _rotate_half(xf)).sum(dim=(0, 1)).reshape(sin.shape).to(sin.dtype)
+    return gx, gcos, gsin
+
+
 def register():
     global _REGISTERED
     if _REGISTERED:
@@ -173,9 +203,10 @@ def register():
     reg("xpu_ops::silu_mul", _silu_mul_backward, setup_context=_silu_mul_setup)
     reg("xpu_ops::dense", _dense_backward, setup_context=_dense_setup)
     reg("xpu_ops::dense_glu", _dense_glu_backward, setup_context=_dense_glu_setup)
+    reg("xpu_ops::rope", _rope_backward, setup_context=_rope_setup)
     # An op that was traced before (an inference compile earlier in the process) has its dispatch decisions cached
     # on the Python side; a stale entry for the Autograd key would keep sending traces to the "no formula" fallback.
-    for name in ("rms_norm", "layer_norm", "silu_mul2", "silu_mul", "dense", "dense_glu"):
+    for name in ("rms_norm", "layer_norm", "silu_mul2", "silu_mul", "dense", "dense_glu", "rope"):
         packet = getattr(torch.ops.xpu_ops, name)
         for overload in packet.overloads():
             getattr(packet, overload)._dispatch_cache.clear()

@@ -13,6 +13,7 @@ import torch
 from torch import fx, nn
 
 from .....config import OptLevel
+from .....fx_utils import FxStage
 from ...pattern import Pattern, PatternGroup
 from ...utils.node_utils import aten, cat_axis, is_call
 from .swiglu import _last_dim_slice
@@ -89,6 +90,7 @@ def match_rope(add):
 class FusedRoPE(Pattern):
     _opt_level = OptLevel.level2
     _pattern_group = PatternGroup.GROUP1
+    _support_stages = [FxStage.inference, FxStage.pregrad]  # rope carries a backward formula
 
     def process(self, gm):
         changed = False
