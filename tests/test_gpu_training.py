@@ -206,3 +206,63 @@ def test_rotary_backward_formula(device, table_grads):
         scale = c.abs().mean().item()
         assert a.shape == c.shape
         assert (a.float() - c).abs().mean().item() <= 1e-2 * scale + 1e-3, (name, (a.float() - c).abs().mean().item(), scale)
+
+
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("kv_heads", [4, 2])
+def test_attention_backward_formula(device, causal, kv_heads):
+    """Gradients of xpu_ops.sdpa (probabilities recomputed in fp32) against autograd of the written-out attention in
+    fp32, with as many or fewer key/value heads than query heads."""
+    import xpu_graph_amd.ops as xops
+
+    xops.enable_autograd()
+    torch.manual_seed(6)
+    B, H, Sq, Skv, D = 2, 4, 96, 96 if causal else 160, 64
+    bf = torch.bfloat16
+    q = torch.randn(B, H, Sq, D, device=device).to(bf).requires_grad_(True)
+    k = torch.randn(B, kv_heads, Skv, D, device=device).to(bf).requires_grad_(True)
+    v = torch.randn(B, kv_heads, Skv, D, device=device).to(bf).requires_grad_(True)
+    dy = torch.randn(B, H, Sq, D, device=device).to(bf)
+    scale = D**-0.5
+    y = torch.ops.xpu_ops.sdpa(q, k, v, causal, scale)
+    g = torch.autograd.grad((y,), (q, k, v), (dy,))
+    fq, fk, fv = (t.detach().float().requires_grad_(True) for t in (q, k, v))
+    rep = H // kv_heads
+    s = (fq @ fk.repeat_interleave(rep, 1).transpose(-1, -2)) * scale
+    if causal:
+        s = s.masked_fill(~torch.ones(Sq, Skv, dtype=torch.bool, device=device).tril(), float("-inf"))
+    ref = torch.softmax(s, -1) @ fv.repeat_interleave(rep, 1)
+    gref = torch.autograd.grad((ref,), (fq, fk, fv), (dy.float(),))
+    torch.testing.assert_close(y.float(), ref, rtol=1.6e-2, atol=2e-2)
+    for name, a, c in zip("q k v".split(), g, gref):
+        scale_ = c.abs().mean().item()
+        assert a.shape == c.shape
+        assert (a.float() - c).abs().mean().item() <= 1e-2 * scale_ + 1e-3, (name, (a.float() - c).abs().mean().item(), scale_)
+
+
+def test_attention_training_step(device):
+    """A causal self-attention layer (projections, rotary-free, F.scaled_dot_product_attention) compiled for training
+    on the mi355x target: the forward graph calls the attention and dense kernels, gradients follow eager."""
+
+    def layer(x, wqkv, wo):
+        B, S, E = x.shape
+        q, k, v = (t.view(B, S, 4, 64).transpose(1, 2) for t in F.linear(x, wqkv).split(E, dim=-1))
+        a = F.scaled_dot_product_attention(q, k, v, is_causal=True)
+        return F.linear(a.transpose(1, 2).reshape(B, S, E), wo)
+
+    torch.manual_seed(7)
+    bf = torch.bfloat16
+    mk = lambda *s, k=1.0: (torch.randn(*s, device=device) * k).to(bf).requires_grad_(True)  # noqa: E731
+    args = [mk(2, 128, 256), mk(768, 256, k=0.06), mk(256, 256, k=0.06)]
+    be = backend()
+    y0 = torch.compile(layer, backend=be, dynamic=False)(*args)
+    g0 = torch.autograd.grad(y0.float().pow(2).mean(), args)
+    fwd_ops = [str(n.target) for n in be.compiled_graphs[1].graph.nodes if n.op == "call_function"]
+    assert fwd_ops.count("xpu_ops.sdpa.default") == 1 and fwd_ops.count("xpu_ops.dense.default") == 2, fwd_ops
+    ref_args = [a.detach().float().requires_grad_(True) for a in args]
+    g1 = torch.autograd.grad(layer(*ref_args).pow(2).mean(), ref_args)
+    eag_args = [a.detach().clone().requires_grad_(True) for a in args]
+    g2 = torch.autograd.grad(layer(*eag_args).float().pow(2).mean(), eag_args)
+    err = lambda a, c: (a.float() - c).abs().mean().item()  # noqa: E731
+    for a, c, e in zip(g0, g1, g2):
+        assert err(a, c) <= 2 * err(e, c) + 1e-2 * c.abs().mean().item(), (err(a, c), err(e, c), c.abs().mean().item())

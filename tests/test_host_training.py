@@ -202,6 +202,24 @@ def test_rotary_embedding_is_one_module_in_pregrad(caplog):
     assert "Pattern.FusedRoPE changed graph" in caplog.text
 
 
+def test_causal_attention_is_one_module_in_pregrad(caplog):
+    """F.scaled_dot_product_attention(is_causal=True) on 16-bit [B, H, S, D] operands leaves the pregrad stage as
+    the attention module of the target (the op has a backward formula)."""
+
+    def attn(q, k, v):
+        return F.scaled_dot_product_attention(q, k, v, is_causal=True) * 2.0
+
+    bf = torch.bfloat16
+    backend = XpuGraph(XpuGraphConfig(is_training=True, target=Target.mi355x, opt_level=OptLevel.level2, enable_cache=False))
+    args = [torch.randn(2, 4, 32, 64).to(bf).requires_grad_(True) for _ in range(3)]
+    with need_xpu_graph_logs(), pytest.raises(NotImplementedError):
+        torch.compile(attn, backend=backend)(*args)
+    pregrad = backend.compiled_graphs[-2]
+    calls = [n for n in pregrad.graph.nodes if n.op == "call_module"]
+    assert [n.target for n in calls] == ["mi355x_sdpa"] and calls[0].args[3] is True
+    assert "Pattern.FusedCausalSDPA changed graph" in caplog.text
+
+
 def test_backward_formulas_reach_ops_that_were_traced_before_registration():
     """An inference compile that traces xpu_ops::dense BEFORE any training backend exists must not hide the
     backward formula registered later: the joint graph then saves the dense operands for the backward pass (in a

@@ -13,6 +13,7 @@ a few microseconds of dispatch, which inference-only processes should not pay.
     dense(x, W, trans, bias, residual, act)   y = act(x W(^T) + bias + residual)
     dense_glu(x, Wg, Wu)       y = silu(x Wg^T) * (x Wu^T)
     rope(x, cos, sin)          y = x * cos + rotate_half(x) * sin,  rotate_half(x) = cat(-x[D/2:], x[:D/2])
+    sdpa(q, k, v, causal, scale)   y = softmax(scale q k^T [+ causal mask]) v
 
 The input gradient of the dense layer is itself a dense layer over the same weight read the other way, so it runs on
 the HIP kernel; the weight gradient needs a transposed left operand, which that kernel does not take, and is an Aten
@@ -192,6 +193,37 @@ def _rope_backward(ctx, gy):
     return gx, gcos, gsin
 
 
+def _sdpa_setup(ctx, inputs, output):
+    q, k, v, ctx.causal, ctx.scale = inputs
+    ctx.save_for_backward(q, k, v)
+
+
+def _sdpa_backward(ctx, gy):
+    # The probabilities are recomputed in fp32 ([B, H, Sq, Skv] at once: a formula for training at moderate sequence
+    # lengths, not a flash backward).  With fewer key/value heads than query heads, query head h reads head h // rep.
+    q, k, v = ctx.saved_tensors
+    B, H, Sq, D = q.shape
+    Hkv, Skv = k.shape[1], k.shape[2]
+    rep = H // Hkv
+    qf, kf, vf, gf = q.float(), k.float(), v.float(), gy.float()
+    if rep > 1:
+        kf, vf = kf.repeat_interleave(rep, dim=1), vf.repeat_interleave(rep, dim=1)
+    s = (qf @ kf.transpose(-1, -2)) * ctx.scale
+    if ctx.causal:
+        visible = torch.ones(Sq, Skv, dtype=torch.bool, device=q.device).tril()
+        s = s.masked_fill(~visible, float("-inf"))
+    p = torch.softmax(s, dim=-1)
+    gv = p.transpose(-1, -2) @ gf
+    gp = gf @ vf.transpose(-1, -2)
+    gs = p * (gp - (gp * p).sum(-1, keepdim=True))
+    gq = (gs @ kf) * ctx.scale
+    gk = (gs.transpose(-1, -2) @ qf) * ctx.scale
+    if rep > 1:
+        gk = gk.reshape(B, Hkv, rep, Skv, D).sum(2)
+        gv = gv.reshape(B, Hkv, rep, Skv, D).sum(2)
+    return gq.to(q.dtype), gk.to(k.dtype), gv.to(v.dtype), None, None
+
+
 def register():
     global _REGISTERED
     if _REGISTERED:
@@ -204,9 +236,10 @@ def register():
     reg("xpu_ops::dense", _dense_backward, setup_context=_dense_setup)
     reg("xpu_ops::dense_glu", _dense_glu_backward, setup_context=_dense_glu_setup)
     reg("xpu_ops::rope", _rope_backward, setup_context=_rope_setup)
+    reg("xpu_ops::sdpa", _sdpa_backward, setup_context=_sdpa_setup)
     # An op that was traced before (an inference compile earlier in the process) has its dispatch decisions cached
     # on the Python side; a stale entry for the Autograd key would keep sending traces to the "no formula" fallback.
-    for name in ("rms_norm", "layer_norm", "silu_mul2", "silu_mul", "dense", "dense_glu", "rope"):
+    for name in ("rms_norm", "layer_norm", "silu_mul2", "silu_mul", "dense", "dense_glu", "rope", "sdpa"):
         packet = getattr(torch.ops.xpu_ops, name)
         for overload in packet.overloads():
             getattr(packet, overload)._dispatch_cache.clear()

@@ -18,7 +18,7 @@ import torch
 from torch import fx, nn
 
 from .....config import OptLevel
-from .....fx_utils import outside_fake_mode
+from .....fx_utils import FxStage, outside_fake_mode
 from ...pattern import Pattern, PatternGroup
 from ...utils.node_utils import VIEW_OPS, aten, is_call, is_getitem, same_shape
 
@@ -163,6 +163,7 @@ def _supported(q, k, v):
 class FusedCausalSDPA(Pattern):
     _opt_level = OptLevel.level2
     _pattern_group = PatternGroup.GROUP1
+    _support_stages = [FxStage.inference, FxStage.pregrad]  # sdpa carries a backward formula
 
     def _emit(self, gm, node, q, k, v, causal, scale, replace):
         if scale is None:
