@@ -266,3 +266,33 @@ def test_attention_training_step(device):
     err = lambda a, c: (a.float() - c).abs().mean().item()  # noqa: E731
     for a, c, e in zip(g0, g1, g2):
         assert err(a, c) <= 2 * err(e, c) + 1e-2 * c.abs().mean().item(), (err(a, c), err(e, c), c.abs().mean().item())
+
+
+def test_llama_block_training_step(device):
+    """The whole decoder block of benchmark config 5 (small batch and sequence), compiled for training on the mi355x
+    target: the forward graph runs on the HIP kernels, and the gradients of every weight follow fp32 autograd as
+    closely as eager bf16 does."""
+    from collections import Counter
+
+    from oracle import eager, inputs
+
+    torch.manual_seed(8)
+    x, p = inputs.c5_llama_block(B=2, S=128, device=device)
+    names = sorted(p)
+
+    def block(x, *w):
+        return eager.llama_block_eager(x, dict(zip(names, w)), n_heads=32)
+
+    args = [x.detach().requires_grad_(True)] + [p[n].detach().requires_grad_(True) for n in names]
+    be = backend()
+    y0 = torch.compile(block, backend=be, dynamic=False)(*args)
+    g0 = torch.autograd.grad(y0.float().pow(2).mean(), args)
+    ops = Counter(str(n.target) for n in be.compiled_graphs[1].graph.nodes if n.op == "call_function")
+    assert ops["xpu_ops.dense_glu.default"] == 1 and ops["xpu_ops.dense.default"] >= 5 and ops["xpu_ops.rope.default"] == 2, ops
+    ref_args = [a.detach().float().requires_grad_(True) for a in args]
+    g1 = torch.autograd.grad(block(*ref_args).pow(2).mean(), ref_args)
+    eag_args = [a.detach().clone().requires_grad_(True) for a in args]
+    g2 = torch.autograd.grad(block(*eag_args).float().pow(2).mean(), eag_args)
+    err = lambda a, c: (a.float() - c).abs().mean().item()  # noqa: E731
+    for name, a, c, e in zip(["x"] + names, g0, g1, g2):
+        assert err(a, c) <= 2 * err(e, c) + 2e-2 * c.abs().mean().item(), (name, err(a, c), err(e, c), c.abs().mean().item())
