@@ -289,6 +289,7 @@ def test_llama_block_training_step(device):
     g0 = torch.autograd.grad(y0.float().pow(2).mean(), args)
     ops = Counter(str(n.target) for n in be.compiled_graphs[1].graph.nodes if n.op == "call_function")
     assert ops["xpu_ops.dense_glu.default"] == 1 and ops["xpu_ops.dense.default"] >= 5 and ops["xpu_ops.rope.default"] == 2, ops
+    assert ops["xpu_ops.add_rms_norm.default"] == 1, ops  # the attention residual add rides in the second norm
     ref_args = [a.detach().float().requires_grad_(True) for a in args]
     g1 = torch.autograd.grad(block(*ref_args).pow(2).mean(), ref_args)
     eag_args = [a.detach().clone().requires_grad_(True) for a in args]
@@ -296,3 +297,40 @@ def test_llama_block_training_step(device):
     err = lambda a, c: (a.float() - c).abs().mean().item()  # noqa: E731
     for name, a, c, e in zip(["x"] + names, g0, g1, g2):
         assert err(a, c) <= 2 * err(e, c) + 2e-2 * c.abs().mean().item(), (name, err(a, c), err(e, c), c.abs().mean().item())
+
+
+@pytest.mark.parametrize("kind", ["rms", "layer"])
+@pytest.mark.parametrize("with_sum", [True, False])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_add_norm_backward_formulas(device, kind, with_sum, dtype):
+    """Gradients of the residual-add + norm ops (both addends, weight, bias; with the sum returned and used, or
+    not returned) against autograd of the written-out formula in fp32."""
+    import xpu_graph_amd.ops as xops
+
+    xops.enable_autograd()
+    torch.manual_seed(9)
+    rows, cols = 96, 512
+    mk = lambda *s: torch.randn(*s, device=device).to(dtype).requires_grad_(True)  # noqa: E731
+    x, r, w, b = mk(rows, cols), mk(rows, cols), mk(cols), mk(cols)
+    dy, dh = torch.randn(rows, cols, device=device).to(dtype), torch.randn(rows, cols, device=device).to(dtype)
+    ops = torch.ops.xpu_ops
+    if kind == "rms":
+        out = ops.add_rms_norm(x, r, w, 1e-6) if with_sum else (ops.add_rms_norm_only(x, r, w, 1e-6),)
+        wrt = (x, r, w)
+    else:
+        out = ops.add_layer_norm(x, r, w, b, 1e-5) if with_sum else (ops.add_layer_norm_only(x, r, w, b, 1e-5),)
+        wrt = (x, r, w, b)
+    g = torch.autograd.grad(tuple(out), wrt, (dy, dh)[: len(out)])
+    fx, fr, fw, fb = (t.detach().float().requires_grad_(True) for t in (x, r, w, b))
+    h = fx + fr
+    if kind == "rms":
+        y = h * torch.rsqrt(h.pow(2).mean(-1, keepdim=True) + 1e-6) * fw
+        fwrt = (fx, fr, fw)
+    else:
+        y = F.layer_norm(h, (cols,), fw, fb, 1e-5)
+        fwrt = (fx, fr, fw, fb)
+    gref = torch.autograd.grad((y, h) if with_sum else (y,), fwrt, (dy.float(), dh.float())[: len(out)])
+    tol = 1e-4 if dtype == torch.float32 else 1.5e-2
+    for name, a, c in zip("x r w b".split(), g, gref):
+        scale = c.abs().mean().item()
+        assert (a.float() - c).abs().mean().item() <= tol * scale + 1e-6, (name, (a.float() - c).abs().mean().item(), scale)

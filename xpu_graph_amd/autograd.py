@@ -14,6 +14,8 @@ a few microseconds of dispatch, which inference-only processes should not pay.
     dense_glu(x, Wg, Wu)       y = silu(x Wg^T) * (x Wu^T)
     rope(x, cos, sin)          y = x * cos + rotate_half(x) * sin,  rotate_half(x) = cat(-x[D/2:], x[:D/2])
     sdpa(q, k, v, causal, scale)   y = softmax(scale q k^T [+ causal mask]) v
+    add_rms_norm(x, r, w, eps) / add_layer_norm(x, r, w, b, eps)   h = x + r, y = norm(h); returns (y, h)
+    add_rms_norm_only / add_layer_norm_only                         the same, returning y alone
 
 The input gradient of the dense layer is itself a dense layer over the same weight read the other way, so it runs on
 the HIP kernel; the weight gradient needs a transposed left operand, which that kernel does not take, and is an Aten
@@ -224,6 +226,44 @@ def _sdpa_backward(ctx, gy):
     return gq.to(q.dtype), gk.to(k.dtype), gv.to(v.dtype), None, None
 
 
+def _add_norm_formulas(layer, with_sum):
+    """(setup, backward) of the residual-add + norm ops: the sum is recomputed, its gradient is the norm's input
+    gradient plus whatever flows into the returned sum, and both addends receive it."""
+
+    def setup(ctx, inputs, output):
+        x, res, w = inputs[:3]
+        b = inputs[3] if layer else None
+        ctx.eps = inputs[-1]
+        ctx.save_for_backward(*(t for t in (x, res, w) if t is not None))
+        ctx.has_w = w is not None
+        ctx.b_meta = (b.shape, b.dtype) if b is not None else None
+
+    def backward(ctx, gy, gh=None):
+        saved = ctx.saved_tensors
+        x, res = saved[0], saved[1]
+        w = saved[2] if ctx.has_w else None
+        need = ctx.needs_input_grad
+        hf, gf = x.float() + res.float(), gy.float()
+        hc = hf - hf.mean(-1, keepdim=True) if layer else hf
+        r = torch.rsqrt(hc.pow(2).mean(-1, keepdim=True) + ctx.eps)
+        hhat = hc * r
+        ghat = gf * w.float() if w is not None else gf
+        g_sum = ghat - hhat * (ghat * hhat).mean(-1, keepdim=True)
+        if layer:
+            g_sum = g_sum - ghat.mean(-1, keepdim=True)
+        g_sum = r * g_sum
+        if gh is not None:
+            g_sum = g_sum + gh.float()
+        g_sum = g_sum.to(x.dtype)
+        gw = _reduce_to(gf * hhat, w.shape).to(w.dtype) if w is not None and need[2] else None
+        if layer:
+            gb = _reduce_to(gf, ctx.b_meta[0]).to(ctx.b_meta[1]) if ctx.b_meta is not None and need[3] else None
+            return g_sum, g_sum, gw, gb, None
+        return g_sum, g_sum, gw, None
+
+    return setup, backward
+
+
 def register():
     global _REGISTERED
     if _REGISTERED:
@@ -237,9 +277,14 @@ def register():
     reg("xpu_ops::dense_glu", _dense_glu_backward, setup_context=_dense_glu_setup)
     reg("xpu_ops::rope", _rope_backward, setup_context=_rope_setup)
     reg("xpu_ops::sdpa", _sdpa_backward, setup_context=_sdpa_setup)
+    for op, layer, with_sum in (("add_rms_norm", False, True), ("add_rms_norm_only", False, False),
+                                ("add_layer_norm", True, True), ("add_layer_norm_only", True, False)):
+        setup, backward = _add_norm_formulas(layer, with_sum)
+        reg(f"xpu_ops::{op}", backward, setup_context=setup)
     # An op that was traced before (an inference compile earlier in the process) has its dispatch decisions cached
     # on the Python side; a stale entry for the Autograd key would keep sending traces to the "no formula" fallback.
-    for name in ("rms_norm", "layer_norm", "silu_mul2", "silu_mul", "dense", "dense_glu", "rope", "sdpa"):
+    for name in ("rms_norm", "layer_norm", "silu_mul2", "silu_mul", "dense", "dense_glu", "rope", "sdpa",
+                 "add_rms_norm", "add_rms_norm_only", "add_layer_norm", "add_layer_norm_only"):
         packet = getattr(torch.ops.xpu_ops, name)
         for overload in packet.overloads():
             getattr(packet, overload)._dispatch_cache.clear()

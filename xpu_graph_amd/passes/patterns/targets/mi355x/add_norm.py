@@ -17,6 +17,7 @@ import torch
 from torch import fx, nn
 
 from .....config import OptLevel
+from .....fx_utils import FxStage
 from ...pattern import Pattern
 from ...utils.node_utils import aten, hoist_users_after, is_call, norm_module_kind, same_shape
 
@@ -96,6 +97,7 @@ def _rewrite(gm, kind):
 
 class FusedAddLayerNorm(Pattern):
     _opt_level = OptLevel.level2
+    _support_stages = [FxStage.inference, FxStage.pregrad]  # the fused ops carry backward formulas
 
     def process(self, gm):
         return _rewrite(gm, "layer_norm")
@@ -103,6 +105,7 @@ class FusedAddLayerNorm(Pattern):
 
 class FusedAddRMSNorm(Pattern):
     _opt_level = OptLevel.level2
+    _support_stages = [FxStage.inference, FxStage.pregrad]  # the fused ops carry backward formulas
 
     def process(self, gm):
         return _rewrite(gm, "rms_norm")
