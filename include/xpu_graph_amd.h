@@ -95,6 +95,17 @@ int xg_add_layer_norm(const void* x, const void* res, const void* w, const void*
  * min(chunk_bytes, 4) for the source side and of chunk_bytes for the output
  * side.  n_outs <= XG_SLICE_CAT_MAX_OUTS.
  *
+ * The table is device memory, so xg_slice_cat cannot look at it without a
+ * synchronisation: an entry outside a row is an out-of-bounds access, not an
+ * error code.  xg_slice_cat_check_table() validates a HOST copy of the table
+ * once, when it is built: every chunk must lie inside the first
+ * `src_row_valid_bytes` bytes of a source row and inside the first
+ * `out_row_valid_bytes[out_id]` bytes of a row of its output, with the
+ * alignment stated above; it launches nothing.  The reference builds its index
+ * tensor from the matched slice list at module construction
+ * (FuseSliceCatSameInputModule_v2.__init__, structure_replacements/__init__.py:66-95)
+ * and has no such check.
+ *
  * replaces torch_mlu_triton::fused_slice_cat
  *   (passes/patterns/targets/mlu/triton_kernel/fused_slice_cat.py:10-73; one
  *   output) and torch_mlu_triton::fused_slice_low_v2
@@ -110,6 +121,8 @@ typedef struct {
 int xg_slice_cat(const void* src, int64_t src_row_bytes, int64_t rows, void* const* outs,
                  const int64_t* out_row_bytes, int n_outs, const xg_chunk* table_dev, int64_t n_chunks,
                  int chunk_bytes, xg_stream_t stream);
+int xg_slice_cat_check_table(const xg_chunk* table_host, int64_t n_chunks, int chunk_bytes, int64_t src_row_valid_bytes,
+                             const int64_t* out_row_valid_bytes, int n_outs);
 
 /* ---------------------------------------------------------------------------
  * add-N: out = ((t0 + t1) + t2) + ... strictly left to right, fp32 accumulate,
@@ -182,6 +195,15 @@ int xg_dense_glu(const void* a, const void* w_gate, const void* w_up, void* out,
  * replaces torch_mlu_ops.matmul as called by DenseLayerModule.forward
  *   (passes/patterns/targets/mlu/structure_replacements/dense_layer_modules.py:4-56).
  *
+ * xg_dense_batched: `batch` independent layers in ONE launch (batch entry on
+ *   the second grid axis, same tiles and kernels as xg_dense).  Entry z reads
+ *   a + z*stride_a, b + z*stride_b, bias + z*stride_bias (0: one bias for all),
+ *   residual + z*stride_res and writes out + z*stride_out, all strides in
+ *   elements and multiples of 8; each entry's out is [M,N] contiguous.
+ *   batch <= 65535.
+ * replaces torch_mlu_ops.batch_matmul as called by BatchDenseLayerModule.forward
+ *   (passes/patterns/targets/mlu/structure_replacements/dense_layer_modules.py:71-111).
+ *
  * xg_dense_fp8: a_q [M,K] and b_q ([K,N] or [N,K], as above) are OCP e4m3fn
  *   bytes; out = act((a_q @ b_q) * a_scale * b_scale[n] + bias) in `out_dtype`
  *   (XG_BF16 / XG_F16 / XG_F32).  b_scale is f32[N], bias f32-or-out_dtype.
@@ -190,6 +212,10 @@ int xg_dense_glu(const void* a, const void* w_gate, const void* w_up, void* out,
 int xg_dense(const void* a, const void* b, const void* bias, const void* residual, void* out, int64_t M,
              int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldr, int b_trans, int act, int dtype,
              int bias_dtype, xg_stream_t stream);
+int xg_dense_batched(const void* a, const void* b, const void* bias, const void* residual, void* out, int64_t batch,
+                     int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldr, int64_t stride_a,
+                     int64_t stride_b, int64_t stride_bias, int64_t stride_res, int64_t stride_out, int b_trans,
+                     int act, int dtype, int bias_dtype, xg_stream_t stream);
 int xg_dense_fp8(const void* a_q, const void* b_q, const float* a_scale_dev, const float* b_scale_dev,
                  const void* bias, void* out, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
                  int b_trans, int act, int out_dtype, int bias_dtype, xg_stream_t stream);

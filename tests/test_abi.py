@@ -19,7 +19,7 @@ def declared_symbols():
 def test_header_declares_the_expected_entry_points():
     syms = declared_symbols()
     for s in ("xg_rms_norm", "xg_layer_norm", "xg_add_rms_norm", "xg_add_layer_norm", "xg_slice_cat", "xg_addn",
-              "xg_combo_sum", "xg_slice_sum_cat", "xg_silu_mul", "xg_silu_mul2", "xg_dense", "xg_dense_glu", "xg_dense_fp8", "xg_sdpa", "xg_rope", "xg_copy_bytes",
+              "xg_combo_sum", "xg_slice_sum_cat", "xg_silu_mul", "xg_silu_mul2", "xg_dense", "xg_dense_batched", "xg_dense_glu", "xg_dense_fp8", "xg_slice_cat_check_table", "xg_sdpa", "xg_rope", "xg_copy_bytes",
               "xg_version", "xg_status_string"):
         assert s in syms
 
@@ -65,6 +65,65 @@ def test_argument_validation_needs_no_gpu():
     assert lib.xg_slice_sum_cat(p, p, 2, 4, 8, 32, 8, i32(0, 0, 0), i32(1, 2, 3), 3, 9, None) == -1  # unknown dtype
     assert lib.xg_slice_sum_cat(p, p, 0, 4, 8, 32, 8, i32(0, 0, 0), i32(1, 2, 3), 3, 0, None) == 0  # empty batch
     assert lib.xg_silu_mul(p, p, 2, 8, 8, 0, None) == -2  # row stride < 2*d
+
+
+def test_slice_table_is_refused_on_the_host_without_a_launch():
+    """xg_slice_cat cannot look at its device-side table; xg_slice_cat_check_table refuses a bad HOST copy when the
+    table is built: offsets outside the source row / the output row, an unknown output, a misaligned entry."""
+    from xpu_graph_amd import _lib
+
+    lib = _lib.lib()
+    i64 = ctypes.c_int64
+
+    def check(entries, chunk=16, src_valid=256, out_valid=(64,)):
+        arr = (_lib.XgChunk * len(entries))(*[_lib.XgChunk(*e, 0) for e in entries])
+        valid = (i64 * len(out_valid))(*out_valid)
+        return lib.xg_slice_cat_check_table(ctypes.cast(arr, ctypes.c_void_p), len(entries), chunk, src_valid, valid, len(out_valid))
+
+    assert check([(0, 0, 0), (240, 48, 0)]) == 0
+    assert check([(244, 0, 0)]) == -2  # reads past the source row
+    assert check([(0, 52, 0)]) == -2  # writes past the output row
+    assert check([(0, 0, 1)]) == -2  # no such output
+    assert check([(-4, 0, 0)]) == -2
+    assert check([(2, 0, 0)]) == -3  # source offsets need 4-byte alignment for 16-byte chunks
+    assert check([(0, 8, 0)]) == -3  # output offsets are whole chunks
+    assert check([(0, 0, 0)], chunk=3) == -7
+    assert check([], chunk=16) == 0
+    assert lib.xg_slice_cat_check_table(None, 1, 16, 256, (i64 * 1)(64), 1) == -4
+
+
+def test_build_slice_table_runs_the_host_check():
+    import torch  # noqa: F401
+
+    from xpu_graph_amd import ops
+
+    table, chunk, out_cols = ops.build_slice_table([[(3, 35), (100, 132)]], 8192, 4, 8192)
+    assert chunk == 16 and out_cols == [64] and table.shape == (16, 4)
+    with pytest.raises(ValueError):
+        ops.build_slice_table([[(8190, 8200)]], 8192, 4, 8192)
+
+
+def test_batched_dense_validation_needs_no_gpu():
+    from xpu_graph_amd import _lib
+
+    lib = _lib.lib()
+    buf = ctypes.create_string_buffer(1 << 16)
+    p = ctypes.c_void_p((ctypes.addressof(buf) + 15) & ~15)
+    ok = dict(batch=2, M=16, N=16, K=16, lda=16, ldb=16, ldr=0, sa=256, sb=256, sbias=0, sres=0, sout=256)
+
+    def call(**kw):
+        a = {**ok, **kw}
+        return lib.xg_dense_batched(p, p, None, None, p, a["batch"], a["M"], a["N"], a["K"], a["lda"], a["ldb"], a["ldr"], a["sa"], a["sb"],
+                                    a["sbias"], a["sres"], a["sout"], 0, 0, 2, 2, None)
+
+    assert call(batch=0) == 0  # nothing to launch
+    assert call(M=0) == 0
+    assert call(batch=-1) == -2
+    assert call(sout=255) == -2  # entries of the output would overlap
+    assert call(sa=260) == -3  # an entry would start off a 16-byte boundary
+    assert call(batch=70000) == -5
+    assert call(K=12) == -3
+    assert lib.xg_dense_batched(None, p, None, None, p, 2, 16, 16, 16, 16, 16, 0, 256, 256, 0, 0, 256, 0, 0, 2, 2, None) == -4
 
 
 def test_a_missing_library_is_an_error_not_a_fallback(monkeypatch, tmp_path):

@@ -1,13 +1,15 @@
 """GPU parity of the MFMA dense layer (torch.ops.xpu_ops.dense -> xg_dense)
 against the eager oracle: bf16 / fp16, weight as [K, N] and as [N, K],
-bias / residual / activation variants, ragged edges.  Tolerance rtol 1.6e-2
-against the fp32-computed reference of the same bf16 inputs (atol scaled to the
-accumulation length)."""
+bias / residual / activation variants, ragged edges.  Anchor: the layer evaluated
+in fp32 on the same 16-bit inputs; rtol 1.6e-2 with the floor of one output ulp
+at max|y| * 2^-7 (tests/tolerance.py).  Comparisons with the unfused 16-bit
+eager graph, which rounds after every op, are a second, looser check and say so."""
 import pytest
 import torch
 import torch.nn.functional as F
 
 from oracle import eager, inputs
+from tests.tolerance import assert_close_16bit, dense_floor
 
 pytestmark = pytest.mark.gpu
 
@@ -28,7 +30,16 @@ def ref32(x, W, weight_trans, bias, residual, act):
 
 
 def close(got, want, k):
-    torch.testing.assert_close(got.float(), want, rtol=1.6e-2, atol=2e-3 * max(1.0, (k / 64) ** 0.5))
+    """Against the fp32 anchor `want` (k, the accumulation length, only labels the record)."""
+    assert_close_16bit(got, want, dense_floor(want, got.dtype), f"dense K={k} {tuple(got.shape)} {got.dtype}")
+
+
+def close_to_eager_16bit(got, want16):
+    """Second, looser check against the UNFUSED 16-bit eager graph, which rounds the matmul, the bias add and the
+    activation separately (up to three half-ulps of values of the size of the pre-activation): rtol 1.6e-2 plus two
+    ulps of the output type at the largest value."""
+    spacing = 2.0 ** (-7 if got.dtype == torch.bfloat16 else -10)
+    torch.testing.assert_close(got.float(), want16.float(), rtol=1.6e-2, atol=2 * spacing * want16.float().abs().max().item())
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
@@ -104,7 +115,7 @@ def test_dense_c4_full_size(device):
     x, W, b = inputs.c4_dense(device=device)
     got = _ops().dense(x, W, False, b, None, "silu")
     want = eager.dense_silu_eager(x, W, b)  # the unfused bf16 graph on the same device
-    torch.testing.assert_close(got, want, rtol=1.6e-2, atol=2e-2)
+    close_to_eager_16bit(got, want)
     rows = torch.tensor([0, 1, 4095, 8191], device=device)
     close(got[rows], ref32(x[rows], W, False, b, None, "silu"), 4096)
     Wt = W.t().contiguous()
@@ -149,9 +160,76 @@ def test_dense_rejects_what_the_kernel_cannot_take(device):
     assert _ops().dense(torch.empty(0, 16, device=device).bfloat16(), torch.randn(16, 8, device=device).bfloat16(), False, None, None, "none").shape == (0, 8)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("weight_trans", [False, True])
+@pytest.mark.parametrize("B,M,K,N", [(5, 32, 256, 256), (3, 300, 128, 520), (16, 64, 64, 72), (2, 1024, 512, 4096)])
+def test_dense_batched_is_one_launch_equal_to_the_per_entry_path(device, dtype, weight_trans, B, M, K, N):
+    """xg_dense_batched (batch on the second grid axis) against B separate xg_dense calls, bit for bit, and against the
+    fp32 anchor; shared and per-entry bias, residual, activation.  The first shape is the reference's
+    (tests/mlu/test_custom_batchdenselayer.py: batch 5, 32 x 256 outputs viewed as [5, 32, 256])."""
+    g = torch.Generator().manual_seed(B * 1000 + M + N)
+    x = torch.randn(B, M, K, generator=g).to(dtype).to(device)
+    w = (torch.randn(B, N, K, generator=g) / K**0.5).to(dtype).to(device)
+    if not weight_trans:
+        w = w.transpose(1, 2).contiguous()
+    bias1 = torch.randn(N, generator=g).to(dtype).to(device)
+    biasb = torch.randn(B, N, generator=g).to(dtype).to(device)
+    res = torch.randn(B, M, N, generator=g).to(dtype).to(device)
+    ops = _ops()
+    for bias, residual, act in [(None, None, "none"), (bias1, None, "silu"), (biasb, res, "gelu"), (biasb.float(), None, "relu")]:
+        got = ops.dense_batched(x, w, weight_trans, bias, residual, act)
+        assert got.shape == (B, M, N) and got.dtype == dtype
+        for i in range(B):
+            bi = None if bias is None else (bias if bias.dim() == 1 else bias[i])
+            ri = None if residual is None else residual[i]
+            one = ops.dense(x[i], w[i], weight_trans, bi, ri, act)
+            assert torch.equal(got[i], one), (i, act)
+            close(got[i], ref32(x[i], w[i], weight_trans, bi, ri, act), K)
+
+
+def test_dense_batched_strided_entries(device):
+    """Batch entries that are views: a batch stride larger than an entry, rows wider than K; a misaligned view is copied."""
+    ops = _ops()
+    big = torch.randn(4, 40, 320, device=device).bfloat16()
+    x = big[:, :32, 64:320]  # [4, 32, 256], row stride 320, batch stride 40 * 320
+    w = (torch.randn(4, 256, 72, device=device) / 16).bfloat16()
+    got = ops.dense_batched(x, w, False, None, None, "none")
+    for i in range(4):
+        assert torch.equal(got[i], ops.dense(x[i].contiguous(), w[i], False, None, None, "none"))
+    odd = big[:, :32, 3:259]  # base 6 bytes off a 16-byte boundary: the wrapper copies
+    got = ops.dense_batched(odd, w, False, None, None, "none")
+    for i in range(4):
+        assert torch.equal(got[i], ops.dense(odd[i].contiguous(), w[i], False, None, None, "none"))
+
+
+def test_dense_takes_column_sliced_views(device):
+    """A linear layer fed by a column slice of a wider tensor: row strides or bases that are not multiples of 16 bytes
+    (what eager accepts anywhere) are copied by the wrapper instead of being refused by the kernel."""
+    ops = _ops()
+    big = torch.randn(128, 100, device=device).bfloat16()
+    w = (torch.randn(64, 72, device=device) / 8).bfloat16()
+    for x in (big[:, :64], big[:, 4:68], big[:, 3:67]):  # pitch 200 bytes; bases 0, 8 and 6 bytes in
+        got = ops.dense(x, w, False, None, None, "none")
+        close(got, ref32(x, w, False, None, None, "none"), 64)
+    wbig = (torch.randn(72, 100, device=device) / 8).bfloat16()
+    got = ops.dense(big[:, 4:68], wbig[:, 4:68], True, None, big[:, 20:92], "silu")  # strided weight and residual too
+    close(got, ref32(big[:, 4:68], wbig[:, 4:68], True, None, big[:, 20:92], "silu"), 64)
+    glu = ops.dense_glu(big[:, 4:68], wbig[:, 4:68], wbig[:, 30:94])
+    close_glu(glu, big[:, 4:68], wbig[:, 4:68], wbig[:, 30:94])
+
+
+def close_glu(got, x, wg, wu):
+    """The gated layer rounds each projection to the storage type before the gate (as the two separate layers it
+    replaces do), so its anchor is silu(round(x Wg^T)) * round(x Wu^T) with the products in fp32."""
+    gate = (x.float() @ wg.float().t()).to(got.dtype).float()
+    up = (x.float() @ wu.float().t()).to(got.dtype).float()
+    want = torch.nn.functional.silu(gate) * up
+    assert_close_16bit(got, want, dense_floor(want, got.dtype), f"dense_glu {tuple(got.shape)} {got.dtype}")
+
+
 @pytest.mark.parametrize("form", ["plain", "bias_act", "residual", "w_trans"])
 def test_batch_dense_compiled(device, form):
-    """bmm-based layers through torch.compile on the mi355x target: one launch per batch entry of the dense kernel."""
+    """bmm-based layers through torch.compile on the mi355x target: all batch entries in one xg_dense_batched launch."""
     from xpu_graph_amd import mi355x_compiler
 
     B, M, K, N = 5, 300, 256, 520
@@ -198,8 +276,7 @@ def test_dense_glu_bit_identical_to_the_unfused_ops(device, dtype, M, N, K):
     got = ops.dense_glu(x, wg, wu)
     two = ops.silu_mul2(ops.dense(x, wg, True, None, None, "none"), ops.dense(x, wu, True, None, None, "none"))
     assert torch.equal(got, two)
-    ref = torch.nn.functional.silu(x.float() @ wg.float().t()) * (x.float() @ wu.float().t())
-    torch.testing.assert_close(got.float(), ref, rtol=1.6e-2, atol=2e-2)
+    close_glu(got, x, wg, wu)
 
 
 @pytest.mark.parametrize("M,N,K", [(1024, 4096, 256), (900, 2056, 128)])
@@ -210,8 +287,7 @@ def test_dense_glu_half_height_grid(device, M, N, K):
     wg = (torch.randn(N, K, generator=g) / K**0.5).bfloat16().to(device)
     wu = (torch.randn(N, K, generator=g) / K**0.5).bfloat16().to(device)
     got = torch.ops.xpu_ops.dense_glu(x, wg, wu)
-    ref = torch.nn.functional.silu(x.float() @ wg.float().t()) * (x.float() @ wu.float().t())
-    torch.testing.assert_close(got.float(), ref, rtol=1.6e-2, atol=2e-2)
+    close_glu(got, x, wg, wu)
     xi = torch.randint(-2, 3, (M, K), generator=g).bfloat16().to(device)
     wi = torch.randint(-2, 3, (N, K), generator=g).bfloat16().to(device)
     gate = (xi.float() @ wi.float().t()).bfloat16().float()
@@ -225,8 +301,7 @@ def test_dense_glu_strided_operands_and_rejects(device):
     x = big[:, 128:384]  # row stride 512, K = 256
     wbig = (torch.randn(2, 40, 256, device=device) / 16).bfloat16()
     got = ops.dense_glu(x, wbig[0], wbig[1])
-    ref = torch.nn.functional.silu(x.float() @ wbig[0].float().t()) * (x.float() @ wbig[1].float().t())
-    torch.testing.assert_close(got.float(), ref, rtol=1.6e-2, atol=2e-2)
+    close_glu(got, x, wbig[0], wbig[1])
     with pytest.raises(ValueError):
         ops.dense_glu(x[:, :96], wbig[0][:, :96], wbig[1][:, :96])  # K not a multiple of 64
     with pytest.raises(ValueError):

@@ -2,7 +2,8 @@
 
 Reference: softmax(q k^T * scale + mask) v evaluated in fp32 on the SAME bf16 /
 fp16 inputs (the oracle's formula with no intermediate rounding), tolerance
-rtol 1.6e-2 with an absolute floor of one bf16 ulp of the value range; the
+rtol 1.6e-2 with the attention floor of tests/tolerance.py (2^-9 of the largest
+output for bf16: the probabilities are rounded to the storage type); the
 oracle itself (which rounds the scores and probabilities to the storage dtype,
 as the HF eager form does) is compared at the same tolerance.  Cases follow the
 reference's tests/common/test_fuse_sdpa.py:14-610: self and cross attention,
@@ -15,6 +16,7 @@ import pytest
 import torch
 
 from oracle import eager
+from tests.tolerance import assert_close_16bit, attention_floor
 
 pytestmark = pytest.mark.gpu
 
@@ -39,7 +41,7 @@ def ref32(q, k, v, causal, scale):
 
 
 def close(got, want):
-    torch.testing.assert_close(got.float(), want, rtol=1.6e-2, atol=8e-3)
+    assert_close_16bit(got, want, attention_floor(want, got.dtype), f"sdpa {tuple(got.shape)} {got.dtype}")
 
 
 def make(B, H, Hkv, Sq, Skv, D, dtype, device, seed=0):
@@ -60,6 +62,21 @@ def test_sdpa_shapes(device, dtype, D, causal, Sq, Skv):
     got = _ops().sdpa(q, k, v, causal, scale)
     assert got.shape == q.shape and got.dtype == dtype
     close(got, ref32(q, k, v, causal, scale))
+
+
+def test_sdpa_and_rope_take_misaligned_views(device):
+    """q / k / v cut out of a wider buffer at an offset that is not a multiple of 16 bytes (eager takes any view): the
+    wrapper copies what the kernels' 16-byte loads cannot read in place."""
+    big = torch.randn(2, 4, 96, 140, device=device).bfloat16()
+    q, k, v = big[..., 3:131], big[..., 4:132], big[..., 7:135]
+    scale = 1.0 / math.sqrt(128)
+    close(_ops().sdpa(q, k, v, True, scale), ref32(q, k, v, True, scale))
+    cos = torch.cos(torch.arange(96 * 128, device=device).reshape(96, 128) * 1e-3)
+    sin = torch.sin(torch.arange(96 * 128, device=device).reshape(96, 128) * 1e-3)
+    got = _ops().rope(q, cos, sin)
+    qf = q.float()
+    want = qf * cos + torch.cat([-qf[..., 64:], qf[..., :64]], -1) * sin
+    torch.testing.assert_close(got.float(), want, rtol=1.6e-2, atol=2.0**-7 * want.abs().max().item())
 
 
 def test_sdpa_matches_oracle_causal(device):

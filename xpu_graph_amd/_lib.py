@@ -50,6 +50,7 @@ _SIGNATURES = {
         c_int,
         [c_void_p, c_int64, c_int64, ctypes.POINTER(c_void_p), ctypes.POINTER(c_int64), c_int, c_void_p, c_int64, c_int, c_void_p],
     ),
+    "xg_slice_cat_check_table": (c_int, [c_void_p, c_int64, c_int, c_int64, ctypes.POINTER(c_int64), c_int]),
     "xg_addn": (c_int, [ctypes.POINTER(c_void_p), c_int, c_void_p, c_int64, c_int, c_void_p]),
     "xg_dense_glu": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64, c_int, c_void_p]),
     "xg_slice_sum_cat": (
@@ -75,6 +76,10 @@ _SIGNATURES = {
     "xg_dense": (
         c_int,
         [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int, c_int, c_int, c_int, c_void_p],
+    ),
+    "xg_dense_batched": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p] + [c_int64] * 12 + [c_int, c_int, c_int, c_int, c_void_p],
     ),
     "xg_dense_fp8": (
         c_int,

@@ -36,6 +36,39 @@ int xg_dense(const void* a, const void* b, const void* bias, const void* residua
   return dtype == XG_BF16 ? gemm::launch_bf16(p, b_trans != 0, st) : gemm::launch_f16(p, b_trans != 0, st);
 }
 
+int xg_dense_batched(const void* a, const void* b, const void* bias, const void* residual, void* out, int64_t batch,
+                     int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldr, int64_t stride_a,
+                     int64_t stride_b, int64_t stride_bias, int64_t stride_res, int64_t stride_out, int b_trans, int act,
+                     int dtype, int bias_dtype, xg_stream_t stream) {
+  using namespace xg;
+  using namespace xg::gemm;
+  if (a == nullptr || b == nullptr || out == nullptr) return XG_ERR_NULL_PTR;
+  if (batch < 0 || M < 0 || N <= 0 || K <= 0 || lda < K || (b_trans ? ldb < K : ldb < N) || (residual && ldr < N)) return XG_ERR_BAD_SHAPE;
+  if (stride_a < 0 || stride_b < 0 || stride_bias < 0 || stride_res < 0 || stride_out < M * N) return XG_ERR_BAD_SHAPE;
+  if (M > 0x7fffffff || N > 0x7fffffff || K > 0x7fffffff || batch > 65535) return XG_ERR_TOO_LARGE;
+  if (dtype != XG_BF16 && dtype != XG_F16) return XG_ERR_BAD_DTYPE;
+  if (bias && bias_dtype != dtype && bias_dtype != XG_F32) return XG_ERR_BAD_DTYPE;
+  if (act < XG_ACT_NONE || act > XG_ACT_SIGMOID) return XG_ERR_BAD_ARG;
+  if (K % 8 != 0 || N % 8 != 0 || lda % 8 != 0 || ldb % 8 != 0 || (residual && ldr % 8 != 0)) return XG_ERR_BAD_ALIGN;
+  // every entry's operands start on a 16-byte boundary
+  if (stride_a % 8 != 0 || stride_b % 8 != 0 || stride_out % 8 != 0 || (residual && stride_res % 8 != 0) ||
+      (bias && stride_bias % (bias_dtype == XG_F32 ? 4 : 8) != 0))
+    return XG_ERR_BAD_ALIGN;
+  if (!aligned_to(a, 16) || !aligned_to(b, 16) || !aligned_to(out, 16) || (bias && !aligned_to(bias, 16)) ||
+      (residual && !aligned_to(residual, 16)))
+    return XG_ERR_BAD_ALIGN;
+  if (M == 0 || batch == 0) return XG_OK;
+  GemmParams p = make_params(a, b, bias, residual, out, M, N, K, lda, ldb, ldr, act, bias && bias_dtype == XG_F32);
+  p.batch = (int)batch;
+  p.a_batch = stride_a * 2;
+  p.b_batch = stride_b * 2;
+  p.bias_batch = stride_bias * (bias && bias_dtype == XG_F32 ? 4 : 2);
+  p.res_batch = stride_res * 2;
+  p.out_batch = stride_out * 2;
+  hipStream_t st = (hipStream_t)stream;
+  return dtype == XG_BF16 ? gemm::launch_bf16(p, b_trans != 0, st) : gemm::launch_f16(p, b_trans != 0, st);
+}
+
 int xg_dense_glu(const void* a, const void* w_gate, const void* w_up, void* out, int64_t M, int64_t N, int64_t K,
                  int64_t lda, int64_t ldb, int dtype, xg_stream_t stream) {
   using namespace xg;

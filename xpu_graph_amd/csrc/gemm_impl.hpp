@@ -98,7 +98,25 @@ struct GemmParams {
   int bias_f32;
   int tiles_m, tiles_n;
   int pf_dist;  // how many slabs ahead the L2 warm-up touches run
+  // Batched layer: grid.y entries, each a dense layer of its own on operands `*_batch` BYTES apart (0: shared by
+  // every entry).  Every kernel starts with for_batch_entry(), so tiles, heuristics and limits are per entry.
+  int batch;
+  int64_t a_batch, b_batch, bias_batch, res_batch, out_batch;
 };
+
+// The parameters of batch entry blockIdx.y.
+__device__ __forceinline__ GemmParams for_batch_entry(const GemmParams& p) {
+  GemmParams q = p;
+  if (p.batch > 1) {
+    const int64_t z = blockIdx.y;
+    q.A = reinterpret_cast<const char*>(p.A) + z * p.a_batch;
+    q.B = reinterpret_cast<const char*>(p.B) + z * p.b_batch;
+    if (p.bias) q.bias = reinterpret_cast<const char*>(p.bias) + z * p.bias_batch;
+    if (p.res) q.res = reinterpret_cast<const char*>(p.res) + z * p.res_batch;
+    q.out = reinterpret_cast<char*>(p.out) + z * p.out_batch;
+  }
+  return q;
+}
 
 // Compile-time loop: the body receives std::integral_constant indices, so every
 // accumulator access has a constant index and the accumulators stay in registers.
@@ -652,7 +670,7 @@ __device__ __forceinline__ void gemm_dma_tile(const GemmParams& p, int bid, int 
 template <typename T, typename OT, BLayout BL>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_dma_kernel(GemmParams p) {
   extern __shared__ __align__(16) char smem[];
-  gemm_dma_tile<T, OT, BL, 4>(p, blockIdx.x, gridDim.x, smem);
+  gemm_dma_tile<T, OT, BL, 4>(for_batch_entry(p), blockIdx.x, gridDim.x, smem);
 }
 
 // One launch for two tile grids: the first n_full workgroups compute the 256 x 256 tiles of `full`, the others the
@@ -663,9 +681,9 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
   extern __shared__ __align__(16) char smem[];
   const int bid = blockIdx.x;  // uniform
   if (bid < n_full) {
-    gemm_dma_tile<T, OT, BL, 4>(full, bid, n_full, smem);
+    gemm_dma_tile<T, OT, BL, 4>(for_batch_entry(full), bid, n_full, smem);
   } else {
-    gemm_dma_tile<T, OT, BL, 2>(rest, bid - n_full, (int)gridDim.x - n_full, smem);
+    gemm_dma_tile<T, OT, BL, 2>(for_batch_entry(rest), bid - n_full, (int)gridDim.x - n_full, smem);
   }
 }
 
@@ -673,7 +691,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
 template <typename T, typename OT, BLayout BL>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_dma_half_kernel(GemmParams p) {
   extern __shared__ __align__(16) char smem[];
-  gemm_dma_tile<T, OT, BL, 2>(p, blockIdx.x, gridDim.x, smem);
+  gemm_dma_tile<T, OT, BL, 2>(for_batch_entry(p), blockIdx.x, gridDim.x, smem);
 }
 
 // The gated layer: same launch shapes as above.
@@ -703,8 +721,9 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
 }
 
 template <typename T, typename OT, BLayout BL>
-__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_staged_kernel(GemmParams p) {
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_staged_kernel(GemmParams p_all) {
   extern __shared__ __align__(16) char smem[];
+  const GemmParams p = for_batch_entry(p_all);
   constexpr int EB = Elem<T>::BYTES;
   constexpr int KSTEPS = Elem<T>::KSTEPS;
   constexpr int SLAB_K = ROW_BYTES / EB;
@@ -827,8 +846,9 @@ static_assert(S_SMEM_BYTES >= 4 * S_TILE * S_TILE * 4, "the four partial tiles m
 // GLU (gated layer, K-contiguous weights): the 64 B rows of a tile are 32 rows of the gate weight (p.B) followed
 // by the same 32 rows of the up weight (p.B2); the output tile is 64 x 32 and p.tiles_n counts 32-column tiles.
 template <typename T, typename OT, BLayout BL, bool GLU = false>
-__global__ __launch_bounds__(kThreads) void gemm_small_kernel(GemmParams p) {
+__global__ __launch_bounds__(kThreads) void gemm_small_kernel(GemmParams p_all) {
   extern __shared__ __align__(16) char smem[];
+  const GemmParams p = for_batch_entry(p_all);
   constexpr int EB = Elem<T>::BYTES;
   constexpr bool F8 = EB == 1;
   static_assert(!F8 || (BL == BLayout::KMajor && !GLU), "fp8: K-contiguous weights, plain layer");
@@ -1029,7 +1049,7 @@ int launch_kernel(K kernel, const GemmParams& p, hipStream_t stream) {
   if (int st = set_smem_once(kernel)) return st;
   const int64_t tiles = (int64_t)p.tiles_m * p.tiles_n;
   if (tiles > 0x7fffffffLL) return XG_ERR_TOO_LARGE;
-  hipLaunchKernelGGL(kernel, dim3((unsigned)tiles), dim3(kThreads), SMEM_BYTES, stream, p);
+  hipLaunchKernelGGL(kernel, dim3((unsigned)tiles, (unsigned)p.batch), dim3(kThreads), SMEM_BYTES, stream, p);
   return status_from_hip(hipGetLastError());
 }
 
@@ -1038,8 +1058,7 @@ template <typename T>
 bool dma_ok(const GemmParams& p, BLayout bl) {
   constexpr int EB = Elem<T>::BYTES;
   constexpr int SLAB_K = ROW_BYTES / EB;
-  static const bool off = getenv("XG_GEMM_NO_DMA") != nullptr;
-  if (off || p.K % SLAB_K != 0) return false;
+  if (p.K % SLAB_K != 0) return false;
   const int64_t lim = 0x7fffffffLL;
   const int64_t a_bytes = ((int64_t)p.M * p.lda) * EB;
   const int64_t b_bytes = bl == BLayout::KMajor ? ((int64_t)p.N * p.ldb) * EB : ((int64_t)SLAB_K * p.ldb + p.N) * EB;
@@ -1062,7 +1081,6 @@ inline int cu_count() {
 // the work fill the machine once, for about 0.55 of a round.  Returns how many tile columns the
 // full-size tiles keep (tn: no split).
 inline int full_tile_columns(int tm, int tn) {
-  static const bool off = getenv("XG_GEMM_NO_SPLIT") != nullptr;
   const int cus = cu_count();
   int g = tm, c = cus;  // gcd
   while (c) {
@@ -1073,20 +1091,14 @@ inline int full_tile_columns(int tm, int tn) {
   const int col_step = cus / g;  // tile columns per whole number of rounds
   const int keep = tn / col_step * col_step;
   const int tail_tiles = tm * (tn - keep);
-  if (off || keep == 0 || keep == tn || 2 * tail_tiles > cus) return tn;
+  if (keep == 0 || keep == tn || 2 * tail_tiles > cus) return tn;
   return keep;
 }
 
 // Large tiles that would leave most compute units idle give way to the 64 x 64 kernel.  Measured crossover on
 // 256 compute units (N = K = 4096, us, 64 x 64 kernel / half-height tiles / full tiles): 64 tiles 54 / 58 / 83,
 // 80 tiles 71 / 62 / 86, 128 tiles 98 / 66 / 88.
-inline int small_tile_limit() {
-  static const int n = [] {
-    const char* e = getenv("XG_GEMM_SMALL_MAX");
-    return e ? atoi(e) : cu_count() / 4;
-  }();
-  return n;
-}
+inline int small_tile_limit() { return cu_count() / 4; }
 
 template <typename T, typename OT, BLayout BL, bool GLU = false>
 int launch_small(GemmParams p, hipStream_t stream) {
@@ -1097,28 +1109,30 @@ int launch_small(GemmParams p, hipStream_t stream) {
   p.tiles_n = (p.N + cols - 1) / cols;
   const int64_t tiles = (int64_t)p.tiles_m * p.tiles_n;
   if (tiles > 0x7fffffffLL) return XG_ERR_TOO_LARGE;
-  hipLaunchKernelGGL(kernel, dim3((unsigned)tiles), dim3(kThreads), S_SMEM_BYTES, stream, p);
+  hipLaunchKernelGGL(kernel, dim3((unsigned)tiles, (unsigned)p.batch), dim3(kThreads), S_SMEM_BYTES, stream, p);
   return status_from_hip(hipGetLastError());
 }
 
 // A half-height (128-row) tile takes 0.55 of a full tile's time for half of its work, so a grid of them pays when
 // the full-size grid leaves much of its last round empty (128 full tiles on 256 units: one round of 256 half tiles,
 // 0.55 instead of 1).  tn: tile columns; the tile rows follow from M.
-inline bool half_height_wins(int M, int tn) {
-  static const bool off = getenv("XG_GEMM_NO_HALF") != nullptr;
+inline bool half_height_wins(int M, int tn, int batch = 1) {
   const int64_t cus = cu_count();
-  const int64_t full = (int64_t)((M + BM - 1) / BM) * tn, half = (int64_t)((M + 127) / 128) * tn;
+  const int64_t full = (int64_t)((M + BM - 1) / BM) * tn * batch, half = (int64_t)((M + 127) / 128) * tn * batch;
   const double t_full = (double)((full + cus - 1) / cus), t_half = 0.55 * (double)((half + cus - 1) / cus);
-  return !off && t_half < 0.95 * t_full;
+  return t_half < 0.95 * t_full;
 }
 
 template <typename T, typename OT, BLayout BL>
 int launch_gemm(const GemmParams& p, hipStream_t stream) {
   if (!dma_ok<T>(p, BL)) return launch_kernel(gemm_staged_kernel<T, OT, BL>, p, stream);
+  // decided per batch entry: the 64 x 64 kernel splits K between its waves and so adds in another order than the
+  // large tiles; a layer must give the same bits whether it runs alone or as one entry of a batch
   if ((int64_t)p.tiles_m * p.tiles_n <= small_tile_limit()) return launch_small<T, OT, BL>(p, stream);
-  const int keep = full_tile_columns(p.tiles_m, p.tiles_n);
+  // the split of the last, partial round is worked out for one tile grid: batched layers run whole tiles
+  const int keep = p.batch > 1 ? p.tiles_n : full_tile_columns(p.tiles_m, p.tiles_n);
   if (keep == p.tiles_n) {
-    if (half_height_wins(p.M, p.tiles_n)) {
+    if (half_height_wins(p.M, p.tiles_n, p.batch)) {
       GemmParams h = p;
       h.tiles_m = (p.M + 127) / 128;
       return launch_kernel(gemm_dma_half_kernel<T, OT, BL>, h, stream);
@@ -1144,7 +1158,7 @@ int launch_gemm(const GemmParams& p, hipStream_t stream) {
   if (int st = set_smem_once(kernel)) return st;
   const int64_t n_full = (int64_t)full.tiles_m * full.tiles_n, n_rest = (int64_t)rest.tiles_m * rest.tiles_n;
   if (n_full + n_rest > 0x7fffffffLL) return XG_ERR_TOO_LARGE;
-  hipLaunchKernelGGL(kernel, dim3((unsigned)(n_full + n_rest)), dim3(kThreads), SMEM_BYTES, stream, full, rest, (int)n_full);
+  hipLaunchKernelGGL(kernel, dim3((unsigned)(n_full + n_rest), 1), dim3(kThreads), SMEM_BYTES, stream, full, rest, (int)n_full);
   return status_from_hip(hipGetLastError());
 }
 
@@ -1203,9 +1217,10 @@ inline GemmParams make_params(const void* a, const void* b, const void* bias, co
   p.act = act;
   p.bias_f32 = bias_f32 ? 1 : 0;
   p.tiles_m = (int)((M + BM - 1) / BM);
-  static const int pf_env = getenv("XG_GEMM_PF") ? atoi(getenv("XG_GEMM_PF")) : 2;
-  p.pf_dist = pf_env < 1 ? 1 : (pf_env > 16 ? 16 : pf_env);
+  p.pf_dist = 2;  // measured: distances 1 to 6 are within noise of each other on C4
   p.tiles_n = (int)((N + BN - 1) / BN);
+  p.batch = 1;
+  p.a_batch = p.b_batch = p.bias_batch = p.res_batch = p.out_batch = 0;
   return p;
 }
 

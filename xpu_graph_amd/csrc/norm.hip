@@ -190,14 +190,6 @@ struct NormArgs {
   hipStream_t stream;
 };
 
-int tuned_tpr() {
-  static int v = [] {
-    const char* s = getenv("XG_NORM_TPR");
-    return s ? atoi(s) : 0;
-  }();
-  return v;
-}
-
 template <typename T, typename WT, int TPR, int VPT, bool LAYER>
 int launch_vec(const NormArgs& a, int nvec) {
   constexpr int BLOCK = TPR > 256 ? TPR : 256;
@@ -229,11 +221,11 @@ int launch_typed(const NormArgs& a) {
                       (a.b == nullptr || aligned_to(a.b, 16)) && a.cols / VN <= 1024 * 8;
   if (vec_ok) {
     const int nvec = (int)(a.cols / VN);
-    int tpr = tuned_tpr();
-    if (tpr == 0) {
-      // Heuristic from measurement on MI355X: short rows stay inside one wavefront
-      // (no LDS, no barrier); from 256 vectors up a 256-thread row with few
-      // vectors per thread streams better than one wavefront with many.
+    // Heuristic from measurement on MI355X: short rows stay inside one wavefront
+    // (no LDS, no barrier); from 256 vectors up a 256-thread row with few
+    // vectors per thread streams better than one wavefront with many.
+    int tpr;
+    {
       if (nvec <= 16 * 2)
         tpr = 16;
       else if (nvec <= 64 * 4)

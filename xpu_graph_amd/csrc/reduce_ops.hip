@@ -75,11 +75,7 @@ int addn_launch(const AddnTable& tbl, int n, T* out, int64_t numel, hipStream_t 
     const int64_t blocks = (nvec + 255) / 256;
     if (blocks > 0x7fffffffLL) return XG_ERR_TOO_LARGE;
     // independent loads in flight per lane; measured on 32 x [4096,256] fp32: 4 -> 24.3 us, 8 -> 28.2, 16 -> 25.9, 31 -> 24.4
-    static int u = [] { const char* e = getenv("XG_ADDN_U"); return e ? atoi(e) : 4; }();
-    if (u == 4) hipLaunchKernelGGL((addn_kernel<T, VN, 4>), dim3((unsigned)blocks), dim3(256), 0, stream, tbl, n, out, nvec);
-    else if (u == 16) hipLaunchKernelGGL((addn_kernel<T, VN, 16>), dim3((unsigned)blocks), dim3(256), 0, stream, tbl, n, out, nvec);
-    else if (u == 31) hipLaunchKernelGGL((addn_kernel<T, VN, 31>), dim3((unsigned)blocks), dim3(256), 0, stream, tbl, n, out, nvec);
-    else hipLaunchKernelGGL((addn_kernel<T, VN, 8>), dim3((unsigned)blocks), dim3(256), 0, stream, tbl, n, out, nvec);
+    hipLaunchKernelGGL((addn_kernel<T, VN, 4>), dim3((unsigned)blocks), dim3(256), 0, stream, tbl, n, out, nvec);
     done = nvec * VN;
   }
   if (done < numel) {

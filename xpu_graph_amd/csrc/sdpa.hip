@@ -258,7 +258,14 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
       static_for<2>([&](auto TI) { static_for<16>([&](auto VI) { mx = fminf(mx, s[decltype(TI)::value][decltype(VI)::value]); }); });
     }
     float mt = mx * cc;
-    mt = fmaxf(mt, __shfl_xor(mt, 32, kWave));
+    {
+      // lanes l and l ^ 32 share a query: one swap of the two register halves hands both partial maxima to both
+      // lanes without a trip through the LDS crossbar.  Written as asm because the compiler folds the two results
+      // of the builtin into one when both inputs are the same value.
+      float lo = mt, hi = mt;
+      asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(lo), "+v"(hi));
+      mt = fmaxf(lo, hi);
+    }
     const float m_new = mt > m_run + kSlack ? mt : m_run;  // -inf + slack = -inf: the first visible key always moves it
     const float m_use = m_new == -INFINITY ? 0.f : m_new;  // a row with no visible key yet
     const float alpha = __builtin_amdgcn_exp2f(m_run - m_use);
@@ -400,7 +407,6 @@ extern "C" int xg_sdpa(const void* q, const void* k, const void* v, void* out, i
   // each XCD is faster (S2048 non-causal 290 vs 315 us, S8192 causal 558 vs 575 us); short causal problems want
   // the heaviest query blocks of all heads first (S2048 causal 176 vs 205 us).
   p.order = (!p.causal || n_qb >= 32) ? 1 : 0;
-  if (const char* e = getenv("XG_SDPA_ORDER")) p.order = atoi(e) == 1 ? 1 : 0;
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   if (dtype == XG_BF16) return D == 128 ? sdpa::launch<bf16_t, 128>(p, st) : sdpa::launch<bf16_t, 64>(p, st);
   return D == 128 ? sdpa::launch<f16_t, 128>(p, st) : sdpa::launch<f16_t, 64>(p, st);

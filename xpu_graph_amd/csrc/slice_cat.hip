@@ -97,25 +97,14 @@ __global__ __launch_bounds__(kBlock) void slice_cat_kernel(const char* __restric
   }
 }
 
-int tuned_rows_per_block() {
-  static int v = [] {
-    const char* s = getenv("XG_SLICE_ROWS_PER_BLOCK");
-    return s ? atoi(s) : 0;
-  }();
-  return v;
-}
-
 template <int CB>
 int launch(const char* src, int64_t src_row_bytes, int64_t rows, const OutTable& outs, int n_outs,
            const xg_chunk* table, int64_t n_chunks, hipStream_t stream) {
   const int64_t gx = (n_chunks + kBlock - 1) / kBlock;
   // Rows per block: enough blocks to cover the 256 CUs several times over, but a
   // strip long enough that each lane amortises its table entry.
-  int rpb = tuned_rows_per_block();
-  if (rpb <= 0) {
-    rpb = 8;
-    while (rpb < 64 && gx * ((rows + rpb - 1) / rpb) > 8192) rpb *= 2;
-  }
+  int rpb = 8;
+  while (rpb < 64 && gx * ((rows + rpb - 1) / rpb) > 8192) rpb *= 2;
   const int64_t gy = (rows + rpb - 1) / rpb;
   if (gx > 0x7fffffffLL || gy > 65535) return XG_ERR_TOO_LARGE;
   dim3 grid((unsigned)gx, (unsigned)gy);
@@ -130,6 +119,27 @@ int launch(const char* src, int64_t src_row_bytes, int64_t rows, const OutTable&
 
 }  // namespace
 }  // namespace xg
+
+extern "C" int xg_slice_cat_check_table(const xg_chunk* table_host, int64_t n_chunks, int chunk_bytes,
+                                        int64_t src_row_valid_bytes, const int64_t* out_row_valid_bytes, int n_outs) {
+  using namespace xg;
+  if (table_host == nullptr || out_row_valid_bytes == nullptr) return XG_ERR_NULL_PTR;
+  if (n_outs < 1 || n_outs > XG_SLICE_CAT_MAX_OUTS) return XG_ERR_TOO_LARGE;
+  if (n_chunks < 0 || src_row_valid_bytes < 0) return XG_ERR_BAD_SHAPE;
+  if (chunk_bytes != 1 && chunk_bytes != 2 && chunk_bytes != 4 && chunk_bytes != 8 && chunk_bytes != 16)
+    return XG_ERR_BAD_ARG;
+  const int src_align = chunk_bytes < 4 ? chunk_bytes : 4;
+  for (int i = 0; i < n_outs; ++i)
+    if (out_row_valid_bytes[i] < 0) return XG_ERR_BAD_SHAPE;
+  for (int64_t i = 0; i < n_chunks; ++i) {
+    const xg_chunk& c = table_host[i];
+    if (c.out_id < 0 || c.out_id >= n_outs) return XG_ERR_BAD_SHAPE;
+    if (c.src_off < 0 || (int64_t)c.src_off + chunk_bytes > src_row_valid_bytes) return XG_ERR_BAD_SHAPE;
+    if (c.dst_off < 0 || (int64_t)c.dst_off + chunk_bytes > out_row_valid_bytes[c.out_id]) return XG_ERR_BAD_SHAPE;
+    if (c.src_off % src_align != 0 || c.dst_off % chunk_bytes != 0) return XG_ERR_BAD_ALIGN;
+  }
+  return XG_OK;
+}
 
 extern "C" int xg_slice_cat(const void* src, int64_t src_row_bytes, int64_t rows, void* const* outs,
                             const int64_t* out_row_bytes, int n_outs, const xg_chunk* table_dev, int64_t n_chunks,

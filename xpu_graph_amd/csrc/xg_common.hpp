@@ -88,11 +88,6 @@ __device__ __forceinline__ void store_vec_nt(V* p, V v) {
 // the LDS crossbar.
 template <int WIDTH = kWave>
 __device__ __forceinline__ float wave_sum(float v) {
-#ifdef XG_PLAIN_SHUFFLE
-#pragma unroll
-  for (int off = WIDTH / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
-  return v;
-#else
   auto dpp = [](float x, auto CTRL) {
     constexpr int ctrl = decltype(CTRL)::value;
     return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), ctrl, 0xF, 0xF, true));
@@ -104,7 +99,6 @@ __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
   for (int off = 16; off < WIDTH; off <<= 1) v += __shfl_xor(v, off, kWave);
   return v;
-#endif
 }
 template <int WIDTH = kWave>
 __device__ __forceinline__ float wave_max(float v) {

@@ -439,6 +439,13 @@ def build_slice_table(slice_lists, src_cols, elem_size, src_row_stride=None):
             dst += nbytes
         out_cols.append(dst // elem_size)
     table = torch.tensor(rows_out, dtype=torch.int32).reshape(-1, 4)
+    if table.shape[0] and _lib.is_built():
+        # the kernel cannot look at its (device) table: refuse a bad one here, once, on the host
+        valid = (ctypes.c_int64 * len(out_cols))(*[c * elem_size for c in out_cols])
+        st = _lib.lib().xg_slice_cat_check_table(
+            ctypes.c_void_p(table.data_ptr()), table.shape[0], chunk, src_cols * elem_size, valid, len(out_cols)
+        )
+        _lib.check(st, "xg_slice_cat_check_table")
     return table, chunk, out_cols
 
 
@@ -464,8 +471,13 @@ def _dense_out_shape(x, weight, weight_trans):
 
 
 def _row_major(t):
-    """2-D tensor with unit last stride (copied only when it is not)."""
-    return t if t.stride(-1) == 1 and t.stride(0) >= t.shape[1] else t.contiguous()
+    """2-D tensor the kernels can read in place: unit last stride, a row stride that is a multiple of 16 bytes and a
+    16-byte aligned base.  Anything else (a column slice at an odd offset, a narrow view of a wider buffer whose
+    pitch is not a multiple of 16 bytes) is copied, as the reference's modules make such inputs contiguous
+    (dense_layer_modules.py:15-16)."""
+    per16 = 16 // t.element_size()
+    ok = t.stride(-1) == 1 and t.stride(0) >= t.shape[1] and t.stride(0) % per16 == 0 and t.data_ptr() % 16 == 0
+    return t if ok else t.contiguous()
 
 
 def _dense_into(x, weight, weight_trans, bias, residual, act, out):
@@ -515,19 +527,56 @@ def _dense_batched_shape(x, weight, weight_trans):
     return x.shape[0], x.shape[1], n
 
 
+def _batch_major(t):
+    """3-D tensor whose [rows, cols] entries the kernels can read in place (see _row_major) at a batch stride that
+    keeps every entry 16-byte aligned."""
+    per16 = 16 // t.element_size()
+    ok = (
+        t.stride(-1) == 1
+        and t.stride(1) >= t.shape[2]
+        and t.stride(1) % per16 == 0
+        and t.stride(0) % per16 == 0
+        and t.data_ptr() % 16 == 0
+    )
+    return t if ok else t.contiguous()
+
+
 def _dense_batched(x, weight, weight_trans, bias, residual, act):
-    """One dense launch per batch entry, on slices of the operands (no copies for contiguous batches).
+    """All batch entries in ONE xg_dense_batched launch (the batch index is the second grid axis of the dense kernels).
     bias: [N] shared or [B, N] per batch; residual: [B, M, N]."""
     b, m, n = _dense_batched_shape(x, weight, weight_trans)
+    k = x.shape[2]
+    if act not in _lib.ACT_CODES:
+        raise ValueError(f"dense_batched: unknown activation {act!r}")
+    if weight.dtype != x.dtype:
+        raise TypeError("dense_batched: x and weight must share a dtype")
     out = torch.empty((b, m, n), dtype=x.dtype, device=x.device)
     if bias is not None and bias.dim() == 2 and bias.shape[0] != b:
         raise ValueError("dense_batched: a 2-D bias must be [B, N]")
-    if residual is not None and tuple(residual.shape) != (b, m, n):
-        raise ValueError("dense_batched: residual must be [B, M, N]")
-    for i in range(b):
-        bi = None if bias is None else (bias if bias.dim() == 1 else bias[i])
-        ri = None if residual is None else residual[i]
-        _dense_into(x[i], weight[i], weight_trans, bi, ri, act, out[i])
+    if residual is not None and (tuple(residual.shape) != (b, m, n) or residual.dtype != x.dtype):
+        raise ValueError("dense_batched: residual must be [B, M, N] in the input dtype")
+    if out.numel() == 0:
+        return out
+    x, weight = _batch_major(x), _batch_major(weight)
+    bias_dt, bias_stride = _code(x.dtype), 0
+    if bias is not None:
+        if bias.shape[-1] != n:
+            raise ValueError("dense_batched: bias must have N elements per entry")
+        bias = bias.contiguous()
+        if bias.dtype != x.dtype:
+            bias = bias.float()
+        bias_dt = _code(bias.dtype)
+        bias_stride = n if bias.dim() == 2 else 0
+    ldr = res_stride = 0
+    if residual is not None:
+        residual = _batch_major(residual)
+        ldr, res_stride = residual.stride(1), residual.stride(0)
+    st = _lib.lib().xg_dense_batched(
+        _ptr(x), _ptr(weight), _ptr(bias), _ptr(residual), _ptr(out), b, m, n, k, x.stride(1), weight.stride(1), ldr,
+        x.stride(0), weight.stride(0), bias_stride, res_stride, m * n,
+        1 if weight_trans else 0, _lib.ACT_CODES[act], _code(x.dtype), bias_dt, _stream(),
+    )
+    _lib.check(st, "xg_dense_batched")
     return out
 
 
@@ -584,7 +633,11 @@ def _sdpa_check(q, k, v):
 
 
 def _unit_last(t):
-    return t if t.stride(-1) == 1 else t.contiguous()
+    """A tensor the attention / rotary kernels can read in place: unit last stride, every other stride a multiple of
+    16 bytes, 16-byte aligned base (their loads are 16 bytes per lane).  Anything else is copied."""
+    per16 = 16 // t.element_size()
+    ok = t.stride(-1) == 1 and all(st % per16 == 0 for st in t.stride()[:-1]) and t.data_ptr() % 16 == 0
+    return t if ok else t.contiguous()
 
 
 def _dense_strides_ok(t):
@@ -666,13 +719,21 @@ def _rope_meta(x, cos, sin):
     return _empty_like_layout(_unit_last(x))
 
 
+_GLU_OPERAND_LIMIT = 2**31 - 1
+
+
 def dense_glu_fits(x_shape, w_shape, dtype):
     """What the gated kernel takes: 2-D x [M, K], two [N, K] weights, K a multiple of 64, N of 8, 16-bit floats."""
     if len(x_shape) != 2 or len(w_shape) != 2 or dtype not in (torch.bfloat16, torch.float16):
         return False
-    k, n = x_shape[1], w_shape[0]
+    m, k, n = x_shape[0], x_shape[1], w_shape[0]
     ints = all(isinstance(d, int) for d in (k, *w_shape))  # the row count may be symbolic
-    return ints and w_shape[1] == k and k % 64 == 0 and n % 8 == 0 and k > 0 and n > 0
+    if not (ints and w_shape[1] == k and k % 64 == 0 and n % 8 == 0 and k > 0 and n > 0):
+        return False
+    # the gated kernel addresses each operand with a 31-bit byte offset and has no other variant: operands known to
+    # be 2 GiB or more stay two dense layers and a gate kernel (a symbolic row count is decided per call, see _dense_glu)
+    m_ok = not isinstance(m, int) or m * k * 2 < _GLU_OPERAND_LIMIT
+    return m_ok and n * k * 2 < _GLU_OPERAND_LIMIT
 
 
 def _dense_glu(x, w_gate, w_up):
@@ -686,6 +747,10 @@ def _dense_glu(x, w_gate, w_up):
         w_gate, w_up = w_gate.contiguous(), w_up.contiguous()
     m, k = x.shape
     n = w_gate.shape[0]
+    if m * x.stride(0) * 2 >= _GLU_OPERAND_LIMIT or n * w_gate.stride(0) * 2 >= _GLU_OPERAND_LIMIT:
+        # a row count that was symbolic at match time turned out too large for the gated kernel's 31-bit operand
+        # offsets: the same result, bit for bit, from two dense launches and the gate kernel
+        return _silu_mul2(_dense(x, w_gate, True, None, None, "none"), _dense(x, w_up, True, None, None, "none"))
     out = torch.empty((m, n), dtype=x.dtype, device=x.device)
     if out.numel() == 0:
         return out
