@@ -13,6 +13,13 @@ events on the launch stream.  `cpu_baseline` is the same eager function on the
 host cores (through this package's default, non-vendor compile path when it is
 available).  `configs` carries the same three figures for the other benchmark
 configurations.
+
+Every GPU figure is taken on warm clocks: before a timed region the same call
+runs for at least WARM_SECONDS (the first ~100 ms of work after an idle spell,
+e.g. after a CPU baseline, run visibly slower), then the --warmup launches,
+then the timed ones.  `roofline.traffic` is not measured by this run: it is
+read from profiles/traffic.json, which the rocprofv3 --pmc recipe printed in
+that file produces, and `roofline.traffic_source` names it.
 """
 import argparse
 import ctypes
@@ -28,6 +35,28 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
 BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 MFMA, published
 FP8_PEAK_TFLOPS = 5000.0
 N_SETS = 6  # rotating buffer sets so that timed launches stream from HBM, not from the 256 MB last-level cache
+WARM_SECONDS = 0.15  # GPU work of the same kind in front of every timed region
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "traffic.json")
+
+
+def _traffic_table():
+    try:
+        with open(TRAFFIC_FILE) as f:
+            return json.load(f)
+    except (OSError, ValueError):
+        return {}
+
+
+def _warm(torch, fn, n_sets):
+    """Run fn for WARM_SECONDS of wall clock so that the timed region starts on warm clocks."""
+    torch.cuda.synchronize()
+    t_end = time.perf_counter() + WARM_SECONDS
+    i = 0
+    while time.perf_counter() < t_end:
+        for _ in range(4):
+            fn(i % n_sets)
+            i += 1
+        torch.cuda.synchronize()
 
 
 def _p(t):
@@ -36,6 +65,7 @@ def _p(t):
 
 def _events_time(torch, fn, n_sets, steps, warmup):
     """Average seconds per call of fn(i) over `steps` back-to-back calls, by HIP events on the current stream."""
+    _warm(torch, fn, n_sets)
     for i in range(warmup):
         fn(i % n_sets)
     torch.cuda.synchronize()
@@ -49,6 +79,7 @@ def _events_time(torch, fn, n_sets, steps, warmup):
 
 
 def _wall_time(torch, fn, n_sets, steps, warmup):
+    _warm(torch, fn, n_sets)
     for i in range(warmup):
         fn(i % n_sets)
     torch.cuda.synchronize()
@@ -59,9 +90,9 @@ def _wall_time(torch, fn, n_sets, steps, warmup):
     return (time.perf_counter() - t0) / steps
 
 
-def _cpu_time(fn, min_iters=3, budget_s=12.0, max_iters=30):
-    fn()  # warm-up (also compiles the default path)
-    fn()
+def _cpu_time(fn, min_iters=3, budget_s=12.0, max_iters=30, warmups=2):
+    for _ in range(warmups):  # also compiles the default path
+        fn()
     times = []
     t_end = time.perf_counter() + budget_s
     while len(times) < min_iters or (time.perf_counter() < t_end and len(times) < max_iters):
@@ -113,8 +144,7 @@ class AddLayerNormC2(Workload):
     dtype = "bf16"
     kernel = "norm_rows_kernel<bf16,bf16,LAYER>"
     work = 4 * 8192 * 4096 * 2 + 2 * 4096 * 2
-    # HBM bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE, scaled by a 64 MiB copy (profiles/membound_fused_ops_bench.md)
-    traffic = 268.6e6
+    traffic_key = "c2_add_layernorm"
 
     def setup(self, torch, dev):
         from oracle import inputs
@@ -158,7 +188,7 @@ class RmsNormC1(Workload):
     dtype = "f32"
     kernel = "norm_rows_kernel<f32,f32,RMS>"
     work = 2 * 2048 * 4096 * 4 + 4096 * 4
-    traffic = 67.3e6
+    traffic_key = "c1_rmsnorm"
 
     def setup(self, torch, dev):
         from oracle import inputs
@@ -197,7 +227,7 @@ class SliceCatC3a(Workload):
     dtype = "b32"
     kernel = "slice_cat_kernel<16>"
     work = 2 * 4096 * 2048 * 4 + 64 * 8
-    traffic = 96.9e6  # unaligned 128-byte slices straddle two 128-byte lines on the read side
+    traffic_key = "c3a_slice_cat"
 
     def setup(self, torch, dev):
         from oracle import inputs
@@ -240,7 +270,7 @@ class AddNC3b(Workload):
     dtype = "f32"
     kernel = "addn_kernel<f32>"
     work = 33 * 4096 * 256 * 4
-    traffic = 138.4e6
+    traffic_key = "c3b_addn"
 
     def setup(self, torch, dev):
         from oracle import inputs
@@ -279,10 +309,9 @@ class DenseC4(Workload):
     unit = "TFLOP/s"
     kernel = "gemm_dma_split_kernel<bf16,[K,N] weight> (256x256 tiles + 128x256 tiles for the last partial round)"
     work = 2 * 8192 * 4096 * 11008
-    # FETCH_SIZE / WRITE_SIZE per launch (profiles/mfma_kernels_bench.md): each XCD's L2 pulls its own copy of the operand panels
-    traffic = 1312.3e6
+    traffic_key = "c4_dense_bf16"
     n_sets = 3
-    cpu_rows = 512
+    cpu_warmups = 1
 
     def setup(self, torch, dev):
         from oracle import inputs
@@ -311,20 +340,16 @@ class DenseC4(Workload):
     def cpu_fn(self, torch):
         from oracle import eager, inputs
 
-        x, W, b = inputs.c4_dense(M=self.cpu_rows, device="cpu", seed=0)
+        x, W, b = inputs.c4_dense(device="cpu", seed=0)
         fn, how = _default_path_compile(eager.dense_silu_eager)
-        return (lambda: fn(x, W, b)), how + f", first {self.cpu_rows} of 8192 rows"
-
-    @property
-    def cpu_work(self):
-        return self.work * self.cpu_rows / 8192
+        return (lambda: fn(x, W, b)), how
 
 
 class DenseFp8C4(DenseC4):
     name = "C4 dense + bias + SiLU fp8 e4m3 (per-tensor x, per-channel W) M8192 K4096 N11008"
     dtype = "fp8"
     kernel = "gemm_dma_split_kernel<e4m3,[N,K] weight>"
-    traffic = 746.7e6  # FETCH_SIZE / WRITE_SIZE per launch (profiles/mfma_kernels_bench.md)
+    traffic_key = "c4_dense_fp8"
 
     def setup(self, torch, dev):
         from oracle import eager, inputs
@@ -363,10 +388,10 @@ class DenseFp8C4(DenseC4):
     def cpu_fn(self, torch):
         from oracle import eager, inputs
 
-        x, W, b = inputs.c4_dense(M=self.cpu_rows, device="cpu", seed=0)
+        x, W, b = inputs.c4_dense(device="cpu", seed=0)
         x_q, s_x = eager.quantize_fp8_per_tensor(x)
         W_q, s_w = eager.quantize_fp8_per_out_channel(W)
-        return (lambda: eager.dense_fp8_silu_eager(x_q, W_q, s_x, s_w, b)), f"eager dequantise + fp32 matmul, first {self.cpu_rows} of 8192 rows"
+        return (lambda: eager.dense_fp8_silu_eager(x_q, W_q, s_x, s_w, b)), "eager dequantise + fp32 matmul"
 
 
 class DenseGluC5(Workload):
@@ -376,9 +401,9 @@ class DenseGluC5(Workload):
     unit = "TFLOP/s"
     kernel = "gemm_glu_kernel<bf16> (256x128 output tiles: gate and up accumulators side by side, SwiGLU in the epilogue)"
     work = 4 * 8192 * 4096 * 11008
-    traffic = 2382.0e6  # FETCH_SIZE / WRITE_SIZE per launch (profiles/mfma_kernels_bench.md)
+    traffic_key = "c5_dense_glu"
     n_sets = 3
-    cpu_rows = 256
+    cpu_warmups = 1
 
     def setup(self, torch, dev):
         from xpu_graph_amd import _lib
@@ -416,13 +441,8 @@ class DenseGluC5(Workload):
         from oracle import eager
 
         x, wg, wu = (t.cpu() for t in self.sets[0])
-        x = x[: self.cpu_rows].contiguous()
         fn, how = _default_path_compile(lambda x, wg, wu: torch.nn.functional.silu(torch.nn.functional.linear(x, wg)) * torch.nn.functional.linear(x, wu))
-        return (lambda: fn(x, wg, wu)), how + f", first {self.cpu_rows} of 8192 rows"
-
-    @property
-    def cpu_work(self):
-        return self.work * self.cpu_rows / 8192
+        return (lambda: fn(x, wg, wu)), how
 
 
 class SdpaC5(Workload):
@@ -432,9 +452,9 @@ class SdpaC5(Workload):
     unit = "TFLOP/s"
     kernel = "sdpa_fwd_kernel<bf16,128>"
     work = 4 * 4 * 32 * 2048 * 2048 * 128 // 2  # two matmuls, lower triangle only
-    traffic = 700.3e6
+    traffic_key = "c5_sdpa"
     n_sets = 3
-    cpu_heads = 8
+    cpu_warmups = 1
 
     def setup(self, torch, dev):
         from xpu_graph_amd import _lib
@@ -468,13 +488,9 @@ class SdpaC5(Workload):
         from oracle import eager
 
         g = torch.Generator().manual_seed(0)
-        q, k, v = (torch.randn(1, self.cpu_heads, 2048, 128, generator=g).bfloat16() for _ in range(3))
+        q, k, v = (torch.randn(4, 32, 2048, 128, generator=g).bfloat16() for _ in range(3))
         fn, how = _default_path_compile(eager.causal_sdpa_eager)
-        return (lambda: fn(q, k, v)), how + f", {self.cpu_heads} of 128 (batch, head) pairs"
-
-    @property
-    def cpu_work(self):
-        return self.work * self.cpu_heads / 128
+        return (lambda: fn(q, k, v)), how
 
 
 class LlamaBlockC5(Workload):
@@ -483,10 +499,10 @@ class LlamaBlockC5(Workload):
     dtype = "bf16"
     unit = "TFLOP/s"
     kernel = "whole compiled block (5 dense + 1 gated dense, attention, 2 rotary, 2 norm kernels)"
-    traffic = None
+    traffic_key = None
     work = 2 * 8192 * (4 * 4096 * 4096 + 3 * 4096 * 11008) + 4 * 4 * 32 * 2048 * 2048 * 128 // 2
     n_sets = 1
-    cpu_tokens = 256
+    cpu_warmups = 1
 
     def setup(self, torch, dev):
         from oracle import eager, inputs
@@ -520,19 +536,94 @@ class LlamaBlockC5(Workload):
     def cpu_fn(self, torch):
         from oracle import eager, inputs
 
-        x, p = inputs.c5_llama_block(B=1, S=self.cpu_tokens, device="cpu")
+        x, p = inputs.c5_llama_block(device="cpu")
         fn, how = _default_path_compile(lambda x: eager.llama_block_eager(x, p, n_heads=32))
 
         def run():
             with torch.no_grad():
                 return fn(x)
 
-        return run, how + f", B1 S{self.cpu_tokens} (1/32 of the tokens)"
+        return run, how
 
-    @property
-    def cpu_work(self):
-        t = self.cpu_tokens
-        return 2 * t * (4 * 4096 * 4096 + 3 * 4096 * 11008) + 4 * 32 * t * t * 128 // 2
+
+# ---- roofline.traffic: HBM bytes per launch from two rocprofv3 --pmc runs of this file -------------------------
+# kernel of each workload as it appears in rocprofv3's Kernel_Name column (mangled or demangled): all of `has`, and
+# any of `any` when given
+TRAFFIC_KERNELS = {
+    "c2_add_layernorm": {"has": ["norm_rows_kernel"], "any": ["Lb1EEE", "true>"]},
+    "c1_rmsnorm": {"has": ["norm_rows_kernel"], "any": ["IffLi", "<float, float"]},
+    "c3a_slice_cat": {"has": ["slice_cat_kernel"]},
+    "c3b_addn": {"has": ["addn_kernel"]},
+    "c4_dense_bf16": {"has": ["gemm_dma_split_kernel"], "any": ["IDF16bDF16b", "<__bf16", "<__hip_bfloat16"]},
+    "c4_dense_fp8": {"has": ["gemm_dma_split_kernel"], "any": ["IhDF16b", "<unsigned char"]},
+    "c5_dense_glu": {"has": ["gemm_glu_"]},
+    "c5_sdpa": {"has": ["sdpa_fwd_kernel"]},
+}
+COPY_YARDSTICK_BYTES = 64 << 20
+
+
+def copy_yardstick(torch, dev):
+    """A few launches of the plain copy kernel over 64 MiB: the known-size dispatch that tells what one unit of
+    FETCH_SIZE / WRITE_SIZE is worth on this box."""
+    from xpu_graph_amd import _lib
+
+    a = torch.empty(COPY_YARDSTICK_BYTES, dtype=torch.uint8, device=dev)
+    b = torch.empty_like(a)
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    for _ in range(5):
+        _lib.check(_lib.lib().xg_copy_bytes(_p(a), _p(b), COPY_YARDSTICK_BYTES, st), "xg_copy_bytes")
+    torch.cuda.synchronize()
+
+
+def _median_counter(csv_dir, counter):
+    """kernel name -> median `counter` per dispatch, from the *_counter_collection.csv files under csv_dir."""
+    import csv
+    import glob
+
+    vals = {}
+    for path in glob.glob(os.path.join(csv_dir, "**", "*counter_collection.csv"), recursive=True):
+        with open(path, newline="") as f:
+            for row in csv.DictReader(f):
+                if row["Counter_Name"] == counter:
+                    vals.setdefault(row["Kernel_Name"], []).append(float(row["Counter_Value"]))
+    out = {}
+    for k, v in vals.items():
+        v.sort()
+        out[k] = (v[len(v) // 2], len(v))
+    return out
+
+
+def traffic_from(fetch_dir, write_dir, out_path=TRAFFIC_FILE):
+    """Turns `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` runs of this file into profiles/traffic.json:
+    bytes per launch = counter x (64 MiB / what the same counter reads for the 64 MiB copy kernel)."""
+    fetch, write = _median_counter(fetch_dir, "FETCH_SIZE"), _median_counter(write_dir, "WRITE_SIZE")
+
+    def pick(table, spec):
+        hits = [(v, k) for k, v in table.items() if all(h in k for h in spec["has"]) and ("any" not in spec or any(a in k for a in spec["any"]))]
+        return max(hits, key=lambda h: h[0][1]) if hits else None  # the variant with the most dispatches is the benchmark's
+
+    copy_spec = {"has": ["xg", "copy_kernel"]}
+    cf, cw = pick(fetch, copy_spec), pick(write, copy_spec)
+    if cf is None or cw is None:
+        raise SystemExit("the counter runs hold no xg copy_kernel dispatch: run bench.py itself under rocprofv3")
+    unit_f, unit_w = COPY_YARDSTICK_BYTES / cf[0][0], COPY_YARDSTICK_BYTES / cw[0][0]
+    table = {}
+    for key, spec in TRAFFIC_KERNELS.items():
+        f, w = pick(fetch, spec), pick(write, spec)
+        if f is None or w is None:
+            continue
+        table[key] = {
+            "bytes_per_launch": round(f[0][0] * unit_f + w[0][0] * unit_w),
+            "fetch_bytes": round(f[0][0] * unit_f),
+            "write_bytes": round(w[0][0] * unit_w),
+            "dispatches": [f[0][1], w[0][1]],
+            "kernel": f[1][:120],
+            "from": f"rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, median per dispatch; one counter unit = {unit_f:.0f} / {unit_w:.0f} bytes by the 64 MiB copy kernel",
+        }
+    with open(out_path, "w") as f:
+        json.dump(table, f, indent=1, sort_keys=True)
+        f.write("\n")
+    print(f"wrote {out_path}: {sorted(table)}")
 
 
 HEADLINE = AddLayerNormC2
@@ -545,6 +636,9 @@ def run_workload(torch, dev, wl, steps, warmup, with_cpu=True):
     peak = HBM_PEAK_GBPS if wl.bound == "hbm" else (FP8_PEAK_TFLOPS if wl.dtype == "fp8" else BF16_PEAK_TFLOPS)
     scale = 1e9 if wl.bound == "hbm" else 1e12
     n_sets = getattr(wl, "n_sets", N_SETS)
+    entry = _traffic_table().get(getattr(wl, "traffic_key", None) or "", None)
+    traffic = entry["bytes_per_launch"] if entry else None
+    traffic_source = f"profiles/traffic.json ({entry['from']})" if entry else None
     t_op = _wall_time(torch, wl.op_call, n_sets, steps, warmup)
     t_k = _events_time(torch, wl.abi_call, n_sets, max(steps, 100), max(warmup, 20))
     res = {
@@ -561,18 +655,20 @@ def run_workload(torch, dev, wl, steps, warmup, with_cpu=True):
             "unit": "GB/s" if wl.bound == "hbm" else "TFLOP/s",
             "frac": wl.work / t_k / scale / peak,
             "kernel_us": t_k * 1e6,
-            "traffic": getattr(wl, "traffic", None),
+            "traffic": traffic,
+            "traffic_source": traffic_source,
         },
     }
     if with_cpu:
         fn, how = wl.cpu_fn(torch)
-        t_cpu, n = _cpu_time(fn)
+        t_cpu, n = _cpu_time(fn, warmups=getattr(wl, "cpu_warmups", 2))
         res["cpu_baseline"] = {
-            "value": getattr(wl, "cpu_work", wl.work) / t_cpu / scale,
+            "value": wl.work / t_cpu / scale,
             "unit": res["unit"],
             "cores": torch.get_num_threads(),
+            "host_cpu_count": os.cpu_count(),
             "kind": "port",
-            "sample": f"{n} timed runs of {'a bounded sample' if hasattr(wl, 'cpu_work') else 'the full-size workload'} through {how}, median {t_cpu * 1e3:.2f} ms",
+            "sample": f"{n} timed runs of the full-size workload through {how}, median {t_cpu * 1e3:.2f} ms",
         }
     if hasattr(wl, "eager_ms"):
         res["eager_gpu_ms"] = wl.eager_ms
@@ -586,7 +682,12 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--only", default=None, help="headline only, or a substring of another workload's name")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--traffic-from", nargs=2, metavar=("FETCH_DIR", "WRITE_DIR"), default=None,
+                    help="no GPU work: read two rocprofv3 --pmc output folders of earlier runs of this file and write profiles/traffic.json")
     args = ap.parse_args()
+    if args.traffic_from:
+        traffic_from(*args.traffic_from)
+        return
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: the hot path has no cross-GPU part; run with --gpus 1", file=sys.stderr)
         sys.exit(2)
@@ -604,8 +705,12 @@ def main():
         if isinstance(handler, logging.StreamHandler):
             handler.setStream(sys.stderr)
 
-    torch.set_num_threads(min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16"))))
+    # The CPU baseline uses the cores this job owns: OMP_NUM_THREADS when the launcher sets it (a GPU box hands one job
+    # a share of a larger host, and more threads than that share only fight each other), else every core.  Both
+    # counts are reported: cpu_baseline.cores (threads used) and cpu_baseline.host_cpu_count.
+    torch.set_num_threads(min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))))
     dev = torch.device("cuda:0")
+    copy_yardstick(torch, dev)
     head = run_workload(torch, dev, HEADLINE(), args.steps, args.warmup, with_cpu=not args.no_cpu)
     out = {
         "metric": "fused-op GB/s (residual-add + LayerNorm, % of HBM peak in roofline.frac)",

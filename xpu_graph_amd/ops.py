@@ -636,7 +636,9 @@ def _unit_last(t):
     """A tensor the attention / rotary kernels can read in place: unit last stride, every other stride a multiple of
     16 bytes, 16-byte aligned base (their loads are 16 bytes per lane).  Anything else is copied."""
     per16 = 16 // t.element_size()
-    ok = t.stride(-1) == 1 and all(st % per16 == 0 for st in t.stride()[:-1]) and t.data_ptr() % 16 == 0
+    # the offset into the storage stands for the base address (allocations are at least 256-byte aligned), so that the
+    # shape-only Meta implementations predict the same layout as the real call
+    ok = t.stride(-1) == 1 and all(st % per16 == 0 for st in t.stride()[:-1]) and t.storage_offset() % per16 == 0
     return t if ok else t.contiguous()
 
 
