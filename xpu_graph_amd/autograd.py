@@ -200,30 +200,52 @@ def _sdpa_setup(ctx, inputs, output):
     ctx.save_for_backward(q, k, v)
 
 
+SDPA_BACKWARD_CHUNK_ELEMS = 32 * 1024 * 1024  # fp32 elements of one [B, H, rows, Skv] temporary (128 MiB)
+
+
 def _sdpa_backward(ctx, gy):
-    # The probabilities are recomputed in fp32 ([B, H, Sq, Skv] at once: a formula for training at moderate sequence
-    # lengths, not a flash backward).  With fewer key/value heads than query heads, query head h reads head h // rep.
+    # The probabilities are recomputed in fp32 Aten ops, a block of query rows at a time: softmax runs along the keys,
+    # so a block of whole rows is exact, and no temporary is larger than SDPA_BACKWARD_CHUNK_ELEMS elements whatever
+    # the sequence length (the whole [B, H, Sq, Skv] matrix is 34 GB per temporary at B4 H32 S8192).  With a causal
+    # mask a block only meets the keys up to its last row.  With fewer key/value heads than query heads, query head
+    # h reads head h // rep.  Not a flash backward kernel: the key/value gradients are accumulated in fp32 tensors.
     q, k, v = ctx.saved_tensors
     B, H, Sq, D = q.shape
     Hkv, Skv = k.shape[1], k.shape[2]
     rep = H // Hkv
-    qf, kf, vf, gf = q.float(), k.float(), v.float(), gy.float()
+    kf, vf = k.float(), v.float()
     if rep > 1:
         kf, vf = kf.repeat_interleave(rep, dim=1), vf.repeat_interleave(rep, dim=1)
-    s = (qf @ kf.transpose(-1, -2)) * ctx.scale
-    if ctx.causal:
-        visible = torch.ones(Sq, Skv, dtype=torch.bool, device=q.device).tril()
-        s = s.masked_fill(~visible, float("-inf"))
-    p = torch.softmax(s, dim=-1)
-    gv = p.transpose(-1, -2) @ gf
-    gp = gf @ vf.transpose(-1, -2)
-    gs = p * (gp - (gp * p).sum(-1, keepdim=True))
-    gq = (gs @ kf) * ctx.scale
-    gk = (gs.transpose(-1, -2) @ qf) * ctx.scale
+    gq = torch.empty_like(q)
+    gk = torch.zeros(B, H, Skv, D, dtype=torch.float32, device=q.device)
+    gv = torch.zeros(B, H, Skv, D, dtype=torch.float32, device=q.device)
+    rows = max(1, min(Sq, SDPA_BACKWARD_CHUNK_ELEMS // max(1, B * H * Skv)))
+    for r0 in range(0, Sq, rows):
+        r1 = min(Sq, r0 + rows)
+        n_keys = min(Skv, r1) if ctx.causal else Skv  # keys a causal block can see: 0 .. its last row
+        if n_keys == 0:
+            gq[:, :, r0:r1] = 0
+            continue
+        qc, gc = q[:, :, r0:r1].float(), gy[:, :, r0:r1].float()
+        kc, vc = kf[:, :, :n_keys], vf[:, :, :n_keys]
+        s = (qc @ kc.transpose(-1, -2)) * ctx.scale
+        if ctx.causal:
+            row = torch.arange(r0, r1, device=q.device).unsqueeze(1)
+            col = torch.arange(n_keys, device=q.device).unsqueeze(0)
+            s = s.masked_fill(col > row, float("-inf"))
+        p = torch.softmax(s, dim=-1)
+        del s
+        gv[:, :, :n_keys] += p.transpose(-1, -2) @ gc
+        gp = gc @ vc.transpose(-1, -2)
+        gs = p * (gp - (gp * p).sum(-1, keepdim=True))
+        del p, gp
+        gq[:, :, r0:r1] = ((gs @ kc) * ctx.scale).to(q.dtype)
+        gk[:, :, :n_keys] += (gs.transpose(-1, -2) @ qc) * ctx.scale
+        del gs
     if rep > 1:
         gk = gk.reshape(B, Hkv, rep, Skv, D).sum(2)
         gv = gv.reshape(B, Hkv, rep, Skv, D).sum(2)
-    return gq.to(q.dtype), gk.to(k.dtype), gv.to(v.dtype), None, None
+    return gq, gk.to(k.dtype), gv.to(v.dtype), None, None
 
 
 def _add_norm_formulas(layer, with_sum):

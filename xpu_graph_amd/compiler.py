@@ -82,9 +82,18 @@ class XpuGraph:
             with local_logger(stage.name):
                 if stage == FxStage.inference:
                     logger.info("decompose graph complete")
+                kept = None
+                if stage == FxStage.inference and self._config.freeze and not self._config.is_training:
+                    kept = self._freeze(gm)
+                    if kept is not None:
+                        sample_inputs = [sample_inputs[i] for i in kept]
                 fake_mode, fake_inputs = fakify_tensors(sample_inputs)
                 hashkey = None
-                if self._cache is not None:
+                # a frozen graph carries its parameters as constants: the text of the graph, which is what the cache
+                # key is made of, no longer identifies it (two models of one architecture would share an artifact)
+                if self._cache is not None and kept is not None:
+                    logger.info("frozen graph: not cached (its constants are this model's parameters)")
+                if self._cache is not None and kept is None:
                     hashkey = self._cache.cache_key(gm, fake_inputs, self._config, stage)
                     cached = self._cache.load_artifact(hashkey)
                     if cached is not None:
@@ -114,10 +123,28 @@ class XpuGraph:
                 # the cache holds the rewritten graph; what the post-pass hook builds around it (recordings of
                 # device graphs) is made again, cheaply, in every process
                 runnable = self._vendor_compile(out, fake_inputs, stage)
+                if kept is not None:
+                    return _drop_frozen_args(runnable, kept)
                 # AOT's runtime wrappers call the compiled stage with one list of arguments
                 return make_boxed_func(runnable) if boxed else runnable
 
         return compile_stage
+
+    def _freeze(self, gm):
+        """Parameters and buffers of an inference graph become constants of the graph (reference
+        fx_utils.py:89-350, `dispatch_graph` with freeze).  Returns the placeholder indices that stay inputs, or
+        None (with a warning) when AOT did not say which inputs are parameters."""
+        from .fx_utils import unlift_params
+
+        ctx = torch._guards.TracingContext.try_get()
+        params_flat = getattr(ctx, "params_flat", None) if ctx is not None else None
+        fw_metadata = getattr(ctx, "fw_metadata", None) if ctx is not None else None
+        if not params_flat or fw_metadata is None:
+            logger.warning("freeze=True has no effect on this graph: it received its parameters as ordinary inputs")
+            return None
+        kept = unlift_params(gm, list(params_flat), fw_metadata)
+        logger.info(f"freeze: {len(params_flat) - sum(1 for i in kept if i < len(params_flat))} parameters became constants, {len(kept)} inputs remain")
+        return kept
 
     def __call__(self, dynamo_gm, example_inputs, *args, **kwargs):
         logger.info(f"{self._config}")
@@ -232,6 +259,18 @@ class XpuGraph:
         import torch._inductor.config as inductor_config
 
         inductor_config.freezing = self._orig_ctx["freezing"]
+
+
+def _drop_frozen_args(runnable, kept):
+    """AOT keeps passing every parameter at run time; the frozen graph takes only the inputs it kept."""
+
+    def call(args):
+        live = [args[i] for i in kept]
+        args.clear()
+        return runnable(*live)
+
+    call._boxed_call = True
+    return call
 
 
 class XpuGraphCompiler:

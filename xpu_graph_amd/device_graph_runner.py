@@ -92,8 +92,11 @@ class HIPGraphRunner(GraphRunner):
             self._output = self._callable_target(*args, **kwargs)
 
     def forward(self, *args, **kwargs):
-        assert self._graph is not None, "capture() first"
-        assert self._copy_param_callback(self._input_buffers, *args, **kwargs), "arguments do not fit the recorded buffers"
+        if self._graph is None:
+            raise RuntimeError("capture() first")
+        # the refresh of the recorded input buffers is work, not a check: it must also happen under `python -O`
+        if not self._copy_param_callback(self._input_buffers, *args, **kwargs):
+            raise RuntimeError("arguments do not fit the recorded buffers")
         self._graph.replay()
         return self._output
 

@@ -93,3 +93,34 @@ def dispatch_pregrad(gm, example_inputs):
     if sig.user_inputs_to_mutate or sig.buffers_to_mutate or getattr(sig, "parameters_to_mutate", None) or sig.input_tokens:
         raise NotImplementedError("the graph mutates its inputs")
     return out
+
+
+def unlift_params(gm, params_flat, fw_metadata):
+    """Freezing (reference fx_utils.py `_unlift_params`): AOT hands the inference compiler a graph whose first
+    len(params_flat) placeholders are the module's parameters and buffers.  Each of them that the graph neither
+    writes nor hands back as (an alias of) an output becomes a `get_attr` constant holding the parameter itself, so
+    that ConstantFolding(folding_freezed_params) can fold weight-side subgraphs (a transposed or pre-scaled weight).
+    Returns the indices of the placeholders that remain graph inputs, in order."""
+    from torch._functorch._aot_autograd.schemas import MutationType
+
+    placeholders = [n for n in gm.graph.nodes if n.op == "placeholder"]
+    aliased = {info.base_idx for info in fw_metadata.output_info if info.base_idx is not None}
+    mutated = {i for i, m in enumerate(fw_metadata.input_info) if m.mutation_type in (MutationType.MUTATED_IN_GRAPH, MutationType.MUTATED_OUT_GRAPH)}
+    kept = []
+    for i, (node, real) in enumerate(zip(placeholders, params_flat)):
+        if i in aliased or i in mutated or not isinstance(real, torch.Tensor):
+            kept.append(i)
+            continue
+        name = f"_xg_frozen_param{i}"
+        if isinstance(real, torch.nn.Parameter):
+            gm.register_parameter(name, real)  # the parameter itself, not a copy
+        else:
+            gm.register_buffer(name, real, persistent=False)
+        with gm.graph.inserting_before(node):
+            const = gm.graph.get_attr(name)
+        const.meta.update({k: v for k, v in node.meta.items() if k in ("val", "tensor_meta")})
+        node.replace_all_uses_with(const)
+        gm.graph.erase_node(node)
+    kept.extend(range(len(params_flat), len(placeholders)))
+    gm.recompile()
+    return kept

@@ -87,6 +87,11 @@ class Cse(Optimizer):
             # factories and copies return fresh storage that later in-place ops may write
             if name.startswith("aten::empty") or name in ("aten::clone", "aten::_to_copy", "aten::copy"):
                 return False
+            # a call with no tensor input (zeros, full, arange, ...) makes a fresh tensor each time: two of them are
+            # two tensors, which the caller may go on to write separately
+            flat, _ = pytree.tree_flatten((node.args, node.kwargs))
+            if not any(isinstance(a, fx.Node) for a in flat):
+                return False
             return True
         return tgt.__module__ == "_operator"
 
@@ -154,6 +159,8 @@ class ConstantFolding(Optimizer):
                 continue
             if not any(isinstance(a, fx.Node) for a in flat) and not self._foldable_factory(node):
                 continue
+            if node.target is torch.ops.aten.clone.default and node.users and all(u.op == "output" for u in node.users):
+                continue  # the copy that keeps a constant from being handed to the caller (see _protect_outputs)
             args, kwargs = pytree.tree_map(lambda a: getattr(gm, a.target) if isinstance(a, fx.Node) else a, (node.args, node.kwargs))
             logger.info(f"start constant folding: {node.name} {node.target}")
             with outside_fake_mode():
@@ -169,4 +176,46 @@ class ConstantFolding(Optimizer):
                 const = graph.get_attr(name)
             node.replace_all_uses_with(const)
             changed = True
+        return self._protect_outputs(gm) or changed
+
+    _VIEW_OPS = (
+        "aten::view", "aten::reshape", "aten::_unsafe_view", "aten::expand", "aten::permute", "aten::transpose", "aten::t",
+        "aten::slice", "aten::select", "aten::unsqueeze", "aten::squeeze", "aten::alias", "aten::detach", "aten::as_strided",
+    )
+
+    @classmethod
+    def _folded_base(cls, gm, node):
+        """The folded constant `node` is (a view of), or None."""
+        while isinstance(node, fx.Node):
+            if node.op == "get_attr":
+                return node if node.target in getattr(gm, "_xg_constants", ()) else None
+            tgt = node.target
+            if node.op == "call_function" and isinstance(tgt, torch._ops.OpOverload) and tgt._schema.name in cls._VIEW_OPS and node.args:
+                node = node.args[0]
+                continue
+            return None
+        return None
+
+    def _protect_outputs(self, gm):
+        """A folded constant lives in the module and would be handed to the caller again on every call: whoever writes
+        into a result (a freshly initialised cache or accumulator) would change the next call's result, and two
+        outputs folded to one constant would alias each other.  Every output that is (a view of) a folded constant is
+        returned as a copy, which is what eager and the unfolded graph return: a fresh tensor."""
+        out_node = next(n for n in reversed(gm.graph.nodes) if n.op == "output")
+        changed = False
+
+        def fix(arg):
+            nonlocal changed
+            if isinstance(arg, fx.Node) and self._folded_base(gm, arg) is not None:
+                with gm.graph.inserting_before(out_node):
+                    fresh = gm.graph.call_function(torch.ops.aten.clone.default, (arg,))
+                if "val" in arg.meta:
+                    fresh.meta["val"] = arg.meta["val"]
+                changed = True
+                return fresh
+            return arg
+
+        new_args = fx.map_arg(out_node.args, fix)
+        if changed:
+            out_node.args = new_args
         return changed
