@@ -235,6 +235,27 @@ int xg_sdpa(const void* q, const void* k, const void* v, void* out, int64_t B, i
             xg_stream_t stream);
 
 /* ---------------------------------------------------------------------------
+ * xg_sdpa with the two operands the general attn_mask form of FusedSDPA carries
+ * (fuse_scaled_dot_product_attention.py:184-234, `attn_mask=` and a tensor
+ * `scale`):
+ *   mask: NULL or an additive mask, element [b,h,i,j] at
+ *     mask + mask_strides[0]*b + mask_strides[1]*h + mask_strides[2]*i + j
+ *     (strides in elements, 0 = broadcast along that axis), dtype `mask_dtype`
+ *     = `dtype` or XG_F32; it is added to q.k^T * scale before the softmax.
+ *     A row whose every key is masked with -inf comes out as NaN, as in eager.
+ *   scale_dev: NULL, or a one-element fp32 DEVICE tensor that holds the scale;
+ *     the kernel reads it (no host read, no synchronisation) and `scale` is
+ *     ignored.  Replaces SDPAWrappedScale.forward, which reads the tensor with
+ *     .item() (passes/patterns/utils/default_replacements.py:39-55).
+ * `causal` may be combined with a mask.
+ * ------------------------------------------------------------------------- */
+int xg_sdpa_masked(const void* q, const void* k, const void* v, void* out, const void* mask,
+                   const int64_t mask_strides[3], int mask_dtype, const float* scale_dev, int64_t B, int64_t H,
+                   int64_t Hkv, int64_t Sq, int64_t Skv, int64_t D, const int64_t q_strides[3],
+                   const int64_t k_strides[3], const int64_t v_strides[3], const int64_t o_strides[3], float scale,
+                   int causal, int dtype, xg_stream_t stream);
+
+/* ---------------------------------------------------------------------------
  * Rotary position embedding, rotate-half convention:
  *   out = x * cos + cat(-x[..., D/2:], x[..., :D/2]) * sin      (fp32 math, one rounding)
  *   x, out [B,H,S,D] with element strides for batch, head, sequence (D has unit stride, D % 16 == 0);

@@ -378,3 +378,54 @@ def test_hand_written_gelu_runs_in_the_dense_epilogue_or_as_aten_gelu(device, fo
     else:
         assert calls == ["custom_dense_layer_replacement", "aten.gelu.default"], calls
     torch._dynamo.reset()
+
+
+def test_sdpa_with_a_tensor_scale_runs_the_kernel_without_a_host_read(device):
+    """The reference's tensor-scale form (tests/common/test_fuse_sdpa.py:608-610, `_sdpa_pattern_tensor_scale`):
+    FusedSDPA wraps it in xpu_graph::sdpa_wrapped_scale, which reads the scale with .item(); on this target the
+    kernel reads the one-element tensor itself."""
+    import math
+
+    from tests.tolerance import assert_close_16bit, attention_floor
+
+    def att_div(q, k, v, s):
+        return torch.matmul(q, k.transpose(-2, -1)).div(s).softmax(dim=-1).matmul(v)
+
+    g = torch.Generator().manual_seed(0)
+    q, k, v = (torch.randn(2, 4, 256, 128, generator=g).bfloat16().to(device) for _ in range(3))
+    s = torch.tensor([math.sqrt(128.0)], device=device)
+    out, mods, rest = run(att_div, q, k, v, s)
+    assert "mi355x_sdpa_masked" in mods and "fused_sdpa" not in mods, (mods, rest)
+    assert not any("softmax" in t or "bmm" in t or "matmul" in t for t in rest), rest
+    want = att_div(q.float(), k.float(), v.float(), s)
+    assert_close_16bit(out, want, attention_floor(want, out.dtype), "sdpa tensor-scale compiled")
+
+
+@pytest.mark.parametrize("mask_kind", ["per_head", "rows_f32", "padding"])
+def test_sdpa_with_an_additive_mask_runs_the_kernel(device, mask_kind):
+    """Masked attention written out in eager (the reference's `_sdpa_pattern_*` forms with a mask): FusedSDPA emits
+    aten.scaled_dot_product_attention(attn_mask=...), the target hands the mask to the kernel."""
+    import math
+
+    from tests.tolerance import assert_close_16bit, attention_floor
+
+    def att(q, k, v, m):
+        return torch.softmax((q @ k.transpose(-2, -1) / math.sqrt(q.size(-1))) + m, dim=-1) @ v
+
+    g = torch.Generator().manual_seed(1)
+    B, H, S, D = 2, 4, 192, 128
+    q, k, v = (torch.randn(B, H, S, D, generator=g).bfloat16().to(device) for _ in range(3))
+    if mask_kind == "per_head":
+        m = torch.randn(1, H, S, S, generator=g).bfloat16().to(device)
+    elif mask_kind == "rows_f32":
+        m = torch.randn(S, S, generator=g).to(device)
+    else:
+        m = torch.zeros(B, 1, S, S)
+        m[0, :, :, 150:] = float("-inf")
+        m[1, :, :, 100:] = float("-inf")
+        m = m.bfloat16().to(device)
+    out, mods, rest = run(att, q, k, v, m)
+    assert "mi355x_sdpa_masked" in mods, (mods, rest)
+    assert not any("softmax" in t or "bmm" in t for t in rest), rest
+    want = att(q.float(), k.float(), v.float(), m.float())
+    assert_close_16bit(out.to(torch.bfloat16) if out.dtype != torch.bfloat16 else out, want, attention_floor(want, torch.bfloat16), f"sdpa masked compiled {mask_kind}")

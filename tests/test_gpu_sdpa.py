@@ -79,6 +79,60 @@ def test_sdpa_and_rope_take_misaligned_views(device):
     torch.testing.assert_close(got.float(), want, rtol=1.6e-2, atol=2.0**-7 * want.abs().max().item())
 
 
+def ref32_masked(q, k, v, mask, causal, scale):
+    qf, kf, vf = q.float(), k.float(), v.float()
+    rep = q.shape[1] // k.shape[1]
+    if rep > 1:
+        kf, vf = kf.repeat_interleave(rep, dim=1), vf.repeat_interleave(rep, dim=1)
+    s = torch.matmul(qf, kf.transpose(-1, -2)) * scale
+    if mask is not None:
+        s = s + mask.float()
+    if causal:
+        s = s + torch.full(s.shape[-2:], float("-inf"), device=q.device).triu(1)
+    return torch.matmul(torch.softmax(s, dim=-1), vf)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("D", [128, 64])
+@pytest.mark.parametrize("mask_shape,mask_dtype", [("full", "same"), ("rows", "f32"), ("per_batch", "same"), ("per_head", "f32")])
+@pytest.mark.parametrize("Sq,Skv", [(256, 256), (130, 77), (1, 300), (200, 333)])
+def test_sdpa_additive_mask(device, dtype, D, mask_shape, mask_dtype, Sq, Skv):
+    """attn_mask of the FusedSDPA form (reference tests/common/test_fuse_sdpa.py: `_sdpa_pattern_*` with a mask
+    operand): any floating-point additive mask, broadcast over batch and / or heads, odd sizes (rows the kernel must
+    read element by element), -inf entries (padding) and a causal flag on top."""
+    B, H, Hkv = 2, 4, 2
+    q, k, v = make(B, H, Hkv, Sq, Skv, D, dtype, device, seed=Sq * 3 + Skv + D)
+    g = torch.Generator().manual_seed(Sq + Skv)
+    shape = {"full": (B, H, Sq, Skv), "rows": (Sq, Skv), "per_batch": (B, 1, Sq, Skv), "per_head": (1, H, Sq, Skv)}[mask_shape]
+    mask = torch.randn(shape, generator=g)
+    pad = torch.rand(shape[:-2] + (1, Skv), generator=g) < 0.2  # padded keys, at least key 0 stays visible
+    pad[..., 0] = False
+    mask = mask.masked_fill(pad.expand(shape), float("-inf")).to(dtype if mask_dtype == "same" else torch.float32).to(device)
+    scale = 1.0 / math.sqrt(D)
+    got = _ops().sdpa_masked(q, k, v, mask, None, False, scale)
+    assert got.shape == q.shape and got.dtype == dtype
+    close(got, ref32_masked(q, k, v, mask, False, scale))
+    if Sq == Skv:
+        close(_ops().sdpa_masked(q, k, v, mask, None, True, scale), ref32_masked(q, k, v, mask, True, scale))
+
+
+def test_sdpa_scale_from_a_device_tensor(device):
+    """The scale arrives as a one-element tensor (the reference's sdpa_wrapped_scale reads it with .item()): the kernel
+    reads it on the device, and the result equals the by-value call bit for bit."""
+    q, k, v = make(2, 4, 4, 192, 160, 128, torch.bfloat16, device, seed=9)
+    for value, dt in ((0.07, torch.float32), (1.0 / math.sqrt(128), torch.bfloat16)):
+        t = torch.tensor([value], dtype=dt, device=device)
+        got = _ops().sdpa_masked(q, k, v, None, t, False, 123.0)  # the by-value scale is ignored
+        assert torch.equal(got, _ops().sdpa(q, k, v, False, t.float().item()))
+    # a fully masked row is NaN, as in eager
+    mask = torch.zeros(192, 160, device=device)
+    mask[5] = float("-inf")
+    out = _ops().sdpa_masked(q, k, v, mask, None, False, 0.1)
+    assert torch.isnan(out[:, :, 5]).all() and not torch.isnan(out[:, :, 4]).any()
+    with pytest.raises(ValueError):
+        _ops().sdpa_masked(q, k, v, torch.zeros(3, 192, 160, device=device), None, False, 0.1)
+
+
 def test_sdpa_matches_oracle_causal(device):
     q, k, v = make(1, 4, 4, 512, 512, 128, torch.bfloat16, device, seed=5)
     got = _ops().sdpa(q, k, v, True, 1.0 / math.sqrt(128))

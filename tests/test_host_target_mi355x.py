@@ -571,3 +571,24 @@ def test_repeated_gather_index_becomes_a_broadcast_view(caplog):
     assert torch.equal(got, real_repeat(x, idx))
     assert "Pattern.FusedGatherToCopy changed graph" not in caplog.text
     torch._dynamo.reset()
+
+
+def test_masked_and_tensor_scale_attention_become_the_masked_kernel_call(caplog, backend):
+    """A non-causal additive mask and the wrapped tensor scale both end in `mi355x_sdpa_masked` (reference forms:
+    tests/common/test_fuse_sdpa.py `_sdpa_pattern_*` with a mask, `_sdpa_pattern_tensor_scale`); a boolean mask
+    stays on aten."""
+    B, H, S, D = 2, 4, 64, 128
+
+    def att_mask(q, k, v, m):
+        return torch.softmax((q @ k.transpose(-2, -1) / math.sqrt(D)) + m, dim=-1) @ v
+
+    def att_tscale(q, k, v, s):
+        return torch.matmul(q, k.transpose(-2, -1)).div(s).softmax(dim=-1).matmul(v)
+
+    q, k, v = (torch.randn(B, H, S, D).to(bf16) for _ in range(3))
+    gm = rewrite(backend, att_mask, q, k, v, torch.randn(1, H, S, S).to(bf16))
+    assert "mi355x_sdpa_masked" in modules_called(gm), (modules_called(gm), aten_ops(gm))
+    assert not any("softmax" in t or "bmm" in t for t in aten_ops(gm))
+    torch._dynamo.reset()
+    gm = rewrite(backend, att_tscale, q, k, v, torch.tensor([math.sqrt(D)]))
+    assert "mi355x_sdpa_masked" in modules_called(gm) and "fused_sdpa" not in modules_called(gm), (modules_called(gm), aten_ops(gm))

@@ -108,6 +108,13 @@ _SIGNATURES = {
             c_void_p,
         ],
     ),
+    "xg_sdpa_masked": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, ctypes.POINTER(c_int64), c_int, c_void_p]
+        + [c_int64] * 6
+        + [ctypes.POINTER(c_int64)] * 4
+        + [c_float, c_int, c_int, c_void_p],
+    ),
     "xg_rope": (
         c_int,
         [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, ctypes.POINTER(c_int64), ctypes.POINTER(c_int64), c_int64, c_int, c_int, c_void_p],

@@ -56,6 +56,11 @@ struct Params {
   int B, H, Hkv, Sq, Skv;
   int64_t qs[3], ks[3], vs[3], os[3];  // element strides of batch, head, sequence
   float c;                             // scale * log2(e)
+  const float* scale_dev;              // when set: the scale is read from this one-element device tensor instead
+  const void* mask;                    // additive mask (MASK kernels only), element [b, h, i, j] at ms[0] b + ms[1] h + ms[2] i + j
+  int64_t ms[3];                       // element strides of batch, head, query row (0: broadcast)
+  int mask_f32;                        // mask elements are fp32 (else the dtype of q)
+  int mask_vec;                        // rows of the mask can be read four elements at a time
   int causal;
   int n_qb;   // query blocks per (batch, head)
   int order;  // 0: heaviest query blocks of ALL heads first; 1: head after head inside each XCD
@@ -97,7 +102,9 @@ __device__ __forceinline__ int swz_v(int r) {
   else return (((r >> 1) & 1) << 2) | ((r >> 2) & 3);
 }
 
-template <typename T, int D>
+// MASK: an additive mask [B | 1, H | 1, Sq, Skv] is added to the scaled scores (aten.scaled_dot_product_attention's
+// attn_mask); rows whose every key is masked with -inf come out as NaN, as they do in eager.
+template <typename T, int D, bool MASK = false>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void sdpa_fwd_kernel(Params p) {
   typedef typename Vec8<T>::type V8;
   constexpr int RB = D * 2;          // bytes per tile row
@@ -113,6 +120,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int l32 = lane & 31, h = lane >> 5;
+  // scale * log2(e): by value, or from a one-element device tensor (a scale that is only known on the device)
+  const float c_eff = p.scale_dev ? *p.scale_dev * 1.44269504088896340736f : p.c;
 
   // ---- which (batch, head, query block).  Blocks are dealt round-robin to the 8 XCDs, so with the
   // number of heads a multiple of 8 both orders keep all query blocks of a head on ONE XCD (one L2).
@@ -235,7 +244,43 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
 
     // scores are s * c in the exponent's base-2 scale.  Tiles that cross the diagonal or the end of
     // the keys are scaled and masked explicitly (cc = 1 afterwards); all others fold c into the FMA.
-    float cc = p.c;
+    float cc = c_eff;
+    if constexpr (MASK) {
+      // scores in the exponent's base-2 scale with the mask added: s * c + m * log2(e); afterwards cc = 1.
+      // Row and key indices are clamped for the loads; what lies past the end is masked by index below.
+      const int mrow = qrow < p.Sq ? qrow : p.Sq - 1;
+      const int64_t mbase = (int64_t)b * p.ms[0] + (int64_t)head * p.ms[1] + (int64_t)mrow * p.ms[2];
+      constexpr float kLog2e = 1.44269504088896340736f;
+      static_for<2>([&](auto TI) {
+        constexpr int t = decltype(TI)::value;
+        static_for<4>([&](auto GI) {
+          constexpr int g = decltype(GI)::value;
+          const int key0 = kv0 + 32 * t + 8 * g + 4 * h;
+          float m4[4];
+          if (p.mask_vec && key0 + 3 < p.Skv) {
+            if (p.mask_f32) {
+              const f32x4 mv = *reinterpret_cast<const f32x4*>(reinterpret_cast<const float*>(p.mask) + mbase + key0);
+              m4[0] = mv[0], m4[1] = mv[1], m4[2] = mv[2], m4[3] = mv[3];
+            } else {
+              typedef T t4 __attribute__((ext_vector_type(4)));
+              const t4 mv = *reinterpret_cast<const t4*>(reinterpret_cast<const T*>(p.mask) + mbase + key0);
+              m4[0] = (float)mv[0], m4[1] = (float)mv[1], m4[2] = (float)mv[2], m4[3] = (float)mv[3];
+            }
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const int key = key0 + e < p.Skv ? key0 + e : p.Skv - 1;
+              m4[e] = p.mask_f32 ? reinterpret_cast<const float*>(p.mask)[mbase + key] : (float)reinterpret_cast<const T*>(p.mask)[mbase + key];
+            }
+          }
+          static_for<4>([&](auto EI) {
+            constexpr int e = decltype(EI)::value;
+            s[t][4 * g + e] = __builtin_fmaf(s[t][4 * g + e], cc, m4[e] * kLog2e);
+          });
+        });
+      });
+      cc = 1.f;
+    }
     const bool need_mask = (p.causal && kv0 + BKV - 1 > qw_min) || (kv0 + BKV > p.Skv);
     if (need_mask) {
       int lim = p.Skv - 1;  // last visible key of this lane's query
@@ -352,10 +397,10 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
   });
 }
 
-template <typename T, int D>
+template <typename T, int D, bool MASK = false>
 int launch(const Params& p, hipStream_t stream) {
   constexpr int SMEM = 2 * 2 * BKV * D * 2;
-  auto kernel = sdpa_fwd_kernel<T, D>;
+  auto kernel = sdpa_fwd_kernel<T, D, MASK>;
   if (int st = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), SMEM)) return st;
   const int64_t blocks = (int64_t)p.B * p.H * p.n_qb;
   hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(kThreads), SMEM, stream, p);
@@ -365,9 +410,12 @@ int launch(const Params& p, hipStream_t stream) {
 }  // namespace sdpa
 }  // namespace xg
 
-extern "C" int xg_sdpa(const void* q, const void* k, const void* v, void* out, int64_t B, int64_t H, int64_t Hkv, int64_t Sq,
-                       int64_t Skv, int64_t D, const int64_t q_strides[3], const int64_t k_strides[3], const int64_t v_strides[3],
-                       const int64_t o_strides[3], float scale, int causal, int dtype, xg_stream_t stream) {
+namespace {
+
+int sdpa_entry(const void* q, const void* k, const void* v, void* out, const void* mask, const int64_t* mask_strides, int mask_dtype,
+               const float* scale_dev, int64_t B, int64_t H, int64_t Hkv, int64_t Sq, int64_t Skv, int64_t D, const int64_t q_strides[3],
+               const int64_t k_strides[3], const int64_t v_strides[3], const int64_t o_strides[3], float scale, int causal, int dtype,
+               xg_stream_t stream) {
   using namespace xg;
   if (dtype != XG_BF16 && dtype != XG_F16) return XG_ERR_BAD_DTYPE;
   if (B < 0 || H < 0 || Hkv < 0 || Sq < 0 || Skv < 0) return XG_ERR_BAD_SHAPE;
@@ -391,6 +439,27 @@ extern "C" int xg_sdpa(const void* q, const void* k, const void* v, void* out, i
   }
   // per-lane tile offsets are 32-bit: 64 rows of K / V must span less than 2 GiB
   if (k_strides[2] > (1 << 23) || v_strides[2] > (1 << 23)) return XG_ERR_TOO_LARGE;
+  p.mask = mask;
+  p.mask_f32 = 0;
+  p.mask_vec = 0;
+  p.ms[0] = p.ms[1] = p.ms[2] = 0;
+  if (mask) {
+    if (!mask_strides) return XG_ERR_NULL_PTR;
+    if (mask_dtype != dtype && mask_dtype != XG_F32) return XG_ERR_BAD_DTYPE;
+    const size_t esz = mask_dtype == XG_F32 ? 4 : 2;
+    if (!aligned_to(mask, esz)) return XG_ERR_BAD_ALIGN;
+    bool vec = aligned_to(mask, 4 * esz);
+    for (int i = 0; i < 3; ++i) {
+      if (mask_strides[i] < 0) return XG_ERR_BAD_SHAPE;
+      p.ms[i] = mask_strides[i];
+      vec = vec && mask_strides[i] % 4 == 0;
+    }
+    if (Sq > 1 && mask_strides[2] != 0 && mask_strides[2] < Skv) return XG_ERR_BAD_SHAPE;  // rows would overlap
+    p.mask_f32 = mask_dtype == XG_F32 ? 1 : 0;
+    p.mask_vec = vec ? 1 : 0;
+  }
+  if (scale_dev && !aligned_to(scale_dev, 4)) return XG_ERR_BAD_ALIGN;
+  p.scale_dev = scale_dev;
   p.q = q;
   p.k = k;
   p.v = v;
@@ -408,6 +477,27 @@ extern "C" int xg_sdpa(const void* q, const void* k, const void* v, void* out, i
   // the heaviest query blocks of all heads first (S2048 causal 176 vs 205 us).
   p.order = (!p.causal || n_qb >= 32) ? 1 : 0;
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  if (mask) {
+    if (dtype == XG_BF16) return D == 128 ? sdpa::launch<bf16_t, 128, true>(p, st) : sdpa::launch<bf16_t, 64, true>(p, st);
+    return D == 128 ? sdpa::launch<f16_t, 128, true>(p, st) : sdpa::launch<f16_t, 64, true>(p, st);
+  }
   if (dtype == XG_BF16) return D == 128 ? sdpa::launch<bf16_t, 128>(p, st) : sdpa::launch<bf16_t, 64>(p, st);
   return D == 128 ? sdpa::launch<f16_t, 128>(p, st) : sdpa::launch<f16_t, 64>(p, st);
+}
+
+}  // namespace
+
+extern "C" int xg_sdpa(const void* q, const void* k, const void* v, void* out, int64_t B, int64_t H, int64_t Hkv, int64_t Sq,
+                       int64_t Skv, int64_t D, const int64_t q_strides[3], const int64_t k_strides[3], const int64_t v_strides[3],
+                       const int64_t o_strides[3], float scale, int causal, int dtype, xg_stream_t stream) {
+  return sdpa_entry(q, k, v, out, nullptr, nullptr, dtype, nullptr, B, H, Hkv, Sq, Skv, D, q_strides, k_strides, v_strides, o_strides, scale,
+                    causal, dtype, stream);
+}
+
+extern "C" int xg_sdpa_masked(const void* q, const void* k, const void* v, void* out, const void* mask, const int64_t mask_strides[3],
+                              int mask_dtype, const float* scale_dev, int64_t B, int64_t H, int64_t Hkv, int64_t Sq, int64_t Skv,
+                              int64_t D, const int64_t q_strides[3], const int64_t k_strides[3], const int64_t v_strides[3],
+                              const int64_t o_strides[3], float scale, int causal, int dtype, xg_stream_t stream) {
+  return sdpa_entry(q, k, v, out, mask, mask_strides, mask_dtype, scale_dev, B, H, Hkv, Sq, Skv, D, q_strides, k_strides, v_strides,
+                    o_strides, scale, causal, dtype, stream);
 }

@@ -457,6 +457,7 @@ _library.define(
     "dense_fp8(Tensor x_q, Tensor w_q, bool weight_trans, Tensor x_scale, Tensor w_scale, Tensor? bias, str act, ScalarType out_dtype) -> Tensor"
 )
 _library.define("sdpa(Tensor q, Tensor k, Tensor v, bool is_causal, float scale) -> Tensor")
+_library.define("sdpa_masked(Tensor q, Tensor k, Tensor v, Tensor? mask, Tensor? scale_t, bool is_causal, float scale) -> Tensor")
 _library.define("rope(Tensor x, Tensor cos, Tensor sin) -> Tensor")
 
 
@@ -679,6 +680,61 @@ def _sdpa(q, k, v, is_causal, scale):
     return out
 
 
+def sdpa_mask_fits(mask_shape, q_shape, skv):
+    """An additive mask the kernel can index: up to 4-D, last two dims exactly [Sq, Skv], leading dims 1 or the
+    batch / head count (broadcast)."""
+    if len(mask_shape) < 2 or len(mask_shape) > 4:
+        return False
+    full = [1] * (4 - len(mask_shape)) + list(mask_shape)
+    B, H, Sq = q_shape[0], q_shape[1], q_shape[2]
+    return full[2] == Sq and full[3] == skv and full[0] in (1, B) and full[1] in (1, H)
+
+
+def _sdpa_masked(q, k, v, mask, scale_t, is_causal, scale):
+    """Attention with an additive mask and / or a scale held in a one-element device tensor (read by the kernel:
+    no .item(), no synchronisation)."""
+    _sdpa_check(q, k, v)
+    if k.dtype != q.dtype or v.dtype != q.dtype:
+        raise TypeError("sdpa: q, k, v must share a dtype")
+    q, k, v = _unit_last(q), _unit_last(k), _unit_last(v)
+    B, H, Sq, D = q.shape
+    Skv = k.shape[2]
+    out = _empty_like_layout(q)
+    if out.numel() == 0:
+        return out
+    S3 = ctypes.c_int64 * 3
+    mask_strides, mask_dt = None, _code(q.dtype)
+    if mask is not None:
+        if not sdpa_mask_fits(tuple(mask.shape), tuple(q.shape), Skv):
+            raise ValueError("sdpa_masked: the mask must be [Sq, Skv] with up to two leading dims of size 1, B or H")
+        if mask.dtype not in (q.dtype, torch.float32):
+            mask = mask.float() if mask.dtype.is_floating_point else None
+            if mask is None:
+                raise TypeError("sdpa_masked: the mask must be a floating-point additive mask")
+        while mask.dim() < 4:
+            mask = mask.unsqueeze(0)
+        if mask.stride(-1) != 1:
+            mask = mask.contiguous()
+        mask_strides = S3(*[0 if mask.shape[i] == 1 else mask.stride(i) for i in range(2)], mask.stride(2) if Sq > 1 else 0)
+        mask_dt = _code(mask.dtype)
+    if scale_t is not None:
+        if scale_t.numel() != 1:
+            raise ValueError("sdpa_masked: the scale tensor must have one element")
+        scale_t = scale_t.reshape(1).to(torch.float32)  # a device op, not a read
+    st = _lib.lib().xg_sdpa_masked(
+        _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(mask), mask_strides, mask_dt, _ptr(scale_t), B, H, k.shape[1], Sq, Skv, D,
+        S3(*q.stride()[:3]), S3(*k.stride()[:3]), S3(*v.stride()[:3]), S3(*out.stride()[:3]), scale, 1 if is_causal else 0,
+        _code(q.dtype), _stream(),
+    )
+    _lib.check(st, "xg_sdpa_masked")
+    return out
+
+
+def _sdpa_masked_meta(q, k, v, mask, scale_t, is_causal, scale):
+    _sdpa_check(q, k, v)
+    return _empty_like_layout(_unit_last(q))
+
+
 def _sdpa_meta(q, k, v, is_causal, scale):
     _sdpa_check(q, k, v)
     return _empty_like_layout(_unit_last(q))
@@ -771,6 +827,8 @@ _library.impl("dense_fp8", _dense_fp8, "CUDA")
 _library.impl("dense_fp8", _dense_fp8_meta, "Meta")
 _library.impl("sdpa", _sdpa, "CUDA")
 _library.impl("sdpa", _sdpa_meta, "Meta")
+_library.impl("sdpa_masked", _sdpa_masked, "CUDA")
+_library.impl("sdpa_masked", _sdpa_masked_meta, "Meta")
 _library.impl("rope", _rope, "CUDA")
 _library.impl("rope", _rope_meta, "Meta")
 

@@ -2,11 +2,17 @@
 
 Handles `aten.scaled_dot_product_attention` (what FusedSDPA emits) and the
 backend-specific ops it decomposes to when the user calls
-F.scaled_dot_product_attention directly.  An additive mask is accepted only if
-it is a compile-time constant equal to the causal mask (-inf or the dtype's
-lowest value strictly above the diagonal, 0 elsewhere); it is then dropped and
-the kernel masks by index.  The reference never detects causality
+F.scaled_dot_product_attention directly.  An additive mask that is a
+compile-time constant equal to the causal mask (-inf or the dtype's lowest
+value strictly above the diagonal, 0 elsewhere) is dropped and the kernel masks
+by index; the reference never detects causality
 (fuse_scaled_dot_product_attention.py:184-234 forwards the mask as attn_mask).
+Any other floating-point additive mask ([Sq, Skv] with broadcast batch / head
+dims) goes to the kernel as an operand, and so does the one-element scale
+tensor of the reference's `xpu_graph::sdpa_wrapped_scale` form
+(utils/default_replacements.py:39-55), which the kernel reads on the device
+instead of the host reading it with .item() (inference graphs only: these two
+forms carry no backward formula).
 
 The rewrite also looks through the contiguous clones and 3-D reshapes FusedSDPA
 puts in front of q, k, v: the kernel takes strides, so the [B, H, S, D] views
@@ -23,6 +29,7 @@ from ...pattern import Pattern, PatternGroup
 from ...utils.node_utils import VIEW_OPS, aten, is_call, is_getitem, same_shape
 
 SDPA_NAME = "mi355x_sdpa"
+SDPA_MASKED_NAME = "mi355x_sdpa_masked"
 _DTYPES = (torch.bfloat16, torch.float16)
 _HEAD_DIMS = (64, 128)
 _MAX_CONST_ELEMS = 1 << 26
@@ -31,6 +38,27 @@ _MAX_CONST_ELEMS = 1 << 26
 class SDPAModule(nn.Module):
     def forward(self, q, k, v, is_causal, scale):
         return torch.ops.xpu_ops.sdpa(q, k, v, is_causal, scale)
+
+
+class SDPAMaskedModule(nn.Module):
+    def forward(self, q, k, v, mask, scale_t, is_causal, scale):
+        return torch.ops.xpu_ops.sdpa_masked(q, k, v, mask, scale_t, is_causal, scale)
+
+
+def _mask_operand_ok(mask, q, k):
+    """A floating-point additive mask the kernel can index (see ops.sdpa_mask_fits), static in its last two dims."""
+    from ..... import ops as _xops
+
+    mv, qv, kv = mask.meta.get("val"), q.meta["val"], k.meta["val"]
+    if not isinstance(mv, torch.Tensor) or not mv.dtype.is_floating_point or mv.dtype not in (qv.dtype, torch.float32):
+        return False
+    if not all(isinstance(d, int) for d in list(mv.shape)[-2:]):
+        return False
+    lead = list(mv.shape)[:-2]
+    if any(not isinstance(d, int) and not same_shape([d], [qv.shape[0]]) for d in lead):
+        return False
+    shape = tuple(d if isinstance(d, int) else qv.shape[0] for d in mv.shape)
+    return _xops.sdpa_mask_fits(shape, tuple(qv.shape), kv.shape[2])
 
 
 def _const_eval(node, memo):
@@ -165,15 +193,28 @@ class FusedCausalSDPA(Pattern):
     _pattern_group = PatternGroup.GROUP1
     _support_stages = [FxStage.inference, FxStage.pregrad]  # sdpa carries a backward formula
 
-    def _emit(self, gm, node, q, k, v, causal, scale, replace):
+    def _emit(self, gm, node, q, k, v, causal, scale, replace, mask=None, scale_t=None):
         if scale is None:
             scale = 1.0 / math.sqrt(q.meta["val"].shape[-1])
         if not isinstance(scale, (int, float)):
             return False
         with gm.graph.inserting_before(node):
-            new = gm.graph.call_module(SDPA_NAME, args=(q, k, v, bool(causal), float(scale)))
+            if mask is None and scale_t is None:
+                new = gm.graph.call_module(SDPA_NAME, args=(q, k, v, bool(causal), float(scale)))
+            else:
+                if not hasattr(gm, SDPA_MASKED_NAME):
+                    gm.add_submodule(SDPA_MASKED_NAME, SDPAMaskedModule())
+                new = gm.graph.call_module(SDPA_MASKED_NAME, args=(q, k, v, mask, scale_t, bool(causal), float(scale)))
         replace(new)
         return True
+
+    def _wrapped_scale_calls(self, gm):
+        """call_module nodes of SDPAWrappedScale (what FusedSDPA emits for a tensor-valued scale)."""
+        from ...utils.default_replacements import SDPAWrappedScale
+
+        for node in list(gm.graph.nodes):
+            if node.op == "call_module" and isinstance(gm.get_submodule(node.target), SDPAWrappedScale) and len(node.args) == 5:
+                yield node
 
     def process(self, gm):
         if not hasattr(gm, SDPA_NAME):
@@ -203,10 +244,17 @@ class FusedCausalSDPA(Pattern):
                 if not all(isinstance(n, fx.Node) and isinstance(n.meta.get("val"), torch.Tensor) and n.meta["val"].dim() == 4 for n in (q, k, v)):
                     continue
                 sq, skv = q.meta["val"].shape[2], k.meta["val"].shape[2]
+                mask_operand = None
                 if mask is not None:
-                    if causal or not is_causal_constant(mask, sq, skv):
+                    if not causal and is_causal_constant(mask, sq, skv):
+                        causal = True
+                    elif self._current_stage == FxStage.inference and isinstance(mask, fx.Node) and _supported(q, k, v) and _mask_operand_ok(mask, q, k):
+                        mask_operand = mask  # the kernel adds it; q, k, v go as they are (no peeling: the mask is indexed by [B, H])
+                    else:
                         continue
-                    causal = True
+                if mask_operand is not None:
+                    changed |= self._emit(gm, node, q, k, v, causal, scale, node.replace_all_uses_with, mask=mask_operand)
+                    continue
                 q2 = _peel_qv(q, q.meta["val"].shape)
                 k2 = _peel_k(k, k.meta["val"].shape)
                 v2 = _peel_qv(v, v.meta["val"].shape)
@@ -253,4 +301,19 @@ class FusedCausalSDPA(Pattern):
                         u.replace_all_uses_with(new)
 
                 changed |= self._emit(gm, node, q, k, v, causal, node.kwargs.get("scale"), replace)
+        if self._current_stage == FxStage.inference:
+            for node in self._wrapped_scale_calls(gm):
+                q, k, v, mask, scale_t = node.args
+                if not all(isinstance(n, fx.Node) and isinstance(n.meta.get("val"), torch.Tensor) for n in (q, k, v, scale_t)):
+                    continue
+                if not _supported(q, k, v) or scale_t.meta["val"].numel() != 1:
+                    continue
+                causal = False
+                if mask is not None:
+                    sq, skv = q.meta["val"].shape[2], k.meta["val"].shape[2]
+                    if isinstance(mask, fx.Node) and is_causal_constant(mask, sq, skv):
+                        mask, causal = None, True
+                    elif not (isinstance(mask, fx.Node) and _mask_operand_ok(mask, q, k)):
+                        continue
+                changed |= self._emit(gm, node, q, k, v, causal, 1.0, node.replace_all_uses_with, mask=mask, scale_t=scale_t)
         return changed
