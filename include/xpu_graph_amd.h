@@ -204,6 +204,14 @@ int xg_dense_glu(const void* a, const void* w_gate, const void* w_up, void* out,
  * replaces torch_mlu_ops.batch_matmul as called by BatchDenseLayerModule.forward
  *   (passes/patterns/targets/mlu/structure_replacements/dense_layer_modules.py:71-111).
  *
+ * xg_dense_at: out[M,N] = a_t^T @ b (+ residual) with a_t [K,M] (row stride
+ *   lda) and b [K,N] (row stride ldb): the left operand arrives transposed, as
+ *   the weight gradient of a dense layer does (dW^T = dY^T X: a_t = dY [tokens,
+ *   out_features], b = X [tokens, in_features]).  M, N, lda, ldb, ldr multiples
+ *   of 8; any K.  fp32 accumulation, one rounding.
+ * replaces the mm(t(grad), x) of the backward graph the reference leaves to
+ *   the device's own matmul (tests/common/test_training.py:1-80 is its bar).
+ *
  * xg_dense_fp8: a_q [M,K] and b_q ([K,N] or [N,K], as above) are OCP e4m3fn
  *   bytes; out = act((a_q @ b_q) * a_scale * b_scale[n] + bias) in `out_dtype`
  *   (XG_BF16 / XG_F16 / XG_F32).  b_scale is f32[N], bias f32-or-out_dtype.
@@ -216,6 +224,8 @@ int xg_dense_batched(const void* a, const void* b, const void* bias, const void*
                      int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldr, int64_t stride_a,
                      int64_t stride_b, int64_t stride_bias, int64_t stride_res, int64_t stride_out, int b_trans,
                      int act, int dtype, int bias_dtype, xg_stream_t stream);
+int xg_dense_at(const void* a_t, const void* b, const void* residual, void* out, int64_t M, int64_t N, int64_t K,
+                int64_t lda, int64_t ldb, int64_t ldr, int dtype, xg_stream_t stream);
 int xg_dense_fp8(const void* a_q, const void* b_q, const float* a_scale_dev, const float* b_scale_dev,
                  const void* bias, void* out, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
                  int b_trans, int act, int out_dtype, int bias_dtype, xg_stream_t stream);

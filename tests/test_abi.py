@@ -19,7 +19,7 @@ def declared_symbols():
 def test_header_declares_the_expected_entry_points():
     syms = declared_symbols()
     for s in ("xg_rms_norm", "xg_layer_norm", "xg_add_rms_norm", "xg_add_layer_norm", "xg_slice_cat", "xg_addn",
-              "xg_combo_sum", "xg_slice_sum_cat", "xg_silu_mul", "xg_silu_mul2", "xg_dense", "xg_dense_batched", "xg_dense_glu", "xg_dense_fp8", "xg_slice_cat_check_table", "xg_sdpa", "xg_sdpa_masked", "xg_rope", "xg_copy_bytes",
+              "xg_combo_sum", "xg_slice_sum_cat", "xg_silu_mul", "xg_silu_mul2", "xg_dense", "xg_dense_batched", "xg_dense_at", "xg_dense_glu", "xg_dense_fp8", "xg_slice_cat_check_table", "xg_sdpa", "xg_sdpa_masked", "xg_rope", "xg_copy_bytes",
               "xg_version", "xg_status_string"):
         assert s in syms
 
@@ -124,6 +124,28 @@ def test_batched_dense_validation_needs_no_gpu():
     assert call(batch=70000) == -5
     assert call(K=12) == -3
     assert lib.xg_dense_batched(None, p, None, None, p, 2, 16, 16, 16, 16, 16, 0, 256, 256, 0, 0, 256, 0, 0, 2, 2, None) == -4
+
+
+def test_transposed_left_operand_validation_needs_no_gpu():
+    from xpu_graph_amd import _lib
+
+    lib = _lib.lib()
+    buf = ctypes.create_string_buffer(1 << 12)
+    p = ctypes.c_void_p((ctypes.addressof(buf) + 15) & ~15)
+    ok = dict(M=16, N=16, K=5, lda=16, ldb=16, ldr=0, dtype=2)
+
+    def call(**kw):
+        a = {**ok, **kw}
+        return lib.xg_dense_at(p, p, None, p, a["M"], a["N"], a["K"], a["lda"], a["ldb"], a["ldr"], a["dtype"], None)
+
+    assert call(M=12) == -3  # 16-byte loads along M
+    assert call(N=20, ldb=24) == -3
+    assert call(lda=8) == -2  # rows narrower than M
+    assert call(K=0) == -2
+    assert call(dtype=0) == -1  # fp32 has no kernel
+    assert lib.xg_dense_at(None, p, None, p, 16, 16, 8, 16, 16, 0, 2, None) == -4
+    off = ctypes.c_void_p(p.value + 2)
+    assert lib.xg_dense_at(off, p, None, p, 16, 16, 8, 16, 16, 0, 2, None) == -3
 
 
 def test_a_missing_library_is_an_error_not_a_fallback(monkeypatch, tmp_path):

@@ -202,6 +202,40 @@ def test_dense_batched_strided_entries(device):
         assert torch.equal(got[i], ops.dense(odd[i].contiguous(), w[i], False, None, None, "none"))
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize(
+    "K,M,N",
+    [(64, 256, 256), (256, 512, 768), (200, 264, 304), (1, 8, 8), (1000, 1032, 72), (4096, 320, 4096), (8192, 1024, 512), (77, 4096, 11008)],
+)
+def test_dense_with_transposed_left_operand(device, dtype, K, M, N):
+    """xg_dense_at: a_t [K, M]^T @ b [K, N], the weight gradient of a dense layer, against the fp32 product of the same
+    16-bit operands; K with and without whole 64-element slabs (direct loads / staged through registers), ragged M
+    and N tiles, with and without a residual."""
+    g = torch.Generator().manual_seed(K + M + N)
+    a_t = (torch.randn(K, M, generator=g) / K**0.25).to(dtype).to(device)
+    b = (torch.randn(K, N, generator=g) / K**0.25).to(dtype).to(device)
+    res = torch.randn(M, N, generator=g).to(dtype).to(device)
+    got = _ops().dense_at(a_t, b, None)
+    assert got.shape == (M, N) and got.dtype == dtype
+    want = a_t.float().t() @ b.float()
+    close(got, want, K)
+    got = _ops().dense_at(a_t, b, res)
+    close(got, want + res.float(), K)
+
+
+def test_dense_at_reads_strided_views_in_place(device):
+    ops = _ops()
+    big_a = torch.randn(300, 200, device=device).bfloat16()
+    big_b = torch.randn(300, 400, device=device).bfloat16()
+    a_t, b = big_a[:, 8:136], big_b[:, 16:336]  # row strides 200 and 400 elements, 16-byte aligned bases
+    got = ops.dense_at(a_t, b, None)
+    close(got, a_t.float().t() @ b.float(), 300)
+    a_t = big_a[:, 3:131]  # base 6 bytes off: the wrapper copies
+    close(ops.dense_at(a_t, b, None), a_t.float().t() @ b.float(), 300)
+    with pytest.raises(ValueError, match="M % 8"):
+        ops.dense_at(big_a[:, :12], b, None)
+
+
 def test_dense_takes_column_sliced_views(device):
     """A linear layer fed by a column slice of a wider tensor: row strides or bases that are not multiples of 16 bytes
     (what eager accepts anywhere) are copied by the wrapper instead of being refused by the kernel."""

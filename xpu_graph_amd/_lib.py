@@ -81,6 +81,7 @@ _SIGNATURES = {
         c_int,
         [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p] + [c_int64] * 12 + [c_int, c_int, c_int, c_int, c_void_p],
     ),
+    "xg_dense_at": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p] + [c_int64] * 6 + [c_int, c_void_p]),
     "xg_dense_fp8": (
         c_int,
         [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64, c_int, c_int, c_int, c_int, c_void_p],

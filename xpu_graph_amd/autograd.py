@@ -18,8 +18,9 @@ a few microseconds of dispatch, which inference-only processes should not pay.
     add_rms_norm_only / add_layer_norm_only                         the same, returning y alone
 
 The input gradient of the dense layer is itself a dense layer over the same weight read the other way, so it runs on
-the HIP kernel; the weight gradient needs a transposed left operand, which that kernel does not take, and is an Aten
-matmul.  For activations whose derivative cannot be told from the output (silu, gelu) the pre-activation is
+the HIP kernel; the weight gradient is a product with a transposed LEFT operand (gz^T x), which the same kernel
+takes in place through xpu_ops::dense_at (shapes it does not take -- a dimension that is no multiple of 8 -- fall to
+an Aten matmul).  For activations whose derivative cannot be told from the output (silu, gelu) the pre-activation is
 recomputed with one more dense call.  The gated layer saves only its inputs: both projections are recomputed on the
 dense kernel, the two input-gradient products run as one chain (the second takes the first as its residual).
 """
@@ -103,6 +104,15 @@ def _silu_mul_backward(ctx, gy):
     return (torch.cat([yf * b * _silu_grad(a), yf * torch.nn.functional.silu(a)], dim=-1).to(x.dtype),)
 
 
+def _weight_grad(a_t, b):
+    """a_t^T @ b for 2-D operands [tokens, M], [tokens, N]: on the dense kernel when it takes the shape."""
+    from . import ops
+
+    if ops.dense_at_fits(tuple(a_t.shape), tuple(b.shape), a_t.dtype) and a_t.dtype == b.dtype:
+        return torch.ops.xpu_ops.dense_at(a_t, b, None)
+    return a_t.t() @ b
+
+
 def _dense_setup(ctx, inputs, output):
     x, weight, weight_trans, bias, residual, act = inputs
     ctx.save_for_backward(x, weight, output, *(t for t in (bias, residual) if t is not None))
@@ -139,7 +149,7 @@ def _dense_backward(ctx, gy):
     gx = torch.ops.xpu_ops.dense(gz, weight, not ctx.trans, None, None, "none") if need[0] else None
     gw = None
     if need[1]:
-        gw = (gz.t() @ x) if ctx.trans else (x.t() @ gz)
+        gw = _weight_grad(gz, x) if ctx.trans else _weight_grad(x, gz)
     gb = gz.float().sum(0).to(bias.dtype) if ctx.has_bias and need[3] else None
     gr = gz if ctx.has_res and need[4] else None
     return gx, gw, None, gb, gr, None
@@ -161,8 +171,8 @@ def _dense_glu_backward(ctx, gy):
     gx = None
     if need[0]:
         gx = dense(d_up, w_up, False, None, dense(d_gate, w_gate, False, None, None, "none"), "none")
-    gwg = d_gate.t() @ x if need[1] else None
-    gwu = d_up.t() @ x if need[2] else None
+    gwg = _weight_grad(d_gate, x) if need[1] else None
+    gwu = _weight_grad(d_up, x) if need[2] else None
     return gx, gwg, gwu
 
 

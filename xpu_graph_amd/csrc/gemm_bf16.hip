@@ -4,6 +4,8 @@
 namespace xg {
 namespace gemm {
 int launch_f16(const GemmParams& p, bool b_trans, hipStream_t st);  // gemm_f16.hip
+int launch_at_f16(const GemmParams& p, hipStream_t st);               // gemm_f16.hip
+int launch_at_bf16(const GemmParams& p, hipStream_t st) { return launch_gemm_at<bf16_t, bf16_t>(p, st); }
 int launch_glu_f16(const GemmParams& p, hipStream_t st);              // gemm_f16.hip
 int launch_glu_bf16(const GemmParams& p, hipStream_t st) { return launch_glu<bf16_t, bf16_t>(p, st); }
 int launch_bf16(const GemmParams& p, bool b_trans, hipStream_t st) {
@@ -67,6 +69,23 @@ int xg_dense_batched(const void* a, const void* b, const void* bias, const void*
   p.out_batch = stride_out * 2;
   hipStream_t st = (hipStream_t)stream;
   return dtype == XG_BF16 ? gemm::launch_bf16(p, b_trans != 0, st) : gemm::launch_f16(p, b_trans != 0, st);
+}
+
+int xg_dense_at(const void* a_t, const void* b, const void* residual, void* out, int64_t M, int64_t N, int64_t K,
+                int64_t lda, int64_t ldb, int64_t ldr, int dtype, xg_stream_t stream) {
+  using namespace xg;
+  using namespace xg::gemm;
+  if (a_t == nullptr || b == nullptr || out == nullptr) return XG_ERR_NULL_PTR;
+  if (M <= 0 || N <= 0 || K <= 0 || lda < M || ldb < N || (residual && ldr < N)) return XG_ERR_BAD_SHAPE;
+  if (M > 0x7fffffff || N > 0x7fffffff || K > 0x7fffffff) return XG_ERR_TOO_LARGE;
+  if (dtype != XG_BF16 && dtype != XG_F16) return XG_ERR_BAD_DTYPE;
+  // 16-byte loads along M and N, 16-byte output stores; K is free (a partial last slab reads as zero)
+  if (M % 8 != 0 || N % 8 != 0 || lda % 8 != 0 || ldb % 8 != 0 || (residual && ldr % 8 != 0)) return XG_ERR_BAD_ALIGN;
+  if (!aligned_to(a_t, 16) || !aligned_to(b, 16) || !aligned_to(out, 16) || (residual && !aligned_to(residual, 16)))
+    return XG_ERR_BAD_ALIGN;
+  const GemmParams p = make_params(a_t, b, nullptr, residual, out, M, N, K, lda, ldb, ldr, XG_ACT_NONE, false);
+  hipStream_t st = (hipStream_t)stream;
+  return dtype == XG_BF16 ? gemm::launch_at_bf16(p, st) : gemm::launch_at_f16(p, st);
 }
 
 int xg_dense_glu(const void* a, const void* w_gate, const void* w_up, void* out, int64_t M, int64_t N, int64_t K,

@@ -82,6 +82,11 @@ constexpr int kXcds = 8;
 constexpr int kGroupM = 8;
 
 enum class BLayout { KMajor, NMajor };  // B stored [N, K] (K contiguous) or [K, N] (N contiguous)
+// A stored [M, K] (K contiguous) or [K, M] (M contiguous: the left operand arrives transposed, as in a weight
+// gradient dW = X^T dY).  An M-contiguous A slab is laid out and read exactly like an N-contiguous B slab --
+// [64 k][256 m] in LDS, fetched with the transposing LDS read -- and is wired for 16-bit elements, N-contiguous B
+// and full-height (256-row) tiles only.
+enum class ALayout { KMajor, MMajor };
 
 struct GemmParams {
   const void* A;
@@ -239,12 +244,21 @@ struct Lane {
 };
 
 // Unit U (0..3: A tile row U, 4..7: B tile column U-4) of the fragments of k-step ks from the slabs at a_s / b_s.
-template <typename T, BLayout BL, int U>
+template <typename T, BLayout BL, int U, ALayout AL = ALayout::KMajor>
 __device__ __forceinline__ void read_unit(const Lane& L, const char* a_s, const char* b_s, int ks, Frag<T> (&fa)[4],
                                           Frag<T> (&fb)[4]) {
   if constexpr (Elem<T>::BYTES == 2) {
     const int ch = ((ks * 2 + L.half) ^ L.fsw) << 4;
-    if constexpr (U < 4) {
+    if constexpr (U < 4 && AL == ALayout::MMajor) {
+      // slab is [64 k][256 m]: the same transposing read as for an N-contiguous B, with this wave's row units
+      const int gran = ((L.wm * 4 + U) ^ L.tr_sw) & 7;
+      const int col = (gran << 6) + (L.blk << 5) + ((L.p16 & 3) << 3);
+      const int row0 = ks * 16 + L.half * 8 + (L.p16 >> 2);
+      const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(a_s + row0 * (BM * 2) + col));
+      const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(a_s + (row0 + 4) * (BM * 2) + col));
+      const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
+      fa[U].v = u32x4{l2.x, l2.y, h2.x, h2.y};
+    } else if constexpr (U < 4) {
       fa[U].v = *reinterpret_cast<const u32x4*>(a_s + L.a_row[U] + ch);
     } else if constexpr (BL == BLayout::KMajor) {
       fb[U - 4].v = *reinterpret_cast<const u32x4*>(b_s + L.b_row[U - 4] + ch);
@@ -273,12 +287,12 @@ __device__ __forceinline__ void read_unit(const Lane& L, const char* a_s, const 
 }
 
 // All fragments of k-step ks (NI A units, 4 B units).
-template <typename T, BLayout BL, int NI = 4>
+template <typename T, BLayout BL, int NI = 4, ALayout AL = ALayout::KMajor>
 __device__ __forceinline__ void read_frags(const Lane& L, const char* a_s, const char* b_s, int ks, Frag<T> (&fa)[4],
                                            Frag<T> (&fb)[4]) {
   static_for<8>([&](auto U) {
     constexpr int u = decltype(U)::value;
-    if constexpr (u >= 4 || u < NI) read_unit<T, BL, u>(L, a_s, b_s, ks, fa, fb);
+    if constexpr (u >= 4 || u < NI) read_unit<T, BL, u, AL>(L, a_s, b_s, ks, fa, fb);
   });
 }
 
@@ -476,9 +490,10 @@ __device__ __forceinline__ void zero_acc(f32x16 (&acc)[4][4]) {
 // the same 128 rows of the up weight, so waves with wn = 0 accumulate x Wg^T and waves with wn = 1 accumulate
 // x Wu^T for the SAME 128 output columns; the epilogue writes silu(gate) * up.  A slabs are shared, so the
 // operand traffic per output element is that of two separate layers minus one read of x.
-template <typename T, typename OT, BLayout BL, int NI, bool GLU = false>
+template <typename T, typename OT, BLayout BL, int NI, bool GLU = false, ALayout AL = ALayout::KMajor>
 __device__ __forceinline__ void gemm_dma_tile(const GemmParams& p, int bid, int nb, char* smem) {
   static_assert(!GLU || BL == BLayout::KMajor, "the gated layer is wired for K-contiguous weights");
+  static_assert(AL == ALayout::KMajor || (BL == BLayout::NMajor && NI == 4 && !GLU), "M-contiguous A: N-contiguous B, full tiles");
   constexpr int EB = Elem<T>::BYTES;
   constexpr int KSTEPS = Elem<T>::KSTEPS;
   constexpr int SLAB_K = ROW_BYTES / EB;
@@ -498,9 +513,19 @@ __device__ __forceinline__ void gemm_dma_tile(const GemmParams& p, int bid, int 
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       const int r = j * 32 + L.wave * 8 + lrow;
-      int gr = m0 + r;
-      gr = gr < p.M ? gr : p.M - 1;  // rows past the edge re-read the last row; their results are never stored
-      a_off[j] = (uint32_t)(((int64_t)gr * p.lda) * EB + lc * 16);
+      if constexpr (AL == ALayout::KMajor) {
+        int gr = m0 + r;
+        gr = gr < p.M ? gr : p.M - 1;  // rows past the edge re-read the last row; their results are never stored
+        a_off[j] = (uint32_t)(((int64_t)gr * p.lda) * EB + lc * 16);
+      } else {
+        const int kr = j * 8 + L.wave * 2 + L.half;
+        const int pc32 = L.lane & 31;
+        const int sw = ((L.wave * 2 + L.half) & 3) | ((j & 1) << 2);
+        const int gran = ((pc32 >> 2) ^ sw) & 7;
+        int gc = m0 + (gran * 4 + (pc32 & 3)) * 8;
+        gc = gc < p.M ? gc : (p.M - 8);  // M % 8 == 0 is checked on the host
+        a_off[j] = (uint32_t)(((int64_t)kr * p.lda + gc) * EB);
+      }
       if constexpr (BL == BLayout::KMajor) {
         int gn = n0 + (GLU ? (r & 127) : r);  // gated: tile rows 128..255 are rows 0..127 again, of the up weight
         gn = gn < p.N ? gn : p.N - 1;
@@ -516,7 +541,7 @@ __device__ __forceinline__ void gemm_dma_tile(const GemmParams& p, int bid, int 
       }
     }
   }
-  const int64_t a_step = ROW_BYTES;
+  const int64_t a_step = AL == ALayout::KMajor ? (int64_t)ROW_BYTES : (int64_t)SLAB_K * p.lda * EB;
   const int64_t b_step = BL == BLayout::KMajor ? (int64_t)ROW_BYTES : (int64_t)SLAB_K * p.ldb * EB;
   const int wave_u = __builtin_amdgcn_readfirstlane(L.wave);  // LDS destinations of direct loads are wavefront-uniform
   const char* const a_base = reinterpret_cast<const char*>(p.A);
@@ -541,9 +566,15 @@ __device__ __forceinline__ void gemm_dma_tile(const GemmParams& p, int bid, int 
   const char* pfa_ptr;
   const char* pfb_ptr;
   {
-    int gr = m0 + L.tid;
-    gr = gr < p.M ? gr : p.M - 1;
-    pfa_ptr = reinterpret_cast<const char*>(p.A) + ((int64_t)gr * p.lda) * EB;
+    if constexpr (AL == ALayout::KMajor) {
+      int gr = m0 + L.tid;
+      gr = gr < p.M ? gr : p.M - 1;
+      pfa_ptr = reinterpret_cast<const char*>(p.A) + ((int64_t)gr * p.lda) * EB;
+    } else {
+      int gc = m0 + (L.tid & 3) * 64;
+      gc = gc < p.M ? gc : (p.M - 8);
+      pfa_ptr = reinterpret_cast<const char*>(p.A) + ((int64_t)(L.tid >> 2) * p.lda + gc) * EB;
+    }
     if constexpr (BL == BLayout::KMajor) {
       int gn = n0 + (GLU ? (L.tid & 127) : L.tid);
       gn = gn < p.N ? gn : p.N - 1;
@@ -596,7 +627,7 @@ __device__ __forceinline__ void gemm_dma_tile(const GemmParams& p, int bid, int 
     wait_vm<0>();
   }
   barrier_only();
-  read_frags<T, BL, NI>(L, smem, smem + SLAB_BYTES, 0, fa[0], fb[0]);
+  read_frags<T, BL, NI, AL>(L, smem, smem + SLAB_BYTES, 0, fa[0], fb[0]);
 
   // One slab of math, written in issue order.  NEXT: slab kt+1 exists (hand it over in front of the last
   // k-step and fetch its first fragments under that step); NEXT2: slab kt+2 exists (its direct loads go
@@ -639,8 +670,8 @@ __device__ __forceinline__ void gemm_dma_tile(const GemmParams& p, int bid, int 
         constexpr int idx = decltype(IDX)::value;
         constexpr int i = idx / 4, j = idx % 4;
         if constexpr (idx < 8 && (idx >= 4 || idx < NI)) {  // units 0..3 are A tile rows: a 128-row tile has two
-          if constexpr (!last_step) read_unit<T, BL, idx>(L, a_s, b_s, ks + 1, fa[(ks + 1) & 1], fb[(ks + 1) & 1]);
-          else if constexpr (next) read_unit<T, BL, idx>(L, a_n, b_n, 0, fa[0], fb[0]);
+          if constexpr (!last_step) read_unit<T, BL, idx, AL>(L, a_s, b_s, ks + 1, fa[(ks + 1) & 1], fb[(ks + 1) & 1]);
+          else if constexpr (next) read_unit<T, BL, idx, AL>(L, a_n, b_n, 0, fa[0], fb[0]);
         }
         // direct loads: the rest of slab kt+1 early in this slab, the head of slab kt+2 after the barrier
         if constexpr (next && ks == 0 && !last_step) {
@@ -667,10 +698,10 @@ __device__ __forceinline__ void gemm_dma_tile(const GemmParams& p, int bid, int 
   else epilogue<OT, NI>(p, L, acc, smem, m0, n0);
 }
 
-template <typename T, typename OT, BLayout BL>
+template <typename T, typename OT, BLayout BL, ALayout AL = ALayout::KMajor>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_dma_kernel(GemmParams p) {
   extern __shared__ __align__(16) char smem[];
-  gemm_dma_tile<T, OT, BL, 4>(for_batch_entry(p), blockIdx.x, gridDim.x, smem);
+  gemm_dma_tile<T, OT, BL, 4, false, AL>(for_batch_entry(p), blockIdx.x, gridDim.x, smem);
 }
 
 // One launch for two tile grids: the first n_full workgroups compute the 256 x 256 tiles of `full`, the others the
@@ -720,7 +751,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
   gemm_dma_tile<T, OT, BLayout::KMajor, 2, true>(p, blockIdx.x, gridDim.x, smem);
 }
 
-template <typename T, typename OT, BLayout BL>
+template <typename T, typename OT, BLayout BL, ALayout AL = ALayout::KMajor>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_staged_kernel(GemmParams p_all) {
   extern __shared__ __align__(16) char smem[];
   const GemmParams p = for_batch_entry(p_all);
@@ -728,6 +759,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
   constexpr int KSTEPS = Elem<T>::KSTEPS;
   constexpr int SLAB_K = ROW_BYTES / EB;
   static_assert(BL == BLayout::KMajor || EB == 2, "the transposing LDS read is wired for 16-bit elements only");
+  static_assert(AL == ALayout::KMajor || BL == BLayout::NMajor, "M-contiguous A goes with N-contiguous B");
 
   int tm, tn;
   tile_of_block(p, blockIdx.x, gridDim.x, tm, tn);
@@ -740,13 +772,27 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
   const char* a_ptr[8];
   const char* b_ptr[8];
   int a_lds[8], b_lds[8];
+  if constexpr (AL == ALayout::KMajor) {
 #pragma unroll
-  for (int j = 0; j < 8; ++j) {
-    const int r = r0 + 32 * j;
-    int gr = m0 + r;
-    gr = gr < p.M ? gr : p.M - 1;
-    a_ptr[j] = reinterpret_cast<const char*>(p.A) + ((int64_t)gr * p.lda) * EB + c8 * 16;
-    a_lds[j] = r * ROW_BYTES + ((c8 ^ swz(r)) << 4);
+    for (int j = 0; j < 8; ++j) {
+      const int r = r0 + 32 * j;
+      int gr = m0 + r;
+      gr = gr < p.M ? gr : p.M - 1;
+      a_ptr[j] = reinterpret_cast<const char*>(p.A) + ((int64_t)gr * p.lda) * EB + c8 * 16;
+      a_lds[j] = r * ROW_BYTES + ((c8 ^ swz(r)) << 4);
+    }
+  } else {
+    // M-major operand: slab is [64 k][256 m], covered like the N-major B slab below
+    const int c32 = tid & 31, kr0 = tid >> 5;
+    int gc = m0 + c32 * 8;
+    gc = gc < p.M ? gc : (p.M - 8);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int kr = kr0 + 8 * j;
+      a_ptr[j] = reinterpret_cast<const char*>(p.A) + ((int64_t)kr * p.lda + gc) * EB;
+      const int sw = (kr & 3) | (((kr >> 3) & 1) << 2);
+      a_lds[j] = kr * (BM * EB) + ((((c32 >> 2) ^ sw) & 7) << 6) + ((c32 & 3) << 4);
+    }
   }
   if constexpr (BL == BLayout::KMajor) {
 #pragma unroll
@@ -774,7 +820,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
   u32x4 ga[8], gb[8];
   auto load_slab = [&](int kt) {
     const int k_left = p.K - kt * SLAB_K;  // elements of K still valid from this slab's start
-    const int64_t koff = (int64_t)kt * ROW_BYTES;
+    const int64_t koff = AL == ALayout::KMajor ? (int64_t)kt * ROW_BYTES : (int64_t)kt * SLAB_K * p.lda * EB;
     const int64_t boff = BL == BLayout::KMajor ? koff : (int64_t)kt * SLAB_K * p.ldb * EB;
     if (k_left >= SLAB_K) {  // uniform: a whole slab, no per-load predicate
 #pragma unroll
@@ -783,8 +829,10 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
       for (int j = 0; j < 8; ++j) gb[j] = *reinterpret_cast<const u32x4*>(b_ptr[j] + boff);
     } else {  // the last, partial slab: chunks past K read as zero
 #pragma unroll
-      for (int j = 0; j < 8; ++j)
-        ga[j] = (c8 * (16 / EB) < k_left) ? *reinterpret_cast<const u32x4*>(a_ptr[j] + koff) : u32x4{0, 0, 0, 0};
+      for (int j = 0; j < 8; ++j) {
+        const bool ok = AL == ALayout::KMajor ? (c8 * (16 / EB) < k_left) : ((tid >> 5) + 8 * j < k_left);
+        ga[j] = ok ? *reinterpret_cast<const u32x4*>(a_ptr[j] + koff) : u32x4{0, 0, 0, 0};
+      }
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         const bool ok = BL == BLayout::KMajor ? (c8 * (16 / EB) < k_left) : ((tid >> 5) + 8 * j < k_left);
@@ -815,7 +863,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ++ks) {
       Frag<T> fa[4], fb[4];
-      read_frags<T, BL>(L, a_s, b_s, ks, fa, fb);
+      read_frags<T, BL, 4, AL>(L, a_s, b_s, ks, fa, fb);
       mma_step<T>(acc, fa, fb);
       if (ks == 0 && kt + 1 < KT) store_slab(stage ^ 1);  // slab kt+1: registers -> the idle LDS stage
       if (ks == 1 && kt + 2 < KT) load_slab(kt + 2);      // slab kt+2: memory -> registers
@@ -1055,12 +1103,12 @@ int launch_kernel(K kernel, const GemmParams& p, hipStream_t stream) {
 
 // The direct-to-LDS kernel needs whole slabs and 31-bit operand offsets.
 template <typename T>
-bool dma_ok(const GemmParams& p, BLayout bl) {
+bool dma_ok(const GemmParams& p, BLayout bl, ALayout al = ALayout::KMajor) {
   constexpr int EB = Elem<T>::BYTES;
   constexpr int SLAB_K = ROW_BYTES / EB;
   if (p.K % SLAB_K != 0) return false;
   const int64_t lim = 0x7fffffffLL;
-  const int64_t a_bytes = ((int64_t)p.M * p.lda) * EB;
+  const int64_t a_bytes = al == ALayout::KMajor ? ((int64_t)p.M * p.lda) * EB : ((int64_t)SLAB_K * p.lda + p.M) * EB;
   const int64_t b_bytes = bl == BLayout::KMajor ? ((int64_t)p.N * p.ldb) * EB : ((int64_t)SLAB_K * p.ldb + p.N) * EB;
   return a_bytes < lim && b_bytes < lim;
 }
@@ -1160,6 +1208,15 @@ int launch_gemm(const GemmParams& p, hipStream_t stream) {
   if (n_full + n_rest > 0x7fffffffLL) return XG_ERR_TOO_LARGE;
   hipLaunchKernelGGL(kernel, dim3((unsigned)(n_full + n_rest), 1), dim3(kThreads), SMEM_BYTES, stream, full, rest, (int)n_full);
   return status_from_hip(hipGetLastError());
+}
+
+// Left operand transposed in memory: out[M, N] = At^T B with At [K, M] (row stride lda) and B [K, N], the shape of a
+// weight gradient.  Full-height tiles only (whole slabs by direct loads, any K through registers).
+template <typename T, typename OT>
+int launch_gemm_at(const GemmParams& p, hipStream_t stream) {
+  if (!dma_ok<T>(p, BLayout::NMajor, ALayout::MMajor))
+    return launch_kernel(gemm_staged_kernel<T, OT, BLayout::NMajor, ALayout::MMajor>, p, stream);
+  return launch_kernel(gemm_dma_kernel<T, OT, BLayout::NMajor, ALayout::MMajor>, p, stream);
 }
 
 // Gated layer: out[M, N] = silu(A Wg^T) * (A Wu^T), Wg = p.B and Wu = p.B2 both [N, K] with row stride ldb.

@@ -45,11 +45,13 @@ struct OutTable {
   int64_t row_bytes[XG_SLICE_CAT_MAX_OUTS];
 };
 
-constexpr int kBlock = 256;
-
-// RU = rows in flight per lane (unrolled loads before the matching stores).
-template <int CB, int RU, bool MULTI>
-__global__ __launch_bounds__(kBlock) void slice_cat_kernel(const char* __restrict__ src, int64_t src_row_bytes,
+// RU = rows in flight per lane (unrolled loads before the matching stores); KB = lanes per block.
+// Loads are ordinary (cached) loads: a slice that straddles a 128-byte line shares that line with the
+// neighbouring lanes' requests and with the next row strip, and measured 3-4 % faster than streaming
+// loads on the 64 x 128-byte-slice case; the stores bypass the cache (streaming stores measured 15 % faster
+// than cached ones there).
+template <int CB, int RU, int KB, bool MULTI>
+__global__ __launch_bounds__(KB) void slice_cat_kernel(const char* __restrict__ src, int64_t src_row_bytes,
                                                            int64_t rows, OutTable outs, int n_outs,
                                                            const xg_chunk* __restrict__ table, int64_t n_chunks,
                                                            int rows_per_block) {
@@ -64,7 +66,7 @@ __global__ __launch_bounds__(kBlock) void slice_cat_kernel(const char* __restric
     }
     __syncthreads();
   }
-  const int64_t ci = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  const int64_t ci = (int64_t)blockIdx.x * KB + threadIdx.x;
   if (ci >= n_chunks) return;
   const xg_chunk ch = table[ci];
   char* dst;
@@ -83,7 +85,7 @@ __global__ __launch_bounds__(kBlock) void slice_cat_kernel(const char* __restric
   for (; r0 + RU <= r_end; r0 += RU) {
     store_t v[RU];
 #pragma unroll
-    for (int u = 0; u < RU; ++u) v[u] = __builtin_nontemporal_load(reinterpret_cast<const load_t*>(s + u * src_row_bytes));
+    for (int u = 0; u < RU; ++u) v[u] = *reinterpret_cast<const load_t*>(s + u * src_row_bytes);
 #pragma unroll
     for (int u = 0; u < RU; ++u) __builtin_nontemporal_store(v[u], reinterpret_cast<store_t*>(d + u * dst_rb));
     s += RU * src_row_bytes;
@@ -97,10 +99,10 @@ __global__ __launch_bounds__(kBlock) void slice_cat_kernel(const char* __restric
   }
 }
 
-template <int CB>
-int launch(const char* src, int64_t src_row_bytes, int64_t rows, const OutTable& outs, int n_outs,
+template <int CB, int KB>
+int launch_kb(const char* src, int64_t src_row_bytes, int64_t rows, const OutTable& outs, int n_outs,
            const xg_chunk* table, int64_t n_chunks, hipStream_t stream) {
-  const int64_t gx = (n_chunks + kBlock - 1) / kBlock;
+  const int64_t gx = (n_chunks + KB - 1) / KB;
   // Rows per block: enough blocks to cover the 256 CUs several times over, but a
   // strip long enough that each lane amortises its table entry.
   int rpb = 8;
@@ -109,12 +111,21 @@ int launch(const char* src, int64_t src_row_bytes, int64_t rows, const OutTable&
   if (gx > 0x7fffffffLL || gy > 65535) return XG_ERR_TOO_LARGE;
   dim3 grid((unsigned)gx, (unsigned)gy);
   if (n_outs == 1)
-    hipLaunchKernelGGL((slice_cat_kernel<CB, 8, false>), grid, dim3(kBlock), 0, stream, src, src_row_bytes, rows, outs,
+    hipLaunchKernelGGL((slice_cat_kernel<CB, 8, KB, false>), grid, dim3(KB), 0, stream, src, src_row_bytes, rows, outs,
                        n_outs, table, n_chunks, rpb);
   else
-    hipLaunchKernelGGL((slice_cat_kernel<CB, 8, true>), grid, dim3(kBlock), 0, stream, src, src_row_bytes, rows, outs,
+    hipLaunchKernelGGL((slice_cat_kernel<CB, 8, KB, true>), grid, dim3(KB), 0, stream, src, src_row_bytes, rows, outs,
                        n_outs, table, n_chunks, rpb);
   return status_from_hip(hipGetLastError());
+}
+
+// 512 lanes per block once a row has that many chunks (one block then spans a whole 8 KiB output row of 16-byte
+// chunks: 4 % faster than two 256-lane blocks on the 64-slice case), 256 otherwise.
+template <int CB>
+int launch(const char* src, int64_t src_row_bytes, int64_t rows, const OutTable& outs, int n_outs,
+           const xg_chunk* table, int64_t n_chunks, hipStream_t stream) {
+  return n_chunks >= 512 ? launch_kb<CB, 512>(src, src_row_bytes, rows, outs, n_outs, table, n_chunks, stream)
+                         : launch_kb<CB, 256>(src, src_row_bytes, rows, outs, n_outs, table, n_chunks, stream);
 }
 
 }  // namespace

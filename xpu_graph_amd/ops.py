@@ -452,6 +452,7 @@ def build_slice_table(slice_lists, src_cols, elem_size, src_row_stride=None):
 # ------------------------------------------------------------- dense / SDPA
 _library.define("dense(Tensor x, Tensor weight, bool weight_trans, Tensor? bias, Tensor? residual, str act) -> Tensor")
 _library.define("dense_batched(Tensor x, Tensor weight, bool weight_trans, Tensor? bias, Tensor? residual, str act) -> Tensor")
+_library.define("dense_at(Tensor a_t, Tensor b, Tensor? residual) -> Tensor")
 _library.define("dense_glu(Tensor x, Tensor w_gate, Tensor w_up) -> Tensor")
 _library.define(
     "dense_fp8(Tensor x_q, Tensor w_q, bool weight_trans, Tensor x_scale, Tensor w_scale, Tensor? bias, str act, ScalarType out_dtype) -> Tensor"
@@ -589,6 +590,44 @@ def _dense_batched_meta(x, weight, weight_trans, bias, residual, act):
 def _dense_meta(x, weight, weight_trans, bias, residual, act):
     m, n, _ = _dense_out_shape(x, weight, weight_trans)
     return torch.empty((m, n), dtype=x.dtype, device=x.device)
+
+
+def dense_at_fits(a_shape, b_shape, dtype):
+    """What xg_dense_at takes: a_t [K, M], b [K, N], M and N multiples of 8, 16-bit floats; any K."""
+    if len(a_shape) != 2 or len(b_shape) != 2 or dtype not in (torch.bfloat16, torch.float16):
+        return False
+    m, n = a_shape[1], b_shape[1]
+    return isinstance(m, int) and isinstance(n, int) and m > 0 and n > 0 and m % 8 == 0 and n % 8 == 0
+
+
+def _dense_at(a_t, b, residual):
+    """a_t.T @ b (+ residual) without materialising the transpose: a_t [K, M], b [K, N] -> [M, N].  The weight gradient
+    of a dense layer (gz.T @ x, or x.T @ gz) in one launch of the dense kernel."""
+    if a_t.dim() != 2 or b.dim() != 2 or a_t.shape[0] != b.shape[0]:
+        raise ValueError("dense_at: a_t must be [K, M] and b [K, N]")
+    if a_t.dtype != b.dtype:
+        raise TypeError("dense_at: operands must share a dtype")
+    k, m = a_t.shape
+    n = b.shape[1]
+    if not dense_at_fits(tuple(a_t.shape), tuple(b.shape), a_t.dtype):
+        raise ValueError("dense_at: needs M % 8 == 0, N % 8 == 0, bf16 or f16")
+    out = torch.empty((m, n), dtype=a_t.dtype, device=a_t.device)
+    if k == 0:
+        return out.zero_() if residual is None else out.copy_(residual)
+    a_t, b = _row_major(a_t), _row_major(b)
+    ldr = 0
+    if residual is not None:
+        if tuple(residual.shape) != (m, n) or residual.dtype != a_t.dtype:
+            raise ValueError("dense_at: residual must be [M, N] in the operand dtype")
+        residual = _row_major(residual)
+        ldr = residual.stride(0)
+    st = _lib.lib().xg_dense_at(_ptr(a_t), _ptr(b), _ptr(residual), _ptr(out), m, n, k, a_t.stride(0), b.stride(0), ldr, _code(a_t.dtype), _stream())
+    _lib.check(st, "xg_dense_at")
+    return out
+
+
+def _dense_at_meta(a_t, b, residual):
+    return torch.empty((a_t.shape[1], b.shape[1]), dtype=a_t.dtype, device=a_t.device)
 
 
 def _dense_fp8(x_q, w_q, weight_trans, x_scale, w_scale, bias, act, out_dtype):
@@ -821,6 +860,8 @@ _library.impl("dense", _dense, "CUDA")
 _library.impl("dense_glu", _dense_glu, "CUDA")
 _library.impl("dense_glu", lambda x, w_gate, w_up: torch.empty((x.shape[0], w_gate.shape[0]), dtype=x.dtype, device=x.device), "Meta")
 _library.impl("dense", _dense_meta, "Meta")
+_library.impl("dense_at", _dense_at, "CUDA")
+_library.impl("dense_at", _dense_at_meta, "Meta")
 _library.impl("dense_batched", _dense_batched, "CUDA")
 _library.impl("dense_batched", _dense_batched_meta, "Meta")
 _library.impl("dense_fp8", _dense_fp8, "CUDA")
