@@ -266,6 +266,32 @@ int xg_sdpa_masked(const void* q, const void* k, const void* v, void* out, const
                    int causal, int dtype, xg_stream_t stream);
 
 /* ---------------------------------------------------------------------------
+ * Attention for graphs that are differentiated (the reference compiles
+ * training graphs through AOT autograd and leaves attention's backward to the
+ * device's own kernels: compiler.py:105-180, tests/common/test_training.py).
+ *   xg_sdpa_lse: xg_sdpa that also writes lse [B,H,Sq] fp32, the natural-log
+ *     sum of exponentials of every query row's scaled (and causally masked)
+ *     scores; -inf for a row that sees no key.
+ *   xg_sdpa_backward: dq [B,H,Sq,D], dk and dv [B,Hkv,Skv,D] (contiguous, in
+ *     `dtype`) from q, k, v, the forward's out and lse, and d_out (strides as
+ *     in xg_sdpa; d_out has its own).  The probabilities are recomputed tile by
+ *     tile from lse: no [Sq,Skv] temporary.  With Hkv < H the gradients of a
+ *     key/value head are summed over its query heads inside the kernel.  Two
+ *     launches on `stream`; results do not depend on scheduling (no atomics).
+ *     delta_ws: [B,H,Sq] fp32 workspace supplied by the caller (row sums of
+ *     d_out * out, written by the first launch and read by the second).
+ * ------------------------------------------------------------------------- */
+int xg_sdpa_lse(const void* q, const void* k, const void* v, void* out, float* lse, int64_t B, int64_t H, int64_t Hkv,
+                int64_t Sq, int64_t Skv, int64_t D, const int64_t q_strides[3], const int64_t k_strides[3],
+                const int64_t v_strides[3], const int64_t o_strides[3], float scale, int causal, int dtype,
+                xg_stream_t stream);
+int xg_sdpa_backward(const void* q, const void* k, const void* v, const void* out, const void* d_out, const float* lse,
+                     void* dq, void* dk, void* dv, float* delta_ws, int64_t B, int64_t H, int64_t Hkv, int64_t Sq,
+                     int64_t Skv, int64_t D, const int64_t q_strides[3], const int64_t k_strides[3],
+                     const int64_t v_strides[3], const int64_t o_strides[3], const int64_t do_strides[3], float scale,
+                     int causal, int dtype, xg_stream_t stream);
+
+/* ---------------------------------------------------------------------------
  * Rotary position embedding, rotate-half convention:
  *   out = x * cos + cat(-x[..., D/2:], x[..., :D/2]) * sin      (fp32 math, one rounding)
  *   x, out [B,H,S,D] with element strides for batch, head, sequence (D has unit stride, D % 16 == 0);

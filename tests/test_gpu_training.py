@@ -211,7 +211,7 @@ def test_rotary_backward_formula(device, table_grads):
 @pytest.mark.parametrize("causal", [True, False])
 @pytest.mark.parametrize("kv_heads", [4, 2])
 def test_attention_backward_formula(device, causal, kv_heads):
-    """Gradients of xpu_ops.sdpa (probabilities recomputed in fp32) against autograd of the written-out attention in
+    """Gradients of xpu_ops.sdpa (the backward kernels, row statistics recomputed) against autograd of the written-out attention in
     fp32, with as many or fewer key/value heads than query heads."""
     import xpu_graph_amd.ops as xops
 
@@ -258,7 +258,10 @@ def test_attention_training_step(device):
     y0 = torch.compile(layer, backend=be, dynamic=False)(*args)
     g0 = torch.autograd.grad(y0.float().pow(2).mean(), args)
     fwd_ops = [str(n.target) for n in be.compiled_graphs[1].graph.nodes if n.op == "call_function"]
-    assert fwd_ops.count("xpu_ops.sdpa.default") == 1 and fwd_ops.count("xpu_ops.dense.default") == 2, fwd_ops
+    # a graph that is differentiated runs the attention that also saves the row statistics for the backward kernels
+    assert fwd_ops.count("xpu_ops.sdpa_lse.default") == 1 and fwd_ops.count("xpu_ops.dense.default") == 2, fwd_ops
+    bwd_ops = [str(n.target) for gm in be.compiled_graphs[2:] for n in gm.graph.nodes if n.op == "call_function"]
+    assert bwd_ops.count("xpu_ops.sdpa_bwd.default") == 1 and bwd_ops.count("xpu_ops.dense_at.default") == 2, bwd_ops
     ref_args = [a.detach().float().requires_grad_(True) for a in args]
     g1 = torch.autograd.grad(layer(*ref_args).pow(2).mean(), ref_args)
     eag_args = [a.detach().clone().requires_grad_(True) for a in args]
@@ -297,6 +300,55 @@ def test_llama_block_training_step(device):
     err = lambda a, c: (a.float() - c).abs().mean().item()  # noqa: E731
     for name, a, c, e in zip(["x"] + names, g0, g1, g2):
         assert err(a, c) <= 2 * err(e, c) + 2e-2 * c.abs().mean().item(), (name, err(a, c), err(e, c), c.abs().mean().item())
+
+
+def test_llama_block_training_step_full_size_holds_no_score_matrix(device):
+    """The block at its benchmark size (B4 S2048, 32 heads of 128): no tensor of the forward or backward graph is as
+    large as one [B, H, S, S] score matrix, the step's peak memory is below eager's (which holds several), the
+    backward runs the attention-backward and transposed-operand dense kernels, and the gradients follow fp32
+    autograd as closely as eager bf16 does."""
+    from collections import Counter
+
+    from oracle import eager, inputs
+
+    torch.manual_seed(9)
+    B, S, H = 4, 2048, 32
+    x, p = inputs.c5_llama_block(B=B, S=S, device=device)
+    names = sorted(p)
+
+    def block(x, *w):
+        return eager.llama_block_eager(x, dict(zip(names, w)), n_heads=H)
+
+    def step(fn, args):
+        torch.cuda.synchronize()
+        torch.cuda.reset_peak_memory_stats()
+        base = torch.cuda.memory_allocated()
+        g = torch.autograd.grad(fn(*args).float().pow(2).mean(), args)
+        torch.cuda.synchronize()
+        return g, torch.cuda.max_memory_allocated() - base
+
+    args = [x.detach().requires_grad_(True)] + [p[n].detach().requires_grad_(True) for n in names]
+    be = backend()
+    compiled = torch.compile(block, backend=be, dynamic=False)
+    step(compiled, args)  # compiles; the second step is the one measured
+    g0, peak_compiled = step(compiled, args)
+    eag_args = [a.detach().clone().requires_grad_(True) for a in args]
+    g2, peak_eager = step(block, eag_args)
+    score_elems = B * H * S * S
+    for gm in be.compiled_graphs[1:]:
+        for n in gm.graph.nodes:
+            val = n.meta.get("val")
+            vals = val if isinstance(val, (list, tuple)) else [val]
+            assert all(not isinstance(t, torch.Tensor) or t.numel() < score_elems for t in vals), (n, [tuple(t.shape) for t in vals if isinstance(t, torch.Tensor)])
+    assert peak_compiled < peak_eager, (peak_compiled, peak_eager)
+    ops = Counter(str(n.target) for gm in be.compiled_graphs[2:] for n in gm.graph.nodes if n.op == "call_function")
+    assert ops["xpu_ops.sdpa_bwd.default"] == 1 and ops["xpu_ops.dense_at.default"] >= 5, ops
+    ref_args = [a.detach().float().requires_grad_(True) for a in args]
+    g1 = torch.autograd.grad(block(*ref_args).pow(2).mean(), ref_args)
+    err = lambda a, c: (a.float() - c).abs().mean().item()  # noqa: E731
+    for name, a, c, e in zip(["x"] + names, g0, g1, g2):
+        assert err(a, c) <= 2 * err(e, c) + 2e-2 * c.abs().mean().item(), (name, err(a, c), err(e, c), c.abs().mean().item())
+    print(f"peak memory of one training step: compiled {peak_compiled / 2**30:.2f} GiB, eager {peak_eager / 2**30:.2f} GiB")
 
 
 @pytest.mark.parametrize("kind", ["rms", "layer"])

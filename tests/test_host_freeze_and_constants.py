@@ -129,37 +129,6 @@ def test_a_view_of_a_folded_constant_is_returned_as_a_copy():
     torch.testing.assert_close(y, torch.ones(4) + 28.0)
 
 
-def test_attention_backward_never_holds_more_than_its_chunk(monkeypatch):
-    """The formula walks the query rows in blocks: same gradients as autograd of the eager form whatever the block
-    size, and no temporary beyond [B, H, rows, Skv]."""
-    from xpu_graph_amd import autograd as ag
-
-    class Ctx:
-        pass
-
-    B, H, Hkv, Sq, Skv, D = 2, 4, 2, 45, 61, 8
-    q = torch.randn(B, H, Sq, D, requires_grad=True)
-    k = torch.randn(B, Hkv, Skv, D, requires_grad=True)
-    v = torch.randn(B, Hkv, Skv, D, requires_grad=True)
-    s = (q @ k.repeat_interleave(2, 1).transpose(-1, -2)) * 0.25
-    s = s.masked_fill(~torch.ones(Sq, Skv, dtype=torch.bool).tril(), float("-inf"))
-    o = torch.softmax(s, -1) @ v.repeat_interleave(2, 1)
-    g = torch.randn_like(o)
-    want = torch.autograd.grad(o, (q, k, v), g)
-    ctx = Ctx()
-    ctx.saved_tensors, ctx.causal, ctx.scale = (q.detach(), k.detach(), v.detach()), True, 0.25
-    seen = []
-    real_softmax = torch.softmax
-    monkeypatch.setattr(torch, "softmax", lambda t, dim: (seen.append(t.numel()), real_softmax(t, dim))[1])
-    for chunk in (ag.SDPA_BACKWARD_CHUNK_ELEMS, B * H * Skv * 7, 1):
-        monkeypatch.setattr(ag, "SDPA_BACKWARD_CHUNK_ELEMS", chunk)
-        seen.clear()
-        got = ag._sdpa_backward(ctx, g)[:3]
-        for a, b in zip(got, want):
-            torch.testing.assert_close(a, b, rtol=1e-4, atol=1e-5)
-        assert max(seen) <= max(chunk, B * H * Skv)
-
-
 def test_graph_runner_refreshes_its_inputs_outside_an_assert():
     import inspect
 

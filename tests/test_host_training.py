@@ -258,3 +258,32 @@ print("FORWARD_OUTPUTS", len(outs))
     assert proc.returncode == 0, proc.stderr[-2000:]
     n_out = int(proc.stdout.split("FORWARD_OUTPUTS")[1].split()[0])
     assert n_out >= 5, n_out  # y + the operands both dense backward formulas keep (x, weights, outputs, bias)
+
+
+def test_written_out_attention_reaches_the_attention_kernel_in_pregrad(caplog):
+    """matmul -> / sqrt(D) -> + causal mask -> softmax in fp32 -> cast -> matmul on [B, H, S, D] operands, as a
+    hand-written decoder block spells it, becomes aten.scaled_dot_product_attention before autograd is traced
+    (beyond the reference, whose FusedSDPA is inference-only); the target pattern recognises the constant causal
+    mask, and the differentiated forward graph runs the attention that saves the row statistics."""
+    import math
+
+    def attn(q, k, v):
+        S, D = q.shape[-2], q.shape[-1]
+        s = torch.matmul(q, k.transpose(2, 3)) / math.sqrt(D)
+        s = s + torch.full((S, S), float("-inf"), dtype=q.dtype).triu(1)
+        p = torch.softmax(s, dim=-1, dtype=torch.float32).to(q.dtype)
+        return torch.matmul(p, v)
+
+    bf = torch.bfloat16
+    backend = XpuGraph(XpuGraphConfig(is_training=True, target=Target.mi355x, opt_level=OptLevel.level2, enable_cache=False))
+    args = [torch.randn(2, 4, 32, 64).to(bf).requires_grad_(True) for _ in range(3)]
+    with need_xpu_graph_logs(), pytest.raises(NotImplementedError):
+        torch.compile(attn, backend=backend)(*args)
+    pregrad, forward = backend.compiled_graphs[-2:]
+    calls = [n for n in pregrad.graph.nodes if n.op == "call_module"]
+    assert [n.target for n in calls] == ["mi355x_sdpa"]
+    assert calls[0].args[3] is True and abs(calls[0].args[4] - 0.125) < 1e-9  # causal by index, scale 1 / sqrt(64)
+    assert not any("softmax" in str(n.target) or "matmul" in str(n.target) for n in pregrad.graph.nodes)
+    fwd_ops = [str(n.target) for n in forward.graph.nodes if n.op == "call_function"]
+    assert fwd_ops.count("xpu_ops.sdpa_lse.default") == 1 and "xpu_ops.sdpa.default" not in fwd_ops, fwd_ops
+    assert "Pattern.FusedSDPA changed graph" in caplog.text

@@ -40,6 +40,8 @@ def ulp_error(got, want32):
     (below that the absolute floor decides, and an ulp of a nearly cancelled sum says nothing about the kernel)."""
     g = got.float()
     big = want32.abs().max()
+    if big == 0:  # an exactly cancelled result: only the absolute floor applies
+        return 0.0
     ok = torch.isfinite(want32) & (want32.abs() >= big * 2.0**-6)
     if not ok.any():
         return 0.0
@@ -67,3 +69,11 @@ def assert_close_16bit(got, want32, floor, label):
     ulps = ulp_error(got, want32)
     RECORDS.append((label, ulps, err.max().item() if err.numel() else 0.0, floor))
     torch.testing.assert_close(got.float(), want32, rtol=RTOL_16BIT, atol=floor, msg=lambda m: f"{label}: {m} (max {ulps:.2f} ulp)")
+
+
+def attention_grad_floor(want32, dtype):
+    """Gradients of attention: the probabilities and the score gradients are rounded to the storage type before
+    they multiply dO / Q / K (as in every tiled attention backward), and a gradient element sums one such product
+    per key (or query), so its error is a random walk of half-ulp steps: 2^-7 of the largest gradient for bf16,
+    2^-10 for fp16."""
+    return want32.abs().max().item() * (2.0**-7 if dtype == torch.bfloat16 else 2.0**-10)

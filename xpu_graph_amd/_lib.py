@@ -116,6 +116,14 @@ _SIGNATURES = {
         + [ctypes.POINTER(c_int64)] * 4
         + [c_float, c_int, c_int, c_void_p],
     ),
+    "xg_sdpa_lse": (
+        c_int,
+        [c_void_p] * 5 + [c_int64] * 6 + [ctypes.POINTER(c_int64)] * 4 + [c_float, c_int, c_int, c_void_p],
+    ),
+    "xg_sdpa_backward": (
+        c_int,
+        [c_void_p] * 10 + [c_int64] * 6 + [ctypes.POINTER(c_int64)] * 5 + [c_float, c_int, c_int, c_void_p],
+    ),
     "xg_rope": (
         c_int,
         [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, ctypes.POINTER(c_int64), ctypes.POINTER(c_int64), c_int64, c_int, c_int, c_void_p],

@@ -14,6 +14,7 @@ a few microseconds of dispatch, which inference-only processes should not pay.
     dense_glu(x, Wg, Wu)       y = silu(x Wg^T) * (x Wu^T)
     rope(x, cos, sin)          y = x * cos + rotate_half(x) * sin,  rotate_half(x) = cat(-x[D/2:], x[:D/2])
     sdpa(q, k, v, causal, scale)   y = softmax(scale q k^T [+ causal mask]) v
+    sdpa_lse(q, k, v, causal, scale)   the same, also returning the log-sum-exp of every row for the backward kernels
     add_rms_norm(x, r, w, eps) / add_layer_norm(x, r, w, b, eps)   h = x + r, y = norm(h); returns (y, h)
     add_rms_norm_only / add_layer_norm_only                         the same, returning y alone
 
@@ -210,52 +211,26 @@ def _sdpa_setup(ctx, inputs, output):
     ctx.save_for_backward(q, k, v)
 
 
-SDPA_BACKWARD_CHUNK_ELEMS = 32 * 1024 * 1024  # fp32 elements of one [B, H, rows, Skv] temporary (128 MiB)
-
-
 def _sdpa_backward(ctx, gy):
-    # The probabilities are recomputed in fp32 Aten ops, a block of query rows at a time: softmax runs along the keys,
-    # so a block of whole rows is exact, and no temporary is larger than SDPA_BACKWARD_CHUNK_ELEMS elements whatever
-    # the sequence length (the whole [B, H, Sq, Skv] matrix is 34 GB per temporary at B4 H32 S8192).  With a causal
-    # mask a block only meets the keys up to its last row.  With fewer key/value heads than query heads, query head
-    # h reads head h // rep.  Not a flash backward kernel: the key/value gradients are accumulated in fp32 tensors.
+    # The plain op saves no row statistics: one more forward launch recomputes the output and its log-sum-exp (bit
+    # for bit the forward's), then the backward kernels run.  Graphs built for training use sdpa_lse instead.
     q, k, v = ctx.saved_tensors
-    B, H, Sq, D = q.shape
-    Hkv, Skv = k.shape[1], k.shape[2]
-    rep = H // Hkv
-    kf, vf = k.float(), v.float()
-    if rep > 1:
-        kf, vf = kf.repeat_interleave(rep, dim=1), vf.repeat_interleave(rep, dim=1)
-    gq = torch.empty_like(q)
-    gk = torch.zeros(B, H, Skv, D, dtype=torch.float32, device=q.device)
-    gv = torch.zeros(B, H, Skv, D, dtype=torch.float32, device=q.device)
-    rows = max(1, min(Sq, SDPA_BACKWARD_CHUNK_ELEMS // max(1, B * H * Skv)))
-    for r0 in range(0, Sq, rows):
-        r1 = min(Sq, r0 + rows)
-        n_keys = min(Skv, r1) if ctx.causal else Skv  # keys a causal block can see: 0 .. its last row
-        if n_keys == 0:
-            gq[:, :, r0:r1] = 0
-            continue
-        qc, gc = q[:, :, r0:r1].float(), gy[:, :, r0:r1].float()
-        kc, vc = kf[:, :, :n_keys], vf[:, :, :n_keys]
-        s = (qc @ kc.transpose(-1, -2)) * ctx.scale
-        if ctx.causal:
-            row = torch.arange(r0, r1, device=q.device).unsqueeze(1)
-            col = torch.arange(n_keys, device=q.device).unsqueeze(0)
-            s = s.masked_fill(col > row, float("-inf"))
-        p = torch.softmax(s, dim=-1)
-        del s
-        gv[:, :, :n_keys] += p.transpose(-1, -2) @ gc
-        gp = gc @ vc.transpose(-1, -2)
-        gs = p * (gp - (gp * p).sum(-1, keepdim=True))
-        del p, gp
-        gq[:, :, r0:r1] = ((gs @ kc) * ctx.scale).to(q.dtype)
-        gk[:, :, :n_keys] += (gs.transpose(-1, -2) @ qc) * ctx.scale
-        del gs
-    if rep > 1:
-        gk = gk.reshape(B, Hkv, rep, Skv, D).sum(2)
-        gv = gv.reshape(B, Hkv, rep, Skv, D).sum(2)
-    return gq, gk.to(k.dtype), gv.to(v.dtype), None, None
+    out, lse = torch.ops.xpu_ops.sdpa_lse(q, k, v, ctx.causal, ctx.scale)
+    gq, gk, gv = torch.ops.xpu_ops.sdpa_bwd(q, k, v, out, gy, lse, ctx.causal, ctx.scale)
+    return gq, gk, gv, None, None
+
+
+def _sdpa_lse_setup(ctx, inputs, output):
+    q, k, v, ctx.causal, ctx.scale = inputs
+    out, lse = output
+    ctx.save_for_backward(q, k, v, out, lse)
+
+
+def _sdpa_lse_backward(ctx, gy, g_lse=None):
+    # the log-sum-exp output exists for this formula; a gradient flowing into it is not supported
+    q, k, v, out, lse = ctx.saved_tensors
+    gq, gk, gv = torch.ops.xpu_ops.sdpa_bwd(q, k, v, out, gy, lse, ctx.causal, ctx.scale)
+    return gq, gk, gv, None, None
 
 
 def _add_norm_formulas(layer, with_sum):
@@ -309,13 +284,14 @@ def register():
     reg("xpu_ops::dense_glu", _dense_glu_backward, setup_context=_dense_glu_setup)
     reg("xpu_ops::rope", _rope_backward, setup_context=_rope_setup)
     reg("xpu_ops::sdpa", _sdpa_backward, setup_context=_sdpa_setup)
+    reg("xpu_ops::sdpa_lse", _sdpa_lse_backward, setup_context=_sdpa_lse_setup)
     for op, layer, with_sum in (("add_rms_norm", False, True), ("add_rms_norm_only", False, False),
                                 ("add_layer_norm", True, True), ("add_layer_norm_only", True, False)):
         setup, backward = _add_norm_formulas(layer, with_sum)
         reg(f"xpu_ops::{op}", backward, setup_context=setup)
     # An op that was traced before (an inference compile earlier in the process) has its dispatch decisions cached
     # on the Python side; a stale entry for the Autograd key would keep sending traces to the "no formula" fallback.
-    for name in ("rms_norm", "layer_norm", "silu_mul2", "silu_mul", "dense", "dense_glu", "rope", "sdpa",
+    for name in ("rms_norm", "layer_norm", "silu_mul2", "silu_mul", "dense", "dense_glu", "rope", "sdpa", "sdpa_lse",
                  "add_rms_norm", "add_rms_norm_only", "add_layer_norm", "add_layer_norm_only"):
         packet = getattr(torch.ops.xpu_ops, name)
         for overload in packet.overloads():

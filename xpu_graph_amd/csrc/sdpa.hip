@@ -26,33 +26,17 @@
 // rows) and the 8-row x 64-byte footprints of the transposing V reads spread over
 // all banks.  The swizzle is applied to the GLOBAL address of each lane of the
 // direct load, since its LDS side is fixed (lane i -> base + 16 i).
-#include "xg_common.hpp"
-
-#include <math.h>
-#include <stdlib.h>
-
-#include <type_traits>
-#include <utility>
+#include "sdpa_common.hpp"
 
 namespace xg {
 namespace sdpa {
-
-typedef float f32x16 __attribute__((ext_vector_type(16)));
-typedef short s16x4 __attribute__((ext_vector_type(4)));
-typedef short s16x8 __attribute__((ext_vector_type(8)));
-typedef __attribute__((address_space(1))) void gvoid;
-typedef __attribute__((address_space(3))) void lvoid;
-typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
-
-constexpr int BQ = 128;   // query rows per workgroup
-constexpr int BKV = 64;   // key rows per step
-constexpr int kThreads = 256;
 
 struct Params {
   const void* q;
   const void* k;
   const void* v;
   void* o;
+  float* lse;  // when set: the natural-log sum of exponentials of every query row, [B, H, Sq] (what a backward pass recomputes the probabilities from)
   int B, H, Hkv, Sq, Skv;
   int64_t qs[3], ks[3], vs[3], os[3];  // element strides of batch, head, sequence
   float c;                             // scale * log2(e)
@@ -65,42 +49,6 @@ struct Params {
   int n_qb;   // query blocks per (batch, head)
   int order;  // 0: heaviest query blocks of ALL heads first; 1: head after head inside each XCD
 };
-
-template <typename F, int... I>
-__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, I...>) {
-  (f(std::integral_constant<int, I>{}), ...);
-}
-template <int N, typename F>
-__device__ __forceinline__ void static_for(F&& f) {
-  static_for_impl(f, std::make_integer_sequence<int, N>{});
-}
-
-template <typename T>
-struct Vec8;
-template <>
-struct Vec8<bf16_t> {
-  typedef bf16x8 type;
-};
-template <>
-struct Vec8<f16_t> {
-  typedef f16x8 type;
-};
-
-__device__ __forceinline__ f32x16 mma(bf16x8 a, bf16x8 b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
-__device__ __forceinline__ f32x16 mma(f16x8 a, f16x8 b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0); }
-
-// Chunk swizzles (16-byte chunks within a row of D elements).
-template <int D>
-__device__ __forceinline__ int swz_k(int r) {
-  if constexpr (D == 128) return r & 15;  // 256-byte rows: 16 rows x one chunk -> 16 distinct bank groups
-  else return (r >> 1) & 7;               // 128-byte rows: two rows per 256 bytes
-}
-template <int D>
-__device__ __forceinline__ int swz_v(int r) {
-  // the transposing read touches 8 consecutive rows x 4 aligned chunks: rows must move the GROUP of four
-  if constexpr (D == 128) return ((r & 3) << 2) | ((r >> 2) & 3);
-  else return (((r >> 1) & 1) << 2) | ((r >> 2) & 3);
-}
 
 // MASK: an additive mask [B | 1, H | 1, Sq, Skv] is added to the scaled scores (aten.scaled_dot_product_attention's
 // attn_mask); rows whose every key is masked with -inf come out as NaN, as they do in eager.
@@ -368,6 +316,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
   // global stores are 16 bytes per lane and whole rows per 16 lanes.
   const float l_tot = l_run + __shfl_xor(l_run, 32, kWave);
   const float inv = 1.f / l_tot;
+  if (p.lse && h == 0 && qrow < p.Sq)  // m_run is in base-2 units; a row without a visible key gives -inf
+    p.lse[(int64_t)bh * p.Sq + qrow] = (m_run + log2f(l_tot)) * 0.69314718055994530942f;
   __syncthreads();  // all waves are done reading K / V tiles
   char* park = smem + wave * (32 * RB);
   static_for<DT>([&](auto DI) {
@@ -412,7 +362,7 @@ int launch(const Params& p, hipStream_t stream) {
 
 namespace {
 
-int sdpa_entry(const void* q, const void* k, const void* v, void* out, const void* mask, const int64_t* mask_strides, int mask_dtype,
+int sdpa_entry(const void* q, const void* k, const void* v, void* out, float* lse, const void* mask, const int64_t* mask_strides, int mask_dtype,
                const float* scale_dev, int64_t B, int64_t H, int64_t Hkv, int64_t Sq, int64_t Skv, int64_t D, const int64_t q_strides[3],
                const int64_t k_strides[3], const int64_t v_strides[3], const int64_t o_strides[3], float scale, int causal, int dtype,
                xg_stream_t stream) {
@@ -460,6 +410,8 @@ int sdpa_entry(const void* q, const void* k, const void* v, void* out, const voi
   }
   if (scale_dev && !aligned_to(scale_dev, 4)) return XG_ERR_BAD_ALIGN;
   p.scale_dev = scale_dev;
+  if (lse && !aligned_to(lse, 4)) return XG_ERR_BAD_ALIGN;
+  p.lse = lse;
   p.q = q;
   p.k = k;
   p.v = v;
@@ -490,7 +442,7 @@ int sdpa_entry(const void* q, const void* k, const void* v, void* out, const voi
 extern "C" int xg_sdpa(const void* q, const void* k, const void* v, void* out, int64_t B, int64_t H, int64_t Hkv, int64_t Sq,
                        int64_t Skv, int64_t D, const int64_t q_strides[3], const int64_t k_strides[3], const int64_t v_strides[3],
                        const int64_t o_strides[3], float scale, int causal, int dtype, xg_stream_t stream) {
-  return sdpa_entry(q, k, v, out, nullptr, nullptr, dtype, nullptr, B, H, Hkv, Sq, Skv, D, q_strides, k_strides, v_strides, o_strides, scale,
+  return sdpa_entry(q, k, v, out, nullptr, nullptr, nullptr, dtype, nullptr, B, H, Hkv, Sq, Skv, D, q_strides, k_strides, v_strides, o_strides, scale,
                     causal, dtype, stream);
 }
 
@@ -498,6 +450,15 @@ extern "C" int xg_sdpa_masked(const void* q, const void* k, const void* v, void*
                               int mask_dtype, const float* scale_dev, int64_t B, int64_t H, int64_t Hkv, int64_t Sq, int64_t Skv,
                               int64_t D, const int64_t q_strides[3], const int64_t k_strides[3], const int64_t v_strides[3],
                               const int64_t o_strides[3], float scale, int causal, int dtype, xg_stream_t stream) {
-  return sdpa_entry(q, k, v, out, mask, mask_strides, mask_dtype, scale_dev, B, H, Hkv, Sq, Skv, D, q_strides, k_strides, v_strides,
+  return sdpa_entry(q, k, v, out, nullptr, mask, mask_strides, mask_dtype, scale_dev, B, H, Hkv, Sq, Skv, D, q_strides, k_strides, v_strides,
                     o_strides, scale, causal, dtype, stream);
+}
+
+extern "C" int xg_sdpa_lse(const void* q, const void* k, const void* v, void* out, float* lse, int64_t B, int64_t H, int64_t Hkv,
+                           int64_t Sq, int64_t Skv, int64_t D, const int64_t q_strides[3], const int64_t k_strides[3],
+                           const int64_t v_strides[3], const int64_t o_strides[3], float scale, int causal, int dtype,
+                           xg_stream_t stream) {
+  if (lse == nullptr && B > 0 && H > 0 && Sq > 0) return XG_ERR_NULL_PTR;
+  return sdpa_entry(q, k, v, out, lse, nullptr, nullptr, dtype, nullptr, B, H, Hkv, Sq, Skv, D, q_strides, k_strides, v_strides, o_strides,
+                    scale, causal, dtype, stream);
 }

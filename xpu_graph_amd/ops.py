@@ -458,6 +458,10 @@ _library.define(
     "dense_fp8(Tensor x_q, Tensor w_q, bool weight_trans, Tensor x_scale, Tensor w_scale, Tensor? bias, str act, ScalarType out_dtype) -> Tensor"
 )
 _library.define("sdpa(Tensor q, Tensor k, Tensor v, bool is_causal, float scale) -> Tensor")
+_library.define("sdpa_lse(Tensor q, Tensor k, Tensor v, bool is_causal, float scale) -> (Tensor, Tensor)")
+_library.define(
+    "sdpa_bwd(Tensor q, Tensor k, Tensor v, Tensor out, Tensor d_out, Tensor lse, bool is_causal, float scale) -> (Tensor, Tensor, Tensor)"
+)
 _library.define("sdpa_masked(Tensor q, Tensor k, Tensor v, Tensor? mask, Tensor? scale_t, bool is_causal, float scale) -> Tensor")
 _library.define("rope(Tensor x, Tensor cos, Tensor sin) -> Tensor")
 
@@ -701,22 +705,62 @@ def _empty_like_layout(t):
     return torch.empty(t.shape, dtype=t.dtype, device=t.device)
 
 
-def _sdpa(q, k, v, is_causal, scale):
+def _sdpa_run(q, k, v, is_causal, scale, want_lse):
     _sdpa_check(q, k, v)
     if k.dtype != q.dtype or v.dtype != q.dtype:
         raise TypeError("sdpa: q, k, v must share a dtype")
     q, k, v = _unit_last(q), _unit_last(k), _unit_last(v)
     B, H, Sq, D = q.shape
     out = _empty_like_layout(q)
+    lse = torch.empty((B, H, Sq), dtype=torch.float32, device=q.device) if want_lse else None
     if out.numel() == 0:
-        return out
+        return out, lse
     S3 = ctypes.c_int64 * 3
-    st = _lib.lib().xg_sdpa(
-        _ptr(q), _ptr(k), _ptr(v), _ptr(out), B, H, k.shape[1], Sq, k.shape[2], D, S3(*q.stride()[:3]), S3(*k.stride()[:3]),
-        S3(*v.stride()[:3]), S3(*out.stride()[:3]), scale, 1 if is_causal else 0, _code(q.dtype), _stream(),
+    shape = (B, H, k.shape[1], Sq, k.shape[2], D, S3(*q.stride()[:3]), S3(*k.stride()[:3]), S3(*v.stride()[:3]), S3(*out.stride()[:3]))
+    tail = (scale, 1 if is_causal else 0, _code(q.dtype), _stream())
+    if want_lse:
+        _lib.check(_lib.lib().xg_sdpa_lse(_ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), *shape, *tail), "xg_sdpa_lse")
+    else:
+        _lib.check(_lib.lib().xg_sdpa(_ptr(q), _ptr(k), _ptr(v), _ptr(out), *shape, *tail), "xg_sdpa")
+    return out, lse
+
+
+def _sdpa(q, k, v, is_causal, scale):
+    return _sdpa_run(q, k, v, is_causal, scale, False)[0]
+
+
+def _sdpa_lse(q, k, v, is_causal, scale):
+    """Attention that also returns the natural-log sum of exponentials of every query row ([B, H, Sq] fp32), from
+    which the backward kernels recompute the probabilities."""
+    return _sdpa_run(q, k, v, is_causal, scale, True)
+
+
+def _sdpa_bwd(q, k, v, out, d_out, lse, is_causal, scale):
+    """Gradients of attention with respect to q, k, v on the flash-style backward kernels: nothing of size
+    [Sq, Skv] is stored.  `delta` ([B, H, Sq] fp32, the row sums of d_out * out) is the one temporary."""
+    _sdpa_check(q, k, v)
+    if out.shape != q.shape or d_out.shape != q.shape or tuple(lse.shape) != tuple(q.shape[:3]):
+        raise ValueError("sdpa_bwd: out and d_out must have the shape of q, lse its first three dims")
+    if any(t.dtype != q.dtype for t in (k, v, out, d_out)) or lse.dtype != torch.float32:
+        raise TypeError("sdpa_bwd: q, k, v, out, d_out must share a dtype; lse is float32")
+    q, k, v, out, d_out = (_unit_last(t) for t in (q, k, v, out, d_out))
+    lse = lse.contiguous()
+    B, H, Sq, D = q.shape
+    Hkv, Skv = k.shape[1], k.shape[2]
+    dq = torch.empty((B, H, Sq, D), dtype=q.dtype, device=q.device)
+    dk = torch.empty((B, Hkv, Skv, D), dtype=q.dtype, device=q.device)
+    dv = torch.empty((B, Hkv, Skv, D), dtype=q.dtype, device=q.device)
+    if dq.numel() == 0 or dk.numel() == 0:
+        return dq.zero_(), dk.zero_(), dv.zero_()
+    delta = torch.empty((B, H, Sq), dtype=torch.float32, device=q.device)
+    S3 = ctypes.c_int64 * 3
+    st = _lib.lib().xg_sdpa_backward(
+        _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(d_out), _ptr(lse), _ptr(dq), _ptr(dk), _ptr(dv), _ptr(delta), B, H, Hkv, Sq, Skv, D,
+        S3(*q.stride()[:3]), S3(*k.stride()[:3]), S3(*v.stride()[:3]), S3(*out.stride()[:3]), S3(*d_out.stride()[:3]), scale,
+        1 if is_causal else 0, _code(q.dtype), _stream(),
     )
-    _lib.check(st, "xg_sdpa")
-    return out
+    _lib.check(st, "xg_sdpa_backward")
+    return dq, dk, dv
 
 
 def sdpa_mask_fits(mask_shape, q_shape, skv):
@@ -777,6 +821,17 @@ def _sdpa_masked_meta(q, k, v, mask, scale_t, is_causal, scale):
 def _sdpa_meta(q, k, v, is_causal, scale):
     _sdpa_check(q, k, v)
     return _empty_like_layout(_unit_last(q))
+
+
+def _sdpa_lse_meta(q, k, v, is_causal, scale):
+    _sdpa_check(q, k, v)
+    return _empty_like_layout(_unit_last(q)), torch.empty(tuple(q.shape[:3]), dtype=torch.float32, device=q.device)
+
+
+def _sdpa_bwd_meta(q, k, v, out, d_out, lse, is_causal, scale):
+    _sdpa_check(q, k, v)
+    return (torch.empty(tuple(q.shape), dtype=q.dtype, device=q.device), torch.empty(tuple(k.shape), dtype=q.dtype, device=q.device),
+            torch.empty(tuple(v.shape), dtype=q.dtype, device=q.device))
 
 
 def _rope_check(x, cos, sin):
@@ -868,6 +923,10 @@ _library.impl("dense_fp8", _dense_fp8, "CUDA")
 _library.impl("dense_fp8", _dense_fp8_meta, "Meta")
 _library.impl("sdpa", _sdpa, "CUDA")
 _library.impl("sdpa", _sdpa_meta, "Meta")
+_library.impl("sdpa_lse", _sdpa_lse, "CUDA")
+_library.impl("sdpa_lse", _sdpa_lse_meta, "Meta")
+_library.impl("sdpa_bwd", _sdpa_bwd, "CUDA")
+_library.impl("sdpa_bwd", _sdpa_bwd_meta, "Meta")
 _library.impl("sdpa_masked", _sdpa_masked, "CUDA")
 _library.impl("sdpa_masked", _sdpa_masked_meta, "Meta")
 _library.impl("rope", _rope, "CUDA")

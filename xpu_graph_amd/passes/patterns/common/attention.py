@@ -113,10 +113,89 @@ def match_attention(node):
     return q, k, v, scale, scale_divides, mask, mask_added, dims
 
 
+def match_attention_predispatch(node):
+    """The same chain as it looks BEFORE dispatch (the `pregrad` stage of a training graph), on 4-D [B, H, S, D]
+    operands: matmul(q, transpose(k)) -> [mul / div by a number] -> [add mask] -> softmax.int(-1[, float32]) ->
+    [cast back] -> matmul(., v).  Returns (q, k, v, scale, mask) or None.  Equal head counts only; the mask, if any,
+    has the dtype of q (what aten.scaled_dot_product_attention accepts)."""
+    if not is_call(node, aten.matmul.default):
+        return None
+    probs, v = arg(node, 0), arg(node, 1)
+    cast_back = is_call(probs, aten._to_copy.default) and set(probs.kwargs) == {"dtype"}
+    softmax = probs.args[0] if cast_back else probs
+    if not is_call(softmax, aten.softmax.int):
+        return None
+    scores, sm_dim, sm_dtype = arg(softmax, 0), arg(softmax, 1), arg(softmax, 2)
+    if not (isinstance(scores, fx.Node) and isinstance(scores.meta.get("val"), torch.Tensor)):
+        return None
+    sm_rank = len(scores.meta["val"].shape)
+    if sm_rank != 4 or not isinstance(sm_dim, int) or sm_dim % sm_rank != sm_rank - 1:
+        return None
+    vv = v.meta.get("val") if isinstance(v, fx.Node) else None
+    if not isinstance(vv, torch.Tensor) or probs.meta["val"].dtype != vv.dtype:
+        return None  # the probabilities must enter the second product in the dtype of v
+    if sm_dtype not in (None, torch.float32, vv.dtype):
+        return None
+    cur = scores
+    mask = None
+    if is_call(cur, aten.add.Tensor) and kwarg(cur, "alpha") in (None, 1):
+        mask, cur = arg(cur, 1), arg(cur, 0)
+        if not (isinstance(mask, fx.Node) and isinstance(mask.meta.get("val"), torch.Tensor) and mask.meta["val"].dtype == vv.dtype):
+            return None
+    scale = 1.0
+    if is_call(cur, aten.mul.Tensor, aten.div.Tensor):
+        factor = arg(cur, 1)
+        if not isinstance(factor, (int, float)) or (cur.target == aten.div.Tensor and factor == 0):
+            return None
+        scale = float(factor) if cur.target == aten.mul.Tensor else 1.0 / float(factor)
+        cur = arg(cur, 0)
+    if not is_call(cur, aten.matmul.default):
+        return None
+    q, kt = arg(cur, 0), arg(cur, 1)
+    if is_call(kt, aten.transpose.int) and {arg(kt, 1) % 4, arg(kt, 2) % 4} == {2, 3}:
+        k = arg(kt, 0)
+    else:
+        return None
+    vals = [t.meta.get("val") if isinstance(t, fx.Node) else None for t in (q, k)]
+    if not all(isinstance(t, torch.Tensor) and t.dim() == 4 and t.dtype == vv.dtype for t in vals) or vv.dim() != 4:
+        return None
+    qv, kv = vals
+    if not (same_shape(qv.shape[:2], kv.shape[:2]) and same_shape(kv.shape[:3], vv.shape[:3]) and same_shape(qv.shape[3], kv.shape[3])):
+        return None
+    if mask is not None:
+        try:
+            full = torch.broadcast_shapes(mask.meta["val"].shape, scores.meta["val"].shape)
+        except Exception:
+            return None
+        if not same_shape(full, scores.meta["val"].shape):
+            return None
+    return q, k, v, scale, mask
+
+
 class FusedSDPA(Pattern):
     _opt_level = OptLevel.level2
+    # pregrad: beyond the reference (inference only, pattern.py:29), so that a hand-written attention in a training
+    # graph reaches the target's attention kernels, which carry a backward
+    _support_stages = [FxStage.inference, FxStage.pregrad]
+
+    def _process_predispatch(self, gm):
+        g = gm.graph
+        changed = False
+        for node in reversed(g.nodes):
+            m = match_attention_predispatch(node)
+            if m is None:
+                continue
+            q, k, v, scale, mask = m
+            with g.inserting_before(node):
+                fused = g.call_function(aten.scaled_dot_product_attention.default, (q, k, v), {"attn_mask": mask, "scale": scale})
+            fused.meta["val"] = node.meta.get("val")
+            node.replace_all_uses_with(fused)
+            changed = True
+        return changed
 
     def process(self, gm):
+        if self._current_stage == FxStage.pregrad:
+            return self._process_predispatch(gm)
         g = gm.graph
         syms = SymShapes(g)
         inference = self._current_stage == FxStage.inference

@@ -37,6 +37,10 @@ _MAX_CONST_ELEMS = 1 << 26
 
 class SDPAModule(nn.Module):
     def forward(self, q, k, v, is_causal, scale):
+        if torch.is_grad_enabled() and (q.requires_grad or k.requires_grad or v.requires_grad):
+            # a graph that will be differentiated: the forward also writes the log-sum-exp of every row, which is
+            # all the backward kernels need beside q, k, v and the output
+            return torch.ops.xpu_ops.sdpa_lse(q, k, v, is_causal, scale)[0]
         return torch.ops.xpu_ops.sdpa(q, k, v, is_causal, scale)
 
 
