@@ -292,6 +292,25 @@ int xg_sdpa_backward(const void* q, const void* k, const void* v, const void* ou
                      int causal, int dtype, xg_stream_t stream);
 
 /* ---------------------------------------------------------------------------
+ * xg_sdpa_backward without the workspace argument, for callers that cannot
+ * allocate device memory (code under HIP graph capture, serving loops and
+ * harnesses that forbid hipMalloc).  No counterpart in the reference.  The
+ * delta workspace is an 8 MiB array that lives in the library's device image,
+ * one per GPU, from load until the process ends: B * H * Sq must not exceed
+ * 2 097 152 query rows (XG_ERR_TOO_LARGE beyond that: use xg_sdpa_backward).
+ * The call allocates and frees nothing.  Every call on a GPU uses that GPU's
+ * one array: calls that overlap in time on the same GPU (different streams)
+ * race; calls on one stream are ordered and need nothing cleared in between
+ * (each call writes every row of the workspace that it later reads).
+ * Results are bit-identical to xg_sdpa_backward.
+ * ------------------------------------------------------------------------- */
+int xg_sdpa_backward_static(const void* q, const void* k, const void* v, const void* out, const void* d_out,
+                            const float* lse, void* dq, void* dk, void* dv, int64_t B, int64_t H, int64_t Hkv,
+                            int64_t Sq, int64_t Skv, int64_t D, const int64_t q_strides[3],
+                            const int64_t k_strides[3], const int64_t v_strides[3], const int64_t o_strides[3],
+                            const int64_t do_strides[3], float scale, int causal, int dtype, xg_stream_t stream);
+
+/* ---------------------------------------------------------------------------
  * Rotary position embedding, rotate-half convention:
  *   out = x * cos + cat(-x[..., D/2:], x[..., :D/2]) * sin      (fp32 math, one rounding)
  *   x, out [B,H,S,D] with element strides for batch, head, sequence (D has unit stride, D % 16 == 0);

@@ -19,7 +19,7 @@ def declared_symbols():
 def test_header_declares_the_expected_entry_points():
     syms = declared_symbols()
     for s in ("xg_rms_norm", "xg_layer_norm", "xg_add_rms_norm", "xg_add_layer_norm", "xg_slice_cat", "xg_addn",
-              "xg_combo_sum", "xg_slice_sum_cat", "xg_silu_mul", "xg_silu_mul2", "xg_dense", "xg_dense_batched", "xg_dense_at", "xg_dense_glu", "xg_dense_fp8", "xg_slice_cat_check_table", "xg_sdpa", "xg_sdpa_masked", "xg_sdpa_lse", "xg_sdpa_backward", "xg_rope", "xg_copy_bytes",
+              "xg_combo_sum", "xg_slice_sum_cat", "xg_silu_mul", "xg_silu_mul2", "xg_dense", "xg_dense_batched", "xg_dense_at", "xg_dense_glu", "xg_dense_fp8", "xg_slice_cat_check_table", "xg_sdpa", "xg_sdpa_masked", "xg_sdpa_lse", "xg_sdpa_backward", "xg_sdpa_backward_static", "xg_rope", "xg_copy_bytes",
               "xg_version", "xg_status_string"):
         assert s in syms
 
@@ -146,6 +146,18 @@ def test_transposed_left_operand_validation_needs_no_gpu():
     assert lib.xg_dense_at(None, p, None, p, 16, 16, 8, 16, 16, 0, 2, None) == -4
     off = ctypes.c_void_p(p.value + 2)
     assert lib.xg_dense_at(off, p, None, p, 16, 16, 8, 16, 16, 0, 2, None) == -3
+
+
+def test_static_workspace_backward_refuses_more_rows_than_it_holds_without_a_gpu():
+    from xpu_graph_amd import _lib
+
+    lib = _lib.lib()
+    S3 = ctypes.c_int64 * 3
+    p = ctypes.c_void_p(256)  # never dereferenced: the size check comes first
+    args = (S3(), S3(), S3(), S3(), S3(), 1.0, 0, 2, None)
+    assert lib.xg_sdpa_backward_static(p, p, p, p, p, p, p, p, p, 1, 1, 1, (1 << 21) + 1, 64, 64, *args) == -5
+    assert lib.xg_sdpa_backward_static(p, p, p, p, p, p, p, p, p, 1 << 11, 1 << 11, 1, 1, 64, 64, *args) == -5
+    assert lib.xg_sdpa_backward_static(p, p, p, p, p, p, p, p, p, 0, 4, 4, 64, 64, 64, *args) == 0  # nothing to do
 
 
 def test_a_missing_library_is_an_error_not_a_fallback(monkeypatch, tmp_path):

@@ -124,6 +124,10 @@ _SIGNATURES = {
         c_int,
         [c_void_p] * 10 + [c_int64] * 6 + [ctypes.POINTER(c_int64)] * 5 + [c_float, c_int, c_int, c_void_p],
     ),
+    "xg_sdpa_backward_static": (
+        c_int,
+        [c_void_p] * 9 + [c_int64] * 6 + [ctypes.POINTER(c_int64)] * 5 + [c_float, c_int, c_int, c_void_p],
+    ),
     "xg_rope": (
         c_int,
         [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, ctypes.POINTER(c_int64), ctypes.POINTER(c_int64), c_int64, c_int, c_int, c_void_p],

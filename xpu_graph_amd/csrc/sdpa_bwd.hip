@@ -22,6 +22,9 @@
 // slots, so the row-wise (A operand) reads of the same tile stay conflict free.
 #include "sdpa_common.hpp"
 
+#include <map>
+#include <mutex>
+
 namespace xg {
 namespace sdpa {
 
@@ -396,11 +399,12 @@ int launch_bwd(const BwdParams& p, hipStream_t stream) {
 }  // namespace sdpa
 }  // namespace xg
 
-extern "C" int xg_sdpa_backward(const void* q, const void* k, const void* v, const void* out, const void* d_out, const float* lse,
-                                void* dq, void* dk, void* dv, float* delta_ws, int64_t B, int64_t H, int64_t Hkv, int64_t Sq,
-                                int64_t Skv, int64_t D, const int64_t q_strides[3], const int64_t k_strides[3],
-                                const int64_t v_strides[3], const int64_t o_strides[3], const int64_t do_strides[3], float scale,
-                                int causal, int dtype, xg_stream_t stream) {
+namespace {
+
+int backward_entry(const void* q, const void* k, const void* v, const void* out, const void* d_out, const float* lse, void* dq, void* dk,
+                   void* dv, float* delta_ws, int64_t B, int64_t H, int64_t Hkv, int64_t Sq, int64_t Skv, int64_t D,
+                   const int64_t q_strides[3], const int64_t k_strides[3], const int64_t v_strides[3], const int64_t o_strides[3],
+                   const int64_t do_strides[3], float scale, int causal, int dtype, xg_stream_t stream) {
   using namespace xg;
   if (dtype != XG_BF16 && dtype != XG_F16) return XG_ERR_BAD_DTYPE;
   if (B < 0 || H < 0 || Hkv < 0 || Sq < 0 || Skv < 0) return XG_ERR_BAD_SHAPE;
@@ -454,4 +458,52 @@ extern "C" int xg_sdpa_backward(const void* q, const void* k, const void* v, con
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   if (dtype == XG_BF16) return D == 128 ? sdpa::launch_bwd<bf16_t, 128>(p, st) : sdpa::launch_bwd<bf16_t, 64>(p, st);
   return D == 128 ? sdpa::launch_bwd<f16_t, 128>(p, st) : sdpa::launch_bwd<f16_t, 64>(p, st);
+}
+
+}  // namespace
+
+// The delta workspace of xg_sdpa_backward_static: one per GPU, held until the process ends.
+constexpr int64_t kScratchFloats = int64_t(1) << 21;  // 8 MiB: B * H * Sq <= 2 097 152 query rows per call
+static __device__ __align__(256) float scratch[kScratchFloats];
+
+// Device address of `scratch` on the current GPU (every GPU holds its own copy of the array at its own address;
+// the array's name is only a host-side handle).  Looked up once per device.
+static int scratch_address(float** out) {
+  static std::mutex mu;
+  static std::map<int, float*> known;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return XG_ERR_LAUNCH;
+  std::lock_guard<std::mutex> lock(mu);
+  auto it = known.find(dev);
+  if (it == known.end()) {
+    void* ptr = nullptr;
+    if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || ptr == nullptr) return XG_ERR_LAUNCH;
+    it = known.emplace(dev, static_cast<float*>(ptr)).first;
+  }
+  *out = it->second;
+  return XG_OK;
+}
+
+extern "C" int xg_sdpa_backward(const void* q, const void* k, const void* v, const void* out, const void* d_out, const float* lse,
+                                void* dq, void* dk, void* dv, float* delta_ws, int64_t B, int64_t H, int64_t Hkv, int64_t Sq,
+                                int64_t Skv, int64_t D, const int64_t q_strides[3], const int64_t k_strides[3],
+                                const int64_t v_strides[3], const int64_t o_strides[3], const int64_t do_strides[3], float scale,
+                                int causal, int dtype, xg_stream_t stream) {
+  return backward_entry(q, k, v, out, d_out, lse, dq, dk, dv, delta_ws, B, H, Hkv, Sq, Skv, D, q_strides, k_strides, v_strides, o_strides,
+                        do_strides, scale, causal, dtype, stream);
+}
+
+extern "C" int xg_sdpa_backward_static(const void* q, const void* k, const void* v, const void* out, const void* d_out,
+                                       const float* lse, void* dq, void* dk, void* dv, int64_t B, int64_t H, int64_t Hkv, int64_t Sq,
+                                       int64_t Skv, int64_t D, const int64_t q_strides[3], const int64_t k_strides[3],
+                                       const int64_t v_strides[3], const int64_t o_strides[3], const int64_t do_strides[3],
+                                       float scale, int causal, int dtype, xg_stream_t stream) {
+  if (B < 0 || H < 0 || Sq < 0) return XG_ERR_BAD_SHAPE;
+  if (B > kScratchFloats || H > kScratchFloats || Sq > kScratchFloats || B * H > kScratchFloats || B * H * Sq > kScratchFloats)
+    return XG_ERR_TOO_LARGE;  // more query rows than the static workspace holds: use xg_sdpa_backward
+  if (B == 0 || H == 0) return XG_OK;
+  float* ws = nullptr;
+  if (int st = scratch_address(&ws)) return st;
+  return backward_entry(q, k, v, out, d_out, lse, dq, dk, dv, ws, B, H, Hkv, Sq, Skv, D, q_strides, k_strides, v_strides, o_strides,
+                        do_strides, scale, causal, dtype, stream);
 }
