@@ -25,14 +25,15 @@
 //    one k-step: the wait-and-barrier that hands slab t+1 over sits in front of
 //    the LAST k-step of slab t (whose fragments are already in registers), so the
 //    first fragments of slab t+1 and the loads of slab t+2 go out under that
-//    step's MFMAs.  One 4-byte touch per 128-byte line warms L2 further ahead,
-//    because one slab of math is too short to cover an L2 miss.  Every memory
-//    wait of the loop is explicit: the direct loads and the touches are issued
-//    as inline asm, because the compiler would otherwise wait for ALL loads in
-//    flight at the loop's back edge (a tracked touch) and in front of every
-//    transposing read (which it cannot prove disjoint from the stage being
-//    loaded), and the hand-over barrier is a bare s_barrier, without the fence
-//    of __syncthreads() that waits for the touches as well.
+//    step's MFMAs.  Every memory wait of the loop is explicit: the direct loads
+//    are issued as inline asm, because the compiler would otherwise wait for ALL
+//    loads in flight in front of every transposing read (which it cannot prove
+//    disjoint from the stage being loaded), and the hand-over barrier is a bare
+//    s_barrier, without the fence of __syncthreads().  Nothing prefetches into
+//    L2 beyond that: 4-byte "touch" loads one to four slabs ahead, from one
+//    tile per group or from every tile, all measured slower than no touches
+//    (8192 x 4096 x 11008 bf16: 616 / 648-659 / 593 us) -- the loop is limited
+//    by memory requests in flight, and every touch is one more.
 //  * gemm_staged_kernel (any K % 8 == 0): slabs pass through registers, which
 //    lets the last, partial slab be zero-filled.
 //
@@ -102,7 +103,6 @@ struct GemmParams {
   int act;
   int bias_f32;
   int tiles_m, tiles_n;
-  int pf_dist;  // how many slabs ahead the L2 warm-up touches run
   // Batched layer: grid.y entries, each a dense layer of its own on operands `*_batch` BYTES apart (0: shared by
   // every entry).  Every kernel starts with for_batch_entry(), so tiles, heuristics and limits are per entry.
   int batch;
@@ -176,16 +176,8 @@ __device__ __forceinline__ f32x16 mma(const Frag<uint8_t>& a, const Frag<uint8_t
   return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(x, y, c, 0, 0, 0, 127, 0, 127);
 }
 
-// L2 warm-up touch: a 4-byte load whose result is never read.  It is written as inline asm so that the compiler
-// does not track it: a tracked load is waited for (together with every direct load issued before it) where its
-// value is handed to the next loop iteration.  All touches write `sink`, which must stay live until a vmcnt(0)
-// wait has passed.
-__device__ __forceinline__ void touch(const char* ptr, uint32_t& sink) {
-  asm volatile("global_load_dword %0, %1, off" : "+v"(sink) : "v"(ptr) : "memory");
-}
-
 // Workgroup barrier without the memory fence of __syncthreads(), which waits for EVERY outstanding memory
-// operation, the L2 touches included.  The caller waits for what it needs with explicit s_waitcnt.
+// operation.  The caller waits for what it needs with explicit s_waitcnt.
 __device__ __forceinline__ void barrier_only() {
   __builtin_amdgcn_sched_barrier(0);
   asm volatile("s_barrier" ::: "memory");
@@ -559,34 +551,6 @@ __device__ __forceinline__ void gemm_dma_tile(const GemmParams& p, int bid, int 
     load_to_lds16(base, off, (uint32_t)(size_t)(lvoid*)dst);
   };
 
-  // L2 warm-up: one 4-byte touch per 128-byte line.  A row panel is shared by the tiles of a tile
-  // row and a B panel by the tiles of a tile column that run on the same XCD at the same time, so
-  // only one tile of each group needs to touch them.
-  const bool pf_a = (tn & 3) == 0, pf_b = (tm & 7) == 0;
-  const char* pfa_ptr;
-  const char* pfb_ptr;
-  {
-    if constexpr (AL == ALayout::KMajor) {
-      int gr = m0 + L.tid;
-      gr = gr < p.M ? gr : p.M - 1;
-      pfa_ptr = reinterpret_cast<const char*>(p.A) + ((int64_t)gr * p.lda) * EB;
-    } else {
-      int gc = m0 + (L.tid & 3) * 64;
-      gc = gc < p.M ? gc : (p.M - 8);
-      pfa_ptr = reinterpret_cast<const char*>(p.A) + ((int64_t)(L.tid >> 2) * p.lda + gc) * EB;
-    }
-    if constexpr (BL == BLayout::KMajor) {
-      int gn = n0 + (GLU ? (L.tid & 127) : L.tid);
-      gn = gn < p.N ? gn : p.N - 1;
-      pfb_ptr = reinterpret_cast<const char*>((GLU && L.tid >= 128) ? p.B2 : p.B) + ((int64_t)gn * p.ldb) * EB;
-    } else {
-      int gc = n0 + (L.tid & 3) * 64;
-      gc = gc < p.N ? gc : (p.N - 8);
-      pfb_ptr = reinterpret_cast<const char*>(p.B) + ((int64_t)(L.tid >> 2) * p.ldb + gc) * EB;
-    }
-  }
-  uint32_t pf_sink = 0;  // every touch lands here; never read
-
   f32x16 acc[4][4];
   zero_acc(acc);
   Frag<T> fa[2][4], fb[2][4];
@@ -639,31 +603,16 @@ __device__ __forceinline__ void gemm_dma_tile(const GemmParams& p, int bid, int 
     const char* b_s = a_s + SLAB_BYTES;
     const char* a_n = smem + (stage ^ 1) * STAGE_BYTES;
     const char* b_n = a_n + SLAB_BYTES;
-    // The L2 touches of this slab go out after its last direct load (the late loads all sit in k-step 0), so
-    // that the hand-over can leave them in flight; how many there are is uniform over the workgroup.
-    const bool do_pf = next && kt + 1 + p.pf_dist < KT;
-    const int touches = do_pf ? (int)pf_a + (int)pf_b : 0;
     static_for<KSTEPS>([&](auto KS) {
       constexpr int ks = decltype(KS)::value;
       constexpr bool last_step = ks + 1 == KSTEPS;
       // the transposing reads are not tracked by the compiler: this step's fragments, read under the previous
       // step, are in registers once the LDS queue is empty (it has had at least eight MFMAs to drain)
-      if constexpr (ks == 1 && next) {
-        if (do_pf && pf_a) touch(pfa_ptr + (int64_t)(kt + 1 + p.pf_dist) * a_step, pf_sink);
-        if (do_pf && pf_b) touch(pfb_ptr + (int64_t)(kt + 1 + p.pf_dist) * b_step, pf_sink);
-      }
       if constexpr (last_step && next) {
         // This step's fragments are in registers, so nothing of slab kt is read from LDS any more, and
-        // every direct load of slab kt+1 must have landed; only the touches, the newest memory reads of this
-        // wave, may stay in flight.
+        // every direct load of slab kt+1 must have landed.
         wait_lgkm0();
-        if (touches == 2) {
-          wait_vm<2>();
-        } else if (touches == 1) {
-          wait_vm<1>();
-        } else {
-          wait_vm<0>();
-        }
+        wait_vm<0>();
         barrier_only();
       }
       static_for<16>([&](auto IDX) {
@@ -693,7 +642,6 @@ __device__ __forceinline__ void gemm_dma_tile(const GemmParams& p, int bid, int 
   slab(std::false_type{}, std::false_type{}, KT - 1);
   __syncthreads();  // the slabs are dead: the epilogue reuses LDS
 
-  asm volatile("s_waitcnt vmcnt(0)" : "+v"(pf_sink)::"memory");  // the last touches have landed: their register is free again
   if constexpr (GLU) epilogue_glu<OT, NI>(p, L, acc, smem, m0, n0);
   else epilogue<OT, NI>(p, L, acc, smem, m0, n0);
 }
@@ -1274,7 +1222,6 @@ inline GemmParams make_params(const void* a, const void* b, const void* bias, co
   p.act = act;
   p.bias_f32 = bias_f32 ? 1 : 0;
   p.tiles_m = (int)((M + BM - 1) / BM);
-  p.pf_dist = 2;  // measured: distances 1 to 6 are within noise of each other on C4
   p.tiles_n = (int)((N + BN - 1) / BN);
   p.batch = 1;
   p.a_batch = p.b_batch = p.bias_batch = p.res_batch = p.out_batch = 0;
