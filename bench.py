@@ -493,6 +493,113 @@ class SdpaC5(Workload):
         return (lambda: fn(q, k, v)), how
 
 
+class SdpaBackwardC5(Workload):
+    name = "C5 causal attention backward bf16 B4 H32 S2048 D128 (dq, dk, dv from the saved row log-sum-exps)"
+    bound = "mfma"
+    dtype = "bf16"
+    unit = "TFLOP/s"
+    kernel = "sdpa_bwd_dq_kernel<bf16,128> + sdpa_bwd_dkv_kernel<bf16,128> (two launches, timed together)"
+    work = 10 * 4 * 32 * 2048 * 2048 * 128 // 2  # five matmuls (S, dP, dV, dK, dQ), lower triangle only
+    cpu_work = work // 4  # the CPU leg runs one of the four batch entries
+    traffic_key = None
+    n_sets = 2
+    cpu_warmups = 0
+
+    def setup(self, torch, dev):
+        from xpu_graph_amd import _lib
+
+        self.torch = torch
+        g = torch.Generator().manual_seed(0)
+        mk = lambda: torch.randn(4, 32, 2048, 128, generator=g).bfloat16().to(dev)  # noqa: E731
+        self.sets = []
+        for _ in range(self.n_sets):
+            q, k, v, do = mk(), mk(), mk(), mk()
+            out, lse = torch.ops.xpu_ops.sdpa_lse(q, k, v, True, 128**-0.5)
+            self.sets.append((q, k, v, out, do, lse))
+        self.grads = [tuple(torch.empty_like(s[0]) for _ in range(3)) for s in self.sets]
+        self.delta = torch.empty(4, 32, 2048, dtype=torch.float32, device=dev)
+        self.lib = _lib.lib()
+        self.st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        self.strides = (ctypes.c_int64 * 3)(32 * 2048 * 128, 2048 * 128, 128)
+        self.scale = ctypes.c_float(128**-0.5)
+
+    def op_call(self, i):
+        q, k, v, out, do, lse = self.sets[i]
+        return self.torch.ops.xpu_ops.sdpa_bwd(q, k, v, out, do, lse, True, 128**-0.5)
+
+    def abi_call(self, i):
+        q, k, v, out, do, lse = self.sets[i]
+        dq, dk, dv = self.grads[i]
+        s = self.strides
+        self.lib.xg_sdpa_backward(_p(q), _p(k), _p(v), _p(out), _p(do), _p(lse), _p(dq), _p(dk), _p(dv), _p(self.delta), 4, 32, 32, 2048, 2048,
+                                  128, s, s, s, s, s, self.scale, 1, 2, self.st)
+
+    def check(self, torch):
+        from oracle import eager
+
+        q, k, v, _, do, _ = (t[:1, :2] for t in self.sets[0])
+        leaves = [t.float().requires_grad_(True) for t in (q, k, v)]
+        want = torch.autograd.grad(eager.causal_sdpa_eager(*leaves), leaves, do.float())
+        got = self.op_call(0)
+        for a, b in zip(got, want):
+            torch.testing.assert_close(a[:1, :2].float(), b, rtol=1.6e-2, atol=b.abs().max().item() * 2.0**-7)
+
+    def cpu_fn(self, torch):
+        from oracle import eager
+
+        g = torch.Generator().manual_seed(0)
+        q, k, v = (torch.randn(1, 32, 2048, 128, generator=g).bfloat16().requires_grad_(True) for _ in range(3))
+        do = torch.randn(1, 32, 2048, 128, generator=g).bfloat16()
+
+        def run():
+            return torch.autograd.grad(eager.causal_sdpa_eager(q, k, v), (q, k, v), do)
+
+        return run, "eager autograd on one batch entry (B1 H32 S2048 D128; forward and backward, the forward's flops not counted)"
+
+
+class DenseWeightGradC4(Workload):
+    name = "C4 dense weight gradient bf16: x[8192,4096]^T @ g[8192,11008] (transposed left operand)"
+    bound = "mfma"
+    dtype = "bf16"
+    unit = "TFLOP/s"
+    kernel = "gemm_dma_kernel<bf16,[K,N] right operand,[K,M] left operand>"
+    work = 2 * 8192 * 4096 * 11008
+    traffic_key = "c4_dense_at"
+    n_sets = 3
+    cpu_warmups = 1
+
+    def setup(self, torch, dev):
+        from xpu_graph_amd import _lib
+
+        self.torch = torch
+        g = torch.Generator().manual_seed(0)
+        self.sets = [(torch.randn(8192, 4096, generator=g).bfloat16().to(dev), (0.02 * torch.randn(8192, 11008, generator=g)).bfloat16().to(dev))
+                     for _ in range(self.n_sets)]
+        self.outs = [torch.empty(4096, 11008, device=dev, dtype=torch.bfloat16) for _ in range(self.n_sets)]
+        self.lib = _lib.lib()
+        self.st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def op_call(self, i):
+        x, g = self.sets[i]
+        return self.torch.ops.xpu_ops.dense_at(x, g, None)
+
+    def abi_call(self, i):
+        x, g = self.sets[i]
+        self.lib.xg_dense_at(_p(x), _p(g), None, _p(self.outs[i]), 4096, 11008, 8192, 4096, 11008, 0, 2, self.st)
+
+    def check(self, torch):
+        x, g = self.sets[0]
+        rows = torch.arange(0, 4096, 97, device=x.device)
+        want = x[:, rows].float().t() @ g.float()
+        torch.testing.assert_close(self.op_call(0)[rows].float(), want, rtol=1.6e-2, atol=want.abs().max().item() * 2.0**-8)
+
+    def cpu_fn(self, torch):
+        g = torch.Generator().manual_seed(0)
+        x = torch.randn(8192, 4096, generator=g).bfloat16()
+        gz = (0.02 * torch.randn(8192, 11008, generator=g)).bfloat16()
+        return (lambda: x.t() @ gz), "eager bf16 matmul (x.t() @ g)"
+
+
 class LlamaBlockC5(Workload):
     name = "C5 Llama decoder block bf16 B4 S2048 hidden4096 H32 inter11008, torch.compile(mi355x) end to end"
     bound = "mfma"
@@ -558,6 +665,7 @@ TRAFFIC_KERNELS = {
     "c4_dense_fp8": {"has": ["gemm_dma_split_kernel"], "any": ["IhDF16b", "<unsigned char"]},
     "c5_dense_glu": {"has": ["gemm_glu_"]},
     "c5_sdpa": {"has": ["sdpa_fwd_kernel"]},
+    "c4_dense_at": {"has": ["gemm_dma_kernel"], "any": ["ALayoutE1", "ALayout)1"]},
 }
 COPY_YARDSTICK_BYTES = 64 << 20
 
@@ -627,7 +735,7 @@ def traffic_from(fetch_dir, write_dir, out_path=TRAFFIC_FILE):
 
 
 HEADLINE = AddLayerNormC2
-OTHERS = [RmsNormC1, SliceCatC3a, AddNC3b, DenseC4, DenseFp8C4, DenseGluC5, SdpaC5, LlamaBlockC5]
+OTHERS = [RmsNormC1, SliceCatC3a, AddNC3b, DenseC4, DenseFp8C4, DenseGluC5, SdpaC5, SdpaBackwardC5, DenseWeightGradC4, LlamaBlockC5]
 
 
 def run_workload(torch, dev, wl, steps, warmup, with_cpu=True):
@@ -663,7 +771,7 @@ def run_workload(torch, dev, wl, steps, warmup, with_cpu=True):
         fn, how = wl.cpu_fn(torch)
         t_cpu, n = _cpu_time(fn, warmups=getattr(wl, "cpu_warmups", 2))
         res["cpu_baseline"] = {
-            "value": wl.work / t_cpu / scale,
+            "value": getattr(wl, "cpu_work", wl.work) / t_cpu / scale,
             "unit": res["unit"],
             "cores": torch.get_num_threads(),
             "host_cpu_count": os.cpu_count(),
