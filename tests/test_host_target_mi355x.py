@@ -334,15 +334,20 @@ def test_library_sdpa_is_causal_flag(caplog, backend):
     assert node.args[3] is True
 
 
-def test_arbitrary_mask_is_not_taken(caplog, backend):
+def test_arbitrary_mask_travels_as_an_operand_and_an_unusable_one_is_not_taken(caplog, backend):
     def fn(q, k, v, m):
         w = torch.matmul(q, k.transpose(2, 3)) / 8.0 + m
         return torch.matmul(torch.softmax(w, dim=-1), v)
 
     q, k, v = (torch.randn(2, 4, 32, 64).to(bf16) for _ in range(3))
-    gm = rewrite(backend, fn, q, k, v, torch.randn(32, 32).to(bf16), must_fail=False)
-    assert "mi355x_sdpa" not in modules_called(gm)
-    assert "aten.scaled_dot_product_attention.default" in aten_ops(gm)
+    gm = rewrite(backend, fn, q, k, v, torch.randn(32, 32).to(bf16))  # a run-time mask: the kernel adds it
+    assert modules_called(gm) == ["mi355x_sdpa_masked"]
+    assert "aten.scaled_dot_product_attention.default" not in aten_ops(gm)
+    # an integer bias is not an attention mask the fused op accepts: no attention call (the two products go to the
+    # batched dense kernel instead)
+    gm = rewrite(backend, fn, q, k, v, torch.randint(-3, 1, (32, 32)))
+    assert not any(m.startswith("mi355x_sdpa") for m in modules_called(gm))
+    assert "aten.scaled_dot_product_attention.default" not in aten_ops(gm)
 
 
 def test_target_none_has_no_structure_patterns(caplog):

@@ -104,6 +104,10 @@ def match_attention(node):
             logger.debug("Flash attention pass: Too many add operations")
         return None
 
+    if has_mask and isinstance(mask, fx.Node) and isinstance(mask.meta.get("val"), torch.Tensor):
+        # what aten.scaled_dot_product_attention accepts as an additive mask: fp32 or the dtype of q
+        if mask.meta["val"].dtype not in (torch.float32, q.meta["val"].dtype):
+            return None
     k_shape = k.meta["val"].shape
     k_shape = tuple(k_shape[:-2]) + (k_shape[-1], k_shape[-2])
     mask_shape = mask.meta["val"].shape if has_mask and isinstance(mask, fx.Node) else []
