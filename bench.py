@@ -776,7 +776,7 @@ def run_workload(torch, dev, wl, steps, warmup, with_cpu=True):
             "cores": torch.get_num_threads(),
             "host_cpu_count": os.cpu_count(),
             "kind": "port",
-            "sample": f"{n} timed runs of the full-size workload through {how}, median {t_cpu * 1e3:.2f} ms",
+            "sample": f"{n} timed runs of {'a bounded sample of the workload' if hasattr(wl, 'cpu_work') else 'the full-size workload'} through {how}, median {t_cpu * 1e3:.2f} ms",
         }
     if hasattr(wl, "eager_ms"):
         res["eager_gpu_ms"] = wl.eager_ms
