@@ -34,6 +34,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
 BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 MFMA, published
 FP8_PEAK_TFLOPS = 5000.0
+FP32_PEAK_TFLOPS = 157.3
 N_SETS = 6  # rotating buffer sets so that timed launches stream from HBM, not from the 256 MB last-level cache
 WARM_SECONDS = 0.15  # GPU work of the same kind in front of every timed region
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "traffic.json")
@@ -343,6 +344,49 @@ class DenseC4(Workload):
         x, W, b = inputs.c4_dense(device="cpu", seed=0)
         fn, how = _default_path_compile(eager.dense_silu_eager)
         return (lambda: fn(x, W, b)), how
+
+
+class DenseFp32(Workload):
+    name = "dense + bias + SiLU fp32 M4096 K4096 N4096 (the dtype of the reference's dense-layer tests)"
+    bound = "mfma"
+    dtype = "f32"
+    unit = "TFLOP/s"
+    kernel = "gemm_dma_kernel<f32,[K,N] weight> (32x32x2 fp32 MFMA)"
+    work = 2 * 4096 * 4096 * 4096
+    traffic_key = None
+    n_sets = 3
+    cpu_warmups = 1
+
+    def setup(self, torch, dev):
+        from xpu_graph_amd import _lib
+
+        self.torch = torch
+        g = torch.Generator().manual_seed(0)
+        self.sets = [(torch.randn(4096, 4096, generator=g).to(dev), (0.02 * torch.randn(4096, 4096, generator=g)).to(dev),
+                      (0.02 * torch.randn(4096, generator=g)).to(dev)) for _ in range(self.n_sets)]
+        self.outs = [torch.empty(4096, 4096, device=dev) for _ in range(self.n_sets)]
+        self.lib = _lib.lib()
+        self.st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def op_call(self, i):
+        x, W, b = self.sets[i]
+        return self.torch.ops.xpu_ops.dense(x, W, False, b, None, "silu")
+
+    def abi_call(self, i):
+        x, W, b = self.sets[i]
+        self.lib.xg_dense(_p(x), _p(W), _p(b), None, _p(self.outs[i]), 4096, 4096, 4096, 4096, 4096, 0, 0, 3, 0, 0, self.st)
+
+    def check(self, torch):
+        x, W, b = self.sets[0]
+        rows = torch.arange(0, 4096, 97, device=x.device)
+        z = x[rows].double() @ W.double() + b.double()
+        want = torch.nn.functional.silu(z)
+        torch.testing.assert_close(self.op_call(0)[rows].double(), want, rtol=1e-5, atol=1.1 * z.abs().max().item() * 64 * 2.0**-24)
+
+    def cpu_fn(self, torch):
+        g = torch.Generator().manual_seed(0)
+        x, W, b = torch.randn(4096, 4096, generator=g), 0.02 * torch.randn(4096, 4096, generator=g), 0.02 * torch.randn(4096, generator=g)
+        return (lambda: torch.nn.functional.silu(x @ W + b)), "eager fp32 matmul + bias + SiLU"
 
 
 class DenseFp8C4(DenseC4):
@@ -735,13 +779,13 @@ def traffic_from(fetch_dir, write_dir, out_path=TRAFFIC_FILE):
 
 
 HEADLINE = AddLayerNormC2
-OTHERS = [RmsNormC1, SliceCatC3a, AddNC3b, DenseC4, DenseFp8C4, DenseGluC5, SdpaC5, SdpaBackwardC5, DenseWeightGradC4, LlamaBlockC5]
+OTHERS = [RmsNormC1, SliceCatC3a, AddNC3b, DenseC4, DenseFp32, DenseFp8C4, DenseGluC5, SdpaC5, SdpaBackwardC5, DenseWeightGradC4, LlamaBlockC5]
 
 
 def run_workload(torch, dev, wl, steps, warmup, with_cpu=True):
     wl.setup(torch, dev)
     wl.check(torch)
-    peak = HBM_PEAK_GBPS if wl.bound == "hbm" else (FP8_PEAK_TFLOPS if wl.dtype == "fp8" else BF16_PEAK_TFLOPS)
+    peak = HBM_PEAK_GBPS if wl.bound == "hbm" else {"fp8": FP8_PEAK_TFLOPS, "f32": FP32_PEAK_TFLOPS}.get(wl.dtype, BF16_PEAK_TFLOPS)
     scale = 1e9 if wl.bound == "hbm" else 1e12
     n_sets = getattr(wl, "n_sets", N_SETS)
     entry = _traffic_table().get(getattr(wl, "traffic_key", None) or "", None)

@@ -191,7 +191,12 @@ int xg_dense_glu(const void* a, const void* w_gate, const void* w_up, void* out,
  *   b_trans == 1 (the nn.Linear weight layout).
  *   bias: NULL or [N] (dtype `dtype` or XG_F32 via bias_dtype).
  *   residual: NULL or [M,N] row stride ldr, added before the activation.
- *   dtype: XG_BF16 or XG_F16 (inputs and output).
+ *   dtype: XG_BF16, XG_F16 or XG_F32 (inputs and output).  16-bit types use
+ *   the 32x32x16 MFMA, fp32 the 32x32x2 fp32 MFMA (plain IEEE fp32 products and
+ *   sums: no reduced-precision passes); fp32 is the dtype of the reference's
+ *   dense-layer tests (tests/mlu/test_custom_denselayer.py:11).  K, lda, ldb,
+ *   ldr multiples of 8 elements (4 for fp32), N a multiple of 8.
+ *   xg_dense_batched and xg_dense_at take the 16-bit types only.
  * replaces torch_mlu_ops.matmul as called by DenseLayerModule.forward
  *   (passes/patterns/targets/mlu/structure_replacements/dense_layer_modules.py:4-56).
  *

@@ -94,6 +94,30 @@ def test_c4_dense_silu(device):
     torch.testing.assert_close(out, eager.dense_silu_eager(x, W, b), rtol=1.6e-2, atol=2e-2)
 
 
+@pytest.mark.parametrize("form", ["mm", "mm_t_bias_sigmoid"])
+def test_fp32_dense_layer_of_the_reference_tests(device, form):
+    """The reference's dense-layer tests are fp32 (tests/mlu/test_custom_denselayer.py:11, 109-119: inputs
+    [4096, 768], weight [768, 16] or [16, 768], bias [16]); compiled for the mi355x target they run on the fp32 MFMA
+    kernel and agree with float64."""
+    x = torch.randn(4096, 768, device=device)
+    b = torch.randn(16, device=device)
+    if form == "mm":
+        w = torch.randn(768, 16, device=device)
+        fn = lambda x, w: torch.matmul(x, w).reshape(128, 32, 16)  # noqa: E731
+        args, want = (x, w), (x.double() @ w.double()).reshape(128, 32, 16)
+        noise = want.abs().max().item() * 768**0.5 * 2.0**-24  # fp32 accumulation of 768 terms
+    else:
+        w = torch.randn(16, 768, device=device)
+        fn = lambda x, w, b: torch.sigmoid(torch.matmul(x, w.transpose(0, 1)) + b)  # noqa: E731
+        z = x.double() @ w.double().t() + b.double()
+        args, want = (x, w, b), torch.sigmoid(z)
+        noise = 0.25 * z.abs().max().item() * 768**0.5 * 2.0**-24  # the same noise through the sigmoid's largest slope
+    out, mods, rest = run(fn, *args)
+    assert mods == ["custom_dense_layer_replacement"], (mods, rest)
+    assert not any("aten.mm" in t or "addmm" in t or "sigmoid" in t for t in rest), rest
+    torch.testing.assert_close(out.double(), want, rtol=1e-5, atol=noise)
+
+
 def test_swiglu(device):
     x = torch.randn(512, 2 * 1408, device=device).bfloat16()
     out, mods, rest = run(eager.silu_mul_eager, x)

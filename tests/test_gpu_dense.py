@@ -236,6 +236,60 @@ def test_dense_at_reads_strided_views_in_place(device):
         ops.dense_at(big_a[:, :12], b, None)
 
 
+def ref64(x, W, weight_trans, bias, residual, act):
+    z = x.double() @ (W.double().t() if weight_trans else W.double())
+    if bias is not None:
+        z = z + bias.double()
+    if residual is not None:
+        z = z + residual.double()
+    return {"none": lambda t: t, "relu": torch.relu, "silu": torch.nn.functional.silu, "gelu": torch.nn.functional.gelu,
+            "sigmoid": torch.sigmoid}[act](z)
+
+
+def close_fp32(got, want64, k):
+    """fp32 layer against the float64 product: products are exact in fp32 MFMA arithmetic and the K-term sum is
+    rounded to fp32 as it grows, a random walk of half-ulp steps at the size of the partial sums -- rtol 1e-5 plus
+    sqrt(K) * 2^-24 of the largest output."""
+    assert got.dtype == torch.float32
+    atol = want64.abs().max().item() * (k**0.5) * 2.0**-24
+    torch.testing.assert_close(got.double(), want64, rtol=1e-5, atol=atol)
+
+
+@pytest.mark.parametrize("weight_trans", [False, True])
+@pytest.mark.parametrize(
+    "M,N,K", [(256, 256, 32), (512, 768, 256), (300, 264, 200), (1, 8, 4), (1000, 1032, 76), (4096, 16, 768), (64, 4096, 4096), (2048, 2048, 2048)]
+)
+def test_dense_fp32_shapes(device, weight_trans, M, N, K):
+    """The fp32 layer (32x32x2 fp32 MFMA): whole and partial 32-element slabs, ragged tiles, the reference's own
+    dense-layer test shape ([4096, 768] x [768, 16], tests/mlu/test_custom_denselayer.py:112-119), both weight
+    layouts, bias / residual / activation in the epilogue."""
+    g = torch.Generator().manual_seed(M + N + K)
+    x = torch.randn(M, K, generator=g).to(device)
+    W = (torch.randn(N, K, generator=g) / K**0.5).to(device)
+    if not weight_trans:
+        W = W.t().contiguous()
+    b = torch.randn(N, generator=g).to(device)
+    res = torch.randn(M, N, generator=g).to(device)
+    got = _ops().dense(x, W, weight_trans, None, None, "none")
+    assert got.shape == (M, N)
+    close_fp32(got, ref64(x, W, weight_trans, None, None, "none"), K)
+    got = _ops().dense(x, W, weight_trans, b, res, "gelu")
+    close_fp32(got, ref64(x, W, weight_trans, b, res, "gelu"), K)
+
+
+def test_dense_fp32_exact_on_small_integers(device):
+    """Integer-valued operands whose products and sums stay below 2^24 come out exact: a dropped k-step, a swapped
+    fragment or a wrong swizzle cannot hide behind a tolerance."""
+    g = torch.Generator().manual_seed(5)
+    for weight_trans in (False, True):
+        x = torch.randint(-8, 9, (520, 328), generator=g).float().to(device)
+        W = torch.randint(-8, 9, (328, 264), generator=g).float().to(device)
+        want = x.double() @ W.double()
+        Wk = W.t().contiguous() if weight_trans else W
+        got = _ops().dense(x, Wk, weight_trans, None, None, "none")
+        assert torch.equal(got.double(), want)
+
+
 def test_dense_takes_column_sliced_views(device):
     """A linear layer fed by a column slice of a wider tensor: row strides or bases that are not multiples of 16 bytes
     (what eager accepts anywhere) are copied by the wrapper instead of being refused by the kernel."""

@@ -286,10 +286,17 @@ def test_c4_dense(caplog, backend, form):
     assert "Pattern.CustomDenseLayer changed graph" in caplog.text
 
 
-def test_dense_constraint_vetoes_fp32_and_odd_sizes(caplog, backend):
-    rewrite(backend, lambda x, w: x @ w, torch.randn(8, 16), torch.randn(16, 8), must_fail=False)  # fp32 stays Aten
+def test_dense_constraint_vetoes_odd_sizes_and_takes_fp32(caplog, backend):
+    """16-byte operand loads: K a multiple of 8 for 16-bit types and of 4 for fp32; N a multiple of 8.  fp32 layers
+    (the dtype of the reference's dense-layer tests, tests/mlu/test_custom_denselayer.py:11) go to the fp32 MFMA kernel."""
     rewrite(backend, lambda x, w: x @ w, torch.randn(8, 12).to(bf16), torch.randn(12, 8).to(bf16), must_fail=False)
+    rewrite(backend, lambda x, w: x @ w, torch.randn(8, 6), torch.randn(6, 8), must_fail=False)
+    rewrite(backend, lambda x, w: x @ w, torch.randn(8, 16), torch.randn(16, 12), must_fail=False)
+    rewrite(backend, lambda x, w: x @ w, torch.randn(8, 16, dtype=torch.float64), torch.randn(16, 8, dtype=torch.float64), must_fail=False)
     assert "Pattern.CustomDenseLayer changed graph" not in caplog.text
+    gm = rewrite(backend, lambda x, w, b: torch.relu(x @ w + b), torch.randn(8, 12), torch.randn(12, 8), torch.randn(8))
+    assert modules_called(gm) == ["custom_dense_layer_replacement"]
+    assert "Pattern.CustomDenseLayer changed graph" in caplog.text
 
 
 def test_swiglu_both_forms(caplog, backend):

@@ -5,6 +5,7 @@ namespace xg {
 namespace gemm {
 int launch_f16(const GemmParams& p, bool b_trans, hipStream_t st);  // gemm_f16.hip
 int launch_at_f16(const GemmParams& p, hipStream_t st);               // gemm_f16.hip
+int launch_f32(const GemmParams& p, bool b_trans, hipStream_t st);  // gemm_f32.hip
 int launch_at_bf16(const GemmParams& p, hipStream_t st) { return launch_gemm_at<bf16_t, bf16_t>(p, st); }
 int launch_glu_f16(const GemmParams& p, hipStream_t st);              // gemm_f16.hip
 int launch_glu_bf16(const GemmParams& p, hipStream_t st) { return launch_glu<bf16_t, bf16_t>(p, st); }
@@ -24,17 +25,19 @@ int xg_dense(const void* a, const void* b, const void* bias, const void* residua
   if (a == nullptr || b == nullptr || out == nullptr) return XG_ERR_NULL_PTR;
   if (M < 0 || N <= 0 || K <= 0 || lda < K || (b_trans ? ldb < K : ldb < N) || (residual && ldr < N)) return XG_ERR_BAD_SHAPE;
   if (M > 0x7fffffff || N > 0x7fffffff || K > 0x7fffffff) return XG_ERR_TOO_LARGE;
-  if (dtype != XG_BF16 && dtype != XG_F16) return XG_ERR_BAD_DTYPE;
+  if (dtype != XG_BF16 && dtype != XG_F16 && dtype != XG_F32) return XG_ERR_BAD_DTYPE;
   if (bias && bias_dtype != dtype && bias_dtype != XG_F32) return XG_ERR_BAD_DTYPE;
   if (act < XG_ACT_NONE || act > XG_ACT_SIGMOID) return XG_ERR_BAD_ARG;
-  // 16-byte operand loads and 16-byte output stores
-  if (K % 8 != 0 || N % 8 != 0 || lda % 8 != 0 || ldb % 8 != 0 || (residual && ldr % 8 != 0)) return XG_ERR_BAD_ALIGN;
+  // 16-byte operand loads (8 elements of a 16-bit type, 4 of fp32); 8 output columns per lane
+  const int64_t per16 = dtype == XG_F32 ? 4 : 8;
+  if (K % per16 != 0 || N % 8 != 0 || lda % per16 != 0 || ldb % per16 != 0 || (residual && ldr % per16 != 0)) return XG_ERR_BAD_ALIGN;
   if (!aligned_to(a, 16) || !aligned_to(b, 16) || !aligned_to(out, 16) || (bias && !aligned_to(bias, 16)) ||
       (residual && !aligned_to(residual, 16)))
     return XG_ERR_BAD_ALIGN;
   if (M == 0) return XG_OK;
   const GemmParams p = make_params(a, b, bias, residual, out, M, N, K, lda, ldb, ldr, act, bias && bias_dtype == XG_F32);
   hipStream_t st = (hipStream_t)stream;
+  if (dtype == XG_F32) return gemm::launch_f32(p, b_trans != 0, st);
   return dtype == XG_BF16 ? gemm::launch_bf16(p, b_trans != 0, st) : gemm::launch_f16(p, b_trans != 0, st);
 }
 

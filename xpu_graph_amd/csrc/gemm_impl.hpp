@@ -147,6 +147,11 @@ struct Elem<f16_t> {
   static constexpr int KSTEPS = 4;
 };
 template <>
+struct Elem<float> {
+  static constexpr int BYTES = 4;
+  static constexpr int KSTEPS = 4;  // a k-step is 8 elements (two 16-byte chunks): 4 x (32x32x2) per lane chunk
+};
+template <>
 struct Elem<uint8_t> {  // OCP e4m3
   static constexpr int BYTES = 1;
   static constexpr int KSTEPS = 2;  // 2 x (32x32x64) per 128-element slab
@@ -168,6 +173,16 @@ __device__ __forceinline__ f32x16 mma(const Frag<bf16_t>& a, const Frag<bf16_t>&
 }
 __device__ __forceinline__ f32x16 mma(const Frag<f16_t>& a, const Frag<f16_t>& b, f32x16 c) {
   return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a.v), __builtin_bit_cast(f16x8, b.v), c, 0, 0, 0);
+}
+// fp32: a lane's 16-byte chunk holds 4 consecutive k of its row; MFMA m of the four takes element m from both
+// operands (lane half h supplies k slot h), so a k-step covers k = 8 ks + 4 h + m.
+__device__ __forceinline__ f32x16 mma(const Frag<float>& a, const Frag<float>& b, f32x16 c) {
+  // the whole vector is reinterpreted first: a bit cast of a single swizzled element (a.v.y) reads element 0
+  const f32x4 x = __builtin_bit_cast(f32x4, a.v), y = __builtin_bit_cast(f32x4, b.v);
+  c = __builtin_amdgcn_mfma_f32_32x32x2f32(x[0], y[0], c, 0, 0, 0);
+  c = __builtin_amdgcn_mfma_f32_32x32x2f32(x[1], y[1], c, 0, 0, 0);
+  c = __builtin_amdgcn_mfma_f32_32x32x2f32(x[2], y[2], c, 0, 0, 0);
+  return __builtin_amdgcn_mfma_f32_32x32x2f32(x[3], y[3], c, 0, 0, 0);
 }
 __device__ __forceinline__ f32x16 mma(const Frag<uint8_t>& a, const Frag<uint8_t>& b, f32x16 c) {
   const i32x8 x = {(int)a.lo.x, (int)a.lo.y, (int)a.lo.z, (int)a.lo.w, (int)a.hi.x, (int)a.hi.y, (int)a.hi.z, (int)a.hi.w};
@@ -239,7 +254,7 @@ struct Lane {
 template <typename T, BLayout BL, int U, ALayout AL = ALayout::KMajor>
 __device__ __forceinline__ void read_unit(const Lane& L, const char* a_s, const char* b_s, int ks, Frag<T> (&fa)[4],
                                           Frag<T> (&fb)[4]) {
-  if constexpr (Elem<T>::BYTES == 2) {
+  if constexpr (Elem<T>::BYTES >= 2) {
     const int ch = ((ks * 2 + L.half) ^ L.fsw) << 4;
     if constexpr (U < 4 && AL == ALayout::MMajor) {
       // slab is [64 k][256 m]: the same transposing read as for an N-contiguous B, with this wave's row units
@@ -254,6 +269,15 @@ __device__ __forceinline__ void read_unit(const Lane& L, const char* a_s, const 
       fa[U].v = *reinterpret_cast<const u32x4*>(a_s + L.a_row[U] + ch);
     } else if constexpr (BL == BLayout::KMajor) {
       fb[U - 4].v = *reinterpret_cast<const u32x4*>(b_s + L.b_row[U - 4] + ch);
+    } else if constexpr (Elem<T>::BYTES == 4) {
+      // fp32 slab is [32 k][256 n], 1 KiB per k row, the two 128-byte halves of every 256 bytes swapped on k rows
+      // with bit 2 set, so that the two lane halves (k rows 4 apart) read different banks.  Four 4-byte reads:
+      // k = 8 ks + 4 half + m at column n.
+      constexpr int j = U - 4;
+      const int n4 = ((L.wn * 128 + j * 32 + L.l32) * 4) ^ (L.half << 7);
+      const char* at = b_s + (ks * 8 + L.half * 4) * 1024 + n4;
+      fb[j].v = u32x4{*reinterpret_cast<const uint32_t*>(at), *reinterpret_cast<const uint32_t*>(at + 1024),
+                      *reinterpret_cast<const uint32_t*>(at + 2048), *reinterpret_cast<const uint32_t*>(at + 3072)};
     } else {
       // slab is [64 k][256 n]: a 16-lane group reads a 4(k) x 16(n) block and gets it back transposed
       constexpr int j = U - 4;
@@ -489,7 +513,8 @@ __device__ __forceinline__ void gemm_dma_tile(const GemmParams& p, int bid, int 
   constexpr int EB = Elem<T>::BYTES;
   constexpr int KSTEPS = Elem<T>::KSTEPS;
   constexpr int SLAB_K = ROW_BYTES / EB;
-  static_assert(BL == BLayout::KMajor || EB == 2, "the transposing LDS read is wired for 16-bit elements only");
+  static_assert(BL == BLayout::KMajor || EB >= 2, "N-contiguous weights: 16-bit (transposing LDS read) or fp32 (4-byte reads)");
+  static_assert(AL == ALayout::KMajor || EB == 2, "M-contiguous A is wired for 16-bit elements only");
 
   int tm, tn;
   tile_of_block(p, bid, nb, tm, tn);
@@ -522,6 +547,13 @@ __device__ __forceinline__ void gemm_dma_tile(const GemmParams& p, int bid, int 
         int gn = n0 + (GLU ? (r & 127) : r);  // gated: tile rows 128..255 are rows 0..127 again, of the up weight
         gn = gn < p.N ? gn : p.N - 1;
         b_off[j] = (uint32_t)(((int64_t)gn * p.ldb) * EB + lc * 16);
+      } else if constexpr (EB == 4) {
+        // load j of this wave fills k row 4 j + wave (1 KiB); lane i lands at chunk i, which holds column chunk
+        // i ^ 8 on k rows with bit 2 set (see read_unit)
+        const int kr = j * 4 + L.wave;
+        int gc = n0 + ((L.lane ^ (((kr >> 2) & 1) << 3)) << 2);
+        gc = gc < p.N ? gc : (p.N - 4);  // N % 8 == 0 is checked on the host
+        b_off[j] = (uint32_t)(((int64_t)kr * p.ldb + gc) * EB);
       } else {
         const int kr = j * 8 + L.wave * 2 + L.half;
         const int pc32 = L.lane & 31;
@@ -706,8 +738,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
   constexpr int EB = Elem<T>::BYTES;
   constexpr int KSTEPS = Elem<T>::KSTEPS;
   constexpr int SLAB_K = ROW_BYTES / EB;
-  static_assert(BL == BLayout::KMajor || EB == 2, "the transposing LDS read is wired for 16-bit elements only");
-  static_assert(AL == ALayout::KMajor || BL == BLayout::NMajor, "M-contiguous A goes with N-contiguous B");
+  static_assert(BL == BLayout::KMajor || EB >= 2, "N-contiguous weights: 16-bit or fp32");
+  static_assert(AL == ALayout::KMajor || (BL == BLayout::NMajor && EB == 2), "M-contiguous A goes with N-contiguous B, 16-bit");
 
   int tm, tn;
   tile_of_block(p, blockIdx.x, gridDim.x, tm, tn);
@@ -751,6 +783,17 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
       b_ptr[j] = reinterpret_cast<const char*>(p.B) + ((int64_t)gr * p.ldb) * EB + c8 * 16;
       b_lds[j] = r * ROW_BYTES + ((c8 ^ swz(r)) << 4);
     }
+  } else if constexpr (EB == 4) {
+    // fp32 N-major operand: slab is [32 k][256 n]; thread covers 16-byte chunk c64 (4 columns) of k rows kr0 + 4 j.
+    const int c64 = tid & 63, kr0 = tid >> 6;
+    int gc = n0 + c64 * 4;
+    gc = gc < p.N ? gc : (p.N - 4);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int kr = kr0 + 4 * j;
+      b_ptr[j] = reinterpret_cast<const char*>(p.B) + ((int64_t)kr * p.ldb + gc) * EB;
+      b_lds[j] = kr * 1024 + ((c64 ^ (((kr >> 2) & 1) << 3)) << 4);
+    }
   } else {
     // N-major operand: slab is [64 k][256 n]; thread covers 16-byte chunk c32 (8 columns) of k rows kr0 + 8 j.
     const int c32 = tid & 31, kr0 = tid >> 5;
@@ -783,7 +826,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
       }
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
-        const bool ok = BL == BLayout::KMajor ? (c8 * (16 / EB) < k_left) : ((tid >> 5) + 8 * j < k_left);
+        const bool ok = BL == BLayout::KMajor ? (c8 * (16 / EB) < k_left) : (EB == 4 ? (tid >> 6) + 4 * j < k_left : (tid >> 5) + 8 * j < k_left);
         gb[j] = ok ? *reinterpret_cast<const u32x4*>(b_ptr[j] + boff) : u32x4{0, 0, 0, 0};
       }
     }
@@ -875,6 +918,15 @@ __global__ __launch_bounds__(kThreads) void gemm_small_kernel(GemmParams p_all) 
       int gn = n0 + (GLU ? (r & 31) : r);  // gated: load 0 of a wavefront fills gate rows, load 1 the same rows of up
       gn = gn < p.N ? gn : p.N - 1;
       b_off[q] = (uint32_t)(((int64_t)gn * p.ldb) * EB + ((slot ^ swz(r)) << 4));
+    } else if constexpr (EB == 4) {
+      // fp32 slab is [32 k][64 n], 256 bytes per k row: a 1 KiB load covers k rows 4 L .. 4 L + 3 (L = q * 4 + wave),
+      // lane i lands at chunk i & 15 of row i >> 4; on the loads with odd L (k bit 2 set) the two 128-byte halves of a
+      // row are swapped so that the lane halves of a fragment read (k rows 4 apart) fall on different banks
+      const int load = q * 4 + wave;
+      const int kr = load * 4 + (lane >> 4);
+      int gc = n0 + (((lane & 15) ^ ((load & 1) << 3)) << 2);
+      gc = gc < p.N ? gc : p.N - 4;  // N % 8 == 0 is checked on the host
+      b_off[q] = (uint32_t)(((int64_t)kr * p.ldb + gc) * EB);
     } else {
       int gc = n0 + ((slot ^ (((r >> 1) & 1) << 2)) << 3);  // r is the k row here
       gc = gc < p.N ? gc : p.N - 8;                          // N % 8 == 0 is checked on the host
@@ -908,6 +960,9 @@ __global__ __launch_bounds__(kThreads) void gemm_small_kernel(GemmParams p_all) 
       b_frag[u] = S_SLAB_BYTES + brow * ROW_BYTES + (((ks * 4 + half * 2) ^ swz(brow)) << 4);
     } else if constexpr (BL == BLayout::KMajor) {
       b_frag[u] = S_SLAB_BYTES + a_frag[u];
+    } else if constexpr (EB == 4) {
+      // k = 8 ks + 4 half + m (m = 0..3: four 4-byte reads 256 bytes apart) at column 32 u + l32
+      b_frag[u] = S_SLAB_BYTES + (ks * 8 + half * 4) * 256 + (((u * 32 + l32) * 4) ^ (half << 7));
     } else {
       const int kr = wave * 16 + half * 8 + (p16 >> 2);
       const int chunk = u * 4 + blk * 2 + ((p16 & 3) >> 1);
@@ -953,6 +1008,11 @@ __global__ __launch_bounds__(kThreads) void gemm_small_kernel(GemmParams p_all) 
       } else if constexpr (BL == BLayout::KMajor) {
         fa[u].v = *reinterpret_cast<const u32x4*>(st + a_frag[u]);
         fb[u].v = *reinterpret_cast<const u32x4*>(st + b_frag[u]);
+      } else if constexpr (EB == 4) {
+        fa[u].v = *reinterpret_cast<const u32x4*>(st + a_frag[u]);
+        const char* at = st + b_frag[u];
+        fb[u].v = u32x4{*reinterpret_cast<const uint32_t*>(at), *reinterpret_cast<const uint32_t*>(at + 256),
+                        *reinterpret_cast<const uint32_t*>(at + 512), *reinterpret_cast<const uint32_t*>(at + 768)};
       } else {
         fa[u].v = *reinterpret_cast<const u32x4*>(st + a_frag[u]);
         const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(st + b_frag[u]));

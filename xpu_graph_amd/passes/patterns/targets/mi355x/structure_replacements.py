@@ -147,10 +147,12 @@ class DenseLayerModule(torch.nn.Module):
 
 
 def can_fuse_custom_denselayer(inputs, weight, weight_trans, bias, act_str):
-    """Match-time veto (arguments are FakeTensors): what the MFMA kernel cannot take stays in Aten."""
+    """Match-time veto (arguments are FakeTensors): what the MFMA kernels cannot take stays in Aten.  bf16 / f16
+    (32x32x16 MFMA) and fp32 (32x32x2 fp32 MFMA, the dtype of the reference's own dense-layer tests,
+    tests/mlu/test_custom_denselayer.py:11)."""
     if act_str not in ("none", "relu", "gelu", "silu", "sigmoid"):
         return False
-    if inputs.dtype not in _DENSE_DTYPES or weight.dtype != inputs.dtype:
+    if inputs.dtype not in (*_DENSE_DTYPES, torch.float32) or weight.dtype != inputs.dtype:
         return False
     if inputs.dim() != 2 or weight.dim() != 2:
         return False
@@ -160,7 +162,8 @@ def can_fuse_custom_denselayer(inputs, weight, weight_trans, bias, act_str):
     n = weight.shape[0] if weight_trans else weight.shape[1]
     if not (isinstance(k, int) and isinstance(n, int)):
         return False
-    return k % 8 == 0 and n % 8 == 0 and k > 0 and n > 0
+    per16 = 16 // inputs.element_size()  # 16-byte operand loads: 8 elements of a 16-bit type, 4 of fp32
+    return k % per16 == 0 and n % 8 == 0 and k > 0 and n > 0
 
 
 class BatchDenseLayerModule(torch.nn.Module):
