@@ -234,15 +234,25 @@ __global__ __launch_bounds__(kThreads) void sdpa_bwd_dq_kernel(BwdParams p) {
     int lim = p.Skv - 1;  // last visible key of this lane's query
     if (p.causal) lim = lim < qrow ? lim : qrow;
     const int rel = lim - kv0 - 4 * h;
+    // only tiles that cross the diagonal or the end of the keys pay for the mask (wave-uniform)
+    const bool need_mask = (p.causal && kv0 + BKV - 1 > qw_max - 31) || (kv0 + BKV > p.Skv);
     static_for<2>([&](auto TI) {
       constexpr int t = decltype(TI)::value;
-      const f32x16 s = rows_times_regs<T, D>(k_s, t, l32, h, sx, qf);
+      f32x16 s = rows_times_regs<T, D>(k_s, t, l32, h, sx, qf);
       const f32x16 dp = rows_times_regs<T, D>(v_s, t, l32, h, sx, dof);
+      float cc = c;
+      if (need_mask) {
+        static_for<16>([&](auto VI) {
+          constexpr int v = decltype(VI)::value;
+          constexpr int key = 32 * t + 8 * (v / 4) + (v % 4);
+          s[v] = key > rel ? -INFINITY : s[v] * cc;  // scaled here so that a negative scale cannot turn -inf around
+        });
+        cc = 1.f;
+      }
       f32x16 ds;
       static_for<16>([&](auto VI) {
         constexpr int v = decltype(VI)::value;
-        constexpr int key = 32 * t + 8 * (v / 4) + (v % 4);
-        const float pr = key > rel ? 0.f : __builtin_amdgcn_exp2f(__builtin_fmaf(s[v], c, -L));
+        const float pr = __builtin_amdgcn_exp2f(__builtin_fmaf(s[v], cc, -L));
         ds[v] = pr * (dp[v] - delta);
       });
       transposed_times_held<T, D>(k_s, t, TL, ds, dq_acc);
@@ -349,8 +359,19 @@ __global__ __launch_bounds__(kThreads) void sdpa_bwd_dkv_kernel(BwdParams p) {
     // sub-tiles' products first and the exponentials of one woven between the MFMAs of the other with scheduling
     // groups -- 689-732 us against 691 us for dq + dk/dv at B4 H32 S2048 D128: with one wave per SIMD the scores sit
     // in accumulation registers, and the moves that hand them to the vector ALU queue behind the MFMAs.)
-    auto soft = [&](auto TI, const f32x16& s, const f32x16& dp, f32x16& pr, f32x16& ds) {
+    // only tiles that cross the diagonal or the end of the queries pay for the mask (wave-uniform)
+    const bool need_mask = (p.causal && qt0 < kw_min + 31) || (qt0 + BKV > p.Sq);
+    auto soft = [&](auto TI, f32x16& s, const f32x16& dp, f32x16& pr, f32x16& ds) {
       constexpr int t = decltype(TI)::value;
+      float cc = c;
+      if (need_mask) {
+        static_for<16>([&](auto VI) {
+          constexpr int v = decltype(VI)::value;
+          constexpr int qi = 32 * t + 8 * (v / 4) + (v % 4);
+          s[v] = (qi < q_lo || qi >= q_hi) ? -INFINITY : s[v] * cc;  // scaled here: a negative scale must not turn -inf around
+        });
+        cc = 1.f;
+      }
       static_for<4>([&](auto GI) {
         constexpr int g = decltype(GI)::value;
         const f32x4 l4 = *reinterpret_cast<const f32x4*>(st_s + (32 * t + 8 * g + 4 * h) * 4);
@@ -358,17 +379,14 @@ __global__ __launch_bounds__(kThreads) void sdpa_bwd_dkv_kernel(BwdParams p) {
         static_for<4>([&](auto EI) {
           constexpr int e = decltype(EI)::value;
           constexpr int v = 4 * g + e;
-          constexpr int qi = 32 * t + 8 * g + e;
-          const bool masked = qi < q_lo || qi >= q_hi;
-          const float e2 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[v], c, -l4[e] * kLog2e));
-          pr[v] = masked ? 0.f : e2;
+          pr[v] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[v], cc, -l4[e] * kLog2e));
           ds[v] = pr[v] * (dp[v] - d4[e]);
         });
       });
     };
     static_for<2>([&](auto TI) {
       constexpr int t = decltype(TI)::value;
-      const f32x16 s = rows_times_regs<T, D>(q_s, t, l32, h, sx, kf);
+      f32x16 s = rows_times_regs<T, D>(q_s, t, l32, h, sx, kf);
       const f32x16 dp = rows_times_regs<T, D>(do_s, t, l32, h, sx, vf);
       f32x16 pr, ds;
       soft(TI, s, dp, pr, ds);
