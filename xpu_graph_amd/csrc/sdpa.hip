@@ -178,15 +178,18 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
     const char* v_s = k_s + TILE;
 
     // S^T tile: s[t][v] = <key 32t + 8(v/4) + 4h + v%4 , query l32>
+    // The two 32-key halves alternate MFMA by MFMA: a dependent MFMA cannot issue until its predecessor has
+    // left the pipe (a chain of eight ran at one MFMA per ~80 clocks in a probe kernel), two interleaved chains can.
     f32x16 s[2];
-    static_for<2>([&](auto TI) {
-      constexpr int t = decltype(TI)::value;
-      s[t] = f32x16{0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-      static_for<KK>([&](auto KI) {
-        constexpr int kk = decltype(KI)::value;
+    s[0] = s[1] = f32x16{0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    static_for<KK>([&](auto KI) {
+      constexpr int kk = decltype(KI)::value;
+      static_for<2>([&](auto TI) {
+        constexpr int t = decltype(TI)::value;
         const int off = l32 * RB + (((2 * kk + h) ^ kx) << 4);
         const V8 kf = *reinterpret_cast<const V8*>(k_s + 32 * t * RB + off);
         s[t] = mma(kf, qf[kk], s[t]);
+        __builtin_amdgcn_sched_barrier(0x7F7);  // everything but MFMAs may move across: the MFMA order stays as written
       });
     });
 
