@@ -697,6 +697,57 @@ class LlamaBlockC5(Workload):
         return run, how
 
 
+class LlamaBlockTrainC5(LlamaBlockC5):
+    name = "C5 Llama decoder block bf16 B4 S2048 training step (forward + backward), torch.compile(mi355x, is_training) end to end"
+    kernel = "whole compiled training step (dense / gated dense and their input- and weight-gradient launches, attention forward with row statistics, the two attention backward kernels, rotary, norms; Aten for the norm and gate formulas)"
+    work = 3 * LlamaBlockC5.work  # one forward, two products per forward product in the backward
+    cpu_work = work // 4            # the CPU leg runs one of the four batch entries
+    cpu_warmups = 0
+
+    def setup(self, torch, dev):
+        from oracle import eager, inputs
+        from xpu_graph_amd import OptLevel, Target, XpuGraph, XpuGraphConfig
+
+        self.torch = torch
+        x, p = inputs.c5_llama_block(device=dev)
+        names = sorted(p)
+
+        def block(x, *ws):
+            return eager.llama_block_eager(x, dict(zip(names, ws)), n_heads=32)
+
+        self.eager_fn = block
+        self.args = [x.requires_grad_(True)] + [p[n].requires_grad_(True) for n in names]
+        backend = XpuGraph(XpuGraphConfig(is_training=True, target=Target.mi355x, opt_level=OptLevel.level2, enable_cache=False))
+        self.fn = torch.compile(block, backend=backend, dynamic=False)
+
+    def _step(self, fn):
+        return self.torch.autograd.grad(fn(*self.args).float().pow(2).mean(), self.args)
+
+    def op_call(self, i):
+        return self._step(self.fn)
+
+    abi_call = op_call
+
+    def check(self, torch):
+        got = self.op_call(0)
+        want = self._step(self.eager_fn)
+        self.eager_ms = _events_time(torch, lambda i: self._step(self.eager_fn), 1, 3, 1) * 1e3
+        for a, b in zip(got, want):  # eager bf16 is the yardstick here; tests/test_gpu_training.py compares both with fp32 autograd
+            assert (a.float() - b.float()).abs().mean().item() <= 0.1 * b.float().abs().mean().item() + 1e-6
+
+    def cpu_fn(self, torch):
+        from oracle import eager, inputs
+
+        x, p = inputs.c5_llama_block(B=1, device="cpu")
+        names = sorted(p)
+        args = [x.requires_grad_(True)] + [p[n].requires_grad_(True) for n in names]
+
+        def run():
+            return torch.autograd.grad(eager.llama_block_eager(args[0], dict(zip(names, args[1:])), n_heads=32).float().pow(2).mean(), args)
+
+        return run, "eager autograd on one batch entry (B1 S2048)"
+
+
 # ---- roofline.traffic: HBM bytes per launch from two rocprofv3 --pmc runs of this file -------------------------
 # kernel of each workload as it appears in rocprofv3's Kernel_Name column (mangled or demangled): all of `has`, and
 # any of `any` when given
@@ -779,7 +830,7 @@ def traffic_from(fetch_dir, write_dir, out_path=TRAFFIC_FILE):
 
 
 HEADLINE = AddLayerNormC2
-OTHERS = [RmsNormC1, SliceCatC3a, AddNC3b, DenseC4, DenseFp32, DenseFp8C4, DenseGluC5, SdpaC5, SdpaBackwardC5, DenseWeightGradC4, LlamaBlockC5]
+OTHERS = [RmsNormC1, SliceCatC3a, AddNC3b, DenseC4, DenseFp32, DenseFp8C4, DenseGluC5, SdpaC5, SdpaBackwardC5, DenseWeightGradC4, LlamaBlockC5, LlamaBlockTrainC5]
 
 
 def run_workload(torch, dev, wl, steps, warmup, with_cpu=True):

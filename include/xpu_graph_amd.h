@@ -84,6 +84,22 @@ int xg_add_layer_norm(const void* x, const void* res, const void* w, const void*
                       int wb_dtype, xg_stream_t stream);
 
 /* ---------------------------------------------------------------------------
+ * Backward of xg_rms_norm / xg_add_rms_norm for training graphs (the reference
+ * differentiates its fused norms through AOT autograd:
+ * tests/common/test_fuse_rmsnorm.py:125-157, tests/common/test_training.py).
+ *   h = x (+ res, rounded to `dtype` as the forward rounds it), r = rsqrt(mean(h^2) + eps), hhat = h r
+ *   gx[rows, cols] (contiguous) = r (gy w - hhat mean(gy w hhat)) (+ gh)   -- the gradient of x, and of res
+ *   gw_part[n_blocks, cols] fp32: block b's share of sum_rows(gy hhat); the caller adds the n_blocks rows
+ *     (NULL when the weight gradient is not wanted; needs w).
+ * res, w, gh may be NULL.  n_blocks workgroups split the rows (1 <= n_blocks <= 65535; when rows < n_blocks the
+ * rows beyond `rows` of gw_part are left unwritten, so pass n_blocks <= rows).  cols a multiple of 8 (4 for fp32)
+ * and at most 16384 (8192 for fp32); strides in elements, multiples of the same.
+ * ------------------------------------------------------------------------- */
+int xg_rms_norm_bwd(const void* x, const void* res, const void* w, const void* gy, const void* gh, void* gx, float* gw_part,
+                    int64_t rows, int64_t cols, int64_t x_stride, int64_t res_stride, int64_t gy_stride, int64_t gh_stride,
+                    float eps, int dtype, int w_dtype, int n_blocks, xg_stream_t stream);
+
+/* ---------------------------------------------------------------------------
  * Column slice + concatenate (bit-exact byte mover, dtype-agnostic).
  *
  * For every row r < rows and every chunk i < n_chunks, copies `chunk_bytes`
@@ -165,11 +181,18 @@ int xg_slice_sum_cat(const void* x, void* out, int64_t batch, int64_t rows, int6
  * replaces torch_npu_triton::fused_silu_mul
  *   (passes/patterns/targets/npu/triton_kernel/fused_silu_mul.py:8-60).
  * xg_silu_mul2 takes gate and up as two separate [rows, d] tensors.
+ * xg_silu_mul2_bwd: the gradients of xg_silu_mul2 for training graphs (the
+ *   reference differentiates its fused gate through AOT autograd,
+ *   tests/common/test_training.py): d_gate = gy * up * s (1 + gate (1 - s)),
+ *   s = sigmoid(gate); d_up = gy * silu(gate); five contiguous tensors of n
+ *   elements, fp32 math, one rounding per output.
  * ------------------------------------------------------------------------- */
 int xg_silu_mul(const void* x, void* y, int64_t rows, int64_t d, int64_t x_stride, int dtype,
                 xg_stream_t stream);
 int xg_silu_mul2(const void* gate, const void* up, void* y, int64_t rows, int64_t d, int64_t gate_stride,
                  int64_t up_stride, int dtype, xg_stream_t stream);
+int xg_silu_mul2_bwd(const void* gate, const void* up, const void* gy, void* d_gate, void* d_up, int64_t n, int dtype,
+                     xg_stream_t stream);
 
 /* ---------------------------------------------------------------------------
  * Gated dense layer (SwiGLU): out[M, N] = silu(a w_gate^T) * (a w_up^T), both

@@ -70,6 +70,60 @@ def test_swiglu_halves_gradient(device):
     torch.testing.assert_close(g0, g1, rtol=1e-4, atol=1e-4)
 
 
+@pytest.mark.parametrize("dtype,wdtype", [(torch.float32, torch.float32), (torch.bfloat16, torch.bfloat16), (torch.bfloat16, torch.float32), (torch.float16, torch.float16)])
+@pytest.mark.parametrize("rows,cols", [(1, 8), (37, 64), (300, 4096), (2050, 1024), (5, 16384), (1500, 2056)])
+@pytest.mark.parametrize("with_res,with_gh,with_w", [(False, False, True), (True, True, True), (True, False, False)])
+def test_rms_norm_backward_kernel(device, dtype, wdtype, rows, cols, with_res, with_gh, with_w):
+    """xg_rms_norm_bwd against float64 autograd of the same forward (the residual sum rounded to the storage type,
+    as the forward kernel rounds it): fp32 row statistics, one rounding of gx; the weight gradient summed over rows
+    from per-block fp32 partials.  Row counts that do not divide among the blocks, one to eight chunks per lane."""
+    import xpu_graph_amd.ops  # noqa: F401
+
+    if dtype == torch.float32 and cols > 8192:
+        pytest.skip("fp32 rows hold at most 8192 columns in the kernel")
+    gen = torch.Generator().manual_seed(rows + cols)
+    x = torch.randn(rows, cols, generator=gen).to(dtype).to(device)
+    res = torch.randn(rows, cols, generator=gen).to(dtype).to(device) if with_res else None
+    w = (1 + 0.2 * torch.randn(cols, generator=gen)).to(wdtype).to(device) if with_w else None
+    gy = torch.randn(rows, cols, generator=gen).to(dtype).to(device)
+    gh = torch.randn(rows, cols, generator=gen).to(dtype).to(device) if with_gh else None
+    gx, gw = torch.ops.xpu_ops.rms_norm_bwd(x, res, w, gy, gh, 1e-6, True)
+    h = (x + res) if with_res else x  # rounded to the storage type
+    h64 = h.double().requires_grad_(True)
+    w64 = w.double().requires_grad_(True) if with_w else None
+    y = h64 * torch.rsqrt(h64.pow(2).mean(-1, keepdim=True) + 1e-6)
+    y = y * w64 if with_w else y
+    grads = torch.autograd.grad(y, (h64, w64) if with_w else (h64,), gy.double())
+    want_gx = grads[0] + (gh.double() if with_gh else 0)
+    ulp = {torch.float32: 2.0**-23, torch.bfloat16: 2.0**-8, torch.float16: 2.0**-11}[dtype]
+    assert gx.shape == x.shape and gx.dtype == dtype
+    torch.testing.assert_close(gx.double(), want_gx, rtol=1.01 * ulp, atol=want_gx.abs().max().item() * max(ulp * 2.0**-6, 2e-6))
+    if with_w:
+        wulp = {torch.float32: 2.0**-23, torch.bfloat16: 2.0**-8, torch.float16: 2.0**-11}[wdtype]
+        assert gw.shape == w.shape and gw.dtype == wdtype
+        torch.testing.assert_close(gw.double(), grads[1], rtol=1.01 * wulp, atol=grads[1].abs().max().item() * max(wulp * 2.0**-6, 1e-5))
+    else:
+        assert gw.numel() == 0
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("shape", [(256, 512), (3, 5, 7), (1, 1), (8192, 1376)])
+def test_gate_backward_kernel(device, dtype, shape):
+    """xg_silu_mul2_bwd against autograd of silu(g) * u evaluated in float64 on the same inputs: fp32 math and one
+    rounding per output (rtol 1e-5 for fp32, half an ulp of the output type otherwise); vector and scalar paths."""
+    import xpu_graph_amd.ops  # noqa: F401
+
+    gen = torch.Generator().manual_seed(sum(shape))
+    g, u, gy = (torch.randn(*shape, generator=gen).to(dtype).to(device) for _ in range(3))
+    dg, du = torch.ops.xpu_ops.silu_mul2_bwd(g, u, gy)
+    g64, u64 = g.double().requires_grad_(True), u.double().requires_grad_(True)
+    wg, wu = torch.autograd.grad(F.silu(g64) * u64, (g64, u64), gy.double())
+    rtol = {torch.float32: 1e-5, torch.bfloat16: 2.0**-8, torch.float16: 2.0**-11}[dtype]
+    for got, want in ((dg, wg), (du, wu)):
+        assert got.dtype == dtype and got.shape == g.shape
+        torch.testing.assert_close(got.double(), want, rtol=rtol * 1.01, atol=1e-6 if dtype == torch.float32 else rtol * 2.0**-10)
+
+
 @pytest.mark.parametrize("act", ["none", "relu", "sigmoid", "silu", "gelu"])
 @pytest.mark.parametrize("weight_trans", [True, False])
 def test_dense_backward_formula(device, act, weight_trans):

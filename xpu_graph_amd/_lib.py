@@ -42,6 +42,7 @@ _SIGNATURES = {
         c_int,
         [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_float, c_int, c_int, c_void_p],
     ),
+    "xg_rms_norm_bwd": (c_int, [c_void_p] * 7 + [c_int64] * 6 + [c_float, c_int, c_int, c_int, c_void_p]),
     "xg_add_layer_norm": (
         c_int,
         [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_float, c_int, c_int, c_void_p],
@@ -81,6 +82,7 @@ _SIGNATURES = {
         c_int,
         [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p] + [c_int64] * 12 + [c_int, c_int, c_int, c_int, c_void_p],
     ),
+    "xg_silu_mul2_bwd": (c_int, [c_void_p] * 5 + [c_int64, c_int, c_void_p]),
     "xg_dense_at": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p] + [c_int64] * 6 + [c_int, c_void_p]),
     "xg_dense_fp8": (
         c_int,

@@ -6,9 +6,11 @@ on the device the tensors live on.  Registered once per process, on demand (`ops
 backend constructed with is_training=True on the mi355x target): a Python autograd formula costs every call of the op
 a few microseconds of dispatch, which inference-only processes should not pay.
 
-    rms_norm(x, w, eps)        y = x * r * w,            r = rsqrt(mean(x^2) + eps)
+    rms_norm(x, w, eps)        y = x * r * w,            r = rsqrt(mean(x^2) + eps)   (gradients: the fused
+                               xg_rms_norm_bwd kernel, also for the add + RMSNorm ops; the Aten formula below is
+                               for shapes the kernel does not take)
     layer_norm(x, w, b, eps)   y = (x - m) * r * w + b,  r = rsqrt(var(x) + eps)
-    silu_mul2(g, u)            y = silu(g) * u
+    silu_mul2(g, u)            y = silu(g) * u          (gradients: the fused xg_silu_mul2_bwd kernel)
     silu_mul(x)                y = silu(x[..., :d]) * x[..., d:]
     dense(x, W, trans, bias, residual, act)   y = act(x W(^T) + bias + residual)
     dense_glu(x, Wg, Wu)       y = silu(x Wg^T) * (x Wu^T)
@@ -42,10 +44,23 @@ def _rms_setup(ctx, inputs, output):
     ctx.has_w, ctx.eps = w is not None, eps
 
 
+def _rms_kernel_backward(x, res, w, gy, gh, eps, want_gw):
+    """(g_sum, gw | None) on the fused backward kernel when it takes the shape, else None."""
+    from . import ops
+
+    if not (x.is_cuda and ops.rms_norm_bwd_fits(x, w)) or (res is not None and res.dtype != x.dtype):
+        return None
+    gx, gw = torch.ops.xpu_ops.rms_norm_bwd(x, res, w, gy, gh, eps, want_gw)
+    return gx, (gw if want_gw and w is not None else None)
+
+
 def _rms_backward(ctx, gy):
     saved = ctx.saved_tensors
     x = saved[0]
     w = saved[1] if ctx.has_w else None
+    fused = _rms_kernel_backward(x, None, w, gy, None, ctx.eps, ctx.needs_input_grad[1])
+    if fused is not None:
+        return fused[0], fused[1], None
     xf, gf = x.float(), gy.float()
     r = torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + ctx.eps)
     xhat = xf * r
@@ -89,8 +104,7 @@ def _silu_mul2_setup(ctx, inputs, output):
 
 def _silu_mul2_backward(ctx, gy):
     g, u = ctx.saved_tensors
-    gf, uf, yf = g.float(), u.float(), gy.float()
-    return (yf * uf * _silu_grad(gf)).to(g.dtype), (yf * torch.nn.functional.silu(gf)).to(u.dtype)
+    return torch.ops.xpu_ops.silu_mul2_bwd(g, u, gy.to(g.dtype))
 
 
 def _silu_mul_setup(ctx, inputs, output):
@@ -128,7 +142,7 @@ def _dense_backward(ctx, gy):
     bias = rest.pop(0) if ctx.has_bias else None
     residual = rest.pop(0) if ctx.has_res else None
     act = ctx.act
-    gf = gy.float()
+    gf = gy if act == "none" else gy.float()  # no activation: the upstream gradient is the pre-activation's, as it is
     if act == "none":
         gz = gf
     elif act == "relu":
@@ -163,11 +177,9 @@ def _dense_glu_setup(ctx, inputs, output):
 def _dense_glu_backward(ctx, gy):
     x, w_gate, w_up = ctx.saved_tensors
     dense = torch.ops.xpu_ops.dense
-    gate = dense(x, w_gate, True, None, None, "none").float()
-    up = dense(x, w_up, True, None, None, "none").float()
-    gf = gy.float()
-    d_gate = (gf * up * _silu_grad(gate)).to(x.dtype)
-    d_up = (gf * torch.nn.functional.silu(gate)).to(x.dtype)
+    gate = dense(x, w_gate, True, None, None, "none")
+    up = dense(x, w_up, True, None, None, "none")
+    d_gate, d_up = torch.ops.xpu_ops.silu_mul2_bwd(gate, up, gy.to(x.dtype))  # one pass instead of a dozen Aten kernels
     need = ctx.needs_input_grad
     gx = None
     if need[0]:
@@ -250,6 +262,10 @@ def _add_norm_formulas(layer, with_sum):
         x, res = saved[0], saved[1]
         w = saved[2] if ctx.has_w else None
         need = ctx.needs_input_grad
+        if not layer:
+            fused = _rms_kernel_backward(x, res, w, gy, gh, ctx.eps, need[2])
+            if fused is not None:
+                return fused[0], fused[0], fused[1], None
         hf, gf = x.float() + res.float(), gy.float()
         hc = hf - hf.mean(-1, keepdim=True) if layer else hf
         r = torch.rsqrt(hc.pow(2).mean(-1, keepdim=True) + ctx.eps)

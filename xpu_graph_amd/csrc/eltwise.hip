@@ -68,6 +68,48 @@ int silu_mul_dispatch(const void* gate, const void* up, void* y, int64_t rows, i
   }
 }
 
+// Backward of y = silu(gate) * up: d_gate = gy * up * s * (1 + gate * (1 - s)) with s = sigmoid(gate), d_up = gy *
+// silu(gate); fp32 math on the storage-type inputs, one rounding per output.  All five tensors are contiguous.
+template <typename T, int VW>
+__global__ __launch_bounds__(256) void silu_mul_bwd_kernel(const T* __restrict__ gate, const T* __restrict__ up,
+                                                           const T* __restrict__ gy, T* __restrict__ d_gate,
+                                                           T* __restrict__ d_up, int64_t nvec) {
+  typedef T VT __attribute__((ext_vector_type(VW)));
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= nvec) return;
+  const VT g = __builtin_nontemporal_load(reinterpret_cast<const VT*>(gate) + i);
+  const VT u = __builtin_nontemporal_load(reinterpret_cast<const VT*>(up) + i);
+  const VT y = __builtin_nontemporal_load(reinterpret_cast<const VT*>(gy) + i);
+  VT dg, du;
+#pragma unroll
+  for (int j = 0; j < VW; ++j) {
+    const float gf = to_f32(g[j]), uf = to_f32(u[j]), yf = to_f32(y[j]);
+    const float sg = sigmoid_f32(gf);
+    dg[j] = from_f32<T>(yf * uf * (sg * (1.f + gf * (1.f - sg))));
+    du[j] = from_f32<T>(yf * (gf * sg));
+  }
+  __builtin_nontemporal_store(dg, reinterpret_cast<VT*>(d_gate) + i);
+  __builtin_nontemporal_store(du, reinterpret_cast<VT*>(d_up) + i);
+}
+
+template <typename T>
+int silu_mul_bwd_typed(const void* gate, const void* up, const void* gy, void* d_gate, void* d_up, int64_t n, hipStream_t stream) {
+  constexpr int VN = VecOf<T>::N;
+  const void* ptrs[] = {gate, up, gy, d_gate, d_up};
+  bool vec_ok = n % VN == 0;
+  for (const void* q : ptrs) vec_ok = vec_ok && aligned_to(q, 16);
+  const int64_t work = vec_ok ? n / VN : n;
+  const int64_t blocks = (work + 255) / 256;
+  if (blocks > 0x7fffffffLL) return XG_ERR_TOO_LARGE;
+  if (vec_ok)
+    hipLaunchKernelGGL((silu_mul_bwd_kernel<T, VN>), dim3((unsigned)blocks), dim3(256), 0, stream, (const T*)gate, (const T*)up,
+                       (const T*)gy, (T*)d_gate, (T*)d_up, work);
+  else
+    hipLaunchKernelGGL((silu_mul_bwd_kernel<T, 1>), dim3((unsigned)blocks), dim3(256), 0, stream, (const T*)gate, (const T*)up,
+                       (const T*)gy, (T*)d_gate, (T*)d_up, work);
+  return status_from_hip(hipGetLastError());
+}
+
 __global__ __launch_bounds__(256) void copy_kernel(const u32x4* __restrict__ src, u32x4* __restrict__ dst, int64_t n) {
   const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (i < n) __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
@@ -89,6 +131,28 @@ int xg_silu_mul(const void* x, void* y, int64_t rows, int64_t d, int64_t x_strid
 int xg_silu_mul2(const void* gate, const void* up, void* y, int64_t rows, int64_t d, int64_t gate_stride,
                  int64_t up_stride, int dtype, xg_stream_t stream) {
   return xg::silu_mul_dispatch(gate, up, y, rows, d, gate_stride, up_stride, dtype, (hipStream_t)stream);
+}
+
+int xg_silu_mul2_bwd(const void* gate, const void* up, const void* gy, void* d_gate, void* d_up, int64_t n, int dtype,
+                     xg_stream_t stream) {
+  using namespace xg;
+  if (!gate || !up || !gy || !d_gate || !d_up) return XG_ERR_NULL_PTR;
+  if (n < 0) return XG_ERR_BAD_SHAPE;
+  if (n == 0) return XG_OK;
+  const size_t esz = dtype == XG_F32 ? 4 : 2;
+  const void* ptrs[] = {gate, up, gy, d_gate, d_up};
+  for (const void* q : ptrs)
+    if (!aligned_to(q, esz)) return XG_ERR_BAD_ALIGN;
+  switch (dtype) {
+    case XG_F32:
+      return silu_mul_bwd_typed<float>(gate, up, gy, d_gate, d_up, n, (hipStream_t)stream);
+    case XG_BF16:
+      return silu_mul_bwd_typed<bf16_t>(gate, up, gy, d_gate, d_up, n, (hipStream_t)stream);
+    case XG_F16:
+      return silu_mul_bwd_typed<f16_t>(gate, up, gy, d_gate, d_up, n, (hipStream_t)stream);
+    default:
+      return XG_ERR_BAD_DTYPE;
+  }
 }
 
 int xg_copy_bytes(const void* src, void* dst, int64_t bytes, xg_stream_t stream) {

@@ -29,6 +29,7 @@ _SCHEMAS = [
     "add_rms_norm_only(Tensor x, Tensor residual, Tensor? weight, float eps) -> Tensor",
     "add_layer_norm(Tensor x, Tensor residual, Tensor? weight, Tensor? bias, float eps) -> (Tensor, Tensor)",
     "add_layer_norm_only(Tensor x, Tensor residual, Tensor? weight, Tensor? bias, float eps) -> Tensor",
+    "rms_norm_bwd(Tensor x, Tensor? residual, Tensor? weight, Tensor gy, Tensor? gh, float eps, bool want_gw) -> (Tensor, Tensor)",
     "slice_cat(Tensor src, Tensor table, int chunk_bytes, int out_cols) -> Tensor",
     "slice_cat_multi(Tensor src, Tensor table, int chunk_bytes, int[] out_cols) -> Tensor[]",
     "slice_stack(Tensor src, Tensor[] tables, int[] chunk_bytes, int slice_len, int num) -> Tensor",
@@ -37,6 +38,7 @@ _SCHEMAS = [
     "slice_sum_cat(Tensor x, int[] starts, int[] ends) -> Tensor",
     "silu_mul(Tensor x) -> Tensor",
     "silu_mul2(Tensor gate, Tensor up) -> Tensor",
+    "silu_mul2_bwd(Tensor gate, Tensor up, Tensor gy) -> (Tensor, Tensor)",
 ]
 for _s in _SCHEMAS:
     _library.define(_s)
@@ -159,12 +161,63 @@ def _add_layer_norm_only(x, residual, weight, bias, eps):
     return _norm_impl("layer", x, residual, weight, bias, eps, False)
 
 
+_RMS_BWD_BLOCKS = 1024  # workgroups that split the rows; each hands back one fp32 partial row of the weight gradient
+
+
+def rms_norm_bwd_fits(x, weight):
+    """What xg_rms_norm_bwd takes: rows of whole 16-byte vectors, at most eight of them per lane of a 256-lane block,
+    a weight that is one row."""
+    per16 = 16 // x.element_size()
+    cols = x.shape[-1]
+    ok = x.dtype in _DTYPE_CODE and isinstance(cols, int) and cols % per16 == 0 and 0 < cols // per16 <= 2048
+    if weight is not None:
+        ok = ok and weight.dim() == 1 and weight.shape[0] == cols and weight.dtype in (x.dtype, torch.float32)
+    return ok
+
+
+def _rms_norm_bwd(x, residual, weight, gy, gh, eps, want_gw):
+    """Gradients of rms_norm / add_rms_norm in one pass per row: (gx, gw); gx also is the residual's gradient.  gw is
+    empty when there is no weight or want_gw is false."""
+    if not rms_norm_bwd_fits(x, weight):
+        raise ValueError("rms_norm_bwd: needs rows of whole 16-byte vectors (at most 2048 of them) and a 1-D weight")
+    cols = x.shape[-1]
+    x2, rows, xs = _rows_2d(x)
+    g2, _, gs = _rows_2d(gy.to(x.dtype))
+    r2 = rs = h2 = hs = None
+    if residual is not None:
+        r2, _, rs = _rows_2d(residual)
+    if gh is not None:
+        h2, _, hs = _rows_2d(gh.to(x.dtype))
+    gx = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+    want_gw = bool(want_gw and weight is not None)
+    n_blocks = max(1, min(_RMS_BWD_BLOCKS, rows))
+    part = torch.empty((n_blocks, cols), dtype=torch.float32, device=x.device) if want_gw else None
+    if rows:
+        st = _lib.lib().xg_rms_norm_bwd(
+            _ptr(x2), _ptr(r2), _ptr(weight.contiguous() if weight is not None else None), _ptr(g2), _ptr(h2), _ptr(gx), _ptr(part), rows, cols,
+            xs, rs or 0, gs, hs or 0, eps, _code(x.dtype), _code(weight.dtype) if weight is not None else _code(x.dtype), n_blocks, _stream(),
+        )
+        _lib.check(st, "xg_rms_norm_bwd")
+    if not want_gw:
+        return gx, torch.empty(0, dtype=x.dtype, device=x.device)
+    return gx, (part.sum(0) if rows else torch.zeros(cols, device=x.device)).to(weight.dtype)
+
+
+def _rms_norm_bwd_meta(x, residual, weight, gy, gh, eps, want_gw):
+    gx = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+    if want_gw and weight is not None:
+        return gx, torch.empty(weight.shape, dtype=weight.dtype, device=x.device)
+    return gx, torch.empty(0, dtype=x.dtype, device=x.device)
+
+
 def _like(x):
     return torch.empty(x.shape, dtype=x.dtype, device=x.device)
 
 
 _library.impl("rms_norm", _rms_norm, "CUDA")
 _library.impl("layer_norm", _layer_norm, "CUDA")
+_library.impl("rms_norm_bwd", _rms_norm_bwd, "CUDA")
+_library.impl("rms_norm_bwd", _rms_norm_bwd_meta, "Meta")
 _library.impl("add_rms_norm", _add_rms_norm, "CUDA")
 _library.impl("add_rms_norm_only", _add_rms_norm_only, "CUDA")
 _library.impl("add_layer_norm", _add_layer_norm, "CUDA")
@@ -392,8 +445,22 @@ def _silu_mul2(gate, up):
     return y
 
 
+def _silu_mul2_bwd(gate, up, gy):
+    """(d_gate, d_up) of silu(gate) * up for the upstream gradient gy, in one pass over the three tensors."""
+    if gate.shape != up.shape or gate.shape != gy.shape or gate.dtype != up.dtype or gate.dtype != gy.dtype:
+        raise ValueError("silu_mul2_bwd: gate, up and gy must match in shape and dtype")
+    gate, up, gy = gate.contiguous(), up.contiguous(), gy.contiguous()
+    d_gate, d_up = torch.empty_like(gate), torch.empty_like(gate)
+    if gate.numel():
+        st = _lib.lib().xg_silu_mul2_bwd(_ptr(gate), _ptr(up), _ptr(gy), _ptr(d_gate), _ptr(d_up), gate.numel(), _code(gate.dtype), _stream())
+        _lib.check(st, "xg_silu_mul2_bwd")
+    return d_gate, d_up
+
+
 _library.impl("silu_mul", _silu_mul, "CUDA")
 _library.impl("silu_mul2", _silu_mul2, "CUDA")
+_library.impl("silu_mul2_bwd", _silu_mul2_bwd, "CUDA")
+_library.impl("silu_mul2_bwd", lambda gate, up, gy: (_like(gate), _like(gate)), "Meta")
 _library.impl(
     "silu_mul",
     lambda x: torch.empty((*x.shape[:-1], x.shape[-1] // 2), dtype=x.dtype, device=x.device),
