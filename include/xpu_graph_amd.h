@@ -206,6 +206,11 @@ int xg_silu_mul2_bwd(const void* gate, const void* up, const void* gy, void* d_g
  * ------------------------------------------------------------------------- */
 int xg_dense_glu(const void* a, const void* w_gate, const void* w_up, void* out, int64_t M, int64_t N, int64_t K,
                  int64_t lda, int64_t ldb, int dtype, xg_stream_t stream);
+/* xg_dense_glu that also writes the two rounded projections (gate_out = a Wg^T, up_out = a Wu^T, [M,N] each, the
+ * values the gate was computed from), for training graphs: the backward needs them and would otherwise run both
+ * projections again.  Same kernel, two more stores per output element. */
+int xg_dense_glu_save(const void* a, const void* w_gate, const void* w_up, void* out, void* gate_out, void* up_out,
+                      int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int dtype, xg_stream_t stream);
 
 /* ---------------------------------------------------------------------------
  * Dense layer: out[M,N] = act(a[M,K] @ B + bias (+ residual)), fp32 accumulate.

@@ -206,6 +206,32 @@ def test_gated_dense_backward_formula(device):
         assert (a.float() - c).abs().mean().item() <= 2e-2 * scale + 1e-3, (name, (a.float() - c).abs().mean().item(), scale)
 
 
+def test_gated_dense_that_saves_its_projections(device):
+    """dense_glu_save returns the gated output bit-identical to dense_glu plus the two projections bit-identical to
+    two dense layers (large tiles and the small-grid kernel), and its backward -- no recomputation -- gives the
+    gradients of the recomputing formula bit for bit."""
+    import xpu_graph_amd.ops as xops
+
+    xops.enable_autograd()
+    ops = torch.ops.xpu_ops
+    for M, K, N in ((4096, 512, 2816), (96, 256, 264)):
+        gen = torch.Generator().manual_seed(M + N)
+        x = torch.randn(M, K, generator=gen).bfloat16().to(device)
+        wg = (torch.randn(N, K, generator=gen) / K**0.5).bfloat16().to(device)
+        wu = (torch.randn(N, K, generator=gen) / K**0.5).bfloat16().to(device)
+        y, gate, up = ops.dense_glu_save(x, wg, wu)
+        assert torch.equal(y, ops.dense_glu(x, wg, wu))
+        assert torch.equal(gate, ops.dense(x, wg, True, None, None, "none")) and torch.equal(up, ops.dense(x, wu, True, None, None, "none"))
+        dy = torch.randn(M, N, generator=gen).bfloat16().to(device)
+        grads = []
+        for op in ("dense_glu", "dense_glu_save"):
+            leaves = [t.clone().requires_grad_(True) for t in (x, wg, wu)]
+            out = getattr(ops, op)(*leaves)
+            out = out[0] if op == "dense_glu_save" else out
+            grads.append(torch.autograd.grad(out, leaves, dy))
+        assert all(torch.equal(a, b) for a, b in zip(*grads))
+
+
 def test_gated_mlp_training_step(device):
     """RMSNorm -> SwiGLU MLP (gate, up, down projections), compiled for training on the mi355x target: the forward
     graph calls the gated dense kernel once and the dense kernel once, loss and gradients follow eager."""
@@ -223,7 +249,8 @@ def test_gated_mlp_training_step(device):
     loss0 = y0.float().pow(2).mean()
     g0 = torch.autograd.grad(loss0, args)
     fwd_ops = [str(n.target) for n in be.compiled_graphs[1].graph.nodes if n.op == "call_function"]
-    assert fwd_ops.count("xpu_ops.dense_glu.default") == 1 and fwd_ops.count("xpu_ops.dense.default") == 1, fwd_ops
+    # a graph that is differentiated runs the gated layer that also saves its two projections for the backward
+    assert fwd_ops.count("xpu_ops.dense_glu_save.default") == 1 and fwd_ops.count("xpu_ops.dense.default") == 1, fwd_ops
     assert not any("aten.mm" in t or "aten.addmm" in t for t in fwd_ops)
     ref_args = [a.detach().float().requires_grad_(True) for a in args]
     loss1 = mlp(*ref_args).pow(2).mean()
@@ -345,7 +372,7 @@ def test_llama_block_training_step(device):
     y0 = torch.compile(block, backend=be, dynamic=False)(*args)
     g0 = torch.autograd.grad(y0.float().pow(2).mean(), args)
     ops = Counter(str(n.target) for n in be.compiled_graphs[1].graph.nodes if n.op == "call_function")
-    assert ops["xpu_ops.dense_glu.default"] == 1 and ops["xpu_ops.dense.default"] >= 5 and ops["xpu_ops.rope.default"] == 2, ops
+    assert ops["xpu_ops.dense_glu_save.default"] == 1 and ops["xpu_ops.dense.default"] >= 5 and ops["xpu_ops.rope.default"] == 2, ops
     assert ops["xpu_ops.add_rms_norm.default"] == 1, ops  # the attention residual add rides in the second norm
     ref_args = [a.detach().float().requires_grad_(True) for a in args]
     g1 = torch.autograd.grad(block(*ref_args).pow(2).mean(), ref_args)

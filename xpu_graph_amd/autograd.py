@@ -174,11 +174,8 @@ def _dense_glu_setup(ctx, inputs, output):
     ctx.save_for_backward(*inputs)
 
 
-def _dense_glu_backward(ctx, gy):
-    x, w_gate, w_up = ctx.saved_tensors
+def _glu_grads(ctx, x, w_gate, w_up, gate, up, gy):
     dense = torch.ops.xpu_ops.dense
-    gate = dense(x, w_gate, True, None, None, "none")
-    up = dense(x, w_up, True, None, None, "none")
     d_gate, d_up = torch.ops.xpu_ops.silu_mul2_bwd(gate, up, gy.to(x.dtype))  # one pass instead of a dozen Aten kernels
     need = ctx.needs_input_grad
     gx = None
@@ -187,6 +184,25 @@ def _dense_glu_backward(ctx, gy):
     gwg = _weight_grad(d_gate, x) if need[1] else None
     gwu = _weight_grad(d_up, x) if need[2] else None
     return gx, gwg, gwu
+
+
+def _dense_glu_backward(ctx, gy):
+    # the plain op saved only its inputs: both projections are run again
+    x, w_gate, w_up = ctx.saved_tensors
+    dense = torch.ops.xpu_ops.dense
+    gate = dense(x, w_gate, True, None, None, "none")
+    up = dense(x, w_up, True, None, None, "none")
+    return _glu_grads(ctx, x, w_gate, w_up, gate, up, gy)
+
+
+def _dense_glu_save_setup(ctx, inputs, output):
+    ctx.save_for_backward(*inputs, output[1], output[2])
+
+
+def _dense_glu_save_backward(ctx, gy, g_gate=None, g_up=None):
+    # the two projection outputs exist for this formula; gradients flowing into them are not supported
+    x, w_gate, w_up, gate, up = ctx.saved_tensors
+    return _glu_grads(ctx, x, w_gate, w_up, gate, up, gy)
 
 
 def _rotate_half(t):
@@ -298,6 +314,7 @@ def register():
     reg("xpu_ops::silu_mul", _silu_mul_backward, setup_context=_silu_mul_setup)
     reg("xpu_ops::dense", _dense_backward, setup_context=_dense_setup)
     reg("xpu_ops::dense_glu", _dense_glu_backward, setup_context=_dense_glu_setup)
+    reg("xpu_ops::dense_glu_save", _dense_glu_save_backward, setup_context=_dense_glu_save_setup)
     reg("xpu_ops::rope", _rope_backward, setup_context=_rope_setup)
     reg("xpu_ops::sdpa", _sdpa_backward, setup_context=_sdpa_setup)
     reg("xpu_ops::sdpa_lse", _sdpa_lse_backward, setup_context=_sdpa_lse_setup)
@@ -307,7 +324,7 @@ def register():
         reg(f"xpu_ops::{op}", backward, setup_context=setup)
     # An op that was traced before (an inference compile earlier in the process) has its dispatch decisions cached
     # on the Python side; a stale entry for the Autograd key would keep sending traces to the "no formula" fallback.
-    for name in ("rms_norm", "layer_norm", "silu_mul2", "silu_mul", "dense", "dense_glu", "rope", "sdpa", "sdpa_lse",
+    for name in ("rms_norm", "layer_norm", "silu_mul2", "silu_mul", "dense", "dense_glu", "dense_glu_save", "rope", "sdpa", "sdpa_lse",
                  "add_rms_norm", "add_rms_norm_only", "add_layer_norm", "add_layer_norm_only"):
         packet = getattr(torch.ops.xpu_ops, name)
         for overload in packet.overloads():

@@ -91,11 +91,13 @@ int xg_dense_at(const void* a_t, const void* b, const void* residual, void* out,
   return dtype == XG_BF16 ? gemm::launch_at_bf16(p, st) : gemm::launch_at_f16(p, st);
 }
 
-int xg_dense_glu(const void* a, const void* w_gate, const void* w_up, void* out, int64_t M, int64_t N, int64_t K,
-                 int64_t lda, int64_t ldb, int dtype, xg_stream_t stream) {
+static int dense_glu_entry(const void* a, const void* w_gate, const void* w_up, void* out, void* gate_out, void* up_out, int64_t M,
+                           int64_t N, int64_t K, int64_t lda, int64_t ldb, int dtype, xg_stream_t stream) {
   using namespace xg;
   using namespace xg::gemm;
   if (a == nullptr || w_gate == nullptr || w_up == nullptr || out == nullptr) return XG_ERR_NULL_PTR;
+  if ((gate_out == nullptr) != (up_out == nullptr)) return XG_ERR_NULL_PTR;
+  if (gate_out && (!aligned_to(gate_out, 16) || !aligned_to(up_out, 16))) return XG_ERR_BAD_ALIGN;
   if (M < 0 || N <= 0 || K <= 0 || lda < K || ldb < K) return XG_ERR_BAD_SHAPE;
   if (M > 0x7fffffff || N > 0x7fffffff || K > 0x7fffffff) return XG_ERR_TOO_LARGE;
   if (dtype != XG_BF16 && dtype != XG_F16) return XG_ERR_BAD_DTYPE;
@@ -105,12 +107,25 @@ int xg_dense_glu(const void* a, const void* w_gate, const void* w_up, void* out,
   if (M == 0) return XG_OK;
   GemmParams p = make_params(a, w_gate, nullptr, nullptr, out, M, N, K, lda, ldb, 0, XG_ACT_NONE, false);
   p.B2 = w_up;
+  p.gate_out = gate_out;
+  p.up_out = up_out;
   p.tiles_n = (int)((N + BN / 2 - 1) / (BN / 2));
   // the direct-to-LDS loads address each operand with a 31-bit lane offset
   const int64_t lim = 0x7fffffffLL;
   if (M * lda * 2 >= lim || N * ldb * 2 >= lim) return XG_ERR_TOO_LARGE;
   hipStream_t st = (hipStream_t)stream;
   return dtype == XG_BF16 ? gemm::launch_glu_bf16(p, st) : gemm::launch_glu_f16(p, st);
+}
+
+int xg_dense_glu(const void* a, const void* w_gate, const void* w_up, void* out, int64_t M, int64_t N, int64_t K,
+                 int64_t lda, int64_t ldb, int dtype, xg_stream_t stream) {
+  return dense_glu_entry(a, w_gate, w_up, out, nullptr, nullptr, M, N, K, lda, ldb, dtype, stream);
+}
+
+int xg_dense_glu_save(const void* a, const void* w_gate, const void* w_up, void* out, void* gate_out, void* up_out, int64_t M,
+                      int64_t N, int64_t K, int64_t lda, int64_t ldb, int dtype, xg_stream_t stream) {
+  if (gate_out == nullptr || up_out == nullptr) return XG_ERR_NULL_PTR;
+  return dense_glu_entry(a, w_gate, w_up, out, gate_out, up_out, M, N, K, lda, ldb, dtype, stream);
 }
 
 }  // extern "C"

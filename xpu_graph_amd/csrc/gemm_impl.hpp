@@ -93,6 +93,8 @@ struct GemmParams {
   const void* A;
   const void* B;
   const void* B2;  // gated layer only: the second ("up") weight; B is then the gate weight
+  void* gate_out;  // gated layer only, optional: where the two rounded projections go as well ([M, N] each, row
+  void* up_out;    // stride ldc), for a backward pass that would otherwise recompute them
   const void* bias;
   const void* res;
   void* out;
@@ -477,14 +479,21 @@ __device__ __forceinline__ void epilogue_glu(const GemmParams& p, const Lane& L,
       if (!(n_ok && m < p.M)) continue;
       const float gv[8] = {g0[0], g0[1], g0[2], g0[3], g1[0], g1[1], g1[2], g1[3]};
       const float uv[8] = {u0[0], u0[1], u0[2], u0[3], u1[0], u1[1], u1[2], u1[3]};
-      O8 o;
+      O8 o, go, uo;
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         // each projection is rounded to the storage type first, as the two separate layers would do
-        const float gr = to_f32(from_f32<OT>(gv[e])), ur = to_f32(from_f32<OT>(uv[e]));
+        const OT g16 = from_f32<OT>(gv[e]), u16 = from_f32<OT>(uv[e]);
+        const float gr = to_f32(g16), ur = to_f32(u16);
         o[e] = from_f32<OT>(silu_f32(gr) * ur);
+        go[e] = g16;
+        uo[e] = u16;
       }
       store_vec_nt(reinterpret_cast<O8*>(reinterpret_cast<OT*>(p.out) + (int64_t)m * p.ldc + n), o);  // written once, read by another kernel
+      if (p.gate_out != nullptr) {
+        store_vec_nt(reinterpret_cast<O8*>(reinterpret_cast<OT*>(p.gate_out) + (int64_t)m * p.ldc + n), go);
+        store_vec_nt(reinterpret_cast<O8*>(reinterpret_cast<OT*>(p.up_out) + (int64_t)m * p.ldc + n), uo);
+      }
     }
     __syncthreads();  // the parks are free for the next half
   });
@@ -1083,14 +1092,21 @@ __global__ __launch_bounds__(kThreads) void gemm_small_kernel(GemmParams p_all) 
       const f32x4 u1 = *reinterpret_cast<const f32x4*>(at + (((9 + 2 * c) ^ (row & 15)) << 4));
       const float gv[8] = {g0[0], g0[1], g0[2], g0[3], g1[0], g1[1], g1[2], g1[3]};
       const float uv[8] = {u0[0], u0[1], u0[2], u0[3], u1[0], u1[1], u1[2], u1[3]};
-      O8 o;
+      O8 o, go, uo;
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         // each projection is rounded to the storage type first, as the two separate layers would do
-        const float gr = to_f32(from_f32<OT>(gv[e])), ur = to_f32(from_f32<OT>(uv[e]));
+        const OT g16 = from_f32<OT>(gv[e]), u16 = from_f32<OT>(uv[e]);
+        const float gr = to_f32(g16), ur = to_f32(u16);
         o[e] = from_f32<OT>(silu_f32(gr) * ur);
+        go[e] = g16;
+        uo[e] = u16;
       }
       store_vec_nt(reinterpret_cast<O8*>(reinterpret_cast<OT*>(p.out) + (int64_t)m * p.ldc + n), o);  // written once, read by another kernel
+      if (p.gate_out != nullptr) {
+        store_vec_nt(reinterpret_cast<O8*>(reinterpret_cast<OT*>(p.gate_out) + (int64_t)m * p.ldc + n), go);
+        store_vec_nt(reinterpret_cast<O8*>(reinterpret_cast<OT*>(p.up_out) + (int64_t)m * p.ldc + n), uo);
+      }
     }
   }
 }
@@ -1253,6 +1269,10 @@ int launch_glu(const GemmParams& p, hipStream_t stream) {
   rest.B = reinterpret_cast<const char*>(p.B) + n_split * p.ldb * EB;
   rest.B2 = reinterpret_cast<const char*>(p.B2) + n_split * p.ldb * EB;
   rest.out = reinterpret_cast<char*>(p.out) + n_split * (int64_t)sizeof(OT);
+  if (p.gate_out) {
+    rest.gate_out = reinterpret_cast<char*>(p.gate_out) + n_split * (int64_t)sizeof(OT);
+    rest.up_out = reinterpret_cast<char*>(p.up_out) + n_split * (int64_t)sizeof(OT);
+  }
   auto kernel = gemm_glu_split_kernel<T, OT>;
   if (int st = set_smem_once(kernel)) return st;
   const int64_t n_full = (int64_t)full.tiles_m * full.tiles_n, n_rest = (int64_t)rest.tiles_m * rest.tiles_n;
@@ -1267,6 +1287,7 @@ inline GemmParams make_params(const void* a, const void* b, const void* bias, co
   p.A = a;
   p.B = b;
   p.B2 = nullptr;
+  p.gate_out = p.up_out = nullptr;
   p.bias = bias;
   p.res = residual;
   p.out = out;

@@ -521,6 +521,7 @@ _library.define("dense(Tensor x, Tensor weight, bool weight_trans, Tensor? bias,
 _library.define("dense_batched(Tensor x, Tensor weight, bool weight_trans, Tensor? bias, Tensor? residual, str act) -> Tensor")
 _library.define("dense_at(Tensor a_t, Tensor b, Tensor? residual) -> Tensor")
 _library.define("dense_glu(Tensor x, Tensor w_gate, Tensor w_up) -> Tensor")
+_library.define("dense_glu_save(Tensor x, Tensor w_gate, Tensor w_up) -> (Tensor, Tensor, Tensor)")
 _library.define(
     "dense_fp8(Tensor x_q, Tensor w_q, bool weight_trans, Tensor x_scale, Tensor w_scale, Tensor? bias, str act, ScalarType out_dtype) -> Tensor"
 )
@@ -955,8 +956,9 @@ def dense_glu_fits(x_shape, w_shape, dtype):
     return m_ok and n * k * 2 < _GLU_OPERAND_LIMIT
 
 
-def _dense_glu(x, w_gate, w_up):
-    """silu(x @ w_gate.T) * (x @ w_up.T) in one launch; weights are [N, K] (torch.nn.Linear layout)."""
+def _dense_glu_run(x, w_gate, w_up, save):
+    """silu(x @ w_gate.T) * (x @ w_up.T) in one launch; weights are [N, K] (torch.nn.Linear layout).  save: also
+    return the two rounded projections the gate was computed from."""
     if w_gate.shape != w_up.shape or w_gate.dtype != x.dtype or w_up.dtype != x.dtype:
         raise ValueError("dense_glu: the two weights must share shape and dtype with each other and with x")
     if not dense_glu_fits(tuple(x.shape), tuple(w_gate.shape), x.dtype):
@@ -969,17 +971,38 @@ def _dense_glu(x, w_gate, w_up):
     if m * x.stride(0) * 2 >= _GLU_OPERAND_LIMIT or n * w_gate.stride(0) * 2 >= _GLU_OPERAND_LIMIT:
         # a row count that was symbolic at match time turned out too large for the gated kernel's 31-bit operand
         # offsets: the same result, bit for bit, from two dense launches and the gate kernel
-        return _silu_mul2(_dense(x, w_gate, True, None, None, "none"), _dense(x, w_up, True, None, None, "none"))
+        gate, up = _dense(x, w_gate, True, None, None, "none"), _dense(x, w_up, True, None, None, "none")
+        return _silu_mul2(gate, up), gate, up
     out = torch.empty((m, n), dtype=x.dtype, device=x.device)
+    gate = torch.empty((m, n), dtype=x.dtype, device=x.device) if save else None
+    up = torch.empty((m, n), dtype=x.dtype, device=x.device) if save else None
     if out.numel() == 0:
-        return out
-    st = _lib.lib().xg_dense_glu(_ptr(x), _ptr(w_gate), _ptr(w_up), _ptr(out), m, n, k, x.stride(0), w_gate.stride(0), _code(x.dtype), _stream())
-    _lib.check(st, "xg_dense_glu")
-    return out
+        return out, gate, up
+    args = (m, n, k, x.stride(0), w_gate.stride(0), _code(x.dtype), _stream())
+    if save:
+        _lib.check(_lib.lib().xg_dense_glu_save(_ptr(x), _ptr(w_gate), _ptr(w_up), _ptr(out), _ptr(gate), _ptr(up), *args), "xg_dense_glu_save")
+    else:
+        _lib.check(_lib.lib().xg_dense_glu(_ptr(x), _ptr(w_gate), _ptr(w_up), _ptr(out), *args), "xg_dense_glu")
+    return out, gate, up
+
+
+def _dense_glu(x, w_gate, w_up):
+    return _dense_glu_run(x, w_gate, w_up, False)[0]
+
+
+def _dense_glu_save(x, w_gate, w_up):
+    return _dense_glu_run(x, w_gate, w_up, True)
+
+
+def _dense_glu_save_meta(x, w_gate, w_up):
+    shape = (x.shape[0], w_gate.shape[0])
+    return tuple(torch.empty(shape, dtype=x.dtype, device=x.device) for _ in range(3))
 
 
 _library.impl("dense", _dense, "CUDA")
 _library.impl("dense_glu", _dense_glu, "CUDA")
+_library.impl("dense_glu_save", _dense_glu_save, "CUDA")
+_library.impl("dense_glu_save", _dense_glu_save_meta, "Meta")
 _library.impl("dense_glu", lambda x, w_gate, w_up: torch.empty((x.shape[0], w_gate.shape[0]), dtype=x.dtype, device=x.device), "Meta")
 _library.impl("dense", _dense_meta, "Meta")
 _library.impl("dense_at", _dense_at, "CUDA")

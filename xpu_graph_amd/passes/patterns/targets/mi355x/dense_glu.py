@@ -24,6 +24,10 @@ SILU_MUL2 = "mi355x_silu_mul2"
 
 class DenseGLUModule(nn.Module):
     def forward(self, x, w_gate, w_up):
+        if torch.is_grad_enabled() and (x.requires_grad or w_gate.requires_grad or w_up.requires_grad):
+            # a graph that will be differentiated: the same launch also writes the two projections, which the backward
+            # needs and would otherwise run again (two more dense layers)
+            return torch.ops.xpu_ops.dense_glu_save(x, w_gate, w_up)[0]
         return torch.ops.xpu_ops.dense_glu(x, w_gate, w_up)
 
 
