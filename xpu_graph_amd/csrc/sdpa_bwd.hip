@@ -140,7 +140,7 @@ __device__ __forceinline__ void store_rows(char* park, const f32x16 (&acc)[D / 3
 
 // ---------------------------------------------------------------------------------------------- dq
 template <typename T, int D>
-__global__ __launch_bounds__(kThreads) void sdpa_bwd_dq_kernel(BwdParams p) {
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void sdpa_bwd_dq_kernel(BwdParams p) {
   typedef typename Vec8<T>::type V8;
   constexpr int RB = D * 2, CH = RB / 16, TILE = BKV * RB, STAGE = 2 * TILE, KK = D / 16, DT = D / 32, LPW = CH / 4;
   extern __shared__ __attribute__((aligned(1024))) char smem[];
