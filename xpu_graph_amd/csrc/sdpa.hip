@@ -55,6 +55,7 @@ struct Params {
 template <typename T, int D, bool MASK = false>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void sdpa_fwd_kernel(Params p) {
   typedef typename Vec8<T>::type V8;
+  typedef __attribute__((address_space(3))) const V8 lds_V8;
   constexpr int RB = D * 2;          // bytes per tile row
   constexpr int CH = RB / 16;        // chunks per row
   constexpr int TILE = BKV * RB;     // one K or V tile
@@ -153,6 +154,24 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
   const int v_row = 4 * h + (a16 >> 2);                          // key row (mod 16) this lane addresses for the V^T fragments
   const int v_chunk = 2 * b16 + ((a16 & 3) >> 1), v_sub = (a16 & 1) << 3;
 
+  // The per-lane LDS byte addresses of every fragment read, formed once and held in registers (the empty asm keeps
+  // the compiler from splitting them up again and redoing the additions in every step).
+  int k_addr[KK], v_addr0[DT], v_addr1[DT];
+  const int lds_base = (int)(uint32_t)(size_t)(lvoid*)smem;
+  static_for<KK>([&](auto KI) {
+    constexpr int kk = decltype(KI)::value;
+    k_addr[kk] = lds_base + l32 * RB + (((2 * kk + h) ^ kx) << 4);
+    asm volatile("" : "+v"(k_addr[kk]));
+  });
+  static_for<DT>([&](auto DI) {
+    constexpr int dt = decltype(DI)::value;
+    // lane a16 of a 16-lane group addresses key row (a16/4), head-dim columns 4(a16%4)..+3 of the group's
+    // 16 columns; the transposing read returns, for result slot e, key row e at column a16.
+    v_addr0[dt] = lds_base + v_row * RB + (((4 * dt + v_chunk) ^ swz_v<D>(v_row)) << 4) + v_sub;
+    v_addr1[dt] = lds_base + (v_row + 8) * RB + (((4 * dt + v_chunk) ^ swz_v<D>(v_row + 8)) << 4) + v_sub;
+    asm volatile("" : "+v"(v_addr0[dt]), "+v"(v_addr1[dt]));
+  });
+
   f32x16 o_acc[DT];
   static_for<DT>([&](auto I) {
     o_acc[decltype(I)::value] = f32x16{0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
@@ -174,21 +193,30 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
     const int kv0 = j * BKV;
     if (p.causal && kv0 > qw_max) return;  // this wave's queries see none of these keys (wave-uniform)
 
-    const char* k_s = smem + stage * STAGE;
-    const char* v_s = k_s + TILE;
 
     // S^T tile: s[t][v] = <key 32t + 8(v/4) + 4h + v%4 , query l32>
     // The two 32-key halves alternate MFMA by MFMA: a dependent MFMA cannot issue until its predecessor has
     // left the pipe (a chain of eight ran at one MFMA per ~80 clocks in a probe kernel), two interleaved chains can.
     f32x16 s[2];
     s[0] = s[1] = f32x16{0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    static_for<KK>([&](auto KI) {
+    // K fragments are read PF k-steps ahead of the MFMAs that use them, so an LDS round trip hides behind MFMAs.
+    constexpr int PF = 2;
+    V8 kf[KK][2];
+    auto read_k = [&](auto KI) {
       constexpr int kk = decltype(KI)::value;
       static_for<2>([&](auto TI) {
         constexpr int t = decltype(TI)::value;
-        const int off = l32 * RB + (((2 * kk + h) ^ kx) << 4);
-        const V8 kf = *reinterpret_cast<const V8*>(k_s + 32 * t * RB + off);
-        s[t] = mma(kf, qf[kk], s[t]);
+        kf[kk][t] = *(lds_V8*)(uint32_t)(k_addr[kk] + stage * STAGE + 32 * t * RB);
+      });
+    };
+    static_for<PF>([&](auto KI) { read_k(KI); });
+    static_for<KK>([&](auto KI) {
+      constexpr int kk = decltype(KI)::value;
+      if constexpr (kk + PF < KK) read_k(std::integral_constant<int, kk + PF>{});
+      __builtin_amdgcn_sched_barrier(0);  // the reads above are issued before the MFMAs below
+      static_for<2>([&](auto TI) {
+        constexpr int t = decltype(TI)::value;
+        s[t] = mma(kf[kk][t], qf[kk], s[t]);
         __builtin_amdgcn_sched_barrier(0x7F7);  // everything but MFMAs may move across: the MFMA order stays as written
       });
     });
@@ -295,13 +323,9 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
         });
         static_for<DT>([&](auto DI) {
           constexpr int dt = decltype(DI)::value;
-          // lane a16 of a 16-lane group addresses key row (a16/4), head-dim columns 4(a16%4)..+3 of the group's
-          // 16 columns; the transposing read returns, for result slot e, key row e at column a16.
-          const int off0 = v_row * RB + (((4 * dt + v_chunk) ^ swz_v<D>(v_row)) << 4) + v_sub;
-          const int off1 = (v_row + 8) * RB + (((4 * dt + v_chunk) ^ swz_v<D>(v_row + 8)) << 4) + v_sub;
-          const char* base = v_s + (32 * t + 16 * st) * RB;
-          const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(base + off0));
-          const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(base + off1));
+          constexpr int base = stage * STAGE + TILE + (32 * t + 16 * st) * RB;
+          const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(uint32_t)(v_addr0[dt] + base));
+          const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(uint32_t)(v_addr1[dt] + base));
           const s16x8 both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
           o_acc[dt] = mma(__builtin_bit_cast(V8, both), pf, o_acc[dt]);
         });
