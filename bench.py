@@ -699,7 +699,7 @@ class LlamaBlockC5(Workload):
 
 class LlamaBlockTrainC5(LlamaBlockC5):
     name = "C5 Llama decoder block bf16 B4 S2048 training step (forward + backward), torch.compile(mi355x, is_training) end to end"
-    kernel = "whole compiled training step (dense / gated dense and their input- and weight-gradient launches, attention forward with row statistics, the two attention backward kernels, rotary, norms; Aten for the norm and gate formulas)"
+    kernel = "whole compiled training step (dense / gated dense and their input- and weight-gradient launches, attention forward with row statistics, the two attention backward kernels, rotary, norms and their backward, gate backward; Aten for the residual and gradient sums)"
     work = 3 * LlamaBlockC5.work  # one forward, two products per forward product in the backward
     cpu_work = work // 4            # the CPU leg runs one of the four batch entries
     cpu_warmups = 0
