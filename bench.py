@@ -576,7 +576,7 @@ class SdpaBackwardC5(Workload):
         dq, dk, dv = self.grads[i]
         s = self.strides
         self.lib.xg_sdpa_backward(_p(q), _p(k), _p(v), _p(out), _p(do), _p(lse), _p(dq), _p(dk), _p(dv), _p(self.delta), 4, 32, 32, 2048, 2048,
-                                  128, s, s, s, s, s, self.scale, 1, 2, self.st)
+                                  128, s, s, s, s, s, s, s, s, self.scale, 1, 2, self.st)
 
     def check(self, torch):
         from oracle import eager

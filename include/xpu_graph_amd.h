@@ -305,9 +305,12 @@ int xg_sdpa_masked(const void* q, const void* k, const void* v, void* out, const
  *   xg_sdpa_lse: xg_sdpa that also writes lse [B,H,Sq] fp32, the natural-log
  *     sum of exponentials of every query row's scaled (and causally masked)
  *     scores; -inf for a row that sees no key.
- *   xg_sdpa_backward: dq [B,H,Sq,D], dk and dv [B,Hkv,Skv,D] (contiguous, in
- *     `dtype`) from q, k, v, the forward's out and lse, and d_out (strides as
- *     in xg_sdpa; d_out has its own).  The probabilities are recomputed tile by
+ *   xg_sdpa_backward: dq [B,H,Sq,D], dk and dv [B,Hkv,Skv,D] (in `dtype`,
+ *     each with its own batch / head / sequence strides like the inputs, so a
+ *     gradient can be written in the layout of the tensor it belongs to; rows
+ *     of D contiguous elements that do not overlap) from q, k, v, the
+ *     forward's out and lse, and d_out (strides as in xg_sdpa; d_out has its
+ *     own).  The probabilities are recomputed tile by
  *     tile from lse: no [Sq,Skv] temporary.  With Hkv < H the gradients of a
  *     key/value head are summed over its query heads inside the kernel.  Two
  *     launches on `stream`; results do not depend on scheduling (no atomics).
@@ -321,7 +324,8 @@ int xg_sdpa_lse(const void* q, const void* k, const void* v, void* out, float* l
 int xg_sdpa_backward(const void* q, const void* k, const void* v, const void* out, const void* d_out, const float* lse,
                      void* dq, void* dk, void* dv, float* delta_ws, int64_t B, int64_t H, int64_t Hkv, int64_t Sq,
                      int64_t Skv, int64_t D, const int64_t q_strides[3], const int64_t k_strides[3],
-                     const int64_t v_strides[3], const int64_t o_strides[3], const int64_t do_strides[3], float scale,
+                     const int64_t v_strides[3], const int64_t o_strides[3], const int64_t do_strides[3],
+                     const int64_t dq_strides[3], const int64_t dk_strides[3], const int64_t dv_strides[3], float scale,
                      int causal, int dtype, xg_stream_t stream);
 
 /* ---------------------------------------------------------------------------
@@ -341,7 +345,8 @@ int xg_sdpa_backward_static(const void* q, const void* k, const void* v, const v
                             const float* lse, void* dq, void* dk, void* dv, int64_t B, int64_t H, int64_t Hkv,
                             int64_t Sq, int64_t Skv, int64_t D, const int64_t q_strides[3],
                             const int64_t k_strides[3], const int64_t v_strides[3], const int64_t o_strides[3],
-                            const int64_t do_strides[3], float scale, int causal, int dtype, xg_stream_t stream);
+                            const int64_t do_strides[3], const int64_t dq_strides[3], const int64_t dk_strides[3],
+                            const int64_t dv_strides[3], float scale, int causal, int dtype, xg_stream_t stream);
 
 /* ---------------------------------------------------------------------------
  * Rotary position embedding, rotate-half convention:

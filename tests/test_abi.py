@@ -154,7 +154,7 @@ def test_static_workspace_backward_refuses_more_rows_than_it_holds_without_a_gpu
     lib = _lib.lib()
     S3 = ctypes.c_int64 * 3
     p = ctypes.c_void_p(256)  # never dereferenced: the size check comes first
-    args = (S3(), S3(), S3(), S3(), S3(), 1.0, 0, 2, None)
+    args = (S3(), S3(), S3(), S3(), S3(), S3(), S3(), S3(), 1.0, 0, 2, None)
     assert lib.xg_sdpa_backward_static(p, p, p, p, p, p, p, p, p, 1, 1, 1, (1 << 21) + 1, 64, 64, *args) == -5
     assert lib.xg_sdpa_backward_static(p, p, p, p, p, p, p, p, p, 1 << 11, 1 << 11, 1, 1, 64, 64, *args) == -5
     assert lib.xg_sdpa_backward_static(p, p, p, p, p, p, p, p, p, 0, 4, 4, 64, 64, 64, *args) == 0  # nothing to do

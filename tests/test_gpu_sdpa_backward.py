@@ -88,6 +88,7 @@ def test_backward_grouped_heads_and_strided_views(device):
     for causal in (True, False):
         out, lse, dq, dk, dv = run_backward(q, k, v, g, causal, 0.09)
         _, wq, wk, wv = ref_grads(q, k, v, g, causal, 0.09)
+        assert dq.stride() == q.stride() and dk.stride() == k.stride() and dv.stride() == v.stride()  # written in place of the layouts they came in
         close_grad(dq, wq, "dq gqa")
         close_grad(dk, wk, "dk gqa")
         close_grad(dv, wv, "dv gqa")

@@ -28,7 +28,7 @@ def _call_both(lib, B, H, Hkv, Sq, Skv, D, causal, seed, device):
     results = []
     for static in (False, True):
         dq, dk, dv = torch.full_like(q, float("nan")), torch.full_like(k, float("nan")), torch.full_like(v, float("nan"))
-        tail = (B, H, Hkv, Sq, Skv, D, st(q), st(k), st(v), st(out), st(d_out), scale, causal, 2, stream)
+        tail = (B, H, Hkv, Sq, Skv, D, st(q), st(k), st(v), st(out), st(d_out), st(dq), st(dk), st(dv), scale, causal, 2, stream)
         if static:
             rc = lib.xg_sdpa_backward_static(P(q), P(k), P(v), P(out), P(d_out), P(lse), P(dq), P(dk), P(dv), *tail)
         else:
@@ -50,4 +50,4 @@ def test_static_workspace_backward_matches_the_workspace_argument_form(device):
     _call_both(lib, 1, 3, 3, 130, 257, 64, 0, 2, device)   # then 390: rows 390.. of the workspace keep the first call's values
     rows = (1 << 21) + 1
     p = ctypes.c_void_p(256)  # never dereferenced: the size check comes first
-    assert lib.xg_sdpa_backward_static(p, p, p, p, p, p, p, p, p, 1, 1, 1, rows, 64, 64, S3(), S3(), S3(), S3(), S3(), 1.0, 0, 2, None) == -5
+    assert lib.xg_sdpa_backward_static(p, p, p, p, p, p, p, p, p, 1, 1, 1, rows, 64, 64, *[S3()] * 8, 1.0, 0, 2, None) == -5

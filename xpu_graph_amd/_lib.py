@@ -125,11 +125,11 @@ _SIGNATURES = {
     ),
     "xg_sdpa_backward": (
         c_int,
-        [c_void_p] * 10 + [c_int64] * 6 + [ctypes.POINTER(c_int64)] * 5 + [c_float, c_int, c_int, c_void_p],
+        [c_void_p] * 10 + [c_int64] * 6 + [ctypes.POINTER(c_int64)] * 8 + [c_float, c_int, c_int, c_void_p],
     ),
     "xg_sdpa_backward_static": (
         c_int,
-        [c_void_p] * 9 + [c_int64] * 6 + [ctypes.POINTER(c_int64)] * 5 + [c_float, c_int, c_int, c_void_p],
+        [c_void_p] * 9 + [c_int64] * 6 + [ctypes.POINTER(c_int64)] * 8 + [c_float, c_int, c_int, c_void_p],
     ),
     "xg_rope": (
         c_int,

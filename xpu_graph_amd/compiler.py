@@ -88,6 +88,13 @@ class XpuGraph:
                     if kept is not None:
                         sample_inputs = [sample_inputs[i] for i in kept]
                 fake_mode, fake_inputs = fakify_tensors(sample_inputs)
+                if stage == FxStage.forward:
+                    # a forward graph returns the caller's results first and the values saved for the backward after
+                    # them; passes that would make two results share storage only need to look at the former
+                    ctx = torch._guards.TracingContext.try_get()
+                    meta = getattr(ctx, "fw_metadata", None) if ctx is not None else None
+                    if meta is not None and hasattr(meta, "num_forward_returns"):
+                        gm.meta["xg_user_outputs"] = int(meta.num_forward_returns)
                 hashkey = None
                 # a frozen graph carries its parameters as constants: the text of the graph, which is what the cache
                 # key is made of, no longer identifies it (two models of one architecture would share an artifact)

@@ -38,11 +38,12 @@ struct BwdParams {
   const void* d_o;
   const float* lse;  // [B, H, Sq] natural log
   float* delta;      // [B, H, Sq] workspace: written by the dq kernel, read by the dk/dv kernel
-  void* dq;          // [B, H, Sq, D] contiguous
-  void* dk;          // [B, Hkv, Skv, D] contiguous
+  void* dq;          // [B, H, Sq, D]
+  void* dk;          // [B, Hkv, Skv, D]
   void* dv;
   int B, H, Hkv, Sq, Skv;
   int64_t qs[3], ks[3], vs[3], os[3], dos[3];  // element strides of batch, head, sequence
+  int64_t dqs[3], dks[3], dvs[3];              // ... of the three outputs (rows of D contiguous elements)
   float scale;
   int causal;
   int n_qb, n_kb;
@@ -108,10 +109,11 @@ __device__ __forceinline__ void transposed_times_held(const char* tile, int t, c
 }
 
 // Write acc^T (lane = row l32 of this wave's 32 rows, registers = columns) times `mul` as rows of D elements of T
-// to dst + row * D, for rows below rows_valid.  `park` is this wave's 32 x D x 2 bytes of LDS; every wave of the
+// to dst + row * row_stride, for rows below rows_valid.  `park` is this wave's 32 x D x 2 bytes of LDS; every wave of the
 // workgroup must make the call (it holds a barrier).
 template <typename T, int D>
-__device__ __forceinline__ void store_rows(char* park, const f32x16 (&acc)[D / 32], float mul, T* dst, int rows_valid, int lane) {
+__device__ __forceinline__ void store_rows(char* park, const f32x16 (&acc)[D / 32], float mul, T* dst, int64_t row_stride, int rows_valid,
+                                           int lane) {
   constexpr int RB = D * 2, DT = D / 32;
   const int l32 = lane & 31, h = lane >> 5;
   static_for<DT>([&](auto DI) {
@@ -134,7 +136,7 @@ __device__ __forceinline__ void store_rows(char* park, const f32x16 (&acc)[D / 3
     const int row = pos / RB, pc = (pos % RB) >> 4;
     const int c = pc ^ swz_k<D>(row);
     const u32x4 val = *reinterpret_cast<const u32x4*>(park + pos);
-    if (row < rows_valid) *reinterpret_cast<u32x4*>(dst + (int64_t)row * D + c * 8) = val;
+    if (row < rows_valid) *reinterpret_cast<u32x4*>(dst + (int64_t)row * row_stride + c * 8) = val;
   });
 }
 
@@ -265,8 +267,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
     if (j + 1 < n_steps) step(std::integral_constant<int, 1>{}, j + 1);
   }
   __syncthreads();  // all waves are done reading tiles: the parks reuse the space
-  T* dst = reinterpret_cast<T*>(p.dq) + ((int64_t)bh * p.Sq + q0 + 32 * wave) * D;
-  store_rows<T, D>(smem + wave * (32 * RB), dq_acc, p.scale, dst, p.Sq - (q0 + 32 * wave), lane);
+  T* dst = reinterpret_cast<T*>(p.dq) + (int64_t)b * p.dqs[0] + (int64_t)head * p.dqs[1] + (int64_t)(q0 + 32 * wave) * p.dqs[2];
+  store_rows<T, D>(smem + wave * (32 * RB), dq_acc, p.scale, dst, p.dqs[2], p.Sq - (q0 + 32 * wave), lane);
 }
 
 // ---------------------------------------------------------------------------------------------- dk, dv
@@ -401,11 +403,13 @@ __global__ __launch_bounds__(kThreads) void sdpa_bwd_dkv_kernel(BwdParams p) {
     if (it + 1 < n_iter) step(std::integral_constant<int, 1>{}, it + 1);
   }
   __syncthreads();
-  const int64_t row0 = (int64_t)bk * p.Skv + k0 + 32 * wave;
+  const int row0 = k0 + 32 * wave;
   char* park = smem + wave * (32 * RB);
-  store_rows<T, D>(park, dk_acc, p.scale, reinterpret_cast<T*>(p.dk) + row0 * D, p.Skv - (k0 + 32 * wave), lane);
+  T* dk_dst = reinterpret_cast<T*>(p.dk) + (int64_t)b * p.dks[0] + (int64_t)hkv * p.dks[1] + (int64_t)row0 * p.dks[2];
+  T* dv_dst = reinterpret_cast<T*>(p.dv) + (int64_t)b * p.dvs[0] + (int64_t)hkv * p.dvs[1] + (int64_t)row0 * p.dvs[2];
+  store_rows<T, D>(park, dk_acc, p.scale, dk_dst, p.dks[2], p.Skv - row0, lane);
   __syncthreads();  // the parks have been read back before they are written again
-  store_rows<T, D>(park, dv_acc, 1.f, reinterpret_cast<T*>(p.dv) + row0 * D, p.Skv - (k0 + 32 * wave), lane);
+  store_rows<T, D>(park, dv_acc, 1.f, dv_dst, p.dvs[2], p.Skv - row0, lane);
 }
 
 template <typename T, int D>
@@ -430,7 +434,8 @@ namespace {
 int backward_entry(const void* q, const void* k, const void* v, const void* out, const void* d_out, const float* lse, void* dq, void* dk,
                    void* dv, float* delta_ws, int64_t B, int64_t H, int64_t Hkv, int64_t Sq, int64_t Skv, int64_t D,
                    const int64_t q_strides[3], const int64_t k_strides[3], const int64_t v_strides[3], const int64_t o_strides[3],
-                   const int64_t do_strides[3], float scale, int causal, int dtype, xg_stream_t stream) {
+                   const int64_t do_strides[3], const int64_t dq_strides[3], const int64_t dk_strides[3], const int64_t dv_strides[3],
+                   float scale, int causal, int dtype, xg_stream_t stream) {
   using namespace xg;
   if (dtype != XG_BF16 && dtype != XG_F16) return XG_ERR_BAD_DTYPE;
   if (B < 0 || H < 0 || Hkv < 0 || Sq < 0 || Skv < 0) return XG_ERR_BAD_SHAPE;
@@ -438,7 +443,7 @@ int backward_entry(const void* q, const void* k, const void* v, const void* out,
   if (B == 0 || H == 0) return XG_OK;
   if (Hkv == 0 || H % Hkv != 0 || Sq == 0 || Skv == 0) return XG_ERR_BAD_SHAPE;
   if (!q || !k || !v || !out || !d_out || !lse || !dq || !dk || !dv || !delta_ws) return XG_ERR_NULL_PTR;
-  if (!q_strides || !k_strides || !v_strides || !o_strides || !do_strides) return XG_ERR_NULL_PTR;
+  if (!q_strides || !k_strides || !v_strides || !o_strides || !do_strides || !dq_strides || !dk_strides || !dv_strides) return XG_ERR_NULL_PTR;
   if (!(scale == scale) || fabsf(scale) > 3.0e38f) return XG_ERR_BAD_ARG;
   if (Sq > (1 << 30) || Skv > (1 << 30)) return XG_ERR_TOO_LARGE;
   const int64_t n_qb = (Sq + sdpa::BQ - 1) / sdpa::BQ, n_kb = (Skv + sdpa::BK - 1) / sdpa::BK;
@@ -449,8 +454,8 @@ int backward_entry(const void* q, const void* k, const void* v, const void* out,
   if (!aligned_to(lse, 4) || !aligned_to(delta_ws, 4)) return XG_ERR_BAD_ALIGN;
   sdpa::BwdParams p;
   for (int i = 0; i < 3; ++i) {
-    const int64_t s5[] = {q_strides[i], k_strides[i], v_strides[i], o_strides[i], do_strides[i]};
-    for (int64_t s : s5) {
+    const int64_t s8[] = {q_strides[i], k_strides[i], v_strides[i], o_strides[i], do_strides[i], dq_strides[i], dk_strides[i], dv_strides[i]};
+    for (int64_t s : s8) {
       if (s < 0) return XG_ERR_BAD_SHAPE;
       if (s % 8) return XG_ERR_BAD_ALIGN;
     }
@@ -459,7 +464,12 @@ int backward_entry(const void* q, const void* k, const void* v, const void* out,
     p.vs[i] = v_strides[i];
     p.os[i] = o_strides[i];
     p.dos[i] = do_strides[i];
+    p.dqs[i] = dq_strides[i];
+    p.dks[i] = dk_strides[i];
+    p.dvs[i] = dv_strides[i];
   }
+  // the outputs are written, so their rows must not overlap: every row holds D elements
+  if (dq_strides[2] < D || dk_strides[2] < D || dv_strides[2] < D) return XG_ERR_BAD_SHAPE;
   // per-lane tile offsets are 32-bit: 64 rows of a streamed operand must span less than 2 GiB
   if (k_strides[2] > (1 << 23) || v_strides[2] > (1 << 23) || q_strides[2] > (1 << 23) || do_strides[2] > (1 << 23)) return XG_ERR_TOO_LARGE;
   p.q = q;
@@ -513,16 +523,18 @@ static int scratch_address(float** out) {
 extern "C" int xg_sdpa_backward(const void* q, const void* k, const void* v, const void* out, const void* d_out, const float* lse,
                                 void* dq, void* dk, void* dv, float* delta_ws, int64_t B, int64_t H, int64_t Hkv, int64_t Sq,
                                 int64_t Skv, int64_t D, const int64_t q_strides[3], const int64_t k_strides[3],
-                                const int64_t v_strides[3], const int64_t o_strides[3], const int64_t do_strides[3], float scale,
+                                const int64_t v_strides[3], const int64_t o_strides[3], const int64_t do_strides[3],
+                                const int64_t dq_strides[3], const int64_t dk_strides[3], const int64_t dv_strides[3], float scale,
                                 int causal, int dtype, xg_stream_t stream) {
   return backward_entry(q, k, v, out, d_out, lse, dq, dk, dv, delta_ws, B, H, Hkv, Sq, Skv, D, q_strides, k_strides, v_strides, o_strides,
-                        do_strides, scale, causal, dtype, stream);
+                        do_strides, dq_strides, dk_strides, dv_strides, scale, causal, dtype, stream);
 }
 
 extern "C" int xg_sdpa_backward_static(const void* q, const void* k, const void* v, const void* out, const void* d_out,
                                        const float* lse, void* dq, void* dk, void* dv, int64_t B, int64_t H, int64_t Hkv, int64_t Sq,
                                        int64_t Skv, int64_t D, const int64_t q_strides[3], const int64_t k_strides[3],
                                        const int64_t v_strides[3], const int64_t o_strides[3], const int64_t do_strides[3],
+                                       const int64_t dq_strides[3], const int64_t dk_strides[3], const int64_t dv_strides[3],
                                        float scale, int causal, int dtype, xg_stream_t stream) {
   if (B < 0 || H < 0 || Sq < 0) return XG_ERR_BAD_SHAPE;
   if (B > kScratchFloats || H > kScratchFloats || Sq > kScratchFloats || B * H > kScratchFloats || B * H * Sq > kScratchFloats)
@@ -531,5 +543,5 @@ extern "C" int xg_sdpa_backward_static(const void* q, const void* k, const void*
   float* ws = nullptr;
   if (int st = scratch_address(&ws)) return st;
   return backward_entry(q, k, v, out, d_out, lse, dq, dk, dv, ws, B, H, Hkv, Sq, Skv, D, q_strides, k_strides, v_strides, o_strides,
-                        do_strides, scale, causal, dtype, stream);
+                        do_strides, dq_strides, dk_strides, dv_strides, scale, causal, dtype, stream);
 }

@@ -815,17 +815,16 @@ def _sdpa_bwd(q, k, v, out, d_out, lse, is_causal, scale):
     lse = lse.contiguous()
     B, H, Sq, D = q.shape
     Hkv, Skv = k.shape[1], k.shape[2]
-    dq = torch.empty((B, H, Sq, D), dtype=q.dtype, device=q.device)
-    dk = torch.empty((B, Hkv, Skv, D), dtype=q.dtype, device=q.device)
-    dv = torch.empty((B, Hkv, Skv, D), dtype=q.dtype, device=q.device)
+    # each gradient in the layout of its tensor: the transpose / reshape that follows in a model's backward is a view
+    dq, dk, dv = _empty_like_layout(q), _empty_like_layout(k), _empty_like_layout(v)
     if dq.numel() == 0 or dk.numel() == 0:
         return dq.zero_(), dk.zero_(), dv.zero_()
     delta = torch.empty((B, H, Sq), dtype=torch.float32, device=q.device)
     S3 = ctypes.c_int64 * 3
     st = _lib.lib().xg_sdpa_backward(
         _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(d_out), _ptr(lse), _ptr(dq), _ptr(dk), _ptr(dv), _ptr(delta), B, H, Hkv, Sq, Skv, D,
-        S3(*q.stride()[:3]), S3(*k.stride()[:3]), S3(*v.stride()[:3]), S3(*out.stride()[:3]), S3(*d_out.stride()[:3]), scale,
-        1 if is_causal else 0, _code(q.dtype), _stream(),
+        S3(*q.stride()[:3]), S3(*k.stride()[:3]), S3(*v.stride()[:3]), S3(*out.stride()[:3]), S3(*d_out.stride()[:3]),
+        S3(*dq.stride()[:3]), S3(*dk.stride()[:3]), S3(*dv.stride()[:3]), scale, 1 if is_causal else 0, _code(q.dtype), _stream(),
     )
     _lib.check(st, "xg_sdpa_backward")
     return dq, dk, dv
@@ -898,8 +897,7 @@ def _sdpa_lse_meta(q, k, v, is_causal, scale):
 
 def _sdpa_bwd_meta(q, k, v, out, d_out, lse, is_causal, scale):
     _sdpa_check(q, k, v)
-    return (torch.empty(tuple(q.shape), dtype=q.dtype, device=q.device), torch.empty(tuple(k.shape), dtype=q.dtype, device=q.device),
-            torch.empty(tuple(v.shape), dtype=q.dtype, device=q.device))
+    return tuple(_empty_like_layout(_unit_last(t)) for t in (q, k, v))
 
 
 def _rope_check(x, cos, sin):
