@@ -100,6 +100,18 @@ int xg_rms_norm_bwd(const void* x, const void* res, const void* w, const void* g
                     float eps, int dtype, int w_dtype, int n_blocks, xg_stream_t stream);
 
 /* ---------------------------------------------------------------------------
+ * Backward of xg_layer_norm / xg_add_layer_norm, same conventions (the
+ * reference's LayerNorm training cases: tests/common/test_fuse_layernorm.py).
+ *   h = x (+ res), mu = mean(h), r = rsqrt(mean((h - mu)^2) + eps), hhat = (h - mu) r
+ *   gx = r (gy w - mean(gy w) - hhat mean(gy w hhat)) (+ gh)
+ *   gw_part[n_blocks, cols] fp32: shares of sum_rows(gy hhat) (needs w);
+ *   gb_part[n_blocks, cols] fp32: shares of sum_rows(gy), the bias gradient; either may be NULL.
+ * ------------------------------------------------------------------------- */
+int xg_layer_norm_bwd(const void* x, const void* res, const void* w, const void* gy, const void* gh, void* gx, float* gw_part,
+                      float* gb_part, int64_t rows, int64_t cols, int64_t x_stride, int64_t res_stride, int64_t gy_stride,
+                      int64_t gh_stride, float eps, int dtype, int w_dtype, int n_blocks, xg_stream_t stream);
+
+/* ---------------------------------------------------------------------------
  * Column slice + concatenate (bit-exact byte mover, dtype-agnostic).
  *
  * For every row r < rows and every chunk i < n_chunks, copies `chunk_bytes`

@@ -106,6 +106,49 @@ def test_rms_norm_backward_kernel(device, dtype, wdtype, rows, cols, with_res, w
         assert gw.numel() == 0
 
 
+@pytest.mark.parametrize("dtype,wdtype", [(torch.float32, torch.float32), (torch.bfloat16, torch.bfloat16), (torch.bfloat16, torch.float32), (torch.float16, torch.float16)])
+@pytest.mark.parametrize("rows,cols", [(1, 8), (37, 64), (300, 4096), (2050, 1024), (5, 16384), (1500, 2056)])
+@pytest.mark.parametrize("with_res,with_gh,with_w", [(False, False, True), (True, True, True), (True, False, False)])
+def test_layer_norm_backward_kernel(device, dtype, wdtype, rows, cols, with_res, with_gh, with_w):
+    """xg_layer_norm_bwd against float64 autograd of the same forward, rows with a mean far from zero (the centred
+    sums must not cancel): gx, the weight gradient and the bias gradient (the column sums of gy)."""
+    import xpu_graph_amd.ops  # noqa: F401
+
+    if dtype == torch.float32 and cols > 8192:
+        pytest.skip("fp32 rows hold at most 8192 columns in the kernel")
+    gen = torch.Generator().manual_seed(rows + 3 * cols)
+    x = (3.0 + torch.randn(rows, cols, generator=gen)).to(dtype).to(device)
+    res = torch.randn(rows, cols, generator=gen).to(dtype).to(device) if with_res else None
+    w = (1 + 0.2 * torch.randn(cols, generator=gen)).to(wdtype).to(device) if with_w else None
+    gy = torch.randn(rows, cols, generator=gen).to(dtype).to(device)
+    gh = torch.randn(rows, cols, generator=gen).to(dtype).to(device) if with_gh else None
+    gx, gw, gb = torch.ops.xpu_ops.layer_norm_bwd(x, res, w, gy, gh, 1e-5, True, True)
+    h = (x + res) if with_res else x  # rounded to the storage type
+    h64 = h.double().requires_grad_(True)
+    w64 = w.double().requires_grad_(True) if with_w else None
+    hc = h64 - h64.mean(-1, keepdim=True)
+    y = hc * torch.rsqrt(hc.pow(2).mean(-1, keepdim=True) + 1e-5)
+    y = y * w64 if with_w else y
+    grads = torch.autograd.grad(y, (h64, w64) if with_w else (h64,), gy.double())
+    want_gx = grads[0] + (gh.double() if with_gh else 0)
+    ulp = {torch.float32: 2.0**-23, torch.bfloat16: 2.0**-8, torch.float16: 2.0**-11}[dtype]
+    assert gx.shape == x.shape and gx.dtype == dtype
+    # the row mean is an fp32 sum of up to 16384 values near 3: its rounding enters every centred value
+    torch.testing.assert_close(gx.double(), want_gx, rtol=1.01 * ulp, atol=want_gx.abs().max().item() * max(ulp * 2.0**-6, 1e-5))
+    out_dt = wdtype if with_w else dtype
+    wulp = {torch.float32: 2.0**-23, torch.bfloat16: 2.0**-8, torch.float16: 2.0**-11}[out_dt]
+    want_gb = gy.double().sum(0)
+    assert gb.shape == (cols,) and gb.dtype == out_dt
+    torch.testing.assert_close(gb.double(), want_gb, rtol=1.01 * wulp, atol=want_gb.abs().max().item() * max(wulp * 2.0**-6, 1e-5))
+    if with_w:
+        assert gw.shape == w.shape and gw.dtype == wdtype
+        torch.testing.assert_close(gw.double(), grads[1], rtol=1.01 * wulp, atol=grads[1].abs().max().item() * max(wulp * 2.0**-6, 1e-5))
+    else:
+        assert gw.numel() == 0
+    only_gx = torch.ops.xpu_ops.layer_norm_bwd(x, res, w, gy, gh, 1e-5, False, False)
+    assert torch.equal(only_gx[0], gx) and only_gx[1].numel() == 0 and only_gx[2].numel() == 0
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("shape", [(256, 512), (3, 5, 7), (1, 1), (8192, 1376)])
 def test_gate_backward_kernel(device, dtype, shape):

@@ -8,7 +8,7 @@ from torch.fx.experimental.proxy_tensor import make_fx
 
 import xpu_graph_amd.ops  # noqa: F401  (defines torch.ops.xpu_ops)
 from xpu_graph_amd.passes.fake_prop import propagate_missing
-from xpu_graph_amd.passes.patterns.targets.mi355x.sum_folds import FoldAddIntoDense, FoldAddIntoRmsNormBackward, FoldCloneOfContiguous
+from xpu_graph_amd.passes.patterns.targets.mi355x.sum_folds import FoldAddIntoDense, FoldAddIntoNormBackward, FoldCloneOfContiguous
 
 bf16 = torch.bfloat16
 xpu = torch.ops.xpu_ops
@@ -88,7 +88,7 @@ def test_gradient_sum_moves_into_the_norm_backward():
         return other + gx, gw
 
     gm = trace(fn, ((4, 8, 256), bf16), ((256,), bf16), ((4, 8, 256), bf16), ((4, 8, 256), bf16))
-    assert FoldAddIntoRmsNormBackward().process(gm)
+    assert FoldAddIntoNormBackward().process(gm)
     gm.graph.lint()
     assert calls(gm, aten.add.Tensor) == []
     (bwd,) = calls(gm, xpu.rms_norm_bwd.default)
@@ -97,13 +97,26 @@ def test_gradient_sum_moves_into_the_norm_backward():
     assert all(o.target is operator.getitem and o.args[0] is bwd for o in outs) and [o.args[1] for o in outs] == [0, 1]
 
 
+def test_gradient_sum_moves_into_the_layer_norm_backward():
+    def fn(x, w, gy, other):
+        gx, gw, gb = xpu.layer_norm_bwd(x, None, w, gy, None, 1e-5, True, True)
+        return gx + other, gw, gb
+
+    gm = trace(fn, ((4, 8, 256), bf16), ((256,), bf16), ((4, 8, 256), bf16), ((4, 8, 256), bf16))
+    assert FoldAddIntoNormBackward().process(gm)
+    gm.graph.lint()
+    assert calls(gm, aten.add.Tensor) == []
+    (bwd,) = calls(gm, xpu.layer_norm_bwd.default)
+    assert bwd.args[4].name == "other_1" and bwd.args[5:] == (1e-5, True, True)
+
+
 def test_norm_backward_that_already_adds_a_gradient_is_left_alone():
     def fn(x, w, gy, gh, other):
         gx, _ = xpu.rms_norm_bwd(x, None, w, gy, gh, 1e-6, False)
         return other + gx
 
     gm = trace(fn, ((8, 256), bf16), ((256,), bf16), *[((8, 256), bf16)] * 3)
-    assert not FoldAddIntoRmsNormBackward().process(gm)
+    assert not FoldAddIntoNormBackward().process(gm)
 
 
 def test_copy_of_a_value_that_is_already_contiguous_is_dropped():

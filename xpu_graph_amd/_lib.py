@@ -43,6 +43,7 @@ _SIGNATURES = {
         [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_float, c_int, c_int, c_void_p],
     ),
     "xg_rms_norm_bwd": (c_int, [c_void_p] * 7 + [c_int64] * 6 + [c_float, c_int, c_int, c_int, c_void_p]),
+    "xg_layer_norm_bwd": (c_int, [c_void_p] * 8 + [c_int64] * 6 + [c_float, c_int, c_int, c_int, c_void_p]),
     "xg_add_layer_norm": (
         c_int,
         [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_float, c_int, c_int, c_void_p],

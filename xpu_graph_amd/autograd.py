@@ -54,6 +54,22 @@ def _rms_kernel_backward(x, res, w, gy, gh, eps, want_gw):
     return gx, (gw if want_gw and w is not None else None)
 
 
+def _bias_is_one_row(b_meta, x):
+    """The bias is a plain [cols] vector: its gradient is the column sum the kernel accumulates."""
+    return b_meta is not None and len(b_meta[0]) == 1 and b_meta[0][0] == x.shape[-1]
+
+
+def _ln_kernel_backward(x, res, w, gy, gh, eps, want_gw, b_meta, want_gb):
+    """(g_sum, gw | None, gb | None) on the fused backward kernel when it takes the shape, else None."""
+    from . import ops
+
+    if not (x.is_cuda and ops.rms_norm_bwd_fits(x, w)) or (res is not None and res.dtype != x.dtype):
+        return None
+    want_gb = bool(want_gb)
+    gx, gw, gb = torch.ops.xpu_ops.layer_norm_bwd(x, res, w, gy, gh, eps, want_gw, want_gb)
+    return gx, (gw if want_gw and w is not None else None), (gb.to(b_meta[1]) if want_gb else None)
+
+
 def _rms_backward(ctx, gy):
     saved = ctx.saved_tensors
     x = saved[0]
@@ -81,6 +97,11 @@ def _ln_backward(ctx, gy):
     saved = ctx.saved_tensors
     x = saved[0]
     w = saved[1] if ctx.has_w else None
+    want_gb = ctx.has_b and ctx.needs_input_grad[2]
+    if not want_gb or _bias_is_one_row(ctx.b_meta, x):
+        fused = _ln_kernel_backward(x, None, w, gy, None, ctx.eps, ctx.needs_input_grad[1], ctx.b_meta, want_gb)
+        if fused is not None:
+            return fused[0], fused[1], fused[2], None
     xf, gf = x.float(), gy.float()
     mean = xf.mean(-1, keepdim=True)
     xc = xf - mean
@@ -282,6 +303,12 @@ def _add_norm_formulas(layer, with_sum):
             fused = _rms_kernel_backward(x, res, w, gy, gh, ctx.eps, need[2])
             if fused is not None:
                 return fused[0], fused[0], fused[1], None
+        else:
+            want_gb = ctx.b_meta is not None and need[3]
+            if not want_gb or _bias_is_one_row(ctx.b_meta, x):
+                fused = _ln_kernel_backward(x, res, w, gy, gh, ctx.eps, need[2], ctx.b_meta, want_gb)
+                if fused is not None:
+                    return fused[0], fused[0], fused[1], fused[2], None
         hf, gf = x.float() + res.float(), gy.float()
         hc = hf - hf.mean(-1, keepdim=True) if layer else hf
         r = torch.rsqrt(hc.pow(2).mean(-1, keepdim=True) + ctx.eps)

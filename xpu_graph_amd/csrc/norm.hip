@@ -275,30 +275,36 @@ int dispatch(const NormArgs& a, int dtype, int wb_dtype) {
 }
 
 
-// ---- backward of RMSNorm with optional residual add ------------------------------------------------
-// h = x (+ res, rounded to the storage type as the forward does), r = rsqrt(mean(h^2) + eps), hhat = h r,
-// ghat = gy w:   g_sum = r (ghat - hhat mean(ghat hhat)) (+ gh)     the gradient of x (and of res)
-//                gw    = sum over rows of gy hhat                   written as one fp32 partial row per block
+// ---- backward of RMSNorm / LayerNorm with optional residual add -------------------------------------
+// h = x (+ res, rounded to the storage type as the forward does), ghat = gy w
+//   RMSNorm:    r = rsqrt(mean(h^2) + eps), hhat = h r
+//               g_sum = r (ghat - hhat mean(ghat hhat)) (+ gh)
+//   LayerNorm:  mu = mean(h), r = rsqrt(mean((h - mu)^2) + eps), hhat = (h - mu) r
+//               g_sum = r (ghat - mean(ghat) - hhat mean(ghat hhat)) (+ gh)
+//   g_sum is the gradient of x (and of res);  gw = sum over rows of gy hhat,  gb = sum over rows of gy (LayerNorm),
+//   each written as one fp32 partial row per block.
 // One block of 256 threads walks a strip of rows; a lane keeps the same CH chunks of 16 bytes of every row, so its
-// share of gw stays in registers across the strip.  One pass over h and gy per row: the two row sums the formula
-// needs (sum h^2 and sum ghat h) are independent of r.
-template <typename T, typename WT, int CH>
-__global__ __launch_bounds__(256) void rms_bwd_kernel(const T* __restrict__ x, const T* __restrict__ res, const WT* __restrict__ w,
-                                                      const T* __restrict__ gy, const T* __restrict__ gh, T* __restrict__ gx,
-                                                      float* __restrict__ gw_part, int64_t rows, int nvec, int64_t x_stride,
-                                                      int64_t res_stride, int64_t gy_stride, int64_t gh_stride, float eps,
-                                                      float inv_cols, int rows_per_block) {
+// share of gw / gb stays in registers across the strip.  One pass over h and gy per row.  RMSNorm needs one round of
+// row sums (sum h^2 and sum ghat h do not depend on r); LayerNorm two, the mean first and the centred sums after it,
+// as its forward does.
+template <typename T, typename WT, int CH, bool LAYER>
+__global__ __launch_bounds__(256) void norm_bwd_kernel(const T* __restrict__ x, const T* __restrict__ res, const WT* __restrict__ w,
+                                                       const T* __restrict__ gy, const T* __restrict__ gh, T* __restrict__ gx,
+                                                       float* __restrict__ gw_part, float* __restrict__ gb_part, int64_t rows, int nvec,
+                                                       int64_t x_stride, int64_t res_stride, int64_t gy_stride, int64_t gh_stride,
+                                                       float eps, float inv_cols, int rows_per_block) {
   typedef typename VecOf<T>::type V;
   constexpr int VN = VecOf<T>::N;
-  __shared__ float red_a[4], red_b[4];
+  __shared__ float red_a[4], red_b[4], red_c[4], red_m[4];
   const int lane = threadIdx.x;
-  float wv[CH][VN], gw_acc[CH][VN];
+  float wv[CH][VN], gw_acc[CH][VN], gb_acc[LAYER ? CH : 1][VN];
 #pragma unroll
   for (int i = 0; i < CH; ++i) {
     const int c = lane + i * 256;
 #pragma unroll
     for (int j = 0; j < VN; ++j) {
       gw_acc[i][j] = 0.f;
+      if constexpr (LAYER) gb_acc[i][j] = 0.f;
       wv[i][j] = (w != nullptr && c < nvec) ? to_f32(w[(int64_t)c * VN + j]) : 1.f;
     }
   }
@@ -306,7 +312,7 @@ __global__ __launch_bounds__(256) void rms_bwd_kernel(const T* __restrict__ x, c
   const int64_t r1 = r0 + rows_per_block < rows ? r0 + rows_per_block : rows;
   for (int64_t row = r0; row < r1; ++row) {
     float hf[CH][VN], gf[CH][VN];
-    float s1 = 0.f, s2 = 0.f;
+    float s0 = 0.f;
 #pragma unroll
     for (int i = 0; i < CH; ++i) {
       const int c = lane + i * 256;
@@ -322,26 +328,50 @@ __global__ __launch_bounds__(256) void rms_bwd_kernel(const T* __restrict__ x, c
         for (int j = 0; j < VN; ++j) {
           hf[i][j] = to_f32(hv[j]);
           gf[i][j] = to_f32(gv[j]);
-          s1 = __builtin_fmaf(hf[i][j], hf[i][j], s1);
-          s2 = __builtin_fmaf(gf[i][j] * wv[i][j], hf[i][j], s2);
+          s0 += hf[i][j];
         }
       } else {
 #pragma unroll
         for (int j = 0; j < VN; ++j) hf[i][j] = gf[i][j] = 0.f;
       }
     }
+    float mean = 0.f;
+    if constexpr (LAYER) {
+      s0 = wave_sum<kWave>(s0);
+      if ((lane & 63) == 0) red_m[lane >> 6] = s0;  // its readers of the previous row passed two barriers since
+      __syncthreads();
+      mean = (red_m[0] + red_m[1] + red_m[2] + red_m[3]) * inv_cols;
+    }
+    float s1 = 0.f, s2 = 0.f, s3 = 0.f;
+#pragma unroll
+    for (int i = 0; i < CH; ++i) {
+      if (lane + i * 256 < nvec) {
+#pragma unroll
+        for (int j = 0; j < VN; ++j) {
+          if constexpr (LAYER) hf[i][j] -= mean;
+          const float ghat = gf[i][j] * wv[i][j];
+          s1 = __builtin_fmaf(hf[i][j], hf[i][j], s1);
+          s2 = __builtin_fmaf(ghat, hf[i][j], s2);
+          if constexpr (LAYER) s3 += ghat;
+        }
+      }
+    }
     s1 = wave_sum<kWave>(s1);
     s2 = wave_sum<kWave>(s2);
-    __syncthreads();  // the previous row's readers are done with red_a / red_b
+    if constexpr (LAYER) s3 = wave_sum<kWave>(s3);
+    __syncthreads();  // the previous row's readers are done with red_a / red_b / red_c
     if ((lane & 63) == 0) {
       red_a[lane >> 6] = s1;
       red_b[lane >> 6] = s2;
+      if constexpr (LAYER) red_c[lane >> 6] = s3;
     }
     __syncthreads();
     s1 = red_a[0] + red_a[1] + red_a[2] + red_a[3];
     s2 = red_b[0] + red_b[1] + red_b[2] + red_b[3];
     const float r = rsqrtf(s1 * inv_cols + eps);
     const float dot = r * s2 * inv_cols;  // mean(ghat * hhat)
+    float gmean = 0.f;
+    if constexpr (LAYER) gmean = (red_c[0] + red_c[1] + red_c[2] + red_c[3]) * inv_cols;
 #pragma unroll
     for (int i = 0; i < CH; ++i) {
       const int c = lane + i * 256;
@@ -352,55 +382,85 @@ __global__ __launch_bounds__(256) void rms_bwd_kernel(const T* __restrict__ x, c
 #pragma unroll
         for (int j = 0; j < VN; ++j) {
           const float hhat = hf[i][j] * r;
-          float g = r * (gf[i][j] * wv[i][j] - hhat * dot);
+          float g = r * (gf[i][j] * wv[i][j] - gmean - hhat * dot);
           if (gh != nullptr) g += to_f32(ghv[j]);
           out[j] = from_f32<T>(g);
           gw_acc[i][j] = __builtin_fmaf(gf[i][j], hhat, gw_acc[i][j]);
+          if constexpr (LAYER) gb_acc[i][j] += gf[i][j];
         }
         store_vec_nt(reinterpret_cast<V*>(gx + row * (int64_t)nvec * VN) + c, out);
       }
     }
   }
-  if (gw_part != nullptr) {
 #pragma unroll
-    for (int i = 0; i < CH; ++i) {
-      const int c = lane + i * 256;
-      if (c < nvec) {
+  for (int i = 0; i < CH; ++i) {
+    const int c = lane + i * 256;
+    if (c < nvec) {
 #pragma unroll
-        for (int j = 0; j < VN; ++j) gw_part[((int64_t)blockIdx.x * nvec + c) * VN + j] = gw_acc[i][j];
+      for (int j = 0; j < VN; ++j) {
+        if (gw_part != nullptr) gw_part[((int64_t)blockIdx.x * nvec + c) * VN + j] = gw_acc[i][j];
+        if constexpr (LAYER) {
+          if (gb_part != nullptr) gb_part[((int64_t)blockIdx.x * nvec + c) * VN + j] = gb_acc[i][j];
+        }
       }
     }
   }
 }
 
-struct RmsBwdArgs {
+struct NormBwdArgs {
   const void *x, *res, *w, *gy, *gh;
   void* gx;
-  float* gw_part;
+  float *gw_part, *gb_part;
   int64_t rows, cols, x_stride, res_stride, gy_stride, gh_stride;
   float eps;
   int n_blocks;
   hipStream_t stream;
 };
 
-template <typename T, typename WT>
-int rms_bwd_typed(const RmsBwdArgs& a) {
+template <typename T, typename WT, bool LAYER>
+int norm_bwd_typed(const NormBwdArgs& a) {
   constexpr int VN = VecOf<T>::N;
   const int nvec = (int)(a.cols / VN);
   const int chunks = (nvec + 255) / 256;
   const int rpb = (int)((a.rows + a.n_blocks - 1) / a.n_blocks);
   const float inv_cols = 1.f / (float)a.cols;
-#define XG_RMS_BWD(CH)                                                                                                        \
-  hipLaunchKernelGGL((rms_bwd_kernel<T, WT, CH>), dim3((unsigned)a.n_blocks), dim3(256), 0, a.stream, (const T*)a.x, (const T*)a.res, \
-                     (const WT*)a.w, (const T*)a.gy, (const T*)a.gh, (T*)a.gx, a.gw_part, a.rows, nvec, a.x_stride, a.res_stride,       \
-                     a.gy_stride, a.gh_stride, a.eps, inv_cols, rpb)
-  if (chunks <= 1) XG_RMS_BWD(1);
-  else if (chunks <= 2) XG_RMS_BWD(2);
-  else if (chunks <= 4) XG_RMS_BWD(4);
-  else if (chunks <= 8) XG_RMS_BWD(8);
+#define XG_NORM_BWD(CH)                                                                                                              \
+  hipLaunchKernelGGL((norm_bwd_kernel<T, WT, CH, LAYER>), dim3((unsigned)a.n_blocks), dim3(256), 0, a.stream, (const T*)a.x,          \
+                     (const T*)a.res, (const WT*)a.w, (const T*)a.gy, (const T*)a.gh, (T*)a.gx, a.gw_part, a.gb_part, a.rows, nvec,   \
+                     a.x_stride, a.res_stride, a.gy_stride, a.gh_stride, a.eps, inv_cols, rpb)
+  if (chunks <= 1) XG_NORM_BWD(1);
+  else if (chunks <= 2) XG_NORM_BWD(2);
+  else if (chunks <= 4) XG_NORM_BWD(4);
+  else if (chunks <= 8) XG_NORM_BWD(8);
   else return XG_ERR_TOO_LARGE;
-#undef XG_RMS_BWD
+#undef XG_NORM_BWD
   return status_from_hip(hipGetLastError());
+}
+
+// Argument checks and type dispatch shared by xg_rms_norm_bwd and xg_layer_norm_bwd.
+template <bool LAYER>
+int norm_bwd_entry(const void* x, const void* res, const void* w, const void* gy, const void* gh, void* gx, float* gw_part, float* gb_part,
+                   int64_t rows, int64_t cols, int64_t x_stride, int64_t res_stride, int64_t gy_stride, int64_t gh_stride, float eps,
+                   int dtype, int w_dtype, int n_blocks, xg_stream_t stream) {
+  if (!x || !gy || !gx) return XG_ERR_NULL_PTR;
+  if (rows < 0 || cols <= 0 || x_stride < cols || gy_stride < cols || (res && res_stride < cols) || (gh && gh_stride < cols)) return XG_ERR_BAD_SHAPE;
+  if (n_blocks < 1 || n_blocks > 65535 || (gw_part && !w)) return XG_ERR_BAD_ARG;
+  if (dtype != XG_F32 && dtype != XG_BF16 && dtype != XG_F16) return XG_ERR_BAD_DTYPE;
+  if (w && w_dtype != dtype && w_dtype != XG_F32) return XG_ERR_BAD_DTYPE;
+  const int64_t per16 = dtype == XG_F32 ? 4 : 8;
+  if (cols % per16 || x_stride % per16 || gy_stride % per16 || (res && res_stride % per16) || (gh && gh_stride % per16)) return XG_ERR_BAD_ALIGN;
+  const void* ptrs[] = {x, res, gy, gh, gx};
+  for (const void* q : ptrs)
+    if (q && !aligned_to(q, 16)) return XG_ERR_BAD_ALIGN;
+  if ((w && !aligned_to(w, 4)) || (gw_part && !aligned_to(gw_part, 4)) || (gb_part && !aligned_to(gb_part, 4))) return XG_ERR_BAD_ALIGN;
+  if (cols / per16 > 8 * 256) return XG_ERR_TOO_LARGE;  // a lane keeps at most eight 16-byte chunks of a row
+  if (rows == 0) return XG_OK;
+  if (n_blocks > rows) n_blocks = (int)rows;
+  NormBwdArgs a{x, res, w, gy, gh, gx, gw_part, gb_part, rows, cols, x_stride, res_stride, gy_stride, gh_stride, eps, n_blocks, (hipStream_t)stream};
+  const bool wf32 = w && w_dtype == XG_F32;
+  if (dtype == XG_F32) return norm_bwd_typed<float, float, LAYER>(a);
+  if (dtype == XG_BF16) return wf32 ? norm_bwd_typed<bf16_t, float, LAYER>(a) : norm_bwd_typed<bf16_t, bf16_t, LAYER>(a);
+  return wf32 ? norm_bwd_typed<f16_t, float, LAYER>(a) : norm_bwd_typed<f16_t, f16_t, LAYER>(a);
 }
 
 }  // namespace
@@ -439,26 +499,15 @@ int xg_add_layer_norm(const void* x, const void* res, const void* w, const void*
 int xg_rms_norm_bwd(const void* x, const void* res, const void* w, const void* gy, const void* gh, void* gx, float* gw_part,
                     int64_t rows, int64_t cols, int64_t x_stride, int64_t res_stride, int64_t gy_stride, int64_t gh_stride,
                     float eps, int dtype, int w_dtype, int n_blocks, xg_stream_t stream) {
-  using namespace xg;
-  if (!x || !gy || !gx) return XG_ERR_NULL_PTR;
-  if (rows < 0 || cols <= 0 || x_stride < cols || gy_stride < cols || (res && res_stride < cols) || (gh && gh_stride < cols)) return XG_ERR_BAD_SHAPE;
-  if (n_blocks < 1 || n_blocks > 65535 || (gw_part && !w)) return XG_ERR_BAD_ARG;
-  if (dtype != XG_F32 && dtype != XG_BF16 && dtype != XG_F16) return XG_ERR_BAD_DTYPE;
-  if (w && w_dtype != dtype && w_dtype != XG_F32) return XG_ERR_BAD_DTYPE;
-  const int64_t per16 = dtype == XG_F32 ? 4 : 8;
-  if (cols % per16 || x_stride % per16 || gy_stride % per16 || (res && res_stride % per16) || (gh && gh_stride % per16)) return XG_ERR_BAD_ALIGN;
-  const void* ptrs[] = {x, res, gy, gh, gx};
-  for (const void* q : ptrs)
-    if (q && !aligned_to(q, 16)) return XG_ERR_BAD_ALIGN;
-  if ((w && !aligned_to(w, 4)) || (gw_part && !aligned_to(gw_part, 4))) return XG_ERR_BAD_ALIGN;
-  if (cols / per16 > 8 * 256) return XG_ERR_TOO_LARGE;  // a lane keeps at most eight 16-byte chunks of a row
-  if (rows == 0) return XG_OK;
-  if (n_blocks > rows) n_blocks = (int)rows;
-  RmsBwdArgs a{x, res, w, gy, gh, gx, gw_part, rows, cols, x_stride, res_stride, gy_stride, gh_stride, eps, n_blocks, (hipStream_t)stream};
-  const bool wf32 = w && w_dtype == XG_F32;
-  if (dtype == XG_F32) return rms_bwd_typed<float, float>(a);
-  if (dtype == XG_BF16) return wf32 ? rms_bwd_typed<bf16_t, float>(a) : rms_bwd_typed<bf16_t, bf16_t>(a);
-  return wf32 ? rms_bwd_typed<f16_t, float>(a) : rms_bwd_typed<f16_t, f16_t>(a);
+  return xg::norm_bwd_entry<false>(x, res, w, gy, gh, gx, gw_part, nullptr, rows, cols, x_stride, res_stride, gy_stride, gh_stride, eps, dtype,
+                                   w_dtype, n_blocks, stream);
+}
+
+int xg_layer_norm_bwd(const void* x, const void* res, const void* w, const void* gy, const void* gh, void* gx, float* gw_part,
+                      float* gb_part, int64_t rows, int64_t cols, int64_t x_stride, int64_t res_stride, int64_t gy_stride,
+                      int64_t gh_stride, float eps, int dtype, int w_dtype, int n_blocks, xg_stream_t stream) {
+  return xg::norm_bwd_entry<true>(x, res, w, gy, gh, gx, gw_part, gb_part, rows, cols, x_stride, res_stride, gy_stride, gh_stride, eps, dtype,
+                                  w_dtype, n_blocks, stream);
 }
 
 }  // extern "C"

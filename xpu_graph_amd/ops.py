@@ -30,6 +30,7 @@ _SCHEMAS = [
     "add_layer_norm(Tensor x, Tensor residual, Tensor? weight, Tensor? bias, float eps) -> (Tensor, Tensor)",
     "add_layer_norm_only(Tensor x, Tensor residual, Tensor? weight, Tensor? bias, float eps) -> Tensor",
     "rms_norm_bwd(Tensor x, Tensor? residual, Tensor? weight, Tensor gy, Tensor? gh, float eps, bool want_gw) -> (Tensor, Tensor)",
+    "layer_norm_bwd(Tensor x, Tensor? residual, Tensor? weight, Tensor gy, Tensor? gh, float eps, bool want_gw, bool want_gb) -> (Tensor, Tensor, Tensor)",
     "slice_cat(Tensor src, Tensor table, int chunk_bytes, int out_cols) -> Tensor",
     "slice_cat_multi(Tensor src, Tensor table, int chunk_bytes, int[] out_cols) -> Tensor[]",
     "slice_stack(Tensor src, Tensor[] tables, int[] chunk_bytes, int slice_len, int num) -> Tensor",
@@ -203,6 +204,51 @@ def _rms_norm_bwd(x, residual, weight, gy, gh, eps, want_gw):
     return gx, (part.sum(0) if rows else torch.zeros(cols, device=x.device)).to(weight.dtype)
 
 
+def _layer_norm_bwd(x, residual, weight, gy, gh, eps, want_gw, want_gb):
+    """Gradients of layer_norm / add_layer_norm in one pass per row: (gx, gw, gb); gx also is the residual's
+    gradient.  gw / gb are empty when not wanted (or, for gw, when there is no weight); gb has the dtype of the
+    weight when there is one, else that of x."""
+    if not rms_norm_bwd_fits(x, weight):
+        raise ValueError("layer_norm_bwd: needs rows of whole 16-byte vectors (at most 2048 of them) and a 1-D weight")
+    cols = x.shape[-1]
+    x2, rows, xs = _rows_2d(x)
+    g2, _, gs = _rows_2d(gy.to(x.dtype))
+    r2 = rs = h2 = hs = None
+    if residual is not None:
+        r2, _, rs = _rows_2d(residual)
+    if gh is not None:
+        h2, _, hs = _rows_2d(gh.to(x.dtype))
+    gx = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+    want_gw = bool(want_gw and weight is not None)
+    n_blocks = max(1, min(_RMS_BWD_BLOCKS, rows))
+    # one buffer for both partial sums: its halves are summed by one reduction
+    n_out = int(want_gw) + int(bool(want_gb))
+    part = torch.empty((n_out, n_blocks, cols), dtype=torch.float32, device=x.device) if n_out else None
+    pw = part[0] if want_gw else None
+    pb = part[n_out - 1] if want_gb else None
+    if rows:
+        st = _lib.lib().xg_layer_norm_bwd(
+            _ptr(x2), _ptr(r2), _ptr(weight.contiguous() if weight is not None else None), _ptr(g2), _ptr(h2), _ptr(gx), _ptr(pw), _ptr(pb),
+            rows, cols, xs, rs or 0, gs, hs or 0, eps, _code(x.dtype), _code(weight.dtype) if weight is not None else _code(x.dtype), n_blocks,
+            _stream(),
+        )
+        _lib.check(st, "xg_layer_norm_bwd")
+    wdt = weight.dtype if weight is not None else x.dtype
+    none = torch.empty(0, dtype=x.dtype, device=x.device)
+    if not n_out:
+        return gx, none, none
+    sums = part.sum(1) if rows else torch.zeros((n_out, cols), device=x.device)
+    return gx, (sums[0].to(wdt) if want_gw else none), (sums[n_out - 1].to(wdt) if want_gb else none)
+
+
+def _layer_norm_bwd_meta(x, residual, weight, gy, gh, eps, want_gw, want_gb):
+    gx = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+    wdt = weight.dtype if weight is not None else x.dtype
+    none = torch.empty(0, dtype=x.dtype, device=x.device)
+    row = lambda: torch.empty((x.shape[-1],), dtype=wdt, device=x.device)  # noqa: E731
+    return gx, (row() if want_gw and weight is not None else none), (row() if want_gb else none)
+
+
 def _rms_norm_bwd_meta(x, residual, weight, gy, gh, eps, want_gw):
     gx = torch.empty(x.shape, dtype=x.dtype, device=x.device)
     if want_gw and weight is not None:
@@ -218,6 +264,8 @@ _library.impl("rms_norm", _rms_norm, "CUDA")
 _library.impl("layer_norm", _layer_norm, "CUDA")
 _library.impl("rms_norm_bwd", _rms_norm_bwd, "CUDA")
 _library.impl("rms_norm_bwd", _rms_norm_bwd_meta, "Meta")
+_library.impl("layer_norm_bwd", _layer_norm_bwd, "CUDA")
+_library.impl("layer_norm_bwd", _layer_norm_bwd_meta, "Meta")
 _library.impl("add_rms_norm", _add_rms_norm, "CUDA")
 _library.impl("add_rms_norm_only", _add_rms_norm_only, "CUDA")
 _library.impl("add_layer_norm", _add_layer_norm, "CUDA")

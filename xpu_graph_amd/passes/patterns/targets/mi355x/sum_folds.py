@@ -2,7 +2,7 @@
 leave these to the vendor compiler; here they are the Aten launches left between the HIP kernels of a training step).
 
     add(dense(x, w, .., residual=None, "none"), t)        ->  dense(x, w, .., residual=t, "none")
-    add(rms_norm_bwd(.., gh=None)[0], t)                  ->  rms_norm_bwd(.., gh=t)[0]
+    add(rms_norm_bwd(.., gh=None)[0], t)                  ->  rms_norm_bwd(.., gh=t)[0]      (layer_norm_bwd alike)
     clone(v) where v is already laid out the way asked    ->  v
 
 The first two appear where autograd sums the gradients of a value with several uses (the three projections of one
@@ -92,7 +92,7 @@ class FoldAddIntoDense(Pattern):
         return changed
 
 
-class FoldAddIntoRmsNormBackward(Pattern):
+class FoldAddIntoNormBackward(Pattern):
     _opt_level = OptLevel.level2
     _support_stages = [FxStage.backward]
 
@@ -107,7 +107,7 @@ class FoldAddIntoRmsNormBackward(Pattern):
                 if not (is_call(mine, operator.getitem) and mine.args[1] == 0):
                     continue
                 bwd = mine.args[0]
-                if not is_call(bwd, _xpu.rms_norm_bwd.default) or len(bwd.args) != 7 or bwd.args[4] is not None:
+                if not is_call(bwd, _xpu.rms_norm_bwd.default, _xpu.layer_norm_bwd.default) or len(bwd.args) < 7 or bwd.args[4] is not None:
                     continue
                 if not (sole_user_is(mine, add) and len(mine.users) == 1):
                     continue
@@ -121,7 +121,7 @@ class FoldAddIntoRmsNormBackward(Pattern):
                 if not all(is_call(u, operator.getitem) and all(order[w] > order[add] for w in u.users) for u in others):
                     continue
                 with g.inserting_before(add):
-                    new = g.call_function(_xpu.rms_norm_bwd.default, bwd.args[:4] + (other,) + bwd.args[5:])
+                    new = g.call_function(bwd.target, bwd.args[:4] + (other,) + bwd.args[5:])
                     item = g.call_function(operator.getitem, (new, 0))
                     moved = [(u, g.call_function(operator.getitem, (new, u.args[1]))) for u in others]
                 add.replace_all_uses_with(item)
