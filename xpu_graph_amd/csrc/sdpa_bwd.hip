@@ -28,7 +28,8 @@
 namespace xg {
 namespace sdpa {
 
-constexpr int BK = 128;  // keys per workgroup of the dk/dv kernel
+constexpr int KW = 8;          // waves per workgroup of the dk/dv kernel, 32 keys each
+constexpr int BK = 32 * KW;   // keys per workgroup of the dk/dv kernel
 
 struct BwdParams {
   const void* q;
@@ -71,6 +72,23 @@ __device__ __forceinline__ f32x16 rows_times_regs(const char* tile, int t, int l
   return acc;
 }
 
+// The same product with the lane's row read from LDS as well: `held` points at the 32 rows of this wave (row l32 is
+// the lane's), laid out like a tile block.
+template <typename T, int D>
+__device__ __forceinline__ f32x16 rows_times_rows(const char* tile, int t, int l32, int h, int sx, const char* held) {
+  typedef typename Vec8<T>::type V8;
+  constexpr int RB = D * 2, KK = D / 16;
+  f32x16 acc = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  static_for<KK>([&](auto KI) {
+    constexpr int kk = decltype(KI)::value;
+    const int off = l32 * RB + (((2 * kk + h) ^ sx) << 4);
+    const V8 a = *reinterpret_cast<const V8*>(tile + 32 * t * RB + off);
+    const V8 b = *reinterpret_cast<const V8*>(held + off);
+    acc = mma(a, b, acc);
+  });
+  return acc;
+}
+
 // Per-lane parts of the transposing-read addresses (see the forward kernel).
 struct TrLane {
   int row, chunk, sub;
@@ -84,17 +102,15 @@ struct TrLane {
 
 // acc[dt][4 g + e] += sum over the 32 rows of tile block t of tile[row][32 dt + 8 g + 4 h + e] * w[row], where
 // w[8 (v / 4) + 4 h + v % 4] for v = 0..15 are the values this lane holds (rounded to T for the product).
+// The held values come rounded and packed: wf[st][jj] = w[8 st + jj].
 template <typename T, int D>
-__device__ __forceinline__ void transposed_times_held(const char* tile, int t, const TrLane& L, const f32x16& w, f32x16 (&acc)[D / 32]) {
+__device__ __forceinline__ void transposed_times_packed(const char* tile, int t, const TrLane& L, const typename Vec8<T>::type (&wfs)[2],
+                                                        f32x16 (&acc)[D / 32]) {
   typedef typename Vec8<T>::type V8;
   constexpr int RB = D * 2, DT = D / 32;
   static_for<2>([&](auto SI) {
     constexpr int st = decltype(SI)::value;
-    V8 wf;
-    static_for<8>([&](auto JI) {
-      constexpr int jj = decltype(JI)::value;
-      wf[jj] = (T)w[8 * st + jj];
-    });
+    const V8 wf = wfs[st];
     static_for<DT>([&](auto DI) {
       constexpr int dt = decltype(DI)::value;
       const int off0 = L.row * RB + (((4 * dt + L.chunk) ^ swz_v<D>(L.row)) << 4) + L.sub;
@@ -106,6 +122,16 @@ __device__ __forceinline__ void transposed_times_held(const char* tile, int t, c
       acc[dt] = mma(__builtin_bit_cast(V8, both), wf, acc[dt]);
     });
   });
+}
+
+template <typename T, int D>
+__device__ __forceinline__ void transposed_times_held(const char* tile, int t, const TrLane& L, const f32x16& w, f32x16 (&acc)[D / 32]) {
+  typename Vec8<T>::type wfs[2];
+  static_for<16>([&](auto VI) {
+    constexpr int v = decltype(VI)::value;
+    wfs[v / 8][v % 8] = (T)w[v];
+  });
+  transposed_times_packed<T, D>(tile, t, L, wfs, acc);
 }
 
 // Write acc^T (lane = row l32 of this wave's 32 rows, registers = columns) times `mul` as rows of D elements of T
@@ -272,11 +298,17 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
 }
 
 // ---------------------------------------------------------------------------------------------- dk, dv
+// Eight waves of 32 keys: two per SIMD, so one wave's exponentials run beside the other's MFMAs.  A lane's dk and
+// dv rows take 128 accumulation registers at D = 128; to stay within the 256 a lane may have at that occupancy only
+// the K row of the lane is held in registers, its V row is read from LDS (the workgroup's 256 V rows are loaded
+// once, each wave its own 32).
 template <typename T, int D>
-__global__ __launch_bounds__(kThreads) void sdpa_bwd_dkv_kernel(BwdParams p) {
+__global__ __launch_bounds__(64 * KW) __attribute__((amdgpu_waves_per_eu(2, 2))) void sdpa_bwd_dkv_kernel(BwdParams p) {
   typedef typename Vec8<T>::type V8;
-  constexpr int RB = D * 2, CH = RB / 16, TILE = BKV * RB, KK = D / 16, DT = D / 32, LPW = CH / 4;
+  constexpr int RB = D * 2, CH = RB / 16, TILE = BKV * RB, KK = D / 16, DT = D / 32, LPW = CH / KW;
+  static_assert(LPW * KW == CH, "tile loads must divide evenly over the waves");
   constexpr int STAGE = 2 * TILE + 1024;  // Q tile, dO tile, 64 log-sum-exps, 64 deltas
+  constexpr int V_ROWS = 2 * STAGE;       // byte offset of the V rows, behind the two stages
   extern __shared__ __attribute__((aligned(1024))) char smem[];
 
   const int tid = threadIdx.x, lane = tid & 63;
@@ -292,14 +324,30 @@ __global__ __launch_bounds__(kThreads) void sdpa_bwd_dkv_kernel(BwdParams p) {
   const int krow = k0 + 32 * wave + l32;
   const int kr = krow < p.Skv ? krow : p.Skv - 1;
 
-  V8 kf[KK], vf[KK];
+  V8 kf[KK];
   {
     const T* kg = reinterpret_cast<const T*>(p.k) + (int64_t)b * p.ks[0] + (int64_t)hkv * p.ks[1] + (int64_t)kr * p.ks[2];
-    const T* vg = reinterpret_cast<const T*>(p.v) + (int64_t)b * p.vs[0] + (int64_t)hkv * p.vs[1] + (int64_t)kr * p.vs[2];
     static_for<KK>([&](auto KI) {
       constexpr int kk = decltype(KI)::value;
       kf[kk] = *reinterpret_cast<const V8*>(kg + 16 * kk + 8 * h);
-      vf[kk] = *reinterpret_cast<const V8*>(vg + 16 * kk + 8 * h);
+    });
+  }
+  // this wave's 32 V rows into LDS, in the layout of a tile block (rows past the end repeat the last valid one);
+  // the wait and barrier of the first step cover them
+  char* v_rows = smem + V_ROWS + wave * (32 * RB);
+  {
+    const char* vb = reinterpret_cast<const char*>(p.v) + ((int64_t)b * p.vs[0] + (int64_t)hkv * p.vs[1]) * 2;
+    const uint32_t v_row_bytes = (uint32_t)(p.vs[2] * 2);
+    const int first = min(k0 + 32 * wave, p.Skv - 1);        // wave-uniform
+    const int n_valid = max(p.Skv - (k0 + 32 * wave), 1);    // rows of this block that exist (the clamped one at least)
+    const char* base = vb + (int64_t)first * v_row_bytes;
+    static_for<32 * RB / 1024>([&](auto I) {
+      constexpr int i = decltype(I)::value;
+      const int pos = i * 1024 + lane * 16;
+      const int row = pos / RB;
+      const int chunk = (((pos % RB) >> 4) ^ swz_v<D>(row)) << 4;
+      const uint32_t src_row = (uint32_t)min(row, n_valid - 1);
+      load_to_lds16(base, src_row * v_row_bytes + chunk, (uint32_t)(size_t)(lvoid*)(v_rows + i * 1024));
     });
   }
 
@@ -363,7 +411,9 @@ __global__ __launch_bounds__(kThreads) void sdpa_bwd_dkv_kernel(BwdParams p) {
     // in accumulation registers, and the moves that hand them to the vector ALU queue behind the MFMAs.)
     // only tiles that cross the diagonal or the end of the queries pay for the mask (wave-uniform)
     const bool need_mask = (p.causal && qt0 < kw_min + 31) || (qt0 + BKV > p.Sq);
-    auto soft = [&](auto TI, f32x16& s, const f32x16& dp, f32x16& pr, f32x16& ds) {
+    // the probabilities and score gradients leave `soft` rounded and packed, eight per 16-byte fragment: four
+    // registers each instead of sixteen, which is what lets two waves share a SIMD's register file
+    auto soft = [&](auto TI, f32x16& s, const f32x16& dp, V8 (&prf)[2], V8 (&dsf)[2]) {
       constexpr int t = decltype(TI)::value;
       float cc = c;
       if (need_mask) {
@@ -381,19 +431,24 @@ __global__ __launch_bounds__(kThreads) void sdpa_bwd_dkv_kernel(BwdParams p) {
         static_for<4>([&](auto EI) {
           constexpr int e = decltype(EI)::value;
           constexpr int v = 4 * g + e;
-          pr[v] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[v], cc, -l4[e] * kLog2e));
-          ds[v] = pr[v] * (dp[v] - d4[e]);
+          const float pr = __builtin_amdgcn_exp2f(__builtin_fmaf(s[v], cc, -l4[e] * kLog2e));
+          prf[v / 8][v % 8] = (T)pr;
+          dsf[v / 8][v % 8] = (T)(pr * (dp[v] - d4[e]));
         });
       });
     };
     static_for<2>([&](auto TI) {
       constexpr int t = decltype(TI)::value;
       f32x16 s = rows_times_regs<T, D>(q_s, t, l32, h, sx, kf);
-      const f32x16 dp = rows_times_regs<T, D>(do_s, t, l32, h, sx, vf);
-      f32x16 pr, ds;
-      soft(TI, s, dp, pr, ds);
-      transposed_times_held<T, D>(do_s, t, TL, pr, dv_acc);
-      transposed_times_held<T, D>(q_s, t, TL, ds, dk_acc);
+      const f32x16 dp = rows_times_rows<T, D>(do_s, t, l32, h, sx, v_rows);
+      V8 prf[2], dsf[2];
+      soft(TI, s, dp, prf, dsf);
+      // nothing of the products below is started before the fragments above exist, and the next sub-tile waits for
+      // this one: what is in flight at once has to fit the 256 registers of a lane
+      __builtin_amdgcn_sched_barrier(0);
+      transposed_times_packed<T, D>(do_s, t, TL, prf, dv_acc);
+      transposed_times_packed<T, D>(q_s, t, TL, dsf, dk_acc);
+      __builtin_amdgcn_sched_barrier(0);
     });
   };
 
@@ -415,14 +470,14 @@ __global__ __launch_bounds__(kThreads) void sdpa_bwd_dkv_kernel(BwdParams p) {
 template <typename T, int D>
 int launch_bwd(const BwdParams& p, hipStream_t stream) {
   constexpr int SMEM_DQ = 2 * 2 * BKV * D * 2;
-  constexpr int SMEM_DKV = 2 * (2 * BKV * D * 2 + 1024);
+  constexpr int SMEM_DKV = 2 * (2 * BKV * D * 2 + 1024) + BK * D * 2;
   auto dq_kernel = sdpa_bwd_dq_kernel<T, D>;
   auto dkv_kernel = sdpa_bwd_dkv_kernel<T, D>;
   if (int st = allow_dynamic_lds(reinterpret_cast<const void*>(dq_kernel), SMEM_DQ)) return st;
   if (int st = allow_dynamic_lds(reinterpret_cast<const void*>(dkv_kernel), SMEM_DKV)) return st;
   hipLaunchKernelGGL(dq_kernel, dim3((unsigned)((int64_t)p.B * p.H * p.n_qb)), dim3(kThreads), SMEM_DQ, stream, p);
   if (hipGetLastError() != hipSuccess) return XG_ERR_LAUNCH;
-  hipLaunchKernelGGL(dkv_kernel, dim3((unsigned)((int64_t)p.B * p.Hkv * p.n_kb)), dim3(kThreads), SMEM_DKV, stream, p);
+  hipLaunchKernelGGL(dkv_kernel, dim3((unsigned)((int64_t)p.B * p.Hkv * p.n_kb)), dim3(64 * KW), SMEM_DKV, stream, p);
   return status_from_hip(hipGetLastError());
 }
 
