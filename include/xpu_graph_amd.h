@@ -207,6 +207,20 @@ int xg_silu_mul2_bwd(const void* gate, const void* up, const void* gy, void* d_g
                      xg_stream_t stream);
 
 /* ---------------------------------------------------------------------------
+ * An activation on its own and its backward, for the dense layer of a training
+ * graph (the reference's FusedDenseLayer takes relu / gelu / silu / sigmoid,
+ * passes/patterns/structure/fuse_denselayer.py; in a differentiated graph the
+ * layer keeps its pre-activation z as eager does, so the backward is one pass
+ * over z and gy instead of a second product):
+ *   xg_activation:     y[i]  = act(x[i])
+ *   xg_activation_bwd: gz[i] = gy[i] * act'(z[i])
+ * n contiguous elements, fp32 math, one rounding; `act` one of XG_ACT_RELU,
+ * _GELU (erf form), _SILU, _SIGMOID (XG_ACT_NONE: XG_ERR_BAD_ARG).
+ * ------------------------------------------------------------------------- */
+int xg_activation(const void* x, void* y, int64_t n, int act, int dtype, xg_stream_t stream);
+int xg_activation_bwd(const void* z, const void* gy, void* gz, int64_t n, int act, int dtype, xg_stream_t stream);
+
+/* ---------------------------------------------------------------------------
  * Gated dense layer (SwiGLU): out[M, N] = silu(a w_gate^T) * (a w_up^T), both
  * weights [N, K] with unit K stride and row stride ldb, a [M, K] with row stride
  * lda, out contiguous [M, N]; bf16 or f16, fp32 accumulation; each projection is

@@ -19,7 +19,7 @@ def declared_symbols():
 def test_header_declares_the_expected_entry_points():
     syms = declared_symbols()
     for s in ("xg_rms_norm", "xg_layer_norm", "xg_add_rms_norm", "xg_add_layer_norm", "xg_rms_norm_bwd", "xg_layer_norm_bwd", "xg_slice_cat", "xg_addn",
-              "xg_combo_sum", "xg_slice_sum_cat", "xg_silu_mul", "xg_silu_mul2", "xg_silu_mul2_bwd", "xg_dense", "xg_dense_batched", "xg_dense_at", "xg_dense_glu", "xg_dense_glu_save", "xg_dense_fp8", "xg_slice_cat_check_table", "xg_sdpa", "xg_sdpa_masked", "xg_sdpa_lse", "xg_sdpa_backward", "xg_sdpa_backward_static", "xg_rope", "xg_copy_bytes",
+              "xg_combo_sum", "xg_slice_sum_cat", "xg_silu_mul", "xg_silu_mul2", "xg_silu_mul2_bwd", "xg_activation", "xg_activation_bwd", "xg_dense", "xg_dense_batched", "xg_dense_at", "xg_dense_glu", "xg_dense_glu_save", "xg_dense_fp8", "xg_slice_cat_check_table", "xg_sdpa", "xg_sdpa_masked", "xg_sdpa_lse", "xg_sdpa_backward", "xg_sdpa_backward_static", "xg_rope", "xg_copy_bytes",
               "xg_version", "xg_status_string"):
         assert s in syms
 

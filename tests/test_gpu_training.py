@@ -195,6 +195,31 @@ def test_dense_backward_formula(device, act, weight_trans):
         assert (a.float() - c).abs().mean().item() <= 2e-2 * scale + 1e-3, (name, (a.float() - c).abs().mean().item(), scale)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("act", ["relu", "gelu", "silu", "sigmoid"])
+@pytest.mark.parametrize("shape", [(256, 512), (3, 5, 7), (1,), (4096, 1376)])
+def test_activation_kernel_and_its_backward(device, dtype, act, shape):
+    """xg_activation / xg_activation_bwd against float64 autograd of the same activation: fp32 math on the stored
+    values, one rounding."""
+    import xpu_graph_amd.ops  # noqa: F401
+
+    gen = torch.Generator().manual_seed(len(shape) + shape[0])
+    z = (2 * torch.randn(*shape, generator=gen)).to(dtype).to(device)
+    gy = torch.randn(*shape, generator=gen).to(dtype).to(device)
+    fn = {"relu": torch.relu, "gelu": F.gelu, "silu": F.silu, "sigmoid": torch.sigmoid}[act]
+    z64 = z.double().requires_grad_(True)
+    want_y = fn(z64)
+    (want_g,) = torch.autograd.grad(want_y, z64, gy.double())
+    y = torch.ops.xpu_ops.act(z, act)
+    gz = torch.ops.xpu_ops.act_bwd(z, gy, act)
+    ulp = {torch.float32: 2.0**-23, torch.bfloat16: 2.0**-8, torch.float16: 2.0**-11}[dtype]
+    assert y.shape == z.shape and y.dtype == dtype and gz.shape == z.shape and gz.dtype == dtype
+    # the hardware exp2 / reciprocal are good to about an ulp of fp32 each; near a zero of the result their error
+    # shows against the size of the terms that cancel
+    torch.testing.assert_close(y.double(), want_y.detach(), rtol=1.01 * ulp + 4e-7, atol=1e-6)
+    torch.testing.assert_close(gz.double(), want_g, rtol=1.01 * ulp + 4e-7, atol=2e-6 * max(1.0, gy.abs().max().item()))
+
+
 def test_mlp_training_step(device):
     """RMSNorm -> linear + bias -> SiLU -> linear, compiled for training on the mi355x target: the forward graph
     calls the HIP norm and dense kernels, loss and gradients follow eager."""
@@ -214,6 +239,11 @@ def test_mlp_training_step(device):
     fwd_ops = [str(n.target) for n in be.compiled_graphs[1].graph.nodes if n.op == "call_function"]
     assert fwd_ops.count("xpu_ops.dense.default") == 2 and "xpu_ops.rms_norm.default" in fwd_ops
     assert not any("aten.mm" in t or "aten.addmm" in t for t in fwd_ops)
+    # the activated layer of a differentiated graph keeps its pre-activation: activation and its backward are one
+    # pass each, and the backward runs no product beyond the input- and weight-gradient ones
+    bwd_ops = [str(n.target) for n in be.compiled_graphs[2].graph.nodes if n.op == "call_function"]
+    assert fwd_ops.count("xpu_ops.act.default") == 1 and bwd_ops.count("xpu_ops.act_bwd.default") == 1, (fwd_ops, bwd_ops)
+    assert bwd_ops.count("xpu_ops.dense.default") == 2 and not any("aten.sigmoid" in t or "aten.silu" in t for t in bwd_ops), bwd_ops
     ref_args = [a.detach().float().requires_grad_(True) for a in args]
     loss1 = mlp(*ref_args).pow(2).mean()
     g1 = torch.autograd.grad(loss1, ref_args)

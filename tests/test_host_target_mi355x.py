@@ -421,6 +421,21 @@ def test_llama_block_graph_has_no_layout_copies(backend):
         assert not any(k in t for t in left for k in ("clone", "cat", "neg", "cos", "sin", "arange", "softmax", "aten.mm", "aten.bmm")), left
 
 
+def test_activation_behind_the_reshape_of_a_linear_layer_joins_the_dense_call(backend):
+    """A linear layer on [B, S, H] input is view -> addmm -> view; the activation that follows commutes with the view
+    and goes into the dense epilogue."""
+
+    def fn(x, w, b):
+        return F.silu(F.linear(x, w, b)) + 1
+
+    gm = rewrite(backend, fn, torch.randn(2, 8, 128).to(bf16), torch.randn(96, 128).to(bf16), torch.randn(96).to(bf16))
+    assert modules_called(gm) == ["custom_dense_layer_replacement"]
+    call = next(n for n in gm.graph.nodes if n.op == "call_module")
+    assert call.args[4] == "silu" and not any("silu" in t for t in aten_ops(gm))
+    out = next(n for n in gm.graph.nodes if n.op == "output").args[0][0]
+    assert tuple(out.meta["val"].shape) == (2, 8, 96)
+
+
 def test_gate_and_up_projections_become_one_gated_dense(caplog, backend):
     def mlp(x, wg, wu):
         return F.silu(F.linear(x, wg)) * F.linear(x, wu)

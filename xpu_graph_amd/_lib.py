@@ -84,6 +84,8 @@ _SIGNATURES = {
         [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p] + [c_int64] * 12 + [c_int, c_int, c_int, c_int, c_void_p],
     ),
     "xg_silu_mul2_bwd": (c_int, [c_void_p] * 5 + [c_int64, c_int, c_void_p]),
+    "xg_activation": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_int, c_void_p]),
+    "xg_activation_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int, c_void_p]),
     "xg_dense_glu_save": (c_int, [c_void_p] * 6 + [c_int64] * 5 + [c_int, c_void_p]),
     "xg_dense_at": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p] + [c_int64] * 6 + [c_int, c_void_p]),
     "xg_dense_fp8": (

@@ -128,6 +128,16 @@ def _silu_mul2_backward(ctx, gy):
     return torch.ops.xpu_ops.silu_mul2_bwd(g, u, gy.to(g.dtype))
 
 
+def _act_setup(ctx, inputs, output):
+    ctx.save_for_backward(inputs[0])
+    ctx.act = inputs[1]
+
+
+def _act_backward(ctx, gy):
+    (z,) = ctx.saved_tensors
+    return torch.ops.xpu_ops.act_bwd(z, gy.to(z.dtype), ctx.act), None
+
+
 def _silu_mul_setup(ctx, inputs, output):
     ctx.save_for_backward(inputs[0])
 
@@ -163,23 +173,19 @@ def _dense_backward(ctx, gy):
     bias = rest.pop(0) if ctx.has_bias else None
     residual = rest.pop(0) if ctx.has_res else None
     act = ctx.act
-    gf = gy if act == "none" else gy.float()  # no activation: the upstream gradient is the pre-activation's, as it is
     if act == "none":
-        gz = gf
+        gz = gy  # the upstream gradient is the pre-activation's, as it is
     elif act == "relu":
-        gz = gf * (y > 0)
+        gz = gy.float() * (y > 0)
     elif act == "sigmoid":
         yf = y.float()
-        gz = gf * yf * (1 - yf)
+        gz = gy.float() * yf * (1 - yf)
+    elif act in ("silu", "gelu"):
+        # the pre-activation is not kept by the fused call: one more product, then one pass over it and gy
+        z = torch.ops.xpu_ops.dense(x, weight, ctx.trans, bias, residual, "none")
+        gz = torch.ops.xpu_ops.act_bwd(z, gy.to(z.dtype), act)
     else:
-        z = torch.ops.xpu_ops.dense(x, weight, ctx.trans, bias, residual, "none").float()
-        if act == "silu":
-            gz = gf * _silu_grad(z)
-        elif act == "gelu":
-            cdf = 0.5 * (1 + torch.erf(z * 0.7071067811865476))
-            gz = gf * (cdf + z * torch.exp(-0.5 * z * z) * 0.3989422804014327)
-        else:
-            raise NotImplementedError(f"dense backward: activation {act!r}")
+        raise NotImplementedError(f"dense backward: activation {act!r}")
     gz = gz.to(x.dtype)
     need = ctx.needs_input_grad
     gx = torch.ops.xpu_ops.dense(gz, weight, not ctx.trans, None, None, "none") if need[0] else None
@@ -338,6 +344,7 @@ def register():
     reg("xpu_ops::rms_norm", _rms_backward, setup_context=_rms_setup)
     reg("xpu_ops::layer_norm", _ln_backward, setup_context=_ln_setup)
     reg("xpu_ops::silu_mul2", _silu_mul2_backward, setup_context=_silu_mul2_setup)
+    reg("xpu_ops::act", _act_backward, setup_context=_act_setup)
     reg("xpu_ops::silu_mul", _silu_mul_backward, setup_context=_silu_mul_setup)
     reg("xpu_ops::dense", _dense_backward, setup_context=_dense_setup)
     reg("xpu_ops::dense_glu", _dense_glu_backward, setup_context=_dense_glu_setup)
@@ -351,7 +358,7 @@ def register():
         reg(f"xpu_ops::{op}", backward, setup_context=setup)
     # An op that was traced before (an inference compile earlier in the process) has its dispatch decisions cached
     # on the Python side; a stale entry for the Autograd key would keep sending traces to the "no formula" fallback.
-    for name in ("rms_norm", "layer_norm", "silu_mul2", "silu_mul", "dense", "dense_glu", "dense_glu_save", "rope", "sdpa", "sdpa_lse",
+    for name in ("rms_norm", "layer_norm", "silu_mul2", "silu_mul", "act", "dense", "dense_glu", "dense_glu_save", "rope", "sdpa", "sdpa_lse",
                  "add_rms_norm", "add_rms_norm_only", "add_layer_norm", "add_layer_norm_only"):
         packet = getattr(torch.ops.xpu_ops, name)
         for overload in packet.overloads():

@@ -110,6 +110,100 @@ int silu_mul_bwd_typed(const void* gate, const void* up, const void* gy, void* d
   return status_from_hip(hipGetLastError());
 }
 
+// An activation on its own, and its backward: y = act(x);  gz = gy * act'(z).  The dense layer of a differentiated graph
+// keeps its pre-activation z (as eager does) and applies the activation with this kernel, so the backward is one pass
+// over z and gy instead of a second product.  fp32 math, one rounding; the same formulas as the dense epilogue.
+template <int ACT>
+__device__ __forceinline__ float act_f32(float t) {
+  if constexpr (ACT == XG_ACT_RELU) return fmaxf(t, 0.f);
+  if constexpr (ACT == XG_ACT_GELU) return 0.5f * t * (1.f + erff(t * 0.70710678118654752f));
+  if constexpr (ACT == XG_ACT_SILU) return silu_f32(t);
+  if constexpr (ACT == XG_ACT_SIGMOID) return sigmoid_f32(t);
+  return t;
+}
+template <int ACT>
+__device__ __forceinline__ float act_grad_f32(float t) {
+  if constexpr (ACT == XG_ACT_RELU) return t > 0.f ? 1.f : 0.f;
+  if constexpr (ACT == XG_ACT_GELU)
+    return 0.5f * (1.f + erff(t * 0.70710678118654752f)) + t * __expf(-0.5f * t * t) * 0.39894228040143268f;
+  if constexpr (ACT == XG_ACT_SILU) {
+    const float sg = sigmoid_f32(t);
+    return sg * (1.f + t * (1.f - sg));
+  }
+  if constexpr (ACT == XG_ACT_SIGMOID) {
+    const float sg = sigmoid_f32(t);
+    return sg * (1.f - sg);
+  }
+  return 1.f;
+}
+
+template <typename T, int VW, int ACT, bool BWD>
+__global__ __launch_bounds__(256) void act_kernel(const T* __restrict__ z, const T* __restrict__ gy, T* __restrict__ out, int64_t nvec) {
+  typedef T VT __attribute__((ext_vector_type(VW)));
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= nvec) return;
+  const VT zv = __builtin_nontemporal_load(reinterpret_cast<const VT*>(z) + i);
+  VT o;
+  if constexpr (BWD) {
+    const VT g = __builtin_nontemporal_load(reinterpret_cast<const VT*>(gy) + i);
+#pragma unroll
+    for (int j = 0; j < VW; ++j) o[j] = from_f32<T>(to_f32(g[j]) * act_grad_f32<ACT>(to_f32(zv[j])));
+  } else {
+#pragma unroll
+    for (int j = 0; j < VW; ++j) o[j] = from_f32<T>(act_f32<ACT>(to_f32(zv[j])));
+  }
+  __builtin_nontemporal_store(o, reinterpret_cast<VT*>(out) + i);
+}
+
+template <typename T, int ACT, bool BWD>
+int act_launch(const void* z, const void* gy, void* out, int64_t n, hipStream_t stream) {
+  constexpr int VN = VecOf<T>::N;
+  const bool vec_ok = n % VN == 0 && aligned_to(z, 16) && aligned_to(out, 16) && (!BWD || aligned_to(gy, 16));
+  const int64_t work = vec_ok ? n / VN : n;
+  const int64_t blocks = (work + 255) / 256;
+  if (blocks > 0x7fffffffLL) return XG_ERR_TOO_LARGE;
+  if (vec_ok)
+    hipLaunchKernelGGL((act_kernel<T, VN, ACT, BWD>), dim3((unsigned)blocks), dim3(256), 0, stream, (const T*)z, (const T*)gy, (T*)out, work);
+  else
+    hipLaunchKernelGGL((act_kernel<T, 1, ACT, BWD>), dim3((unsigned)blocks), dim3(256), 0, stream, (const T*)z, (const T*)gy, (T*)out, work);
+  return status_from_hip(hipGetLastError());
+}
+
+template <typename T, bool BWD>
+int act_typed(const void* z, const void* gy, void* out, int64_t n, int act, hipStream_t stream) {
+  switch (act) {
+    case XG_ACT_RELU:
+      return act_launch<T, XG_ACT_RELU, BWD>(z, gy, out, n, stream);
+    case XG_ACT_GELU:
+      return act_launch<T, XG_ACT_GELU, BWD>(z, gy, out, n, stream);
+    case XG_ACT_SILU:
+      return act_launch<T, XG_ACT_SILU, BWD>(z, gy, out, n, stream);
+    case XG_ACT_SIGMOID:
+      return act_launch<T, XG_ACT_SIGMOID, BWD>(z, gy, out, n, stream);
+    default:
+      return XG_ERR_BAD_ARG;  // "none" has nothing to compute
+  }
+}
+
+template <bool BWD>
+int act_entry(const void* z, const void* gy, void* out, int64_t n, int act, int dtype, xg_stream_t stream) {
+  if (!z || !out || (BWD && !gy)) return XG_ERR_NULL_PTR;
+  if (n < 0) return XG_ERR_BAD_SHAPE;
+  if (n == 0) return XG_OK;
+  const size_t esz = dtype == XG_F32 ? 4 : 2;
+  if (!aligned_to(z, esz) || !aligned_to(out, esz) || (BWD && !aligned_to(gy, esz))) return XG_ERR_BAD_ALIGN;
+  switch (dtype) {
+    case XG_F32:
+      return act_typed<float, BWD>(z, gy, out, n, act, (hipStream_t)stream);
+    case XG_BF16:
+      return act_typed<bf16_t, BWD>(z, gy, out, n, act, (hipStream_t)stream);
+    case XG_F16:
+      return act_typed<f16_t, BWD>(z, gy, out, n, act, (hipStream_t)stream);
+    default:
+      return XG_ERR_BAD_DTYPE;
+  }
+}
+
 __global__ __launch_bounds__(256) void copy_kernel(const u32x4* __restrict__ src, u32x4* __restrict__ dst, int64_t n) {
   const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (i < n) __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
@@ -153,6 +247,14 @@ int xg_silu_mul2_bwd(const void* gate, const void* up, const void* gy, void* d_g
     default:
       return XG_ERR_BAD_DTYPE;
   }
+}
+
+int xg_activation(const void* x, void* y, int64_t n, int act, int dtype, xg_stream_t stream) {
+  return xg::act_entry<false>(x, nullptr, y, n, act, dtype, stream);
+}
+
+int xg_activation_bwd(const void* z, const void* gy, void* gz, int64_t n, int act, int dtype, xg_stream_t stream) {
+  return xg::act_entry<true>(z, gy, gz, n, act, dtype, stream);
 }
 
 int xg_copy_bytes(const void* src, void* dst, int64_t bytes, xg_stream_t stream) {

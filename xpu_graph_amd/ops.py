@@ -40,6 +40,8 @@ _SCHEMAS = [
     "silu_mul(Tensor x) -> Tensor",
     "silu_mul2(Tensor gate, Tensor up) -> Tensor",
     "silu_mul2_bwd(Tensor gate, Tensor up, Tensor gy) -> (Tensor, Tensor)",
+    "act(Tensor x, str act) -> Tensor",
+    "act_bwd(Tensor z, Tensor gy, str act) -> Tensor",
 ]
 for _s in _SCHEMAS:
     _library.define(_s)
@@ -505,6 +507,39 @@ def _silu_mul2_bwd(gate, up, gy):
     return d_gate, d_up
 
 
+def _act_code(act):
+    code = _lib.ACT_CODES.get(act)
+    if not code:
+        raise ValueError(f"act: unknown activation {act!r} (relu, gelu, silu, sigmoid)")
+    return code
+
+
+def _act(x, act):
+    """An activation of the dense layer on its own (what the layer of a differentiated graph runs after its product)."""
+    code = _act_code(act)
+    x = x.contiguous()
+    y = torch.empty_like(x)
+    if x.numel():
+        _lib.check(_lib.lib().xg_activation(_ptr(x), _ptr(y), x.numel(), code, _code(x.dtype), _stream()), "xg_activation")
+    return y
+
+
+def _act_bwd(z, gy, act):
+    """gy * act'(z) in one pass."""
+    code = _act_code(act)
+    if z.shape != gy.shape or z.dtype != gy.dtype:
+        raise ValueError("act_bwd: z and gy must match in shape and dtype")
+    z, gy = z.contiguous(), gy.contiguous()
+    gz = torch.empty_like(z)
+    if z.numel():
+        _lib.check(_lib.lib().xg_activation_bwd(_ptr(z), _ptr(gy), _ptr(gz), z.numel(), code, _code(z.dtype), _stream()), "xg_activation_bwd")
+    return gz
+
+
+_library.impl("act", _act, "CUDA")
+_library.impl("act", lambda x, act: _like(x), "Meta")
+_library.impl("act_bwd", _act_bwd, "CUDA")
+_library.impl("act_bwd", lambda z, gy, act: _like(z), "Meta")
 _library.impl("silu_mul", _silu_mul, "CUDA")
 _library.impl("silu_mul2", _silu_mul2, "CUDA")
 _library.impl("silu_mul2_bwd", _silu_mul2_bwd, "CUDA")

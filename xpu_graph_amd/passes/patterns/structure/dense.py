@@ -9,19 +9,25 @@ from torch import fx
 from ....config import OptLevel
 from ....fx_utils import FxStage
 from ..pattern import Pattern
-from ..utils.node_utils import activation_name, arg, aten, is_call, mm_operands, sole_user_is, strip_transpose
+from ..utils.node_utils import VIEW_OPS, activation_name, arg, aten, is_call, mm_operands, sole_user_is, strip_transpose
 
 DENSE_NAME = "custom_dense_layer_replacement"
 
 
 def match_dense(node):
+    """([x, w, trans, bias, act], product node, reshape node | None): an activation applied to the product directly,
+    or to one reshape of it (a linear layer on [B, S, H] input is view -> addmm -> view -> activation; an elementwise
+    activation commutes with the view, which is then re-applied to the fused result)."""
     act = activation_name(node)
+    view = None
     if act is None:
         act, lin = "none", node
     else:
         lin = node.args[0]
         if not isinstance(lin, fx.Node) or not sole_user_is(lin, node):
             return None
+        if is_call(lin, *VIEW_OPS) and isinstance(lin.args[0], fx.Node) and sole_user_is(lin.args[0], lin):
+            view, lin = lin, lin.args[0]
     ops = mm_operands(lin) if isinstance(lin, fx.Node) else None
     if ops is not None:
         x, w, bias = ops[0], ops[1], None
@@ -32,7 +38,7 @@ def match_dense(node):
     else:
         return None
     trans, w = strip_transpose(w)
-    return [x, w, trans, bias, act], lin
+    return [x, w, trans, bias, act], lin, view
 
 
 class CustomDenseLayer(Pattern):
@@ -54,13 +60,17 @@ class CustomDenseLayer(Pattern):
             m = match_dense(node)
             if m is None:
                 continue
-            params, lin = m
+            params, lin, view = m
             if not self.constraint_fn(*fx.map_arg(params, lambda n: n.meta["val"])):
                 continue
             with g.inserting_before(node):
                 new = g.call_module(DENSE_NAME, tuple(params))
+                if view is not None:
+                    new = g.call_function(view.target, (new,) + tuple(view.args[1:]), dict(view.kwargs))
             node.replace_all_uses_with(new)
             g.erase_node(node)
+            if view is not None:
+                g.erase_node(view)
             if lin is not node:
                 g.erase_node(lin)
             changed = True

@@ -1,7 +1,10 @@
 """silu(x Wg^T) * (x Wu^T): two dense calls and the SwiGLU gate -> one gated dense kernel.
 
     silu_mul2(reshape?(dense(x, Wg, True, None, "none")), reshape?(dense(x, Wu, True, None, "none")))
+    mul(reshape?(dense(x, Wg, True, None, "silu")), reshape?(dense(x, Wu, True, None, "none")))
         ->  reshape?(dense_glu(x, Wg, Wu))
+
+(the second spelling is what is left when the dense pattern has already taken the SiLU into the gate projection)
 
 Both projections read the same activations, both weights are [N, K] (torch.nn.Linear layout) of one shape, and each
 dense result (and its reshape) has no other user.  The kernel computes both projections in one workgroup -- the A
@@ -31,8 +34,9 @@ class DenseGLUModule(nn.Module):
         return torch.ops.xpu_ops.dense_glu(x, w_gate, w_up)
 
 
-def _plain_dense(node):
-    """(dense call, reshape or None) for `dense` or `reshape(dense)` with single users, no bias, no activation, [N, K] weight."""
+def _plain_dense(node, want_act="none"):
+    """(dense call, reshape or None) for `dense` or `reshape(dense)` with single users, no bias, [N, K] weight and the
+    activation `want_act`."""
     view = None
     if is_call(node, *VIEW_OPS) and len(node.users) == 1:
         view, node = node, node.args[0]
@@ -41,9 +45,26 @@ def _plain_dense(node):
     if len(node.args) != 5 or node.kwargs:
         return None, None
     _, _, weight_trans, bias, act = node.args
-    if weight_trans is not True or bias is not None or act != "none":
+    if weight_trans is not True or bias is not None or act != want_act:
         return None, None
     return node, view
+
+
+def _gate_and_up(node):
+    """((gate dense, its reshape), (up dense, its reshape)) for the two spellings of the gated product: the SwiGLU
+    module over two plain projections, or a multiplication whose one factor is a projection that already took the
+    SiLU into its epilogue."""
+    none = ((None, None), (None, None))
+    if node.op == "call_module" and node.target == SILU_MUL2 and len(node.args) == 2:
+        return _plain_dense(node.args[0]), _plain_dense(node.args[1])
+    if is_call(node, aten.mul.Tensor) and len(node.args) == 2 and all(isinstance(a, fx.Node) for a in node.args):
+        for a, b in (node.args, node.args[::-1]):
+            gate, up = _plain_dense(a, "silu"), _plain_dense(b)
+            if gate[0] is not None and up[0] is not None:
+                va, vb, vo = (n.meta.get("val") for n in (a, b, node))
+                if all(isinstance(v, torch.Tensor) for v in (va, vb, vo)) and va.shape == vb.shape == vo.shape and va.dtype == vb.dtype == vo.dtype:
+                    return gate, up
+    return none
 
 
 class FusedDenseGLU(Pattern):
@@ -57,9 +78,7 @@ class FusedDenseGLU(Pattern):
         g = gm.graph
         changed = False
         for node in list(g.nodes):
-            if not (node.op == "call_module" and node.target == SILU_MUL2 and len(node.args) == 2):
-                continue
-            (dg, vg), (du, vu) = _plain_dense(node.args[0]), _plain_dense(node.args[1])
+            (dg, vg), (du, vu) = _gate_and_up(node)
             if dg is None or du is None or dg is du or dg.args[0] is not du.args[0]:
                 continue
             x, wg, wu = dg.args[0], dg.args[1], du.args[1]

@@ -143,6 +143,13 @@ class DenseLayerModule(torch.nn.Module):
             else:
                 residual = bias if tuple(bias.shape) == (m, n) else bias.broadcast_to((m, n)).contiguous()
                 bias = None
+        if act != "none" and torch.is_grad_enabled() and any(
+            t is not None and t.requires_grad for t in (inputs, weight, bias, residual)
+        ):
+            # a graph that will be differentiated keeps the pre-activation, as eager does: the backward is then one
+            # pass over it (xpu_ops::act_bwd) instead of a second product and a chain of fp32 Aten formulas
+            z = torch.ops.xpu_ops.dense(inputs, weight, weight_trans, bias, residual, "none")
+            return torch.ops.xpu_ops.act(z, act)
         return torch.ops.xpu_ops.dense(inputs, weight, weight_trans, bias, residual, act)
 
 
