@@ -19,7 +19,8 @@ runs for at least WARM_SECONDS (the first ~100 ms of work after an idle spell,
 e.g. after a CPU baseline, run visibly slower), then the --warmup launches,
 then the timed ones.  `roofline.traffic` is not measured by this run: it is
 read from profiles/traffic.json, which the rocprofv3 --pmc recipe printed in
-that file produces, and `roofline.traffic_source` names it.
+that file produces, and the top-level `traffic_source` names it (once for every
+workload of the line).
 """
 import argparse
 import ctypes
@@ -308,7 +309,7 @@ class DenseC4(Workload):
     bound = "mfma"
     dtype = "bf16"
     unit = "TFLOP/s"
-    kernel = "gemm_dma_split_kernel<bf16,[K,N] weight> (256x256 tiles + 128x256 tiles for the last partial round)"
+    kernel = "gemm_dma_split_kernel<bf16,[K,N]>"
     work = 2 * 8192 * 4096 * 11008
     traffic_key = "c4_dense_bf16"
     n_sets = 3
@@ -347,11 +348,11 @@ class DenseC4(Workload):
 
 
 class DenseFp32(Workload):
-    name = "dense + bias + SiLU fp32 M4096 K4096 N4096 (the dtype of the reference's dense-layer tests)"
+    name = "dense + bias + SiLU fp32 M4096 K4096 N4096"
     bound = "mfma"
     dtype = "f32"
     unit = "TFLOP/s"
-    kernel = "gemm_dma_kernel<f32,[K,N] weight> (32x32x2 fp32 MFMA)"
+    kernel = "gemm_dma_kernel<f32,[K,N]>"
     work = 2 * 4096 * 4096 * 4096
     traffic_key = None
     n_sets = 3
@@ -390,9 +391,9 @@ class DenseFp32(Workload):
 
 
 class DenseFp8C4(DenseC4):
-    name = "C4 dense + bias + SiLU fp8 e4m3 (per-tensor x, per-channel W) M8192 K4096 N11008"
+    name = "C4 dense + bias + SiLU fp8 e4m3 M8192 K4096 N11008"
     dtype = "fp8"
-    kernel = "gemm_dma_split_kernel<e4m3,[N,K] weight>"
+    kernel = "gemm_dma_split_kernel<e4m3,[N,K]>"
     traffic_key = "c4_dense_fp8"
 
     def setup(self, torch, dev):
@@ -439,11 +440,11 @@ class DenseFp8C4(DenseC4):
 
 
 class DenseGluC5(Workload):
-    name = "C5 MLP gate+up: silu(x Wg^T) * (x Wu^T) bf16 M8192 K4096 N11008 (gated dense, one kernel)"
+    name = "C5 MLP gate+up gated dense bf16 M8192 K4096 N11008"
     bound = "mfma"
     dtype = "bf16"
     unit = "TFLOP/s"
-    kernel = "gemm_glu_kernel<bf16> (256x128 output tiles: gate and up accumulators side by side, SwiGLU in the epilogue)"
+    kernel = "gemm_glu_kernel<bf16>"
     work = 4 * 8192 * 4096 * 11008
     traffic_key = "c5_dense_glu"
     n_sets = 3
@@ -538,11 +539,11 @@ class SdpaC5(Workload):
 
 
 class SdpaBackwardC5(Workload):
-    name = "C5 causal attention backward bf16 B4 H32 S2048 D128 (dq, dk, dv from the saved row log-sum-exps)"
+    name = "C5 causal attention backward bf16 B4 H32 S2048 D128"
     bound = "mfma"
     dtype = "bf16"
     unit = "TFLOP/s"
-    kernel = "sdpa_bwd_dq_kernel<bf16,128> + sdpa_bwd_dkv_kernel<bf16,128> (two launches, timed together)"
+    kernel = "sdpa_bwd_dq_kernel + sdpa_bwd_dkv_kernel"
     work = 10 * 4 * 32 * 2048 * 2048 * 128 // 2  # five matmuls (S, dP, dV, dK, dQ), lower triangle only
     cpu_work = work // 4  # the CPU leg runs one of the four batch entries
     traffic_key = None
@@ -602,11 +603,11 @@ class SdpaBackwardC5(Workload):
 
 
 class DenseWeightGradC4(Workload):
-    name = "C4 dense weight gradient bf16: x[8192,4096]^T @ g[8192,11008] (transposed left operand)"
+    name = "C4 dense weight gradient bf16 x[8192,4096]^T g[8192,11008]"
     bound = "mfma"
     dtype = "bf16"
     unit = "TFLOP/s"
-    kernel = "gemm_dma_kernel<bf16,[K,N] right operand,[K,M] left operand>"
+    kernel = "gemm_dma_kernel<bf16,[K,N],A[K,M]>"
     work = 2 * 8192 * 4096 * 11008
     traffic_key = "c4_dense_at"
     n_sets = 3
@@ -645,11 +646,11 @@ class DenseWeightGradC4(Workload):
 
 
 class LlamaBlockC5(Workload):
-    name = "C5 Llama decoder block bf16 B4 S2048 hidden4096 H32 inter11008, torch.compile(mi355x) end to end"
+    name = "C5 Llama decoder block bf16 B4 S2048 compiled"
     bound = "mfma"
     dtype = "bf16"
     unit = "TFLOP/s"
-    kernel = "whole compiled block (5 dense + 1 gated dense, attention, 2 rotary, 2 norm kernels)"
+    kernel = "compiled block"
     traffic_key = None
     work = 2 * 8192 * (4 * 4096 * 4096 + 3 * 4096 * 11008) + 4 * 4 * 32 * 2048 * 2048 * 128 // 2
     n_sets = 1
@@ -698,8 +699,8 @@ class LlamaBlockC5(Workload):
 
 
 class LlamaBlockTrainC5(LlamaBlockC5):
-    name = "C5 Llama decoder block bf16 B4 S2048 training step (forward + backward), torch.compile(mi355x, is_training) end to end"
-    kernel = "whole compiled training step (dense / gated dense and their input- and weight-gradient launches, attention forward with row statistics, the two attention backward kernels, rotary, norms and their backward, gate backward; Aten for the residual and gradient sums)"
+    name = "C5 Llama decoder block bf16 B4 S2048 compiled training step"
+    kernel = "compiled training step"
     work = 3 * LlamaBlockC5.work  # one forward, two products per forward product in the backward
     cpu_work = work // 4            # the CPU leg runs one of the four batch entries
     cpu_warmups = 0
@@ -841,7 +842,6 @@ def run_workload(torch, dev, wl, steps, warmup, with_cpu=True):
     n_sets = getattr(wl, "n_sets", N_SETS)
     entry = _traffic_table().get(getattr(wl, "traffic_key", None) or "", None)
     traffic = entry["bytes_per_launch"] if entry else None
-    traffic_source = f"profiles/traffic.json ({entry['from']})" if entry else None
     t_op = _wall_time(torch, wl.op_call, n_sets, steps, warmup)
     t_k = _events_time(torch, wl.abi_call, n_sets, max(steps, 100), max(warmup, 20))
     res = {
@@ -859,7 +859,6 @@ def run_workload(torch, dev, wl, steps, warmup, with_cpu=True):
             "frac": wl.work / t_k / scale / peak,
             "kernel_us": t_k * 1e6,
             "traffic": traffic,
-            "traffic_source": traffic_source,
         },
     }
     if with_cpu:
@@ -871,11 +870,23 @@ def run_workload(torch, dev, wl, steps, warmup, with_cpu=True):
             "cores": torch.get_num_threads(),
             "host_cpu_count": os.cpu_count(),
             "kind": "port",
-            "sample": f"{n} timed runs of {'a bounded sample of the workload' if hasattr(wl, 'cpu_work') else 'the full-size workload'} through {how}, median {t_cpu * 1e3:.2f} ms",
+            "sample": f"{'bounded sample' if hasattr(wl, 'cpu_work') else 'full size'}, {n} runs, median {t_cpu * 1e3:.1f} ms",
         }
+        print(f"[bench] cpu baseline of {wl.name}: {how}", file=sys.stderr)
     if hasattr(wl, "eager_ms"):
         res["eager_gpu_ms"] = wl.eager_ms
     return res
+
+
+def _rounded(obj):
+    """Floats to six significant digits: the line is read by people and by a log tail of bounded length."""
+    if isinstance(obj, float):
+        return float(f"{obj:.6g}")
+    if isinstance(obj, dict):
+        return {k: _rounded(v) for k, v in obj.items()}
+    if isinstance(obj, (list, tuple)):
+        return [_rounded(v) for v in obj]
+    return obj
 
 
 def main():
@@ -943,7 +954,10 @@ def main():
             del wl
             torch.cuda.empty_cache()
     out["configs"] = others
-    print(json.dumps(out))
+    entries = [e for e in _traffic_table().values() if e.get("from")]
+    # said once for every roofline.traffic in the line (the whole line has to stay well under the 16 000 characters a log tail keeps)
+    out["traffic_source"] = f"profiles/traffic.json ({entries[0]['from']})" if entries else None
+    print(json.dumps(_rounded(out), separators=(",", ":")))
 
 
 if __name__ == "__main__":

@@ -361,7 +361,10 @@ int xg_sdpa_backward(const void* q, const void* k, const void* v, const void* ou
  * delta workspace is an 8 MiB array that lives in the library's device image,
  * one per GPU, from load until the process ends: B * H * Sq must not exceed
  * 2 097 152 query rows (XG_ERR_TOO_LARGE beyond that: use xg_sdpa_backward).
- * The call allocates and frees nothing.  Every call on a GPU uses that GPU's
+ * The call allocates and frees nothing.  The first call on a GPU also looks
+ * up the array's device address and raises the kernels' LDS limit (host-side
+ * set-up, no stream work): make it outside a stream capture; every later call
+ * on that GPU only enqueues the two kernels.  Every call on a GPU uses that GPU's
  * one array: calls that overlap in time on the same GPU (different streams)
  * race; calls on one stream are ordered and need nothing cleared in between
  * (each call writes every row of the workspace that it later reads).

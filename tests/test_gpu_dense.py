@@ -187,6 +187,38 @@ def test_dense_batched_is_one_launch_equal_to_the_per_entry_path(device, dtype, 
             close(got[i], ref32(x[i], w[i], weight_trans, bi, ri, act), K)
 
 
+def test_dense_batched_beyond_one_launch(device, monkeypatch):
+    """More batch entries than one launch holds (the batch is the second grid axis: 65535) go out in slices with every
+    operand moved on by its batch stride: a real batch of 65540 tiny layers, and a small batch with the limit lowered so
+    that per-entry bias, residual and strided views cross several slice boundaries."""
+    import xpu_graph_amd.ops as xops
+
+    ops = _ops()
+    g = torch.Generator().manual_seed(65540)
+    B = 65540
+    x = torch.randn(B, 8, 8, generator=g).bfloat16().to(device)
+    w = torch.randn(B, 8, 8, generator=g).bfloat16().to(device)
+    got = ops.dense_batched(x, w, False, None, None, "none")
+    want = torch.bmm(x.float(), w.float())
+    close(got, want, 8)
+    for i in (0, 65534, 65535, 65539):
+        assert torch.equal(got[i], ops.dense(x[i], w[i], False, None, None, "none")), i
+
+    B = 8
+    big = torch.randn(B, 40, 320, generator=g).bfloat16().to(device)
+    xs = big[:, :32, 64:320]
+    ws = (torch.randn(B, 72, 256, generator=g) / 16).bfloat16().to(device)
+    biasb = torch.randn(B, 72, generator=g).bfloat16().to(device)
+    res = torch.randn(B, 32, 72, generator=g).bfloat16().to(device)
+    whole = ops.dense_batched(xs, ws, True, biasb, res, "silu")
+    monkeypatch.setattr(xops, "MAX_BATCH_PER_LAUNCH", 3)
+    sliced = ops.dense_batched(xs, ws, True, biasb, res, "silu")
+    assert torch.equal(whole, sliced)
+    sliced = ops.dense_batched(xs, ws, True, biasb.float(), None, "none")
+    monkeypatch.setattr(xops, "MAX_BATCH_PER_LAUNCH", 65535)
+    assert torch.equal(ops.dense_batched(xs, ws, True, biasb.float(), None, "none"), sliced)
+
+
 def test_dense_batched_strided_entries(device):
     """Batch entries that are views: a batch stride larger than an entry, rows wider than K; a misaligned view is copied."""
     ops = _ops()

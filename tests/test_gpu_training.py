@@ -195,6 +195,32 @@ def test_dense_backward_formula(device, act, weight_trans):
         assert (a.float() - c).abs().mean().item() <= 2e-2 * scale + 1e-3, (name, (a.float() - c).abs().mean().item(), scale)
 
 
+@pytest.mark.parametrize("in_features", [76, 100, 64])
+def test_fp32_linear_trains_when_in_features_is_4_mod_8(device, in_features):
+    """An fp32 Linear whose in_features is a multiple of 4 and not of 8 fuses (the forward loads four floats at a time)
+    and its input gradient - a product whose OUTPUT width is in_features - does not fit the kernel: the backward
+    formula takes the Aten product there.  Loss and gradients against eager autograd."""
+
+    def layer(x, w, b):
+        return F.silu(F.linear(x, w, b))
+
+    torch.manual_seed(in_features)
+    x = torch.randn(40, in_features, device=device, requires_grad=True)
+    w = (torch.randn(64, in_features, device=device) / in_features**0.5).requires_grad_(True)
+    b = torch.randn(64, device=device, requires_grad=True)
+    be = backend()
+    y = torch.compile(layer, backend=be, dynamic=False)(x, w, b)
+    fwd_ops = [str(n.target) for n in be.compiled_graphs[1].graph.nodes if n.op == "call_function"]
+    assert "xpu_ops.dense.default" in fwd_ops, fwd_ops
+    g = torch.autograd.grad(y.pow(2).mean(), (x, w, b))
+    args = [t.detach().double().requires_grad_(True) for t in (x, w, b)]
+    want_y = layer(*args)
+    want = torch.autograd.grad(want_y.pow(2).mean(), args)
+    torch.testing.assert_close(y.double(), want_y, rtol=1e-5, atol=1e-5)
+    for a, c in zip(g, want):
+        torch.testing.assert_close(a.double(), c, rtol=1e-4, atol=1e-6)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("act", ["relu", "gelu", "silu", "sigmoid"])
 @pytest.mark.parametrize("shape", [(256, 512), (3, 5, 7), (1,), (4096, 1376)])

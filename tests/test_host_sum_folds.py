@@ -161,3 +161,22 @@ def test_saved_activations_of_a_forward_graph_may_share_storage():
     gm.meta["xg_user_outputs"] = 1
     assert FoldCloneOfContiguous().process(gm)
     assert calls(gm, aten.clone.default) == []
+
+
+def test_a_returned_copy_never_shares_storage_with_a_saved_activation():
+    """The caller may write into a result between forward and backward (legal in eager): a copy it sees stays a copy
+    when its source is saved for the backward, and the other way round."""
+
+    def returned_copy(x, w):
+        y = xpu.dense(x, w, False, None, None, "none")
+        return y.clone(), y  # result for the caller, source saved
+
+    def returned_source(x, w):
+        y = xpu.dense(x, w, False, None, None, "none")
+        return y, y.clone()  # source for the caller, copy saved
+
+    for fn in (returned_copy, returned_source):
+        gm = trace(fn, ((16, 32), bf16), ((32, 48), bf16))
+        gm.meta["xg_user_outputs"] = 1
+        assert not FoldCloneOfContiguous().process(gm), fn.__name__
+        assert len(calls(gm, aten.clone.default)) == 1

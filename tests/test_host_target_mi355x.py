@@ -536,6 +536,11 @@ def test_batch_dense_layer_vetoes(backend):
     x, w = torch.randn(2, 8, 12).to(bf16), torch.randn(2, 12, 8).to(bf16)  # K not a multiple of 8
     gm = rewrite(mi355x_compiler(), lambda x, w: torch.bmm(x, w), x, w, must_fail=False)
     assert modules_called(gm) == []
+    torch._dynamo.reset()
+    # a batch beyond one launch's grid (65535 entries) still fuses: the op wrapper sends it out in slices
+    x, w = torch.randn(70000, 8, 8).to(bf16), torch.randn(70000, 8, 8).to(bf16)
+    gm = rewrite(mi355x_compiler(), lambda x, w: torch.bmm(x, w), x, w)
+    assert len(modules_called(gm)) == 1
 
 
 def test_tanh_gelu_is_not_taken_for_the_erf_gelu_of_the_dense_kernel():

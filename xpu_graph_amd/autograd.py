@@ -188,7 +188,17 @@ def _dense_backward(ctx, gy):
         raise NotImplementedError(f"dense backward: activation {act!r}")
     gz = gz.to(x.dtype)
     need = ctx.needs_input_grad
-    gx = torch.ops.xpu_ops.dense(gz, weight, not ctx.trans, None, None, "none") if need[0] else None
+    gx = None
+    if need[0]:
+        # gz [M, N] times the weight read the other way: the product's inner size is N, its output width K.  The
+        # kernel wants both as the forward wants K and N; an fp32 layer with K % 8 == 4 passes the forward's check
+        # (4-element loads) and not this one, and then takes the Aten product.
+        from . import ops
+
+        if ops.dense_fits(gz.shape[1], x.shape[1], gz.dtype):
+            gx = torch.ops.xpu_ops.dense(gz, weight, not ctx.trans, None, None, "none")
+        else:
+            gx = gz @ (weight if ctx.trans else weight.t())
     gw = None
     if need[1]:
         gw = _weight_grad(gz, x) if ctx.trans else _weight_grad(x, gz)
@@ -224,10 +234,15 @@ def _dense_glu_backward(ctx, gy):
 
 def _dense_glu_save_setup(ctx, inputs, output):
     ctx.save_for_backward(*inputs, output[1], output[2])
+    ctx.set_materialize_grads(False)  # an unused output then hands over None, not zeros: a used one can be told apart
 
 
 def _dense_glu_save_backward(ctx, gy, g_gate=None, g_up=None):
-    # the two projection outputs exist for this formula; gradients flowing into them are not supported
+    # the two projection outputs exist for this formula; a gradient flowing into them is refused, not dropped
+    if g_gate is not None or g_up is not None:
+        raise NotImplementedError("xpu_ops::dense_glu_save: only its first output (the gated product) is differentiable")
+    if gy is None:
+        return None, None, None
     x, w_gate, w_up, gate, up = ctx.saved_tensors
     return _glu_grads(ctx, x, w_gate, w_up, gate, up, gy)
 
@@ -279,10 +294,15 @@ def _sdpa_lse_setup(ctx, inputs, output):
     q, k, v, ctx.causal, ctx.scale = inputs
     out, lse = output
     ctx.save_for_backward(q, k, v, out, lse)
+    ctx.set_materialize_grads(False)  # an unused log-sum-exp then hands over None, not zeros
 
 
 def _sdpa_lse_backward(ctx, gy, g_lse=None):
-    # the log-sum-exp output exists for this formula; a gradient flowing into it is not supported
+    # the log-sum-exp output exists for this formula; a gradient flowing into it is refused, not dropped
+    if g_lse is not None:
+        raise NotImplementedError("xpu_ops::sdpa_lse: only its first output (the attention result) is differentiable")
+    if gy is None:
+        return None, None, None, None, None
     q, k, v, out, lse = ctx.saved_tensors
     gq, gk, gv = torch.ops.xpu_ops.sdpa_bwd(q, k, v, out, gy, lse, ctx.causal, ctx.scale)
     return gq, gk, gv, None, None

@@ -431,6 +431,9 @@ __global__ __launch_bounds__(64 * KW) __attribute__((amdgpu_waves_per_eu(2, 2)))
         static_for<4>([&](auto EI) {
           constexpr int e = decltype(EI)::value;
           constexpr int v = 4 * g + e;
+          // l4 is finite: a causal row sees at least key 0 and additive masks are refused by the entry point.  A
+          // backward that admits rows without any visible key (log-sum-exp -inf) has to map -inf to 0 here, as the
+          // dq kernel does, or -inf - (-inf) gives NaN.
           const float pr = __builtin_amdgcn_exp2f(__builtin_fmaf(s[v], cc, -l4[e] * kLog2e));
           prf[v / 8][v % 8] = (T)pr;
           dsf[v / 8][v % 8] = (T)(pr * (dp[v] - d4[e]));

@@ -669,9 +669,21 @@ def _dense_into(x, weight, weight_trans, bias, residual, act, out):
     return out
 
 
+def dense_fits(k, n, dtype):
+    """What xg_dense takes: static K a multiple of one 16-byte operand load (8 elements of a 16-bit type, 4 of
+    fp32), static N a multiple of 8."""
+    if dtype not in (torch.bfloat16, torch.float16, torch.float32):
+        return False
+    per16 = 16 // torch.empty((), dtype=dtype).element_size()
+    return isinstance(k, int) and isinstance(n, int) and k > 0 and n > 0 and k % per16 == 0 and n % 8 == 0
+
+
 def _dense(x, weight, weight_trans, bias, residual, act):
     m, n, _ = _dense_out_shape(x, weight, weight_trans)
     return _dense_into(x, weight, weight_trans, bias, residual, act, torch.empty((m, n), dtype=x.dtype, device=x.device))
+
+
+MAX_BATCH_PER_LAUNCH = 65535  # gridDim.y of xg_dense_batched
 
 
 def _dense_batched_shape(x, weight, weight_trans):
@@ -728,12 +740,22 @@ def _dense_batched(x, weight, weight_trans, bias, residual, act):
     if residual is not None:
         residual = _batch_major(residual)
         ldr, res_stride = residual.stride(1), residual.stride(0)
-    st = _lib.lib().xg_dense_batched(
-        _ptr(x), _ptr(weight), _ptr(bias), _ptr(residual), _ptr(out), b, m, n, k, x.stride(1), weight.stride(1), ldr,
-        x.stride(0), weight.stride(0), bias_stride, res_stride, m * n,
-        1 if weight_trans else 0, _lib.ACT_CODES[act], _code(x.dtype), bias_dt, _stream(),
-    )
-    _lib.check(st, "xg_dense_batched")
+    # the batch entry is the second grid axis of the kernels (at most MAX_BATCH_PER_LAUNCH entries a launch): a larger
+    # batch goes out in slices, every operand moved on by its batch stride
+    esz = x.element_size()
+    for b0 in range(0, b, MAX_BATCH_PER_LAUNCH):
+        nb = min(MAX_BATCH_PER_LAUNCH, b - b0)
+
+        def at(t, stride, size=esz):
+            return t.data_ptr() + b0 * stride * size if t is not None else None
+
+        st = _lib.lib().xg_dense_batched(
+            at(x, x.stride(0)), at(weight, weight.stride(0)), at(bias, bias_stride, bias.element_size() if bias is not None else 0),
+            at(residual, res_stride), at(out, m * n), nb, m, n, k, x.stride(1), weight.stride(1), ldr,
+            x.stride(0), weight.stride(0), bias_stride, res_stride, m * n,
+            1 if weight_trans else 0, _lib.ACT_CODES[act], _code(x.dtype), bias_dt, _stream(),
+        )
+        _lib.check(st, "xg_dense_batched")
     return out
 
 

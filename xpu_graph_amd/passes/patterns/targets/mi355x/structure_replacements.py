@@ -167,10 +167,7 @@ def can_fuse_custom_denselayer(inputs, weight, weight_trans, bias, act_str):
         return False
     k = inputs.shape[1]
     n = weight.shape[0] if weight_trans else weight.shape[1]
-    if not (isinstance(k, int) and isinstance(n, int)):
-        return False
-    per16 = 16 // inputs.element_size()  # 16-byte operand loads: 8 elements of a 16-bit type, 4 of fp32
-    return k % per16 == 0 and n % 8 == 0 and k > 0 and n > 0
+    return _xops.dense_fits(k, n, inputs.dtype)
 
 
 class BatchDenseLayerModule(torch.nn.Module):

@@ -166,21 +166,25 @@ def _views_of(node, stop=None):
 
 
 def _visible_outputs(gm):
-    """The output values a caller can see and write to: all of them, except in a forward graph, where AOT
-    appends the values saved for the backward after the `xg_user_outputs` it returns to the caller."""
+    """(visible, all): the output values a caller can see and write to, and every output value.  The two differ
+    only in a forward graph, where AOT appends the values saved for the backward after the `xg_user_outputs` it
+    returns to the caller."""
     out = next(n for n in gm.graph.nodes if n.op == "output")
     results = out.args[0] if isinstance(out.args[0], (tuple, list)) else (out.args[0],)
     k = gm.meta.get("xg_user_outputs")
-    found = []
-    fx.node.map_arg(tuple(results) if k is None else tuple(results[:k]), lambda n: found.append(n))
-    return found
+    visible, every = [], []
+    fx.node.map_arg(tuple(results) if k is None else tuple(results[:k]), lambda n: visible.append(n))
+    fx.node.map_arg(tuple(results), lambda n: every.append(n))
+    return visible, every
 
 
 class FoldCloneOfContiguous(Pattern):
     """clone(v) / clone(v, memory_format=contiguous) of a value that is already contiguous and whose storage this
     graph made itself: graphs at these stages are functional (nothing writes into v or the clone), so the copy
-    only costs a pass over memory.  Kept when both the copy and its source (or views of them) are handed to the
-    caller: two results that were separate tensors must not come back sharing storage."""
+    only costs a pass over memory.  Kept when the copy and its source (or views of them) both leave the graph and
+    the caller sees at least one of them: two results that were separate tensors must not come back sharing
+    storage, and a result the caller may write into between forward and backward must not be the tensor that the
+    backward saved.  Two values that are both only saved for the backward may share."""
 
     _opt_level = OptLevel.level2
     _support_stages = _POST_AOT
@@ -203,8 +207,11 @@ class FoldCloneOfContiguous(Pattern):
             if not (isinstance(root, fx.Node) and root.op in ("call_function", "call_module")) or _is_view_of_first_arg(root):
                 continue  # an input, a constant, or a view of something this walk cannot follow
             if visible is None:
-                visible = _visible_outputs(gm)
-            if any(n in visible for n in _views_of(node)) and any(n in visible for n in _views_of(root, stop=node)):
+                visible, every = _visible_outputs(gm)
+            copy_side, source_side = list(_views_of(node)), list(_views_of(root, stop=node))
+            copy_seen, source_seen = any(n in visible for n in copy_side), any(n in visible for n in source_side)
+            copy_out, source_out = any(n in every for n in copy_side), any(n in every for n in source_side)
+            if (copy_seen and source_out) or (source_seen and copy_out):
                 continue
             node.replace_all_uses_with(src)
             g.erase_node(node)
