@@ -88,9 +88,10 @@ def test_c4_dense_silu(device):
     x, W, b = inputs.c4_dense(device=device)
     out, mods, rest = run(eager.dense_silu_eager, x, W, b)
     assert len(mods) == 1 and rest == [], (mods, rest)
-    rows = torch.arange(0, 8192, 37, device=device)
-    want = torch.nn.functional.silu(x[rows].float() @ W.float() + b.float())
-    torch.testing.assert_close(out[rows].float(), want, rtol=1.6e-2, atol=2e-2)
+    Wf, bf = W.float(), b.float()
+    for r0 in range(0, 8192, 1024):  # every row against the fp32 evaluation
+        want = torch.nn.functional.silu(x[r0 : r0 + 1024].float() @ Wf + bf)
+        torch.testing.assert_close(out[r0 : r0 + 1024].float(), want, rtol=1.6e-2, atol=2e-2)
     torch.testing.assert_close(out, eager.dense_silu_eager(x, W, b), rtol=1.6e-2, atol=2e-2)
 
 
@@ -453,3 +454,30 @@ def test_sdpa_with_an_additive_mask_runs_the_kernel(device, mask_kind):
     assert not any("softmax" in t or "bmm" in t for t in rest), rest
     want = att(q.float(), k.float(), v.float(), m.float())
     assert_close_16bit(out.to(torch.bfloat16) if out.dtype != torch.bfloat16 else out, want, attention_floor(want, torch.bfloat16), f"sdpa masked compiled {mask_kind}")
+
+
+@pytest.mark.parametrize("form", ["permuted_fp32_softmax", "permuted_prescaled_query", "permuted_divide", "decoder_output_transposed"])
+def test_permuted_input_sdpa_forms_reach_the_kernel(device, form):
+    """The reference's attention forms whose operands arrive as [B, S, H, E] and are permuted inside the function
+    (tests/common/test_fuse_sdpa.py:166-262, `_sdpa_pattern_7` .. `_12`), and the decoder form that hands its result
+    on transposed and contiguous (`_sdpa_pattern_transformer_1`, :490-506): each is rewritten to the HIP attention
+    kernel, reads the permuted storage in place, and follows the fp32 evaluation of the same function."""
+    from tests.test_host_sdpa_reference_forms import decoder, permuted_divide, permuted_fp32_softmax, permuted_prescaled_query
+    from tests.tolerance import assert_close_16bit, attention_floor
+
+    g = torch.Generator().manual_seed(7)
+    B, S, H, D = 2, 320, 8, 128
+    bf = torch.bfloat16
+    if form == "decoder_output_transposed":
+        q, k, v = (torch.randn(B, H, S, D, generator=g).to(bf).to(device) for _ in range(3))
+        fn, args = decoder, (q, k, v)
+    else:
+        q, k, v = (torch.randn(B, S, H, D, generator=g).to(bf).to(device) for _ in range(3))
+        fn = {"permuted_fp32_softmax": permuted_fp32_softmax, "permuted_prescaled_query": permuted_prescaled_query, "permuted_divide": permuted_divide}[form]
+        args = (q, k, v, D**0.5) if form == "permuted_divide" else (q, k, v)
+    out, mods, rest = run(fn, *args)
+    assert any(m.startswith("mi355x_sdpa") for m in mods), (mods, rest)
+    assert not any("softmax" in t or "bmm" in t or "matmul" in t for t in rest), rest
+    want = fn(*(a.float() if torch.is_tensor(a) else a for a in args))
+    assert out.shape == want.shape and out.dtype == bf
+    assert_close_16bit(out, want, attention_floor(want, bf), f"sdpa compiled {form}")
