@@ -861,6 +861,10 @@ def run_workload(torch, dev, wl, steps, warmup, with_cpu=True):
             "traffic": traffic,
         },
     }
+    if traffic and wl.bound == "hbm":
+        # what the bytes that really moved (whole 128-byte lines) amount to per second: beside `frac`, which prices the
+        # algorithmic bytes only
+        res["roofline"]["traffic_gbps"] = traffic / t_k / 1e9
     if with_cpu:
         fn, how = wl.cpu_fn(torch)
         t_cpu, n = _cpu_time(fn, warmups=getattr(wl, "cpu_warmups", 2))

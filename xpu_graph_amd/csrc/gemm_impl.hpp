@@ -332,35 +332,63 @@ __device__ __forceinline__ void mma_step(f32x16 (&acc)[4][4], const Frag<T> (&fa
 // All the arithmetic therefore exists once, in a loop a few dozen instructions long, instead of
 // 256 unrolled copies; the per-lane bias and scale values are loop invariant.
 template <typename OT, int ACT>
+__device__ __forceinline__ void epilogue_one_row(const GemmParams& p, const f32x4 lo, const f32x4 hi, const float (&sv)[8],
+                                                 const float (&bv)[8], const OT* res_at, OT* out_at) {
+  typedef OT O8 __attribute__((ext_vector_type(8)));
+  float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+#pragma unroll
+  for (int e = 0; e < 8; ++e) v[e] = v[e] * sv[e] + bv[e];
+  if (p.res) {
+    const O8 r = *reinterpret_cast<const O8*>(res_at);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] += to_f32(r[e]);
+  }
+  O8 o;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    float t = v[e];
+    if constexpr (ACT == XG_ACT_RELU) t = fmaxf(t, 0.f);
+    if constexpr (ACT == XG_ACT_GELU) t = 0.5f * t * (1.f + erff(t * 0.70710678118654752f));
+    if constexpr (ACT == XG_ACT_SILU) t = silu_f32(t);
+    if constexpr (ACT == XG_ACT_SIGMOID) t = sigmoid_f32(t);
+    o[e] = from_f32<OT>(t);
+  }
+  store_vec_nt(reinterpret_cast<O8*>(out_at), o);  // written once, read by another kernel
+}
+
+template <typename OT, int ACT>
 __device__ __forceinline__ void epilogue_rows(const GemmParams& p, const char* park, int lane, int m_base, int n, bool n_ok,
                                               const float (&sv)[8], const float (&bv)[8], int passes) {
-  typedef OT O8 __attribute__((ext_vector_type(8)));
   const int c = lane & 7, rr = lane >> 3;
+  // Pass `it` handles row it * 8 + rr, whose chunk permutation (row & 15) alternates between rr and rr | 8: the LDS
+  // addresses of an even and of an odd pass are formed once and only advanced, and the output / residual pointers
+  // step by eight rows -- the loop then holds the arithmetic and little else (it is issue-bound: one wave per SIMD).
+  const char* pk = park + rr * 256;
+  const int lo_e = ((2 * c) ^ rr) << 4, hi_e = ((2 * c + 1) ^ rr) << 4, lo_o = lo_e ^ 128, hi_o = hi_e ^ 128;
+  OT* out_at = reinterpret_cast<OT*>(p.out) + (int64_t)(m_base + rr) * p.ldc + n;
+  const OT* res_at = p.res ? reinterpret_cast<const OT*>(p.res) + (int64_t)(m_base + rr) * p.ldr + n : nullptr;
+  const int64_t out_step = 8 * p.ldc, res_step = 8 * p.ldr;
+  // whole wave inside the matrix (uniform): no per-lane predicates
+  const bool inside = __builtin_amdgcn_ballot_w64(!n_ok) == 0 && m_base + passes * 8 <= p.M;
+  if (inside && (passes & 1) == 0) {
+    for (int it = 0; it < passes; it += 2) {
+      const f32x4 lo0 = *reinterpret_cast<const f32x4*>(pk + lo_e), hi0 = *reinterpret_cast<const f32x4*>(pk + hi_e);
+      const f32x4 lo1 = *reinterpret_cast<const f32x4*>(pk + 2048 + lo_o), hi1 = *reinterpret_cast<const f32x4*>(pk + 2048 + hi_o);
+      epilogue_one_row<OT, ACT>(p, lo0, hi0, sv, bv, res_at, out_at);
+      epilogue_one_row<OT, ACT>(p, lo1, hi1, sv, bv, res_at + res_step, out_at + out_step);
+      pk += 4096;
+      out_at += 2 * out_step;
+      res_at += 2 * res_step;
+    }
+    return;
+  }
   for (int it = 0; it < passes; ++it) {
-    const int row = it * 8 + rr;
-    const int m = m_base + row;
-    const f32x4 lo = *reinterpret_cast<const f32x4*>(park + row * 256 + (((2 * c) ^ (row & 15)) << 4));
-    const f32x4 hi = *reinterpret_cast<const f32x4*>(park + row * 256 + (((2 * c + 1) ^ (row & 15)) << 4));
-    if (!(n_ok && m < p.M)) continue;
-    float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-#pragma unroll
-    for (int e = 0; e < 8; ++e) v[e] = v[e] * sv[e] + bv[e];
-    if (p.res) {
-      const O8 r = *reinterpret_cast<const O8*>(reinterpret_cast<const OT*>(p.res) + (int64_t)m * p.ldr + n);
-#pragma unroll
-      for (int e = 0; e < 8; ++e) v[e] += to_f32(r[e]);
-    }
-    O8 o;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      float t = v[e];
-      if constexpr (ACT == XG_ACT_RELU) t = fmaxf(t, 0.f);
-      if constexpr (ACT == XG_ACT_GELU) t = 0.5f * t * (1.f + erff(t * 0.70710678118654752f));
-      if constexpr (ACT == XG_ACT_SILU) t = silu_f32(t);
-      if constexpr (ACT == XG_ACT_SIGMOID) t = sigmoid_f32(t);
-      o[e] = from_f32<OT>(t);
-    }
-    store_vec_nt(reinterpret_cast<O8*>(reinterpret_cast<OT*>(p.out) + (int64_t)m * p.ldc + n), o);  // written once, read by another kernel
+    const bool odd = it & 1;
+    const f32x4 lo = *reinterpret_cast<const f32x4*>(pk + (odd ? lo_o : lo_e)), hi = *reinterpret_cast<const f32x4*>(pk + (odd ? hi_o : hi_e));
+    if (n_ok && m_base + it * 8 + rr < p.M) epilogue_one_row<OT, ACT>(p, lo, hi, sv, bv, res_at, out_at);
+    pk += 2048;
+    out_at += out_step;
+    res_at += res_step;
   }
 }
 
@@ -437,6 +465,12 @@ __device__ __forceinline__ void epilogue(const GemmParams& p, const Lane& L, f32
     const bool n_ok = n < p.N;  // N % 8 == 0: the 8 columns are in or out together
     float sv[8], bv[8];
     column_terms<OT>(p, n, n_ok, a_sc, sv, bv);
+#ifndef XG_NO_EPI_WAIT
+    // The bias and scale loads are waited for HERE.  Left pending into the row loop, the compiler's wait (it counts
+    // loads and stores with one counter) would sit inside the loop and also wait, in every pass, for the previous
+    // pass's output store to be acknowledged by memory.
+    wait_vm<0>();
+#endif
     epilogue_rows_act<OT>(p, park, L.lane, m_base, n, n_ok, sv, bv, NI * 4);
   });
 }
