@@ -504,29 +504,54 @@ __device__ __forceinline__ void epilogue_glu(const GemmParams& p, const Lane& L,
     __syncthreads();  // both parks of the pair are complete
     const int n = n0 + h * 64 + c * 8;
     const bool n_ok = n < p.N;  // N % 8 == 0: the 8 columns are in or out together
-    for (int it = 0; it < NI * 2; ++it) {
-      const int row = L.wn * (NI * 16) + it * 8 + rr;
-      const int m = m_base + row;
-      const int o0 = row * 256 + (((2 * c) ^ (row & 15)) << 4), o1 = row * 256 + (((2 * c + 1) ^ (row & 15)) << 4);
-      const f32x4 g0 = *reinterpret_cast<const f32x4*>(gate + o0), g1 = *reinterpret_cast<const f32x4*>(gate + o1);
-      const f32x4 u0 = *reinterpret_cast<const f32x4*>(up + o0), u1 = *reinterpret_cast<const f32x4*>(up + o1);
-      if (!(n_ok && m < p.M)) continue;
+    // One row of the pair's result: each projection is rounded to the storage type first, as the two separate
+    // layers would do.
+    auto one_row = [&](const f32x4 g0, const f32x4 g1, const f32x4 u0, const f32x4 u1, int64_t at) {
       const float gv[8] = {g0[0], g0[1], g0[2], g0[3], g1[0], g1[1], g1[2], g1[3]};
       const float uv[8] = {u0[0], u0[1], u0[2], u0[3], u1[0], u1[1], u1[2], u1[3]};
       O8 o, go, uo;
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        // each projection is rounded to the storage type first, as the two separate layers would do
         const OT g16 = from_f32<OT>(gv[e]), u16 = from_f32<OT>(uv[e]);
         const float gr = to_f32(g16), ur = to_f32(u16);
         o[e] = from_f32<OT>(silu_f32(gr) * ur);
         go[e] = g16;
         uo[e] = u16;
       }
-      store_vec_nt(reinterpret_cast<O8*>(reinterpret_cast<OT*>(p.out) + (int64_t)m * p.ldc + n), o);  // written once, read by another kernel
+      store_vec_nt(reinterpret_cast<O8*>(reinterpret_cast<OT*>(p.out) + at), o);  // written once, read by another kernel
       if (p.gate_out != nullptr) {
-        store_vec_nt(reinterpret_cast<O8*>(reinterpret_cast<OT*>(p.gate_out) + (int64_t)m * p.ldc + n), go);
-        store_vec_nt(reinterpret_cast<O8*>(reinterpret_cast<OT*>(p.up_out) + (int64_t)m * p.ldc + n), uo);
+        store_vec_nt(reinterpret_cast<O8*>(reinterpret_cast<OT*>(p.gate_out) + at), go);
+        store_vec_nt(reinterpret_cast<O8*>(reinterpret_cast<OT*>(p.up_out) + at), uo);
+      }
+    };
+    // Pass `it` handles row r0 + it * 8, whose chunk permutation (row & 15) alternates between rr and rr | 8: the
+    // LDS offsets of an even and of an odd pass are formed once and advanced, as is the output offset.
+    const int r0 = L.wn * (NI * 16) + rr;
+    int off = r0 * 256;
+    const int lo_e = ((2 * c) ^ rr) << 4, hi_e = ((2 * c + 1) ^ rr) << 4, lo_o = lo_e ^ 128, hi_o = hi_e ^ 128;
+    int64_t at = (int64_t)(m_base + r0) * p.ldc + n;
+    const int64_t step = 8 * p.ldc;
+    const bool inside = __builtin_amdgcn_ballot_w64(!n_ok) == 0 && m_base + L.wn * (NI * 16) + NI * 16 <= p.M;  // uniform
+    if (inside) {
+      for (int it = 0; it < NI * 2; it += 2) {
+        const f32x4 g0 = *reinterpret_cast<const f32x4*>(gate + off + lo_e), g1 = *reinterpret_cast<const f32x4*>(gate + off + hi_e);
+        const f32x4 u0 = *reinterpret_cast<const f32x4*>(up + off + lo_e), u1 = *reinterpret_cast<const f32x4*>(up + off + hi_e);
+        const f32x4 g2 = *reinterpret_cast<const f32x4*>(gate + off + 2048 + lo_o), g3 = *reinterpret_cast<const f32x4*>(gate + off + 2048 + hi_o);
+        const f32x4 u2 = *reinterpret_cast<const f32x4*>(up + off + 2048 + lo_o), u3 = *reinterpret_cast<const f32x4*>(up + off + 2048 + hi_o);
+        one_row(g0, g1, u0, u1, at);
+        one_row(g2, g3, u2, u3, at + step);
+        off += 4096;
+        at += 2 * step;
+      }
+    } else {
+      for (int it = 0; it < NI * 2; ++it) {
+        const bool odd = it & 1;
+        const int o0 = off + (odd ? lo_o : lo_e), o1 = off + (odd ? hi_o : hi_e);
+        const f32x4 g0 = *reinterpret_cast<const f32x4*>(gate + o0), g1 = *reinterpret_cast<const f32x4*>(gate + o1);
+        const f32x4 u0 = *reinterpret_cast<const f32x4*>(up + o0), u1 = *reinterpret_cast<const f32x4*>(up + o1);
+        if (n_ok && m_base + r0 + it * 8 < p.M) one_row(g0, g1, u0, u1, at);
+        off += 2048;
+        at += step;
       }
     }
     __syncthreads();  // the parks are free for the next half
