@@ -77,22 +77,14 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
   int bh, qb;
   {
     const int id = blockIdx.x, nbh = p.B * p.H;
-    if (p.order >= 2 && (nbh & 7) == 0) {
-      // p.order heads at a time inside each XCD, their query blocks interleaved heaviest first
-      const int xcd = id & 7, slot = id >> 3;
-      const int per = p.order * p.n_qb;
-      const int g = slot / per, r = slot % per;
-      const int left = (nbh >> 3) - g * p.order;
-      const int gsz = left < p.order ? left : p.order;
-      bh = (g * p.order + r % gsz) * 8 + xcd;
-      qb = p.n_qb - 1 - r / gsz;
-    } else if (p.order == 1 && (nbh & 7) == 0) {
+    if (p.order == 1 && (nbh & 7) == 0) {
       const int xcd = id & 7, slot = id >> 3;
       bh = (slot / p.n_qb) * 8 + xcd;
       qb = p.n_qb - 1 - slot % p.n_qb;
     } else {
-      bh = id % nbh;
-      qb = p.n_qb - 1 - id / nbh;  // causal: late query blocks have the most keys, start them first
+      int rank;
+      grouped_block_order(id, nbh, p.n_qb, p.order, bh, rank);  // causal: late query blocks have the most keys, start them first
+      qb = p.n_qb - 1 - rank;
     }
   }
   const int b = bh / p.H, head = bh % p.H, hkv = head / (p.H / p.Hkv);
@@ -465,11 +457,7 @@ int sdpa_entry(const void* q, const void* k, const void* v, void* out, float* ls
   // heads at a time per XCD, so that the blocks in flight share their keys in L2 (a CU streams 117 GB/s from L2, 27 GB/s
   // from the last-level cache): B4 H32 S2048 163 -> 158 us against all sixteen heads of an XCD at once, B2 H16 S8192
   // 533 (head after head) -> 511 us.
-  p.order = !p.causal ? 1 : 0;
-  if (p.causal && (B * H) % 8 == 0) {
-    const int64_t per_xcd = B * H / 8;
-    p.order = per_xcd < 2 ? 1 : (int)(per_xcd < 8 ? per_xcd : 8);
-  }
+  p.order = p.causal ? sdpa::block_order_group(B * H) : 1;
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   if (mask) {
     if (dtype == XG_BF16) return D == 128 ? sdpa::launch<bf16_t, 128, true>(p, st) : sdpa::launch<bf16_t, 64, true>(p, st);

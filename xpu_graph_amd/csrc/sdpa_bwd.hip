@@ -48,6 +48,7 @@ struct BwdParams {
   float scale;
   int causal;
   int n_qb, n_kb;
+  int group_q, group_k;  // block order of the two kernels (grouped_block_order)
 };
 
 constexpr float kLog2e = 1.44269504088896340736f;
@@ -179,8 +180,9 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
   const float c = p.scale * kLog2e;
 
   const int nbh = p.B * p.H;
-  const int bh = blockIdx.x % nbh;
-  const int qb = p.n_qb - 1 - blockIdx.x / nbh;  // causal: late query blocks have the most keys, start them first
+  int bh, rank;
+  grouped_block_order(blockIdx.x, nbh, p.n_qb, p.group_q, bh, rank);
+  const int qb = p.n_qb - 1 - rank;  // causal: late query blocks have the most keys, start them first
   const int b = bh / p.H, head = bh % p.H, hkv = head / (p.H / p.Hkv);
   const int q0 = qb * BQ;
   const int qrow = q0 + 32 * wave + l32;
@@ -317,8 +319,8 @@ __global__ __launch_bounds__(64 * KW) __attribute__((amdgpu_waves_per_eu(2, 2)))
   const float c = p.scale * kLog2e;
 
   const int nbk = p.B * p.Hkv, rep = p.H / p.Hkv;
-  const int bk = blockIdx.x % nbk;
-  const int kb = blockIdx.x / nbk;  // causal: early key blocks meet the most queries, start them first
+  int bk, kb;  // causal: early key blocks meet the most queries, start them first
+  grouped_block_order(blockIdx.x, nbk, p.n_kb, p.group_k, bk, kb);
   const int b = bk / p.Hkv, hkv = bk % p.Hkv;
   const int k0 = kb * BK;
   const int krow = k0 + 32 * wave + l32;
@@ -549,6 +551,8 @@ int backward_entry(const void* q, const void* k, const void* v, const void* out,
   p.causal = causal ? 1 : 0;
   p.n_qb = (int)n_qb;
   p.n_kb = (int)n_kb;
+  p.group_q = sdpa::block_order_group(B * H);
+  p.group_k = sdpa::block_order_group(B * Hkv);
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   if (dtype == XG_BF16) return D == 128 ? sdpa::launch_bwd<bf16_t, 128>(p, st) : sdpa::launch_bwd<bf16_t, 64>(p, st);
   return D == 128 ? sdpa::launch_bwd<f16_t, 128>(p, st) : sdpa::launch_bwd<f16_t, 64>(p, st);

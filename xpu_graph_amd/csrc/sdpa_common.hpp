@@ -46,6 +46,33 @@ struct Vec8<f16_t> {
 __device__ __forceinline__ f32x16 mma(bf16x8 a, bf16x8 b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
 __device__ __forceinline__ f32x16 mma(f16x8 a, f16x8 b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0); }
 
+// Which problem (batch x head) and which of its blocks a workgroup takes, rank 0 being the heaviest block.  Workgroup
+// ids are dealt to the 8 XCDs round-robin; with `group` >= 2 (and a problem count that is a multiple of 8) every XCD
+// walks its own problems `group` at a time, their blocks interleaved heaviest first: the blocks in flight on an XCD then
+// belong to few problems and find each other's tiles in its L2.  Otherwise: the heaviest blocks of all problems first.
+__device__ __forceinline__ void grouped_block_order(int id, int n_prob, int n_blk, int group, int& prob, int& rank) {
+  if (group >= 2 && (n_prob & 7) == 0) {
+    const int xcd = id & 7, slot = id >> 3;
+    const int per = group * n_blk;
+    const int g = slot / per, r = slot % per;
+    const int left = (n_prob >> 3) - g * group;
+    const int gsz = left < group ? left : group;
+    prob = (g * group + r % gsz) * 8 + xcd;
+    rank = r / gsz;
+  } else {
+    prob = id % n_prob;
+    rank = id / n_prob;
+  }
+}
+// Problems per XCD taken at a time by grouped_block_order: all of them up to eight (0: no grouping).
+inline int block_order_group(int64_t n_prob) {
+#ifdef XG_NO_BLOCK_GROUPS
+  return 0;
+#endif
+  if (n_prob % 8 != 0 || n_prob / 8 < 2) return 0;
+  return (int)(n_prob / 8 < 8 ? n_prob / 8 : 8);
+}
+
 // Chunk swizzles (16-byte chunks within a row of D elements).
 template <int D>
 __device__ __forceinline__ int swz_k(int r) {
