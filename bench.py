@@ -92,6 +92,39 @@ def _wall_time(torch, fn, n_sets, steps, warmup):
     return (time.perf_counter() - t0) / steps
 
 
+NOMINAL_CLOCK_GHZ = 2.4  # MI355X peak engine clock: the published MFMA peaks are quoted at it
+
+
+def _shader_clock_ghz(torch, fn, n_sets, t_call, label=""):
+    """Median engine clock while `fn` runs back to back: a one-wave probe kernel on a second stream samples the shader
+    clock against the constant-rate wall clock in 20 us windows for 8 ms (xg_clock_probe); the second half counts, by
+    which the power management has settled on this load."""
+    from xpu_graph_amd import _lib
+
+    lib = _lib.lib()
+    khz = int(lib.xg_wall_clock_khz())
+    if khz <= 0:
+        return None
+    n_win, win_us = 400, 20
+    buf = torch.zeros(2 * n_win, dtype=torch.int64, device="cuda")
+    side = torch.cuda.Stream()
+    warm = min(2000, max(3, int(0.02 / t_call)))                      # ~20 ms of this load first
+    reps = max(3, int(1.5 * n_win * win_us * 1e-6 / t_call) + 2)      # outlasts the probe
+    for i in range(warm):
+        fn(i % n_sets)
+    torch.cuda.synchronize()
+    fn(0)
+    _lib.check(lib.xg_clock_probe(_p(buf), n_win, win_us * khz // 1000, ctypes.c_void_p(side.cuda_stream)), "xg_clock_probe")
+    for i in range(reps):
+        fn(i % n_sets)
+    torch.cuda.synchronize()
+    d = buf.view(n_win, 2).double()
+    ghz = d[:, 0] / d[:, 1].clamp(min=1) * khz / 1e6
+    quarters = [float(ghz[i * n_win // 4:(i + 1) * n_win // 4].median().item()) for i in range(4)]
+    print(f"[bench] shader clock under {label}: median GHz per 2 ms quarter {' '.join(f'{q:.2f}' for q in quarters)}", file=sys.stderr)
+    return float(ghz[n_win // 2:].median().item())
+
+
 def _cpu_time(fn, min_iters=3, budget_s=12.0, max_iters=30, warmups=2):
     for _ in range(warmups):  # also compiles the default path
         fn()
@@ -305,6 +338,7 @@ class AddNC3b(Workload):
 
 
 class DenseC4(Workload):
+    zero_operands = True
     name = "C4 dense + bias + SiLU bf16 M8192 K4096 N11008"
     bound = "mfma"
     dtype = "bf16"
@@ -440,6 +474,7 @@ class DenseFp8C4(DenseC4):
 
 
 class DenseGluC5(Workload):
+    zero_operands = True
     name = "C5 MLP gate+up gated dense bf16 M8192 K4096 N11008"
     bound = "mfma"
     dtype = "bf16"
@@ -491,6 +526,7 @@ class DenseGluC5(Workload):
 
 
 class SdpaC5(Workload):
+    zero_operands = True
     name = "C5 causal attention bf16 B4 H32 S2048 D128"
     bound = "mfma"
     dtype = "bf16"
@@ -603,6 +639,7 @@ class SdpaBackwardC5(Workload):
 
 
 class DenseWeightGradC4(Workload):
+    zero_operands = True
     name = "C4 dense weight gradient bf16 x[8192,4096]^T g[8192,11008]"
     bound = "mfma"
     dtype = "bf16"
@@ -861,6 +898,27 @@ def run_workload(torch, dev, wl, steps, warmup, with_cpu=True):
             "traffic": traffic,
         },
     }
+    clock = _shader_clock_ghz(torch, wl.abi_call, n_sets, t_k, wl.name)
+    if clock:
+        # the engine clock the GPU held under this kernel; for an MFMA kernel also the fraction of the peak scaled to that
+        # clock (`frac` prices against the published peak, which assumes the nominal clock)
+        res["roofline"]["clock_ghz"] = clock
+        if wl.bound == "mfma":
+            res["roofline"]["frac_at_clock"] = res["roofline"]["frac"] * NOMINAL_CLOCK_GHZ / clock
+    if getattr(wl, "zero_operands", False):
+        # The same launches with every matrix operand zeroed: the identical instruction stream at the power of operands
+        # that toggle no bits.  Beside `frac` it tells how much of the gap to the peak is the engine clock the GPU gives
+        # this kernel on random data, and how much is the kernel's own.
+        for group in wl.sets:
+            for t in group:
+                if t.dim() >= 2:
+                    t.zero_()
+        t_z = _events_time(torch, wl.abi_call, n_sets, max(steps, 100), max(warmup, 20))
+        res["roofline"]["zero_operands"] = {
+            "kernel_us": t_z * 1e6,
+            "frac": wl.work / t_z / scale / peak,
+            "clock_ghz": _shader_clock_ghz(torch, wl.abi_call, n_sets, t_z, wl.name + " (zero operands)"),
+        }
     if traffic and wl.bound == "hbm":
         # what the bytes that really moved (whole 128-byte lines) amount to per second: beside `frac`, which prices the
         # algorithmic bytes only

@@ -395,6 +395,21 @@ int xg_rope(const void* x, const void* cos_table, const void* sin_table, void* o
  * ------------------------------------------------------------------------- */
 int xg_copy_bytes(const void* src, void* dst, int64_t bytes, xg_stream_t stream);
 
+/* ---------------------------------------------------------------------------
+ * Shader-clock probe for benchmarks: one wavefront that, for each of
+ * `n_windows` windows of `window_ticks` ticks of the constant-rate wall clock
+ * (xg_wall_clock_khz, 100 MHz on gfx950), writes out[2w] = shader-clock ticks
+ * and out[2w + 1] = wall-clock ticks that went by.  Launched on a second
+ * stream beside the kernel under test, it tells the engine clock the GPU
+ * sustains under that kernel: out[2w] / out[2w + 1] x wall-clock rate.
+ *   out: device memory, 2 x n_windows uint64; n_windows <= 65536;
+ *   0 < window_ticks <= 1000000.  Every window ends after a bounded number
+ *   of polls, so the kernel always finishes.
+ * No counterpart in the reference.
+ * ------------------------------------------------------------------------- */
+int xg_clock_probe(uint64_t* out, int n_windows, int64_t window_ticks, xg_stream_t stream);
+int64_t xg_wall_clock_khz(void);
+
 #ifdef __cplusplus
 }
 #endif

@@ -139,6 +139,8 @@ _SIGNATURES = {
         [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, ctypes.POINTER(c_int64), ctypes.POINTER(c_int64), c_int64, c_int, c_int, c_void_p],
     ),
     "xg_copy_bytes": (c_int, [c_void_p, c_void_p, c_int64, c_void_p]),
+    "xg_clock_probe": (c_int, [c_void_p, c_int, c_int64, c_void_p]),
+    "xg_wall_clock_khz": (c_int64, []),
 }
 
 

@@ -204,6 +204,24 @@ int act_entry(const void* z, const void* gy, void* out, int64_t n, int act, int 
   }
 }
 
+// One lane: for each of `n_windows` windows of `window_ticks` ticks of the constant-rate wall clock, the ticks of the
+// shader clock and of the wall clock that went by.  Every window ends after a bounded number of polls.
+__global__ void clock_probe_kernel(unsigned long long* out, int n_windows, unsigned window_ticks) {
+  if (threadIdx.x != 0) return;
+  for (int w = 0; w < n_windows; ++w) {
+    const unsigned long long r0 = wall_clock64();
+    const unsigned long long c0 = clock64();
+    unsigned long long r1 = r0;
+    for (int poll = 0; poll < (1 << 20) && r1 - r0 < window_ticks; ++poll) {
+      __builtin_amdgcn_s_sleep(8);
+      r1 = wall_clock64();
+    }
+    const unsigned long long c1 = clock64();
+    out[2 * w] = c1 - c0;
+    out[2 * w + 1] = r1 - r0;
+  }
+}
+
 __global__ __launch_bounds__(256) void copy_kernel(const u32x4* __restrict__ src, u32x4* __restrict__ dst, int64_t n) {
   const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (i < n) __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
@@ -294,6 +312,25 @@ const char* xg_status_string(int status) {
     default:
       return "unknown status";
   }
+}
+
+
+int xg_clock_probe(uint64_t* out, int n_windows, int64_t window_ticks, xg_stream_t stream) {
+  using namespace xg;
+  if (out == nullptr) return XG_ERR_NULL_PTR;
+  if (n_windows < 0 || n_windows > (1 << 16) || window_ticks <= 0 || window_ticks > 1000000) return XG_ERR_BAD_ARG;
+  if (!aligned_to(out, 8)) return XG_ERR_BAD_ALIGN;
+  if (n_windows == 0) return XG_OK;
+  hipLaunchKernelGGL(clock_probe_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, (unsigned long long*)out, n_windows,
+                     (unsigned)window_ticks);
+  return status_from_hip(hipGetLastError());
+}
+
+int64_t xg_wall_clock_khz(void) {
+  int dev = 0, khz = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return 0;
+  if (hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, dev) != hipSuccess) return 0;
+  return khz;
 }
 
 }  // extern "C"
