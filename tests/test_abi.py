@@ -19,7 +19,7 @@ def declared_symbols():
 def test_header_declares_the_expected_entry_points():
     syms = declared_symbols()
     for s in ("xg_rms_norm", "xg_layer_norm", "xg_add_rms_norm", "xg_add_layer_norm", "xg_rms_norm_bwd", "xg_layer_norm_bwd", "xg_slice_cat", "xg_addn",
-              "xg_combo_sum", "xg_slice_sum_cat", "xg_silu_mul", "xg_silu_mul2", "xg_silu_mul2_bwd", "xg_activation", "xg_activation_bwd", "xg_dense", "xg_dense_batched", "xg_dense_at", "xg_dense_glu", "xg_dense_glu_save", "xg_dense_fp8", "xg_slice_cat_check_table", "xg_sdpa", "xg_sdpa_masked", "xg_sdpa_lse", "xg_sdpa_backward", "xg_sdpa_backward_static", "xg_rope", "xg_copy_bytes",
+              "xg_combo_sum", "xg_slice_sum_cat", "xg_silu_mul", "xg_silu_mul2", "xg_silu_mul2_bwd", "xg_activation", "xg_activation_bwd", "xg_dense", "xg_dense_batched", "xg_dense_at", "xg_dense_glu", "xg_dense_glu_save", "xg_dense_fp8", "xg_slice_cat_check_table", "xg_sdpa", "xg_sdpa_masked", "xg_sdpa_lse", "xg_sdpa_backward", "xg_sdpa_backward_static", "xg_rope", "xg_copy_bytes", "xg_clock_probe", "xg_wall_clock_khz",
               "xg_version", "xg_status_string"):
         assert s in syms
 
@@ -58,6 +58,10 @@ def test_argument_validation_needs_no_gpu():
     assert lib.xg_rms_norm(p, None, p, 4, 8, 8, 1e-6, 7, 7, None) == -1  # unknown dtype
     assert lib.xg_rms_norm(p, None, p, 0, 8, 8, 1e-6, 0, 0, None) == 0  # empty: nothing to launch
     assert lib.xg_copy_bytes(p, p, 24, None) == -2  # not a multiple of 16
+    assert lib.xg_clock_probe(None, 4, 2000, None) == -4  # NULL output
+    assert lib.xg_clock_probe(p, 4, 0, None) == -7  # empty window
+    assert lib.xg_clock_probe(p, 1 << 20, 2000, None) == -7  # more windows than the probe takes
+    assert lib.xg_clock_probe(p, 0, 2000, None) == 0  # nothing to launch
     i32 = ctypes.c_int32 * 3
     assert lib.xg_slice_sum_cat(p, p, 2, 4, 8, 32, 8, None, None, 3, 0, None) == -4  # NULL bounds
     assert lib.xg_slice_sum_cat(p, p, 2, 4, 8, 32, 4, i32(0, 0, 0), i32(1, 2, 3), 3, 0, None) == -2  # row stride < cols

@@ -192,3 +192,30 @@ def test_slice_sum_cat_rejects(device):
         _ops().slice_sum_cat(x, list(range(65)), list(range(65)))
     with pytest.raises(NotImplementedError):
         _ops().slice_sum_cat(x[0], [0], [1])
+
+
+def test_clock_probe_reads_a_plausible_engine_clock(device):
+    """xg_clock_probe on a side stream: every window reports wall-clock ticks at least the window length and a
+    shader clock between 50 MHz and 3 GHz; a plain copy beside it does not disturb the launch."""
+    import ctypes
+
+    from xpu_graph_amd import _lib
+
+    lib = _lib.lib()
+    khz = int(lib.xg_wall_clock_khz())
+    assert khz > 0
+    n_win, win_us = 25, 20
+    buf = torch.zeros(2 * n_win, dtype=torch.int64, device=device)
+    a = torch.randn(1 << 22, device=device)
+    b = torch.empty_like(a)
+    side = torch.cuda.Stream()
+    torch.cuda.synchronize()
+    assert lib.xg_clock_probe(ctypes.c_void_p(buf.data_ptr()), n_win, win_us * khz // 1000, ctypes.c_void_p(side.cuda_stream)) == 0
+    for _ in range(20):
+        b.copy_(a)
+    torch.cuda.synchronize()
+    d = buf.view(n_win, 2).double().cpu()
+    assert (d[:, 1] >= win_us * khz // 1000).all()
+    ghz = d[:, 0] / d[:, 1] * khz / 1e6
+    assert ((ghz > 0.05) & (ghz < 3.0)).all(), ghz
+    assert torch.equal(a, b)
