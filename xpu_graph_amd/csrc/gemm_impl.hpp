@@ -1170,6 +1170,140 @@ __global__ __launch_bounds__(kThreads) void gemm_small_kernel(GemmParams p_all) 
   }
 }
 
+// ---- 128 x 128 tiles: between the 64 x 64 kernel and the large tiles -------------------------------------------
+// A problem whose 256 x 256 grid fills a fraction of the compute units, or just over a whole number of rounds, has four
+// times as many 128 x 128 tiles: each of the four wavefronts owns a 64 x 64 quadrant (2 x 2 MFMA tiles) over the whole
+// of K, so every output element sees the same sequence of MFMAs as in the large-tile kernels and the results are the
+// same bits.  Slabs (128 rows x 128 bytes per operand) reach LDS by direct loads, four stages deep (three slabs in
+// flight: a slab of math, 16 MFMAs per wavefront, is far shorter than the memory latency); one workgroup per compute unit.
+// K-contiguous operands of 16-bit types, plain layer.
+constexpr int MID_TILE = 128;
+#ifndef XG_MID_STAGES
+#define XG_MID_STAGES 4
+#endif
+constexpr int MID_STAGES = XG_MID_STAGES;
+constexpr int MID_SLAB_BYTES = MID_TILE * ROW_BYTES;  // 16 KiB per operand per stage
+constexpr int MID_STAGE_BYTES = 2 * MID_SLAB_BYTES;
+constexpr int MID_SMEM_BYTES = MID_STAGES * MID_STAGE_BYTES;  // 128 KiB; the epilogue parks 4 x (64 x 64 fp32) in the same space
+
+template <typename T, typename OT>
+__global__ __launch_bounds__(kThreads) void gemm_mid_kernel(GemmParams p_all) {
+  extern __shared__ __align__(16) char smem[];
+  const GemmParams p = for_batch_entry(p_all);
+  constexpr int EB = Elem<T>::BYTES;
+  static_assert(EB == 2, "16-bit operands");
+  constexpr int SLAB_K = ROW_BYTES / EB;
+
+  int tm, tn;
+  tile_of_block(p, blockIdx.x, gridDim.x, tm, tn);
+  const int m0 = tm * MID_TILE, n0 = tn * MID_TILE;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+  const int l32 = lane & 31, half = lane >> 5;
+
+  // direct loads: per slab and operand 16 wavefront loads of 1 KiB (8 rows), four per wavefront
+  uint32_t a_off[4], b_off[4];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const int r = (q * 4 + wave) * 8 + (lane >> 3);
+    const int slot = lane & 7;
+    int gr = m0 + r;
+    gr = gr < p.M ? gr : p.M - 1;  // rows past the edge re-read the last row; their results are never stored
+    a_off[q] = (uint32_t)(((int64_t)gr * p.lda) * EB + ((slot ^ swz(r)) << 4));
+    int gn = n0 + r;
+    gn = gn < p.N ? gn : p.N - 1;
+    b_off[q] = (uint32_t)(((int64_t)gn * p.ldb) * EB + ((slot ^ swz(r)) << 4));
+  }
+  const char* const a_base = reinterpret_cast<const char*>(p.A);
+  const char* const b_base = reinterpret_cast<const char*>(p.B);
+  auto issue = [&](int kt) {
+    char* dst = smem + (kt % MID_STAGES) * MID_STAGE_BYTES + wave * 1024;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) load_to_lds16(a_base + (int64_t)kt * ROW_BYTES, a_off[q], (uint32_t)(size_t)(lvoid*)(dst + q * 4096));
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+      load_to_lds16(b_base + (int64_t)kt * ROW_BYTES, b_off[q], (uint32_t)(size_t)(lvoid*)(dst + MID_SLAB_BYTES + q * 4096));
+  };
+
+  // fragment rows of this wavefront's quadrant inside a stage; the chunk of k-step ks is (2 ks + half) ^ swz(row)
+  int a_row[2], b_row[2], sw[2];
+#pragma unroll
+  for (int u = 0; u < 2; ++u) {
+    a_row[u] = (wm * 64 + u * 32 + l32) * ROW_BYTES;
+    b_row[u] = MID_SLAB_BYTES + (wn * 64 + u * 32 + l32) * ROW_BYTES;
+    sw[u] = swz(u * 32 + l32);  // swz() looks at the low four bits of the row only: the same for both operands
+  }
+
+  f32x16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+  const int KT = p.K / SLAB_K;
+  for (int s = 0; s < MID_STAGES - 1 && s < KT; ++s) issue(s);
+  for (int kt = 0; kt < KT; ++kt) {
+    // slab kt has landed when only the (at most two) slabs issued after it are in flight: 8 loads each
+    const int after = KT - 1 - kt;  // slabs issued after slab kt: at most MID_STAGES - 2 are in flight, 8 loads each
+    if (after >= MID_STAGES - 2) {
+      wait_vm<8 * (MID_STAGES - 2)>();
+    } else if (after >= 3) {
+      wait_vm<24>();
+    } else if (after == 2) {
+      wait_vm<16>();
+    } else if (after == 1) {
+      wait_vm<8>();
+    } else {
+      wait_vm<0>();
+    }
+    barrier_only();  // slab kt is visible to all, and all are done with slab kt-1 ...
+    if (kt + MID_STAGES - 1 < KT) issue(kt + MID_STAGES - 1);  // ... whose stage takes the next slab
+    const char* st = smem + (kt % MID_STAGES) * MID_STAGE_BYTES;
+    // every fragment of the slab is requested before the first MFMA: one LDS round trip per slab is exposed instead of
+    // one per k-step (one wavefront per SIMD: nobody else hides it)
+    Frag<T> fa[4][2], fb[4][2];
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const int ch = ((ks * 2 + half) ^ sw[u]) << 4;
+        fa[ks][u].v = *reinterpret_cast<const u32x4*>(st + a_row[u] + ch);
+        fb[ks][u].v = *reinterpret_cast<const u32x4*>(st + b_row[u] + ch);
+      }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = mma(fb[ks][j], fa[ks][i], acc[i][j]);
+  }
+  __syncthreads();  // the slabs are dead: the quadrants take their place
+
+  // park this wavefront's quadrant in its own 16 KiB: row r at r * 256, 16-byte chunk (4 columns) c at slot c ^ (r & 15)
+  char* park = smem + wave * (64 * 64 * 4);
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int row = i * 32 + l32;
+        const int chunk = (j * 8 + g * 2 + half) ^ (row & 15);
+        const f32x16& a = acc[i][j];
+        *reinterpret_cast<f32x4*>(park + row * 256 + (chunk << 4)) = f32x4{a[4 * g], a[4 * g + 1], a[4 * g + 2], a[4 * g + 3]};
+      }
+  __syncthreads();
+  const int n = n0 + wn * 64 + (lane & 7) * 8;
+  const bool n_ok = n < p.N;
+  float sv[8], bv[8];
+  column_terms<OT>(p, n, n_ok, 1.f, sv, bv);
+  epilogue_rows_act<OT>(p, park, lane, m0 + wm * 64, n, n_ok, sv, bv, 8);
+}
+
 template <typename K>
 int set_smem_once(K kernel) {
   return allow_dynamic_lds(reinterpret_cast<const void*>(kernel), SMEM_BYTES);
@@ -1254,9 +1388,59 @@ inline bool half_height_wins(int M, int tn, int batch = 1) {
   return t_half < 0.95 * t_full;
 }
 
+// Whether the 128 x 128 kernel beats what launch_gemm would otherwise pick, by measured times (us, bf16, 256 compute
+// units; s = K / 64 slabs): a round of 256 x 256 tiles 10.6 + 1.525 s, of 128 x 256 tiles 0.55 of that, of 128 x 128
+// tiles 4 + 0.57 s (bound by the operand stream: 32 KiB per slab and tile), the 64 x 64 kernel 3 + 0.19 s up to 256
+// tiles and 0.047 s / 64 per tile beyond.  It wins where its grid fills a whole number of rounds and the others'
+// do not: M = 1024, N = K = 4096 46 us against 53 (64 x 64), M = 1024, N = 4096, K = 11008 99 against 129,
+// M = 4096, N = 1024, K = 8192 76 against 88.  Decided from M, N and K alone, never from the batch count: a layer gives
+// the same bits alone and as one entry of a batch (the 64 x 64 kernel adds in another order).
+inline bool mid_tiles_win(const GemmParams& p) {
+#ifdef XG_FORCE_MID
+  return true;
+#endif
+  const double cus = cu_count();
+  const double s = p.K / 64.0;
+  const double t_full = 10.6 + 1.525 * s, t_half = 0.55 * t_full, t_mid = 4.0 + 0.57 * s;
+  const int64_t tm = p.tiles_m, tn = p.tiles_n, t256 = tm * tn;
+  const int64_t t128 = (int64_t)((p.M + 127) / 128) * ((p.N + 127) / 128);
+  const double est_mid = (double)((t128 + (int64_t)cus - 1) / (int64_t)cus) * t_mid;
+  double est;
+  if (t256 <= small_tile_limit()) {
+    const int64_t t64 = (int64_t)((p.M + 63) / 64) * ((p.N + 63) / 64);
+    est = 3.0 + 0.19 * s + (t64 > 256 ? (double)(t64 - 256) * 0.047 * s / 64.0 : 0.0);
+  } else {
+    const int keep = full_tile_columns((int)tm, (int)tn);
+    if (keep != tn) {
+      est = (double)(tm * keep) / cus * t_full + t_half;
+    } else if (half_height_wins(p.M, (int)tn)) {
+      const int64_t th = (int64_t)((p.M + 127) / 128) * tn;
+      est = (double)((th + (int64_t)cus - 1) / (int64_t)cus) * t_half;
+    } else {
+      est = (double)((t256 + (int64_t)cus - 1) / (int64_t)cus) * t_full;
+    }
+  }
+  return est_mid < 0.92 * est;
+}
+
+template <typename T, typename OT>
+int launch_mid(GemmParams p, hipStream_t stream) {
+  auto kernel = gemm_mid_kernel<T, OT>;
+  if (int st = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), MID_SMEM_BYTES)) return st;
+  p.tiles_m = (p.M + MID_TILE - 1) / MID_TILE;
+  p.tiles_n = (p.N + MID_TILE - 1) / MID_TILE;
+  const int64_t tiles = (int64_t)p.tiles_m * p.tiles_n;
+  if (tiles > 0x7fffffffLL) return XG_ERR_TOO_LARGE;
+  hipLaunchKernelGGL(kernel, dim3((unsigned)tiles, (unsigned)p.batch), dim3(kThreads), MID_SMEM_BYTES, stream, p);
+  return status_from_hip(hipGetLastError());
+}
+
 template <typename T, typename OT, BLayout BL>
 int launch_gemm(const GemmParams& p, hipStream_t stream) {
   if (!dma_ok<T>(p, BL)) return launch_kernel(gemm_staged_kernel<T, OT, BL>, p, stream);
+  if constexpr (Elem<T>::BYTES == 2 && BL == BLayout::KMajor) {
+    if (mid_tiles_win(p)) return launch_mid<T, OT>(p, stream);
+  }
   // decided per batch entry: the 64 x 64 kernel splits K between its waves and so adds in another order than the
   // large tiles; a layer must give the same bits whether it runs alone or as one entry of a batch
   if ((int64_t)p.tiles_m * p.tiles_n <= small_tile_limit()) return launch_small<T, OT, BL>(p, stream);
