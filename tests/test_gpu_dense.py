@@ -146,22 +146,25 @@ def test_dense_c4_full_size_permutation_properties(device):
     assert torch.equal(glu, ops.silu_mul2(z, z))
 
 
+@pytest.mark.parametrize("weight_trans", [True, False])
 @pytest.mark.parametrize("M,N,K", [(1024, 4096, 4096), (1024, 4096, 11008), (1000, 4000, 4096), (512, 8192, 8192)])
-def test_dense_128_tile_kernel_matches_the_large_tiles(device, M, N, K):
-    """Shapes whose 128 x 128 grid fills a round of compute units ([N, K] weights) take the 128 x 128 kernel: every
+def test_dense_128_tile_kernel_matches_the_large_tiles(device, M, N, K, weight_trans):
+    """Shapes whose 128 x 128 grid fills a round of compute units take the 128 x 128 kernel (either weight layout): every
     output element sees the MFMAs of the large-tile kernels in the same order, so the rows come out BIT FOR BIT as the
     same rows of a four times taller problem (which runs on large tiles), and close to the fp32 anchor."""
     g = torch.Generator().manual_seed(M + N)
     x = torch.randn(4 * M, K, generator=g).bfloat16().to(device)
     W = (torch.randn(N, K, generator=g) / K**0.5).bfloat16().to(device)
+    if not weight_trans:
+        W = W.t().contiguous()
     b = torch.randn(N, generator=g).bfloat16().to(device)
     res = torch.randn(4 * M, N, generator=g).bfloat16().to(device)
     ops = _ops()
-    tall = ops.dense(x, W, True, b, res, "silu")
+    tall = ops.dense(x, W, weight_trans, b, res, "silu")
     for r0 in (0, M, 3 * M):
-        got = ops.dense(x[r0 : r0 + M], W, True, b, res[r0 : r0 + M], "silu")
+        got = ops.dense(x[r0 : r0 + M], W, weight_trans, b, res[r0 : r0 + M], "silu")
         assert torch.equal(got, tall[r0 : r0 + M])
-    close(tall[:M], ref32(x[:M], W, True, b, res[:M], "silu"), K)
+    close(tall[:M], ref32(x[:M], W, weight_trans, b, res[:M], "silu"), K)
 
 
 def test_dense_rejects_what_the_kernel_cannot_take(device):

@@ -1176,7 +1176,7 @@ __global__ __launch_bounds__(kThreads) void gemm_small_kernel(GemmParams p_all) 
 // of K, so every output element sees the same sequence of MFMAs as in the large-tile kernels and the results are the
 // same bits.  Slabs (128 rows x 128 bytes per operand) reach LDS by direct loads, four stages deep (three slabs in
 // flight: a slab of math, 16 MFMAs per wavefront, is far shorter than the memory latency); one workgroup per compute unit.
-// K-contiguous operands of 16-bit types, plain layer.
+// 16-bit types, both weight layouts, plain layer.
 constexpr int MID_TILE = 128;
 #ifndef XG_MID_STAGES
 #define XG_MID_STAGES 4
@@ -1186,7 +1186,7 @@ constexpr int MID_SLAB_BYTES = MID_TILE * ROW_BYTES;  // 16 KiB per operand per 
 constexpr int MID_STAGE_BYTES = 2 * MID_SLAB_BYTES;
 constexpr int MID_SMEM_BYTES = MID_STAGES * MID_STAGE_BYTES;  // 128 KiB; the epilogue parks 4 x (64 x 64 fp32) in the same space
 
-template <typename T, typename OT>
+template <typename T, typename OT, BLayout BL>
 __global__ __launch_bounds__(kThreads) void gemm_mid_kernel(GemmParams p_all) {
   extern __shared__ __align__(16) char smem[];
   const GemmParams p = for_batch_entry(p_all);
@@ -1200,9 +1200,12 @@ __global__ __launch_bounds__(kThreads) void gemm_mid_kernel(GemmParams p_all) {
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave >> 1, wn = wave & 1;
-  const int l32 = lane & 31, half = lane >> 5;
+  const int l32 = lane & 31, half = lane >> 5, p16 = lane & 15, blk = (lane >> 4) & 1;
 
-  // direct loads: per slab and operand 16 wavefront loads of 1 KiB (8 rows), four per wavefront
+  // direct loads: per slab and operand 16 wavefront loads of 1 KiB, four per wavefront.  A, and B when K-contiguous: 8
+  // rows of 128 bytes per load.  An N-contiguous B slab is [64 k][128 n], 256 bytes per k row: a load covers 4 k rows,
+  // lane i lands at chunk i & 15 of row i >> 4, and the four 64-byte granules of a row are XOR-ed with k & 3 so that
+  // the four k rows a 16-lane group of the transposing read touches fall on different banks.
   uint32_t a_off[4], b_off[4];
 #pragma unroll
   for (int q = 0; q < 4; ++q) {
@@ -1211,19 +1214,28 @@ __global__ __launch_bounds__(kThreads) void gemm_mid_kernel(GemmParams p_all) {
     int gr = m0 + r;
     gr = gr < p.M ? gr : p.M - 1;  // rows past the edge re-read the last row; their results are never stored
     a_off[q] = (uint32_t)(((int64_t)gr * p.lda) * EB + ((slot ^ swz(r)) << 4));
-    int gn = n0 + r;
-    gn = gn < p.N ? gn : p.N - 1;
-    b_off[q] = (uint32_t)(((int64_t)gn * p.ldb) * EB + ((slot ^ swz(r)) << 4));
+    if constexpr (BL == BLayout::KMajor) {
+      int gn = n0 + r;
+      gn = gn < p.N ? gn : p.N - 1;
+      b_off[q] = (uint32_t)(((int64_t)gn * p.ldb) * EB + ((slot ^ swz(r)) << 4));
+    } else {
+      const int kr = (q * 4 + wave) * 4 + (lane >> 4);
+      const int chunk = (((p16 >> 2) ^ (kr & 3)) << 2) | (p16 & 3);  // logical 16-byte chunk (8 columns) this LDS slot holds
+      int gc = n0 + chunk * 8;
+      gc = gc < p.N ? gc : p.N - 8;  // N % 8 == 0 is checked on the host
+      b_off[q] = (uint32_t)(((int64_t)kr * p.ldb + gc) * EB);
+    }
   }
   const char* const a_base = reinterpret_cast<const char*>(p.A);
   const char* const b_base = reinterpret_cast<const char*>(p.B);
+  const int64_t b_step = BL == BLayout::KMajor ? (int64_t)ROW_BYTES : (int64_t)SLAB_K * p.ldb * EB;
   auto issue = [&](int kt) {
     char* dst = smem + (kt % MID_STAGES) * MID_STAGE_BYTES + wave * 1024;
 #pragma unroll
     for (int q = 0; q < 4; ++q) load_to_lds16(a_base + (int64_t)kt * ROW_BYTES, a_off[q], (uint32_t)(size_t)(lvoid*)(dst + q * 4096));
 #pragma unroll
     for (int q = 0; q < 4; ++q)
-      load_to_lds16(b_base + (int64_t)kt * ROW_BYTES, b_off[q], (uint32_t)(size_t)(lvoid*)(dst + MID_SLAB_BYTES + q * 4096));
+      load_to_lds16(b_base + kt * b_step, b_off[q], (uint32_t)(size_t)(lvoid*)(dst + MID_SLAB_BYTES + q * 4096));
   };
 
   // fragment rows of this wavefront's quadrant inside a stage; the chunk of k-step ks is (2 ks + half) ^ swz(row)
@@ -1231,8 +1243,16 @@ __global__ __launch_bounds__(kThreads) void gemm_mid_kernel(GemmParams p_all) {
 #pragma unroll
   for (int u = 0; u < 2; ++u) {
     a_row[u] = (wm * 64 + u * 32 + l32) * ROW_BYTES;
-    b_row[u] = MID_SLAB_BYTES + (wn * 64 + u * 32 + l32) * ROW_BYTES;
     sw[u] = swz(u * 32 + l32);  // swz() looks at the low four bits of the row only: the same for both operands
+    if constexpr (BL == BLayout::KMajor) {
+      b_row[u] = MID_SLAB_BYTES + (wn * 64 + u * 32 + l32) * ROW_BYTES;
+    } else {
+      // transposing read of k-step 0: k row half * 8 + p16 / 4, granule (32 columns) 2 wn + u at slot granule ^ (k & 3),
+      // inside it 32 bytes per 16-lane block and 8 bytes per lane; k-step ks is 16 rows (4 KiB) further, the upper four
+      // k of a lane 4 rows (1 KiB) further (same k & 3, same slot)
+      const int kr = half * 8 + (p16 >> 2);
+      b_row[u] = MID_SLAB_BYTES + kr * 256 + ((((wn * 2 + u) ^ (kr & 3)) & 3) << 6) + (blk << 5) + ((p16 & 3) << 3);
+    }
   }
 
   f32x16 acc[2][2];
@@ -1271,7 +1291,14 @@ __global__ __launch_bounds__(kThreads) void gemm_mid_kernel(GemmParams p_all) {
       for (int u = 0; u < 2; ++u) {
         const int ch = ((ks * 2 + half) ^ sw[u]) << 4;
         fa[ks][u].v = *reinterpret_cast<const u32x4*>(st + a_row[u] + ch);
-        fb[ks][u].v = *reinterpret_cast<const u32x4*>(st + b_row[u] + ch);
+        if constexpr (BL == BLayout::KMajor) {
+          fb[ks][u].v = *reinterpret_cast<const u32x4*>(st + b_row[u] + ch);
+        } else {
+          const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(st + b_row[u] + ks * 4096));
+          const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(st + b_row[u] + ks * 4096 + 1024));
+          const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
+          fb[ks][u].v = u32x4{l2.x, l2.y, h2.x, h2.y};
+        }
       }
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -1423,9 +1450,9 @@ inline bool mid_tiles_win(const GemmParams& p) {
   return est_mid < 0.92 * est;
 }
 
-template <typename T, typename OT>
+template <typename T, typename OT, BLayout BL>
 int launch_mid(GemmParams p, hipStream_t stream) {
-  auto kernel = gemm_mid_kernel<T, OT>;
+  auto kernel = gemm_mid_kernel<T, OT, BL>;
   if (int st = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), MID_SMEM_BYTES)) return st;
   p.tiles_m = (p.M + MID_TILE - 1) / MID_TILE;
   p.tiles_n = (p.N + MID_TILE - 1) / MID_TILE;
@@ -1438,8 +1465,8 @@ int launch_mid(GemmParams p, hipStream_t stream) {
 template <typename T, typename OT, BLayout BL>
 int launch_gemm(const GemmParams& p, hipStream_t stream) {
   if (!dma_ok<T>(p, BL)) return launch_kernel(gemm_staged_kernel<T, OT, BL>, p, stream);
-  if constexpr (Elem<T>::BYTES == 2 && BL == BLayout::KMajor) {
-    if (mid_tiles_win(p)) return launch_mid<T, OT>(p, stream);
+  if constexpr (Elem<T>::BYTES == 2) {
+    if (mid_tiles_win(p)) return launch_mid<T, OT, BL>(p, stream);
   }
   // decided per batch entry: the 64 x 64 kernel splits K between its waves and so adds in another order than the
   // large tiles; a layer must give the same bits whether it runs alone or as one entry of a batch
