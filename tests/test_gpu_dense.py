@@ -167,6 +167,26 @@ def test_dense_128_tile_kernel_matches_the_large_tiles(device, M, N, K, weight_t
     close(tall[:M], ref32(x[:M], W, weight_trans, b, res[:M], "silu"), K)
 
 
+@pytest.mark.parametrize("weight_trans", [True, False])
+@pytest.mark.parametrize("M,N,K", [(1536, 11008, 4096), (3072, 6144, 1024), (1300, 11008, 512), (4352, 4096, 2048)])
+def test_dense_grid_of_a_round_and_a_little_runs_in_two_launches_with_the_same_bits(device, M, N, K, weight_trans):
+    """A tile grid of whole rounds of compute units plus a few tiles is split: full tiles on the columns (or rows) that
+    fill the rounds, a second launch for the strip that is left.  Every kernel involved adds in the same order, so the
+    rows must equal the same rows of a taller problem BIT FOR BIT, bias, residual and activation included."""
+    g = torch.Generator().manual_seed(M * 3 + N)
+    x = torch.randn(2 * M + 512, K, generator=g).bfloat16().to(device)
+    W = (torch.randn(N, K, generator=g) / K**0.5).bfloat16().to(device)
+    if not weight_trans:
+        W = W.t().contiguous()
+    b = torch.randn(N, generator=g).bfloat16().to(device)
+    res = torch.randn(2 * M + 512, N, generator=g).bfloat16().to(device)
+    ops = _ops()
+    tall = ops.dense(x, W, weight_trans, b, res, "gelu")
+    got = ops.dense(x[:M], W, weight_trans, b, res[:M], "gelu")
+    assert torch.equal(got, tall[:M])
+    close(got[::7], ref32(x[:M:7], W, weight_trans, b, res[:M:7], "gelu"), K)
+
+
 def test_dense_rejects_what_the_kernel_cannot_take(device):
     from xpu_graph_amd._lib import XgError
 

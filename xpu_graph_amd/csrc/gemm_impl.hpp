@@ -1415,6 +1415,26 @@ inline bool half_height_wins(int M, int tn, int batch = 1) {
   return t_half < 0.95 * t_full;
 }
 
+// Estimated time (us) of the single launch that launch_gemm picks without the 128 x 128 kernel: the 64 x 64 kernel for
+// few tiles, full tiles with the last tile columns at half height, half-height tiles, or full tiles.
+inline double single_launch_estimate(const GemmParams& p) {
+  const double cus = cu_count();
+  const double s = p.K / 64.0;
+  const double t_full = 10.6 + 1.525 * s, t_half = 0.55 * t_full;
+  const int64_t tm = p.tiles_m, tn = p.tiles_n, t256 = tm * tn;
+  if (t256 <= small_tile_limit()) {
+    const int64_t t64 = (int64_t)((p.M + 63) / 64) * ((p.N + 63) / 64);
+    return 3.0 + 0.19 * s + (t64 > 256 ? (double)(t64 - 256) * 0.047 * s / 64.0 : 0.0);
+  }
+  const int keep = full_tile_columns((int)tm, (int)tn);
+  if (keep != tn) return (double)(tm * keep) / cus * t_full + t_half;
+  if (half_height_wins(p.M, (int)tn)) {
+    const int64_t th = (int64_t)((p.M + 127) / 128) * tn;
+    return (double)((th + (int64_t)cus - 1) / (int64_t)cus) * t_half;
+  }
+  return (double)((t256 + (int64_t)cus - 1) / (int64_t)cus) * t_full;
+}
+
 // Whether the 128 x 128 kernel beats what launch_gemm would otherwise pick, by measured times (us, bf16, 256 compute
 // units; s = K / 64 slabs): a round of 256 x 256 tiles 10.6 + 1.525 s, of 128 x 256 tiles 0.55 of that, of 128 x 128
 // tiles 4 + 0.57 s (bound by the operand stream: 32 KiB per slab and tile), the 64 x 64 kernel 3 + 0.19 s up to 256
@@ -1428,26 +1448,10 @@ inline bool mid_tiles_win(const GemmParams& p) {
 #endif
   const double cus = cu_count();
   const double s = p.K / 64.0;
-  const double t_full = 10.6 + 1.525 * s, t_half = 0.55 * t_full, t_mid = 4.0 + 0.57 * s;
-  const int64_t tm = p.tiles_m, tn = p.tiles_n, t256 = tm * tn;
+  const double t_mid = 4.0 + 0.57 * s;
   const int64_t t128 = (int64_t)((p.M + 127) / 128) * ((p.N + 127) / 128);
   const double est_mid = (double)((t128 + (int64_t)cus - 1) / (int64_t)cus) * t_mid;
-  double est;
-  if (t256 <= small_tile_limit()) {
-    const int64_t t64 = (int64_t)((p.M + 63) / 64) * ((p.N + 63) / 64);
-    est = 3.0 + 0.19 * s + (t64 > 256 ? (double)(t64 - 256) * 0.047 * s / 64.0 : 0.0);
-  } else {
-    const int keep = full_tile_columns((int)tm, (int)tn);
-    if (keep != tn) {
-      est = (double)(tm * keep) / cus * t_full + t_half;
-    } else if (half_height_wins(p.M, (int)tn)) {
-      const int64_t th = (int64_t)((p.M + 127) / 128) * tn;
-      est = (double)((th + (int64_t)cus - 1) / (int64_t)cus) * t_half;
-    } else {
-      est = (double)((t256 + (int64_t)cus - 1) / (int64_t)cus) * t_full;
-    }
-  }
-  return est_mid < 0.92 * est;
+  return est_mid < 0.92 * single_launch_estimate(p);
 }
 
 template <typename T, typename OT, BLayout BL>
@@ -1462,6 +1466,80 @@ int launch_mid(GemmParams p, hipStream_t stream) {
   return status_from_hip(hipGetLastError());
 }
 
+// ---- two launches for a grid of a whole number of rounds plus a little --------------------------------------------
+// Measured round times as in mid_tiles_win (us; s = K / 64 slabs).
+struct RoundTimes {
+  double full, half, mid;
+  explicit RoundTimes(int K) {
+    const double s = K / 64.0;
+    full = 10.6 + 1.525 * s;
+    half = 0.55 * full;
+    mid = 4.0 + 0.57 * s;
+  }
+};
+enum class TileKind { Full, Half, Mid };
+
+// Cheapest of the three kernels that add in the large-tile order for an M x N problem, and its estimated time.
+inline double best_same_order_plan(int M, int N, const RoundTimes& t, TileKind& kind) {
+  const int64_t cus = cu_count();
+  auto rounds = [&](int64_t tiles) { return (double)((tiles + cus - 1) / cus); };
+  const int64_t tn = (N + BN - 1) / BN;
+  const double e_full = rounds((int64_t)((M + BM - 1) / BM) * tn) * t.full;
+  const double e_half = rounds((int64_t)((M + 127) / 128) * tn) * t.half;
+  const double e_mid = rounds((int64_t)((M + 127) / 128) * ((N + 127) / 128)) * t.mid;
+  kind = TileKind::Full;
+  double best = e_full;
+  if (e_half < best) best = e_half, kind = TileKind::Half;
+  if (e_mid < best) best = e_mid, kind = TileKind::Mid;
+  return best;
+}
+
+// A grid of r whole rounds of full tiles and a few more pays a whole extra round for them (or runs on half-height tiles
+// throughout, which quantise the same way).  Instead: full tiles on as many tile columns (or tile rows) as fill r rounds,
+// then a second launch for the strip that is left, with whichever of the full / half-height / 128 x 128 kernels takes
+// it fastest -- all three add in the same order, so the result is the same bits as one launch.  Taken when the estimate
+// beats the single launch's by 8 %: M = 1536, N = 11008 169 -> 148 us, M = 3072, N = 6144 170 -> 150 us (K = 4096).
+struct TwoPart {
+  bool by_rows;   // the strip is the last rows (else the last columns)
+  int split;      // first row / column of the strip
+  TileKind rest;  // kernel of the strip
+};
+inline bool two_part_plan(const GemmParams& p, double est_single, TwoPart& out) {
+  const int64_t cus = cu_count();
+  const RoundTimes t(p.K);
+  const int64_t tm = p.tiles_m, tn = p.tiles_n;
+  const int64_t r = tm * tn / cus;
+  if (r < 1 || tm * tn == r * cus) return false;
+  double best = 0.92 * est_single;
+  bool found = false;
+  const double gap = 3.0;  // second launch
+  const int64_t keep_c = r * cus / tm < tn - 1 ? r * cus / tm : tn - 1;
+  if (keep_c >= 1) {
+    TileKind k;
+    const double e = (double)((tm * keep_c + cus - 1) / cus) * t.full + best_same_order_plan(p.M, p.N - (int)(keep_c * BN), t, k) + gap;
+    if (e < best) best = e, found = true, out = TwoPart{false, (int)(keep_c * BN), k};
+  }
+  const int64_t keep_r = r * cus / tn < tm - 1 ? r * cus / tn : tm - 1;
+  if (keep_r >= 1) {
+    TileKind k;
+    const double e = (double)((keep_r * tn + cus - 1) / cus) * t.full + best_same_order_plan(p.M - (int)(keep_r * BM), p.N, t, k) + gap;
+    if (e < best) best = e, found = true, out = TwoPart{true, (int)(keep_r * BM), k};
+  }
+  return found;
+}
+
+template <typename T, typename OT, BLayout BL>
+int launch_same_order(GemmParams p, TileKind kind, hipStream_t stream) {
+  p.tiles_n = (p.N + BN - 1) / BN;
+  if (kind == TileKind::Mid) return launch_mid<T, OT, BL>(p, stream);
+  if (kind == TileKind::Half) {
+    p.tiles_m = (p.M + 127) / 128;
+    return launch_kernel(gemm_dma_half_kernel<T, OT, BL>, p, stream);
+  }
+  p.tiles_m = (p.M + BM - 1) / BM;
+  return launch_kernel(gemm_dma_kernel<T, OT, BL>, p, stream);
+}
+
 template <typename T, typename OT, BLayout BL>
 int launch_gemm(const GemmParams& p, hipStream_t stream) {
   if (!dma_ok<T>(p, BL)) return launch_kernel(gemm_staged_kernel<T, OT, BL>, p, stream);
@@ -1473,6 +1551,32 @@ int launch_gemm(const GemmParams& p, hipStream_t stream) {
   if ((int64_t)p.tiles_m * p.tiles_n <= small_tile_limit()) return launch_small<T, OT, BL>(p, stream);
   // the split of the last, partial round is worked out for one tile grid: batched layers run whole tiles
   const int keep = p.batch > 1 ? p.tiles_n : full_tile_columns(p.tiles_m, p.tiles_n);
+  if constexpr (Elem<T>::BYTES == 2) {
+    TwoPart tp;
+#ifndef XG_NO_TWO_PART
+    if (p.batch == 1 && two_part_plan(p, single_launch_estimate(p), tp)) {
+      constexpr int EB2 = Elem<T>::BYTES;
+      GemmParams first = p, rest = p;
+      if (tp.by_rows) {
+        first.M = tp.split;
+        rest.M = p.M - tp.split;
+        rest.A = reinterpret_cast<const char*>(p.A) + (int64_t)tp.split * p.lda * EB2;
+        if (p.res) rest.res = reinterpret_cast<const char*>(p.res) + (int64_t)tp.split * p.ldr * (int64_t)sizeof(OT);
+        rest.out = reinterpret_cast<char*>(p.out) + (int64_t)tp.split * p.ldc * (int64_t)sizeof(OT);
+      } else {
+        const int64_t n_split = tp.split;
+        first.N = tp.split;
+        rest.N = p.N - tp.split;
+        rest.B = reinterpret_cast<const char*>(p.B) + (BL == BLayout::KMajor ? n_split * p.ldb * EB2 : n_split * EB2);
+        if (p.bias) rest.bias = reinterpret_cast<const char*>(p.bias) + n_split * (p.bias_f32 ? 4 : (int64_t)sizeof(OT));
+        if (p.res) rest.res = reinterpret_cast<const char*>(p.res) + n_split * (int64_t)sizeof(OT);
+        rest.out = reinterpret_cast<char*>(p.out) + n_split * (int64_t)sizeof(OT);
+      }
+      if (int st = launch_same_order<T, OT, BL>(first, TileKind::Full, stream)) return st;
+      return launch_same_order<T, OT, BL>(rest, tp.rest, stream);
+    }
+#endif
+  }
   if (keep == p.tiles_n) {
     if (half_height_wins(p.M, p.tiles_n, p.batch)) {
       GemmParams h = p;
