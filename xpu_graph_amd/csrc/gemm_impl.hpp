@@ -465,12 +465,10 @@ __device__ __forceinline__ void epilogue(const GemmParams& p, const Lane& L, f32
     const bool n_ok = n < p.N;  // N % 8 == 0: the 8 columns are in or out together
     float sv[8], bv[8];
     column_terms<OT>(p, n, n_ok, a_sc, sv, bv);
-#ifndef XG_NO_EPI_WAIT
     // The bias and scale loads are waited for HERE.  Left pending into the row loop, the compiler's wait (it counts
     // loads and stores with one counter) would sit inside the loop and also wait, in every pass, for the previous
     // pass's output store to be acknowledged by memory.
     wait_vm<0>();
-#endif
     epilogue_rows_act<OT>(p, park, L.lane, m_base, n, n_ok, sv, bv, NI * 4);
   });
 }
@@ -1178,10 +1176,7 @@ __global__ __launch_bounds__(kThreads) void gemm_small_kernel(GemmParams p_all) 
 // flight: a slab of math, 16 MFMAs per wavefront, is far shorter than the memory latency); one workgroup per compute unit.
 // 16-bit types, both weight layouts, plain layer.
 constexpr int MID_TILE = 128;
-#ifndef XG_MID_STAGES
-#define XG_MID_STAGES 4
-#endif
-constexpr int MID_STAGES = XG_MID_STAGES;
+constexpr int MID_STAGES = 4;
 constexpr int MID_SLAB_BYTES = MID_TILE * ROW_BYTES;  // 16 KiB per operand per stage
 constexpr int MID_STAGE_BYTES = 2 * MID_SLAB_BYTES;
 constexpr int MID_SMEM_BYTES = MID_STAGES * MID_STAGE_BYTES;  // 128 KiB; the epilogue parks 4 x (64 x 64 fp32) in the same space
@@ -1443,9 +1438,6 @@ inline double single_launch_estimate(const GemmParams& p) {
 // M = 4096, N = 1024, K = 8192 76 against 88.  Decided from M, N and K alone, never from the batch count: a layer gives
 // the same bits alone and as one entry of a batch (the 64 x 64 kernel adds in another order).
 inline bool mid_tiles_win(const GemmParams& p) {
-#ifdef XG_FORCE_MID
-  return true;
-#endif
   const double cus = cu_count();
   const double s = p.K / 64.0;
   const double t_mid = 4.0 + 0.57 * s;
@@ -1553,7 +1545,6 @@ int launch_gemm(const GemmParams& p, hipStream_t stream) {
   const int keep = p.batch > 1 ? p.tiles_n : full_tile_columns(p.tiles_m, p.tiles_n);
   if constexpr (Elem<T>::BYTES == 2) {
     TwoPart tp;
-#ifndef XG_NO_TWO_PART
     if (p.batch == 1 && two_part_plan(p, single_launch_estimate(p), tp)) {
       constexpr int EB2 = Elem<T>::BYTES;
       GemmParams first = p, rest = p;
@@ -1575,7 +1566,6 @@ int launch_gemm(const GemmParams& p, hipStream_t stream) {
       if (int st = launch_same_order<T, OT, BL>(first, TileKind::Full, stream)) return st;
       return launch_same_order<T, OT, BL>(rest, tp.rest, stream);
     }
-#endif
   }
   if (keep == p.tiles_n) {
     if (half_height_wins(p.M, p.tiles_n, p.batch)) {

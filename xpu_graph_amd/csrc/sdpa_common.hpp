@@ -66,9 +66,6 @@ __device__ __forceinline__ void grouped_block_order(int id, int n_prob, int n_bl
 }
 // Problems per XCD taken at a time by grouped_block_order: all of them up to eight (0: no grouping).
 inline int block_order_group(int64_t n_prob) {
-#ifdef XG_NO_BLOCK_GROUPS
-  return 0;
-#endif
   if (n_prob % 8 != 0 || n_prob / 8 < 2) return 0;
   return (int)(n_prob / 8 < 8 ? n_prob / 8 : 8);
 }
