@@ -187,6 +187,28 @@ def test_dense_grid_of_a_round_and_a_little_runs_in_two_launches_with_the_same_b
     close(got[::7], ref32(x[:M:7], W, weight_trans, b, res[:M:7], "gelu"), K)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M,N,K", [(1, 4096, 4096), (3, 11008, 4096), (16, 4096, 11008), (13, 1032, 640), (32, 4096, 512), (17, 520, 1152)])
+def test_dense_decode_sizes_stream_the_weights(device, dtype, M, N, K):
+    """A few activation rows against [N, K] weights take the row-streaming kernel (16 output columns per workgroup, K
+    split over its four waves): against the fp32 anchor with bias, residual and every activation, ragged M and N, and a
+    batch of such layers must equal the layers one by one bit for bit."""
+    g = torch.Generator().manual_seed(M + N + K)
+    x = torch.randn(M, K, generator=g).to(dtype).to(device)
+    W = (torch.randn(N, K, generator=g) / K**0.5).to(dtype).to(device)
+    b = torch.randn(N, generator=g).to(dtype).to(device)
+    res = torch.randn(M, N, generator=g).to(dtype).to(device)
+    ops = _ops()
+    for act in ("none", "silu", "gelu"):
+        close(ops.dense(x, W, True, b, res, act), ref32(x, W, True, b, res, act), K)
+    close(ops.dense(x, W, True, None, None, "relu"), ref32(x, W, True, None, None, "relu"), K)
+    xb = torch.randn(3, M, K, generator=g).to(dtype).to(device)
+    wb = (torch.randn(3, N, K, generator=g) / K**0.5).to(dtype).to(device)
+    got = ops.dense_batched(xb, wb, True, None, None, "none")
+    for i in range(3):
+        assert torch.equal(got[i], ops.dense(xb[i], wb[i], True, None, None, "none"))
+
+
 def test_dense_rejects_what_the_kernel_cannot_take(device):
     from xpu_graph_amd._lib import XgError
 

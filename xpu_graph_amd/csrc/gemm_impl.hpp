@@ -193,6 +193,15 @@ __device__ __forceinline__ f32x16 mma(const Frag<uint8_t>& a, const Frag<uint8_t
   return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(x, y, c, 0, 0, 0, 127, 0, 127);
 }
 
+// 16 x 16 x 32 (16-bit types): lane = 16 q + l16 supplies row (or column) l16 and the 8 k of chunk q; the accumulator holds
+// output rows 4 q .. 4 q + 3 (rows of a) at column l16 (row of b).
+__device__ __forceinline__ f32x4 mma16(const Frag<bf16_t>& a, const Frag<bf16_t>& b, f32x4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a.v), __builtin_bit_cast(bf16x8, b.v), c, 0, 0, 0);
+}
+__device__ __forceinline__ f32x4 mma16(const Frag<f16_t>& a, const Frag<f16_t>& b, f32x4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a.v), __builtin_bit_cast(f16x8, b.v), c, 0, 0, 0);
+}
+
 // Workgroup barrier without the memory fence of __syncthreads(), which waits for EVERY outstanding memory
 // operation.  The caller waits for what it needs with explicit s_waitcnt.
 __device__ __forceinline__ void barrier_only() {
@@ -1168,6 +1177,96 @@ __global__ __launch_bounds__(kThreads) void gemm_small_kernel(GemmParams p_all) 
   }
 }
 
+// ---- at most 32 rows: a decode step ---------------------------------------------------------------------------
+// out[M <= 32, N] = A W^T with K-contiguous 16-bit W is weight streaming: every weight is used M times.  A workgroup owns 16
+// output columns, i.e. 16 whole rows of W, and its four wavefronts a quarter of K each, so a wavefront walks its 16 rows
+// front to back in 64-byte steps -- sequential in memory, where the 64 x 64 kernel's slabs take 128 bytes of each of 64 rows
+// 2 K bytes apart.  Fragments go from global memory straight to registers in 16 x 16 x 32 MFMA layout (lane = 16 q + l16:
+// row l16, k chunk q), U k-steps of loads in flight behind U k-steps of math; the four partial tiles meet in LDS.
+// The accumulation order is this kernel's own, as the 64 x 64 kernel's is.
+template <typename T, typename OT, int MT>
+__global__ __launch_bounds__(kThreads) void gemm_skinny_kernel(GemmParams p_all) {
+  static_assert(Elem<T>::BYTES == 2, "16-bit operands");
+  constexpr int U = MT == 1 ? 8 : 4;
+  __shared__ float part[4][MT][16][16];
+  const GemmParams p = for_batch_entry(p_all);
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l16 = lane & 15, q = lane >> 4;
+  const int n0 = blockIdx.x * 16;
+  int n = n0 + l16;
+  n = n < p.N ? n : p.N - 1;  // columns past the edge re-read the last row of W; their results are never stored
+  const int kq = p.K / 4;     // K % 128 == 0 is checked on the host: every quarter is a whole number of k-steps
+  const T* w_at = reinterpret_cast<const T*>(p.B) + (int64_t)n * p.ldb + wave * kq + 8 * q;
+  const T* x_at[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    int m = 16 * t + l16;
+    m = m < p.M ? m : p.M - 1;
+    x_at[t] = reinterpret_cast<const T*>(p.A) + (int64_t)m * p.lda + wave * kq + 8 * q;
+  }
+  f32x4 acc[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  Frag<T> fw[2][U], fx[2][MT][U];
+  auto load = [&](int buf, int k) {  // k-steps k .. k + U - 1 of this wavefront's quarter
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      fw[buf][u].v = *reinterpret_cast<const u32x4*>(w_at + (k + u) * 32);
+#pragma unroll
+      for (int t = 0; t < MT; ++t) fx[buf][t][u].v = *reinterpret_cast<const u32x4*>(x_at[t] + (k + u) * 32);
+    }
+  };
+  auto math = [&](int buf) {
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int t = 0; t < MT; ++t) acc[t] = mma16(fw[buf][u], fx[buf][t][u], acc[t]);
+  };
+  const int steps = kq / 32, groups = steps / U;
+  if (groups > 0) load(0, 0);
+  for (int g = 0; g + 1 < groups; g += 2) {  // two groups per trip: the buffer indices stay compile-time
+    load(1, (g + 1) * U);
+    math(0);
+    if (g + 2 < groups) load(0, (g + 2) * U);
+    math(1);
+  }
+  if (groups & 1) math(0);
+  for (int k = groups * U; k < steps; ++k) {  // what does not fill a group
+    Frag<T> a, b;
+    a.v = *reinterpret_cast<const u32x4*>(w_at + k * 32);
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+      b.v = *reinterpret_cast<const u32x4*>(x_at[t] + k * 32);
+      acc[t] = mma16(a, b, acc[t]);
+    }
+  }
+
+  // accumulator t of a lane: output rows 16 t + l16 (A rows), columns n0 + 4 q .. + 3
+#pragma unroll
+  for (int t = 0; t < MT; ++t)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) part[wave][t][4 * q + e][l16] = acc[t][e];
+  __syncthreads();
+  for (int idx = tid; idx < MT * 256; idx += kThreads) {
+    const int nl = idx & 15, ml = (idx >> 4) & 15, t = idx >> 8;
+    const int m = 16 * t + ml, nn = n0 + nl;
+    if (m >= p.M || nn >= p.N) continue;
+    float v = (part[0][t][nl][ml] + part[1][t][nl][ml]) + (part[2][t][nl][ml] + part[3][t][nl][ml]);
+    if (p.bias) v += p.bias_f32 ? reinterpret_cast<const float*>(p.bias)[nn] : to_f32(reinterpret_cast<const OT*>(p.bias)[nn]);
+    if (p.res) v += to_f32(reinterpret_cast<const OT*>(p.res)[(int64_t)m * p.ldr + nn]);
+    switch (p.act) {
+      case XG_ACT_RELU: v = fmaxf(v, 0.f); break;
+      case XG_ACT_GELU: v = 0.5f * v * (1.f + erff(v * 0.70710678118654752f)); break;
+      case XG_ACT_SILU: v = silu_f32(v); break;
+      case XG_ACT_SIGMOID: v = sigmoid_f32(v); break;
+      default: break;
+    }
+    reinterpret_cast<OT*>(p.out)[(int64_t)m * p.ldc + nn] = from_f32<OT>(v);
+  }
+}
+
 // ---- 128 x 128 tiles: between the 64 x 64 kernel and the large tiles -------------------------------------------
 // A problem whose 256 x 256 grid fills a fraction of the compute units, or just over a whole number of rounds, has four
 // times as many 128 x 128 tiles: each of the four wavefronts owns a 64 x 64 quadrant (2 x 2 MFMA tiles) over the whole
@@ -1446,6 +1545,27 @@ inline bool mid_tiles_win(const GemmParams& p) {
   return est_mid < 0.92 * single_launch_estimate(p);
 }
 
+// A decode step with K-contiguous weights streams them row by row where the 64 x 64 kernel's grid (N / 64 workgroups) is
+// too small to pull the weights at memory speed.  Every workgroup re-reads the M activation rows, M / 16 of what it reads
+// of W, so it pays for few rows and moderate N only.  Measured (us, bf16, this kernel / the 64 x 64 kernel): M = 1, N = K =
+// 4096 11.2 / 14.9; M = 16 11.1 / 14.9; M = 32 12.8 / 15; M = 64 20.3 / 15.5; M = 16, N = 4096, K = 11008 21.7 / 33.7; M = 1,
+// N = K = 8192 20.4 / 26.0; M = 16, N = 11008, K = 4096 23.0 / 15.9 (172 workgroups already stream at 5.6 TB/s).  Decided
+// from M, N and K alone, like every choice between kernels that add in different orders.
+inline bool skinny_fits(const GemmParams& p) {
+  if (p.N < 512 || p.K < 512 || p.K % 128 != 0) return false;
+  return p.M <= 4 || (p.M <= 16 && p.N <= 4608) || (p.M <= 32 && p.N <= 4096);
+}
+
+template <typename T, typename OT>
+int launch_skinny(const GemmParams& p, hipStream_t stream) {
+  const int64_t blocks = (p.N + 15) / 16;
+  if (blocks > 0x7fffffffLL) return XG_ERR_TOO_LARGE;
+  const dim3 grid((unsigned)blocks, (unsigned)p.batch);
+  if (p.M <= 16) hipLaunchKernelGGL((gemm_skinny_kernel<T, OT, 1>), grid, dim3(kThreads), 0, stream, p);
+  else hipLaunchKernelGGL((gemm_skinny_kernel<T, OT, 2>), grid, dim3(kThreads), 0, stream, p);
+  return status_from_hip(hipGetLastError());
+}
+
 template <typename T, typename OT, BLayout BL>
 int launch_mid(GemmParams p, hipStream_t stream) {
   auto kernel = gemm_mid_kernel<T, OT, BL>;
@@ -1535,6 +1655,9 @@ int launch_same_order(GemmParams p, TileKind kind, hipStream_t stream) {
 template <typename T, typename OT, BLayout BL>
 int launch_gemm(const GemmParams& p, hipStream_t stream) {
   if (!dma_ok<T>(p, BL)) return launch_kernel(gemm_staged_kernel<T, OT, BL>, p, stream);
+  if constexpr (Elem<T>::BYTES == 2 && BL == BLayout::KMajor) {
+    if (skinny_fits(p)) return launch_skinny<T, OT>(p, stream);
+  }
   if constexpr (Elem<T>::BYTES == 2) {
     if (mid_tiles_win(p)) return launch_mid<T, OT, BL>(p, stream);
   }
