@@ -313,6 +313,10 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
 
     // O^T += V^T P^T.  k-step (t, st) uses keys 32t + 16st + {4h..4h+3} and 32t + 16st + 8 + {4h..4h+3}:
     // exactly registers 8st..8st+7 of s[t] in this lane.
+    // This phase issues two transposing reads per MFMA; with the wave's priority raised its reads and MFMAs go
+    // ahead of the vector work of the other wave on the SIMD (B4 H32 S2048 D128 under sustained load: causal
+    // 160.8 -> 157.2 us, unmasked 274.5 -> 263.3 us; the same priority on the score MFMAs as well takes it back).
+    __builtin_amdgcn_s_setprio(1);
     static_for<2>([&](auto TI) {
       constexpr int t = decltype(TI)::value;
       static_for<2>([&](auto SI) {
@@ -332,6 +336,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
         });
       });
     });
+    __builtin_amdgcn_s_setprio(0);
   };
 
   issue(0, std::integral_constant<int, 0>{});
