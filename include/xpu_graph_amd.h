@@ -355,6 +355,31 @@ int xg_sdpa_backward(const void* q, const void* k, const void* v, const void* ou
                      int causal, int dtype, xg_stream_t stream);
 
 /* ---------------------------------------------------------------------------
+ * The two calls above for the attn_mask / tensor-scale form (xg_sdpa_masked):
+ *   xg_sdpa_masked_lse: xg_sdpa_masked that also writes lse [B,H,Sq] fp32.
+ *   xg_sdpa_backward_masked: xg_sdpa_backward with the forward's `mask`
+ *     (NULL or an additive mask, indexed as in xg_sdpa_masked) and `scale_dev`
+ *     (NULL or the one-element device scale).  dq, dk, dv only: the mask and
+ *     the scale tensor get no gradient.  A row that the mask hides completely
+ *     gives NaN gradients, as its forward result is NaN.
+ * replaces the Aten backward of the attn_mask form FusedSDPA emits
+ *   (passes/patterns/common/fuse_scaled_dot_product_attention.py:184-234) in
+ *   training graphs.
+ * ------------------------------------------------------------------------- */
+int xg_sdpa_masked_lse(const void* q, const void* k, const void* v, void* out, float* lse, const void* mask,
+                       const int64_t mask_strides[3], int mask_dtype, const float* scale_dev, int64_t B, int64_t H,
+                       int64_t Hkv, int64_t Sq, int64_t Skv, int64_t D, const int64_t q_strides[3],
+                       const int64_t k_strides[3], const int64_t v_strides[3], const int64_t o_strides[3], float scale,
+                       int causal, int dtype, xg_stream_t stream);
+int xg_sdpa_backward_masked(const void* q, const void* k, const void* v, const void* out, const void* d_out,
+                            const float* lse, const void* mask, const int64_t mask_strides[3], int mask_dtype,
+                            const float* scale_dev, void* dq, void* dk, void* dv, float* delta_ws, int64_t B, int64_t H,
+                            int64_t Hkv, int64_t Sq, int64_t Skv, int64_t D, const int64_t q_strides[3],
+                            const int64_t k_strides[3], const int64_t v_strides[3], const int64_t o_strides[3],
+                            const int64_t do_strides[3], const int64_t dq_strides[3], const int64_t dk_strides[3],
+                            const int64_t dv_strides[3], float scale, int causal, int dtype, xg_stream_t stream);
+
+/* ---------------------------------------------------------------------------
  * xg_sdpa_backward without the workspace argument, for callers that cannot
  * allocate device memory (code under HIP graph capture, serving loops and
  * harnesses that forbid hipMalloc).  No counterpart in the reference.  The

@@ -19,7 +19,7 @@ def declared_symbols():
 def test_header_declares_the_expected_entry_points():
     syms = declared_symbols()
     for s in ("xg_rms_norm", "xg_layer_norm", "xg_add_rms_norm", "xg_add_layer_norm", "xg_rms_norm_bwd", "xg_layer_norm_bwd", "xg_slice_cat", "xg_addn",
-              "xg_combo_sum", "xg_slice_sum_cat", "xg_silu_mul", "xg_silu_mul2", "xg_silu_mul2_bwd", "xg_activation", "xg_activation_bwd", "xg_dense", "xg_dense_batched", "xg_dense_at", "xg_dense_glu", "xg_dense_glu_save", "xg_dense_fp8", "xg_slice_cat_check_table", "xg_sdpa", "xg_sdpa_masked", "xg_sdpa_lse", "xg_sdpa_backward", "xg_sdpa_backward_static", "xg_rope", "xg_copy_bytes", "xg_clock_probe", "xg_wall_clock_khz",
+              "xg_combo_sum", "xg_slice_sum_cat", "xg_silu_mul", "xg_silu_mul2", "xg_silu_mul2_bwd", "xg_activation", "xg_activation_bwd", "xg_dense", "xg_dense_batched", "xg_dense_at", "xg_dense_glu", "xg_dense_glu_save", "xg_dense_fp8", "xg_slice_cat_check_table", "xg_sdpa", "xg_sdpa_masked", "xg_sdpa_lse", "xg_sdpa_backward", "xg_sdpa_masked_lse", "xg_sdpa_backward_masked", "xg_sdpa_backward_static", "xg_rope", "xg_copy_bytes", "xg_clock_probe", "xg_wall_clock_khz",
               "xg_version", "xg_status_string"):
         assert s in syms
 
@@ -162,6 +162,29 @@ def test_static_workspace_backward_refuses_more_rows_than_it_holds_without_a_gpu
     assert lib.xg_sdpa_backward_static(p, p, p, p, p, p, p, p, p, 1, 1, 1, (1 << 21) + 1, 64, 64, *args) == -5
     assert lib.xg_sdpa_backward_static(p, p, p, p, p, p, p, p, p, 1 << 11, 1 << 11, 1, 1, 64, 64, *args) == -5
     assert lib.xg_sdpa_backward_static(p, p, p, p, p, p, p, p, p, 0, 4, 4, 64, 64, 64, *args) == 0  # nothing to do
+
+
+def test_masked_backward_validation_needs_no_gpu():
+    """The mask operand of the backward call is checked like the forward's: strides present, dtype fp32 or the
+    tensors', rows that do not overlap; the device scale must be 4-byte aligned.  No pointer is dereferenced."""
+    from xpu_graph_amd import _lib
+
+    lib = _lib.lib()
+    S3 = ctypes.c_int64 * 3
+    p = ctypes.c_void_p(256)
+    st = S3(64 * 64 * 4, 64 * 64, 64)
+    shape = (1, 4, 4, 64, 64, 64, st, st, st, st, st, st, st, st, 0.125, 0, 2, None)
+
+    def call(mask, mask_strides, mask_dtype, scale_dev):
+        return lib.xg_sdpa_backward_masked(p, p, p, p, p, p, mask, mask_strides, mask_dtype, scale_dev, p, p, p, p, *shape)
+
+    assert call(p, None, 2, None) == -4              # a mask without strides
+    assert call(p, S3(0, 0, 64), 1, None) == -1      # bf16 tensors, an fp16 mask (neither bf16 nor fp32)
+    assert call(p, S3(0, 0, 32), 2, None) == -2      # mask rows of 64 keys at a pitch of 32 overlap
+    assert call(p, S3(0, 0, -64), 2, None) == -2
+    assert call(ctypes.c_void_p(257), S3(0, 0, 64), 2, None) == -3
+    assert call(None, None, 2, ctypes.c_void_p(258)) == -3
+    assert lib.xg_sdpa_masked_lse(p, p, p, p, None, None, None, 2, None, 1, 4, 4, 64, 64, 64, st, st, st, st, 0.125, 0, 2, None) == -4
 
 
 def test_a_missing_library_is_an_error_not_a_fallback(monkeypatch, tmp_path):

@@ -12,7 +12,7 @@ import math
 import pytest
 import torch
 
-from tests.test_gpu_sdpa import make, ref32
+from tests.test_gpu_sdpa import make, ref32, ref32_masked
 from tests.tolerance import assert_close_16bit, attention_floor, attention_grad_floor
 
 pytestmark = pytest.mark.gpu
@@ -124,6 +124,89 @@ def test_autograd_runs_the_backward_kernels(device):
         out.backward(g)
         for leaf, want in zip(leaves, (dq, dk, dv)):
             assert torch.equal(leaf.grad, want), op
+
+
+def ref_grads_masked(q, k, v, g, mask, causal, scale):
+    qf, kf, vf = (t.detach().float().requires_grad_(True) for t in (q, k, v))
+    out = ref32_masked(qf, kf, vf, mask, causal, scale)
+    return (out.detach(), *torch.autograd.grad(out, (qf, kf, vf), g.float()))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("D", [128, 64])
+@pytest.mark.parametrize("mask_shape,mask_dtype", [("full", "same"), ("rows", "f32"), ("per_batch", "same"), ("per_head", "f32")])
+@pytest.mark.parametrize("Sq,Skv", [(256, 256), (130, 77), (1, 300), (200, 333), (320, 512)])
+def test_backward_with_an_additive_mask(device, dtype, D, mask_shape, mask_dtype, Sq, Skv):
+    """Gradients of the attn_mask form (reference passes/patterns/common/fuse_scaled_dot_product_attention.py:184-234
+    in a training graph): the backward kernels add the mask to the recomputed scores.  Masks broadcast over batch and /
+    or heads, in the tensors' dtype or fp32, with -inf entries (padded keys; key 0 stays visible so that no row is
+    empty), odd sizes, grouped heads, and a causal flag on top where the problem is square."""
+    B, H, Hkv = 2, 4, 2
+    q, k, v = make(B, H, Hkv, Sq, Skv, D, dtype, device, seed=Sq * 5 + Skv + D)
+    gen = torch.Generator().manual_seed(Sq + 2 * Skv)
+    shape = {"full": (B, H, Sq, Skv), "rows": (Sq, Skv), "per_batch": (B, 1, Sq, Skv), "per_head": (1, H, Sq, Skv)}[mask_shape]
+    mask = torch.randn(shape, generator=gen)
+    pad = torch.rand(shape[:-2] + (1, Skv), generator=gen) < 0.2
+    pad[..., 0] = False
+    mask = mask.masked_fill(pad.expand(shape), float("-inf")).to(dtype if mask_dtype == "same" else torch.float32).to(device)
+    g = torch.randn(q.shape, generator=gen).to(dtype).to(device)
+    scale = 1.0 / math.sqrt(D)
+    for causal in ((False, True) if Sq == Skv else (False,)):
+        out, lse = _ops().sdpa_masked_lse(q, k, v, mask, None, causal, scale)
+        assert torch.equal(out, _ops().sdpa_masked(q, k, v, mask, None, causal, scale))
+        dq, dk, dv = _ops().sdpa_masked_bwd(q, k, v, out, g, lse, mask, None, causal, scale)
+        want_out, wq, wk, wv = ref_grads_masked(q, k, v, g, mask, causal, scale)
+        assert_close_16bit(out, want_out, attention_floor(want_out, dtype), f"sdpa masked {tuple(out.shape)} {dtype}")
+        noise = cancel_noise(q, k, v, g, scale)
+        close_grad(dq, wq, f"dq mask {mask_shape}", noise)
+        close_grad(dk, wk, f"dk mask {mask_shape}", noise)
+        close_grad(dv, wv, f"dv mask {mask_shape}")
+
+
+def test_backward_with_the_scale_in_a_device_tensor(device):
+    """The tensor-scale form (reference passes/patterns/utils/default_replacements.py:39-55): the backward kernels read
+    the scale on the device too; without a mask the gradients equal the by-value call's bit for bit, with one they
+    match fp32 autograd."""
+    q, k, v = make(2, 4, 2, 200, 264, 128, torch.bfloat16, device, seed=31)
+    g = torch.randn(q.shape, generator=torch.Generator().manual_seed(3)).bfloat16().to(device)
+    t = torch.tensor([0.07], device=device)
+    out, lse = _ops().sdpa_masked_lse(q, k, v, None, t, False, 123.0)  # the by-value scale is ignored
+    got = _ops().sdpa_masked_bwd(q, k, v, out, g, lse, None, t, False, 123.0)
+    _, _, dq, dk, dv = run_backward(q, k, v, g, False, t.item())
+    for a, b in zip(got, (dq, dk, dv)):
+        assert torch.equal(a, b)
+    mask = torch.randn(2, 1, 200, 264, generator=torch.Generator().manual_seed(5)).to(device)
+    out, lse = _ops().sdpa_masked_lse(q, k, v, mask, t, False, 123.0)
+    dq, dk, dv = _ops().sdpa_masked_bwd(q, k, v, out, g, lse, mask, t, False, 123.0)
+    _, wq, wk, wv = ref_grads_masked(q, k, v, g, mask, False, 0.07)
+    noise = cancel_noise(q, k, v, g, 0.07)
+    close_grad(dq, wq, "dq mask + tensor scale", noise)
+    close_grad(dk, wk, "dk mask + tensor scale", noise)
+    close_grad(dv, wv, "dv mask + tensor scale")
+
+
+def test_autograd_of_the_masked_op(device):
+    """loss.backward() through sdpa_masked (which recomputes the row statistics) and sdpa_masked_lse gives the
+    kernels' gradients bit for bit; a mask or a scale tensor that wants a gradient is refused, not ignored."""
+    import xpu_graph_amd.ops as xops
+
+    xops.enable_autograd()
+    q, k, v = make(2, 4, 4, 192, 160, 64, torch.float16, device, seed=23)
+    g = torch.randn(q.shape, generator=torch.Generator().manual_seed(9)).half().to(device)
+    mask = torch.randn(1, 4, 192, 160, generator=torch.Generator().manual_seed(2)).to(device)
+    out, lse = _ops().sdpa_masked_lse(q, k, v, mask, None, False, 0.1)
+    want = _ops().sdpa_masked_bwd(q, k, v, out, g, lse, mask, None, False, 0.1)
+    for op in ("sdpa_masked", "sdpa_masked_lse"):
+        leaves = [t.clone().requires_grad_(True) for t in (q, k, v)]
+        res = getattr(_ops(), op)(*leaves, mask, None, False, 0.1)
+        res = res[0] if op == "sdpa_masked_lse" else res
+        res.backward(g)
+        for leaf, w in zip(leaves, want):
+            assert torch.equal(leaf.grad, w), op
+    leaves = [t.clone().requires_grad_(True) for t in (q, k, v)]
+    learned = mask.clone().requires_grad_(True)
+    with pytest.raises(NotImplementedError):
+        _ops().sdpa_masked(*leaves, learned, None, False, 0.1).backward(g)
 
 
 def test_backward_c5_full_size_holds_no_score_matrix(device):

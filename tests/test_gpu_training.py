@@ -451,6 +451,57 @@ def test_attention_training_step(device):
         assert err(a, c) <= 2 * err(e, c) + 1e-2 * c.abs().mean().item(), (err(a, c), err(e, c), c.abs().mean().item())
 
 
+def test_attention_with_a_padding_mask_trains_on_the_kernels(device):
+    """The attn_mask form in a training graph (reference passes/patterns/common/fuse_scaled_dot_product_attention.py:
+    184-234): a mask that needs no gradient (padded keys, given as a graph input) goes to the attention kernels, forward
+    and backward; a learned additive bias does need one, so that attention stays on Aten and the bias is trained."""
+
+    def layer(x, wqkv, wo, mask):
+        B, S, E = x.shape
+        q, k, v = (t.view(B, S, 4, 64).transpose(1, 2) for t in F.linear(x, wqkv).split(E, dim=-1))
+        a = F.scaled_dot_product_attention(q, k, v, attn_mask=mask)
+        return F.linear(a.transpose(1, 2).reshape(B, S, E), wo)
+
+    torch.manual_seed(11)
+    bf = torch.bfloat16
+    mk = lambda *s, k=1.0: (torch.randn(*s, device=device) * k).to(bf).requires_grad_(True)  # noqa: E731
+    args = [mk(2, 128, 256), mk(768, 256, k=0.06), mk(256, 256, k=0.06)]
+    pad = torch.zeros(2, 1, 128, 128, device=device, dtype=bf)
+    pad[0, :, :, 100:] = float("-inf")
+    pad[1, :, :, 77:] = float("-inf")
+    be = backend()
+    y0 = torch.compile(layer, backend=be, dynamic=False)(*args, pad)
+    g0 = torch.autograd.grad(y0.float().pow(2).mean(), args)
+    fwd_ops = [str(n.target) for n in be.compiled_graphs[1].graph.nodes if n.op == "call_function"]
+    assert fwd_ops.count("xpu_ops.sdpa_masked_lse.default") == 1, fwd_ops
+    bwd_ops = [str(n.target) for gm in be.compiled_graphs[2:] for n in gm.graph.nodes if n.op == "call_function"]
+    assert bwd_ops.count("xpu_ops.sdpa_masked_bwd.default") == 1, bwd_ops
+    ref_args = [a.detach().float().requires_grad_(True) for a in args]
+    g1 = torch.autograd.grad(layer(*ref_args, pad.float()).pow(2).mean(), ref_args)
+    eag_args = [a.detach().clone().requires_grad_(True) for a in args]
+    g2 = torch.autograd.grad(layer(*eag_args, pad).float().pow(2).mean(), eag_args)
+    err = lambda a, c: (a.float() - c).abs().mean().item()  # noqa: E731
+    for a, c, e in zip(g0, g1, g2):
+        assert err(a, c) <= 2 * err(e, c) + 1e-2 * c.abs().mean().item(), (err(a, c), err(e, c), c.abs().mean().item())
+
+    bias = (torch.randn(1, 4, 128, 128, device=device) * 0.5).to(bf).requires_grad_(True)
+    be2 = backend()
+    y = torch.compile(layer, backend=be2, dynamic=False)(*args, bias)
+    gb = torch.autograd.grad(y.float().pow(2).mean(), [bias])[0]
+    ops2 = [str(n.target) for gm in be2.compiled_graphs[1:] for n in gm.graph.nodes if n.op == "call_function"]
+    assert not any("sdpa_masked" in o for o in ops2), ops2
+
+    def written_out(x, wqkv, wo, mask):  # (eager's fused attention backward refuses a bias that alone needs a gradient)
+        B, S, E = x.shape
+        q, k, v = (t.view(B, S, 4, 64).transpose(1, 2) for t in F.linear(x, wqkv).split(E, dim=-1))
+        a = torch.softmax(q @ k.transpose(-1, -2) / 8.0 + mask, dim=-1) @ v
+        return F.linear(a.transpose(1, 2).reshape(B, S, E), wo)
+
+    ref_bias = bias.detach().float().requires_grad_(True)
+    want = torch.autograd.grad(written_out(*[a.detach().float() for a in args], ref_bias).pow(2).mean(), [ref_bias])[0]
+    assert (gb.float() - want).abs().mean().item() <= 0.1 * want.abs().mean().item() + 1e-6
+
+
 def test_llama_block_training_step(device):
     """The whole decoder block of benchmark config 5 (small batch and sequence), compiled for training on the mi355x
     target: the forward graph runs on the HIP kernels, and the gradients of every weight follow fp32 autograd as

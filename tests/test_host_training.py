@@ -287,3 +287,26 @@ def test_written_out_attention_reaches_the_attention_kernel_in_pregrad(caplog):
     fwd_ops = [str(n.target) for n in forward.graph.nodes if n.op == "call_function"]
     assert fwd_ops.count("xpu_ops.sdpa_lse.default") == 1 and "xpu_ops.sdpa.default" not in fwd_ops, fwd_ops
     assert "Pattern.FusedSDPA changed graph" in caplog.text
+
+
+def test_masked_attention_in_pregrad_depends_on_who_needs_a_gradient(caplog):
+    """The attn_mask form in a training graph: a mask computed from inputs that need no gradient (padding) goes to the
+    masked attention module, whose op has backward kernels for q, k, v; a mask computed from a parameter (a learned
+    bias) would lose its gradient there, so that attention stays as the Aten op."""
+
+    def attn(q, k, v, pad, bias):
+        a = F.scaled_dot_product_attention(q, k, v, attn_mask=pad * 2.0)
+        b = F.scaled_dot_product_attention(q, k, v, attn_mask=bias + pad)
+        return a + b
+
+    bf = torch.bfloat16
+    backend = XpuGraph(XpuGraphConfig(is_training=True, target=Target.mi355x, opt_level=OptLevel.level2, enable_cache=False))
+    args = [torch.randn(2, 4, 32, 64).to(bf).requires_grad_(True) for _ in range(3)]
+    args += [torch.zeros(2, 1, 32, 32).to(bf), torch.zeros(1, 4, 32, 32).to(bf).requires_grad_(True)]
+    with need_xpu_graph_logs(), pytest.raises(NotImplementedError):
+        torch.compile(attn, backend=backend)(*args)
+    pregrad, forward = backend.compiled_graphs[-2:]
+    assert [n.target for n in pregrad.graph.nodes if n.op == "call_module"] == ["mi355x_sdpa_masked"]
+    assert sum(1 for n in pregrad.graph.nodes if "scaled_dot_product_attention" in str(n.target)) == 1
+    fwd_ops = [str(n.target) for n in forward.graph.nodes if n.op == "call_function"]
+    assert fwd_ops.count("xpu_ops.sdpa_masked_lse.default") == 1 and "xpu_ops.sdpa_masked.default" not in fwd_ops, fwd_ops

@@ -130,6 +130,15 @@ _SIGNATURES = {
         c_int,
         [c_void_p] * 10 + [c_int64] * 6 + [ctypes.POINTER(c_int64)] * 8 + [c_float, c_int, c_int, c_void_p],
     ),
+    "xg_sdpa_masked_lse": (
+        c_int,
+        [c_void_p] * 6 + [ctypes.POINTER(c_int64), c_int, c_void_p] + [c_int64] * 6 + [ctypes.POINTER(c_int64)] * 4 + [c_float, c_int, c_int, c_void_p],
+    ),
+    "xg_sdpa_backward_masked": (
+        c_int,
+        [c_void_p] * 7 + [ctypes.POINTER(c_int64), c_int, c_void_p] + [c_void_p] * 4 + [c_int64] * 6 + [ctypes.POINTER(c_int64)] * 8
+        + [c_float, c_int, c_int, c_void_p],
+    ),
     "xg_sdpa_backward_static": (
         c_int,
         [c_void_p] * 9 + [c_int64] * 6 + [ctypes.POINTER(c_int64)] * 8 + [c_float, c_int, c_int, c_void_p],

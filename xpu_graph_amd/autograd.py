@@ -17,6 +17,8 @@ a few microseconds of dispatch, which inference-only processes should not pay.
     rope(x, cos, sin)          y = x * cos + rotate_half(x) * sin,  rotate_half(x) = cat(-x[D/2:], x[:D/2])
     sdpa(q, k, v, causal, scale)   y = softmax(scale q k^T [+ causal mask]) v
     sdpa_lse(q, k, v, causal, scale)   the same, also returning the log-sum-exp of every row for the backward kernels
+    sdpa_masked(q, k, v, mask, scale_t, causal, scale) / sdpa_masked_lse   with an additive mask and / or the scale in a
+                               one-element tensor: gradients for q, k, v (the mask and the scale tensor get none)
     add_rms_norm(x, r, w, eps) / add_layer_norm(x, r, w, b, eps)   h = x + r, y = norm(h); returns (y, h)
     add_rms_norm_only / add_layer_norm_only                         the same, returning y alone
 
@@ -308,6 +310,54 @@ def _sdpa_lse_backward(ctx, gy, g_lse=None):
     return gq, gk, gv, None, None
 
 
+def _refuse_mask_or_scale_grad(ctx, name):
+    if ctx.needs_input_grad[3] or ctx.needs_input_grad[4]:
+        raise NotImplementedError(f"xpu_ops::{name}: no gradient for the mask or the scale tensor (only q, k, v are differentiable)")
+
+
+def _sdpa_masked_setup(ctx, inputs, output):
+    q, k, v, mask, scale_t, ctx.causal, ctx.scale = inputs
+    ctx.has_mask, ctx.has_scale = mask is not None, scale_t is not None
+    ctx.save_for_backward(q, k, v, *(t for t in (mask, scale_t) if t is not None))
+
+
+def _masked_operands(ctx, rest):
+    rest = list(rest)
+    mask = rest.pop(0) if ctx.has_mask else None
+    scale_t = rest.pop(0) if ctx.has_scale else None
+    return mask, scale_t
+
+
+def _sdpa_masked_backward(ctx, gy):
+    # as for the plain op: one more forward launch for the row statistics, then the backward kernels
+    _refuse_mask_or_scale_grad(ctx, "sdpa_masked")
+    q, k, v, *rest = ctx.saved_tensors
+    mask, scale_t = _masked_operands(ctx, rest)
+    out, lse = torch.ops.xpu_ops.sdpa_masked_lse(q, k, v, mask, scale_t, ctx.causal, ctx.scale)
+    gq, gk, gv = torch.ops.xpu_ops.sdpa_masked_bwd(q, k, v, out, gy, lse, mask, scale_t, ctx.causal, ctx.scale)
+    return gq, gk, gv, None, None, None, None
+
+
+def _sdpa_masked_lse_setup(ctx, inputs, output):
+    q, k, v, mask, scale_t, ctx.causal, ctx.scale = inputs
+    out, lse = output
+    ctx.has_mask, ctx.has_scale = mask is not None, scale_t is not None
+    ctx.save_for_backward(q, k, v, out, lse, *(t for t in (mask, scale_t) if t is not None))
+    ctx.set_materialize_grads(False)
+
+
+def _sdpa_masked_lse_backward(ctx, gy, g_lse=None):
+    if g_lse is not None:
+        raise NotImplementedError("xpu_ops::sdpa_masked_lse: only its first output (the attention result) is differentiable")
+    if gy is None:
+        return (None,) * 7
+    _refuse_mask_or_scale_grad(ctx, "sdpa_masked_lse")
+    q, k, v, out, lse, *rest = ctx.saved_tensors
+    mask, scale_t = _masked_operands(ctx, rest)
+    gq, gk, gv = torch.ops.xpu_ops.sdpa_masked_bwd(q, k, v, out, gy, lse, mask, scale_t, ctx.causal, ctx.scale)
+    return gq, gk, gv, None, None, None, None
+
+
 def _add_norm_formulas(layer, with_sum):
     """(setup, backward) of the residual-add + norm ops: the sum is recomputed, its gradient is the norm's input
     gradient plus whatever flows into the returned sum, and both addends receive it."""
@@ -372,6 +422,8 @@ def register():
     reg("xpu_ops::rope", _rope_backward, setup_context=_rope_setup)
     reg("xpu_ops::sdpa", _sdpa_backward, setup_context=_sdpa_setup)
     reg("xpu_ops::sdpa_lse", _sdpa_lse_backward, setup_context=_sdpa_lse_setup)
+    reg("xpu_ops::sdpa_masked", _sdpa_masked_backward, setup_context=_sdpa_masked_setup)
+    reg("xpu_ops::sdpa_masked_lse", _sdpa_masked_lse_backward, setup_context=_sdpa_masked_lse_setup)
     for op, layer, with_sum in (("add_rms_norm", False, True), ("add_rms_norm_only", False, False),
                                 ("add_layer_norm", True, True), ("add_layer_norm_only", True, False)):
         setup, backward = _add_norm_formulas(layer, with_sum)
@@ -379,7 +431,7 @@ def register():
     # An op that was traced before (an inference compile earlier in the process) has its dispatch decisions cached
     # on the Python side; a stale entry for the Autograd key would keep sending traces to the "no formula" fallback.
     for name in ("rms_norm", "layer_norm", "silu_mul2", "silu_mul", "act", "dense", "dense_glu", "dense_glu_save", "rope", "sdpa", "sdpa_lse",
-                 "add_rms_norm", "add_rms_norm_only", "add_layer_norm", "add_layer_norm_only"):
+                 "sdpa_masked", "sdpa_masked_lse", "add_rms_norm", "add_rms_norm_only", "add_layer_norm", "add_layer_norm_only"):
         packet = getattr(torch.ops.xpu_ops, name)
         for overload in packet.overloads():
             getattr(packet, overload)._dispatch_cache.clear()

@@ -251,6 +251,12 @@ class XpuGraph:
             return None
         logger.info("decompose graph complete")
         logger.debug("after decompose, graph like:\n %s", dispatched.print_readable(print_output=False))
+        # The exported graph's metadata does not say which inputs will be differentiated; patterns that may only take
+        # operands without a gradient (an attention mask) read it from the placeholders.
+        placeholders = [n for n in dispatched.graph.nodes if n.op == "placeholder"]
+        if len(placeholders) == len(example_inputs):
+            for node, real in zip(placeholders, example_inputs):
+                node.meta["xg_requires_grad"] = bool(isinstance(real, torch.Tensor) and real.requires_grad)
         return self._get_compiler(FxStage.pregrad, boxed=False)(dispatched, example_inputs)
 
     def get_pattern_manager(self):

@@ -497,3 +497,13 @@ extern "C" int xg_sdpa_lse(const void* q, const void* k, const void* v, void* ou
   return sdpa_entry(q, k, v, out, lse, nullptr, nullptr, dtype, nullptr, B, H, Hkv, Sq, Skv, D, q_strides, k_strides, v_strides, o_strides,
                     scale, causal, dtype, stream);
 }
+
+extern "C" int xg_sdpa_masked_lse(const void* q, const void* k, const void* v, void* out, float* lse, const void* mask,
+                                  const int64_t mask_strides[3], int mask_dtype, const float* scale_dev, int64_t B, int64_t H,
+                                  int64_t Hkv, int64_t Sq, int64_t Skv, int64_t D, const int64_t q_strides[3],
+                                  const int64_t k_strides[3], const int64_t v_strides[3], const int64_t o_strides[3], float scale,
+                                  int causal, int dtype, xg_stream_t stream) {
+  if (lse == nullptr && B > 0 && H > 0 && Sq > 0) return XG_ERR_NULL_PTR;
+  return sdpa_entry(q, k, v, out, lse, mask, mask_strides, mask_dtype, scale_dev, B, H, Hkv, Sq, Skv, D, q_strides, k_strides, v_strides,
+                    o_strides, scale, causal, dtype, stream);
+}

@@ -46,6 +46,11 @@ struct BwdParams {
   int64_t qs[3], ks[3], vs[3], os[3], dos[3];  // element strides of batch, head, sequence
   int64_t dqs[3], dks[3], dvs[3];              // ... of the three outputs (rows of D contiguous elements)
   float scale;
+  const float* scale_dev;  // when set: the scale is read from this one-element device tensor instead
+  const void* mask;        // additive mask (MASK kernels only), element [b, h, i, j] at ms[0] b + ms[1] h + ms[2] i + j
+  int64_t ms[3];           // element strides of batch, head, query row (0: broadcast)
+  int mask_f32;            // mask elements are fp32 (else the dtype of q)
+  int mask_vec;            // rows of the mask can be read four elements at a time
   int causal;
   int n_qb, n_kb;
   int group_q, group_k;  // block order of the two kernels (grouped_block_order)
@@ -168,7 +173,9 @@ __device__ __forceinline__ void store_rows(char* park, const f32x16 (&acc)[D / 3
 }
 
 // ---------------------------------------------------------------------------------------------- dq
-template <typename T, int D>
+// MASK: the forward added an additive mask to the scaled scores; the probabilities are recomputed with it (the mask
+// itself gets no gradient).
+template <typename T, int D, bool MASK = false>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void sdpa_bwd_dq_kernel(BwdParams p) {
   typedef typename Vec8<T>::type V8;
   constexpr int RB = D * 2, CH = RB / 16, TILE = BKV * RB, STAGE = 2 * TILE, KK = D / 16, DT = D / 32, LPW = CH / 4;
@@ -177,7 +184,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int l32 = lane & 31, h = lane >> 5;
-  const float c = p.scale * kLog2e;
+  const float scale = p.scale_dev ? *p.scale_dev : p.scale;
+  const float c = scale * kLog2e;
 
   const int nbh = p.B * p.H;
   int bh, rank;
@@ -246,6 +254,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
   const int qw_max = q0 + 32 * wave + 31;
   const int sx = swz_v<D>(l32);
   const TrLane TL(lane);
+  const int64_t mbase = MASK ? (int64_t)b * p.ms[0] + (int64_t)head * p.ms[1] + (int64_t)qr * p.ms[2] : 0;
 
   f32x16 dq_acc[DT];
   static_for<DT>([&](auto I) {
@@ -271,6 +280,36 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
       f32x16 s = rows_times_regs<T, D>(k_s, t, l32, h, sx, qf);
       const f32x16 dp = rows_times_regs<T, D>(v_s, t, l32, h, sx, dof);
       float cc = c;
+      if constexpr (MASK) {
+        // scores in the exponent's base-2 scale with the mask added, as the forward formed them; afterwards cc = 1.
+        // Key indices are clamped for the loads; what lies past the end is masked by index below.
+        static_for<4>([&](auto GI) {
+          constexpr int g = decltype(GI)::value;
+          const int key0 = kv0 + 32 * t + 8 * g + 4 * h;
+          float m4[4];
+          if (p.mask_vec && key0 + 3 < p.Skv) {
+            if (p.mask_f32) {
+              const f32x4 mv = *reinterpret_cast<const f32x4*>(reinterpret_cast<const float*>(p.mask) + mbase + key0);
+              m4[0] = mv[0], m4[1] = mv[1], m4[2] = mv[2], m4[3] = mv[3];
+            } else {
+              typedef T t4 __attribute__((ext_vector_type(4)));
+              const t4 mv = *reinterpret_cast<const t4*>(reinterpret_cast<const T*>(p.mask) + mbase + key0);
+              m4[0] = (float)mv[0], m4[1] = (float)mv[1], m4[2] = (float)mv[2], m4[3] = (float)mv[3];
+            }
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const int key = key0 + e < p.Skv ? key0 + e : p.Skv - 1;
+              m4[e] = p.mask_f32 ? reinterpret_cast<const float*>(p.mask)[mbase + key] : (float)reinterpret_cast<const T*>(p.mask)[mbase + key];
+            }
+          }
+          static_for<4>([&](auto EI) {
+            constexpr int e = decltype(EI)::value;
+            s[4 * g + e] = __builtin_fmaf(s[4 * g + e], cc, m4[e] * kLog2e);
+          });
+        });
+        cc = 1.f;
+      }
       if (need_mask) {
         static_for<16>([&](auto VI) {
           constexpr int v = decltype(VI)::value;
@@ -296,7 +335,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
   }
   __syncthreads();  // all waves are done reading tiles: the parks reuse the space
   T* dst = reinterpret_cast<T*>(p.dq) + (int64_t)b * p.dqs[0] + (int64_t)head * p.dqs[1] + (int64_t)(q0 + 32 * wave) * p.dqs[2];
-  store_rows<T, D>(smem + wave * (32 * RB), dq_acc, p.scale, dst, p.dqs[2], p.Sq - (q0 + 32 * wave), lane);
+  store_rows<T, D>(smem + wave * (32 * RB), dq_acc, scale, dst, p.dqs[2], p.Sq - (q0 + 32 * wave), lane);
 }
 
 // ---------------------------------------------------------------------------------------------- dk, dv
@@ -304,7 +343,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
 // dv rows take 128 accumulation registers at D = 128; to stay within the 256 a lane may have at that occupancy only
 // the K row of the lane is held in registers, its V row is read from LDS (the workgroup's 256 V rows are loaded
 // once, each wave its own 32).
-template <typename T, int D>
+template <typename T, int D, bool MASK = false>
 __global__ __launch_bounds__(64 * KW) __attribute__((amdgpu_waves_per_eu(2, 2))) void sdpa_bwd_dkv_kernel(BwdParams p) {
   typedef typename Vec8<T>::type V8;
   constexpr int RB = D * 2, CH = RB / 16, TILE = BKV * RB, KK = D / 16, DT = D / 32, LPW = CH / KW;
@@ -316,7 +355,8 @@ __global__ __launch_bounds__(64 * KW) __attribute__((amdgpu_waves_per_eu(2, 2)))
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int l32 = lane & 31, h = lane >> 5;
-  const float c = p.scale * kLog2e;
+  const float scale = p.scale_dev ? *p.scale_dev : p.scale;
+  const float c = scale * kLog2e;
 
   const int nbk = p.B * p.Hkv, rep = p.H / p.Hkv;
   int bk, kb;  // causal: early key blocks meet the most queries, start them first
@@ -418,6 +458,21 @@ __global__ __launch_bounds__(64 * KW) __attribute__((amdgpu_waves_per_eu(2, 2)))
     auto soft = [&](auto TI, f32x16& s, const f32x16& dp, V8 (&prf)[2], V8 (&dsf)[2]) {
       constexpr int t = decltype(TI)::value;
       float cc = c;
+      if constexpr (MASK) {
+        // the mask element of (query, this lane's key), one load per score: lanes of a half-wave read neighbouring
+        // keys of one mask row.  Rows and keys past the end are clamped for the load and masked by index below.
+        const int head = hkv * rep + it / nj;
+        const int64_t mb = (int64_t)b * p.ms[0] + (int64_t)head * p.ms[1] + kr;
+        static_for<16>([&](auto VI) {
+          constexpr int v = decltype(VI)::value;
+          int qi = qt0 + 32 * t + 8 * (v / 4) + 4 * h + (v % 4);
+          qi = qi < p.Sq ? qi : p.Sq - 1;
+          const int64_t at = mb + (int64_t)qi * p.ms[2];
+          const float m = p.mask_f32 ? reinterpret_cast<const float*>(p.mask)[at] : (float)reinterpret_cast<const T*>(p.mask)[at];
+          s[v] = __builtin_fmaf(s[v], cc, m * kLog2e);
+        });
+        cc = 1.f;
+      }
       if (need_mask) {
         static_for<16>([&](auto VI) {
           constexpr int v = decltype(VI)::value;
@@ -433,9 +488,9 @@ __global__ __launch_bounds__(64 * KW) __attribute__((amdgpu_waves_per_eu(2, 2)))
         static_for<4>([&](auto EI) {
           constexpr int e = decltype(EI)::value;
           constexpr int v = 4 * g + e;
-          // l4 is finite: a causal row sees at least key 0 and additive masks are refused by the entry point.  A
-          // backward that admits rows without any visible key (log-sum-exp -inf) has to map -inf to 0 here, as the
-          // dq kernel does, or -inf - (-inf) gives NaN.
+          // l4 is finite when the row sees a key: a causal row sees at least key 0.  A row that an additive mask
+          // hides completely has log-sum-exp -inf and gives NaN here (-inf - (-inf)), as its forward result already
+          // is and as the unfused graph's gradients are.
           const float pr = __builtin_amdgcn_exp2f(__builtin_fmaf(s[v], cc, -l4[e] * kLog2e));
           prf[v / 8][v % 8] = (T)pr;
           dsf[v / 8][v % 8] = (T)(pr * (dp[v] - d4[e]));
@@ -467,17 +522,17 @@ __global__ __launch_bounds__(64 * KW) __attribute__((amdgpu_waves_per_eu(2, 2)))
   char* park = smem + wave * (32 * RB);
   T* dk_dst = reinterpret_cast<T*>(p.dk) + (int64_t)b * p.dks[0] + (int64_t)hkv * p.dks[1] + (int64_t)row0 * p.dks[2];
   T* dv_dst = reinterpret_cast<T*>(p.dv) + (int64_t)b * p.dvs[0] + (int64_t)hkv * p.dvs[1] + (int64_t)row0 * p.dvs[2];
-  store_rows<T, D>(park, dk_acc, p.scale, dk_dst, p.dks[2], p.Skv - row0, lane);
+  store_rows<T, D>(park, dk_acc, scale, dk_dst, p.dks[2], p.Skv - row0, lane);
   __syncthreads();  // the parks have been read back before they are written again
   store_rows<T, D>(park, dv_acc, 1.f, dv_dst, p.dvs[2], p.Skv - row0, lane);
 }
 
-template <typename T, int D>
+template <typename T, int D, bool MASK = false>
 int launch_bwd(const BwdParams& p, hipStream_t stream) {
   constexpr int SMEM_DQ = 2 * 2 * BKV * D * 2;
   constexpr int SMEM_DKV = 2 * (2 * BKV * D * 2 + 1024) + BK * D * 2;
-  auto dq_kernel = sdpa_bwd_dq_kernel<T, D>;
-  auto dkv_kernel = sdpa_bwd_dkv_kernel<T, D>;
+  auto dq_kernel = sdpa_bwd_dq_kernel<T, D, MASK>;
+  auto dkv_kernel = sdpa_bwd_dkv_kernel<T, D, MASK>;
   if (int st = allow_dynamic_lds(reinterpret_cast<const void*>(dq_kernel), SMEM_DQ)) return st;
   if (int st = allow_dynamic_lds(reinterpret_cast<const void*>(dkv_kernel), SMEM_DKV)) return st;
   hipLaunchKernelGGL(dq_kernel, dim3((unsigned)((int64_t)p.B * p.H * p.n_qb)), dim3(kThreads), SMEM_DQ, stream, p);
@@ -491,8 +546,8 @@ int launch_bwd(const BwdParams& p, hipStream_t stream) {
 
 namespace {
 
-int backward_entry(const void* q, const void* k, const void* v, const void* out, const void* d_out, const float* lse, void* dq, void* dk,
-                   void* dv, float* delta_ws, int64_t B, int64_t H, int64_t Hkv, int64_t Sq, int64_t Skv, int64_t D,
+int backward_entry(const void* q, const void* k, const void* v, const void* out, const void* d_out, const float* lse, const void* mask,
+                   const int64_t* mask_strides, int mask_dtype, const float* scale_dev, void* dq, void* dk, void* dv, float* delta_ws, int64_t B, int64_t H, int64_t Hkv, int64_t Sq, int64_t Skv, int64_t D,
                    const int64_t q_strides[3], const int64_t k_strides[3], const int64_t v_strides[3], const int64_t o_strides[3],
                    const int64_t do_strides[3], const int64_t dq_strides[3], const int64_t dk_strides[3], const int64_t dv_strides[3],
                    float scale, int causal, int dtype, xg_stream_t stream) {
@@ -548,12 +603,37 @@ int backward_entry(const void* q, const void* k, const void* v, const void* out,
   p.Sq = (int)Sq;
   p.Skv = (int)Skv;
   p.scale = scale;
+  if (scale_dev && !aligned_to(scale_dev, 4)) return XG_ERR_BAD_ALIGN;
+  p.scale_dev = scale_dev;
+  p.mask = mask;
+  p.mask_f32 = 0;
+  p.mask_vec = 0;
+  p.ms[0] = p.ms[1] = p.ms[2] = 0;
+  if (mask) {  // the same conditions as the forward's
+    if (!mask_strides) return XG_ERR_NULL_PTR;
+    if (mask_dtype != dtype && mask_dtype != XG_F32) return XG_ERR_BAD_DTYPE;
+    const size_t esz = mask_dtype == XG_F32 ? 4 : 2;
+    if (!aligned_to(mask, esz)) return XG_ERR_BAD_ALIGN;
+    bool vec = aligned_to(mask, 4 * esz);
+    for (int i = 0; i < 3; ++i) {
+      if (mask_strides[i] < 0) return XG_ERR_BAD_SHAPE;
+      p.ms[i] = mask_strides[i];
+      vec = vec && mask_strides[i] % 4 == 0;
+    }
+    if (Sq > 1 && mask_strides[2] != 0 && mask_strides[2] < Skv) return XG_ERR_BAD_SHAPE;  // rows would overlap
+    p.mask_f32 = mask_dtype == XG_F32 ? 1 : 0;
+    p.mask_vec = vec ? 1 : 0;
+  }
   p.causal = causal ? 1 : 0;
   p.n_qb = (int)n_qb;
   p.n_kb = (int)n_kb;
   p.group_q = sdpa::block_order_group(B * H);
   p.group_k = sdpa::block_order_group(B * Hkv);
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  if (mask) {
+    if (dtype == XG_BF16) return D == 128 ? sdpa::launch_bwd<bf16_t, 128, true>(p, st) : sdpa::launch_bwd<bf16_t, 64, true>(p, st);
+    return D == 128 ? sdpa::launch_bwd<f16_t, 128, true>(p, st) : sdpa::launch_bwd<f16_t, 64, true>(p, st);
+  }
   if (dtype == XG_BF16) return D == 128 ? sdpa::launch_bwd<bf16_t, 128>(p, st) : sdpa::launch_bwd<bf16_t, 64>(p, st);
   return D == 128 ? sdpa::launch_bwd<f16_t, 128>(p, st) : sdpa::launch_bwd<f16_t, 64>(p, st);
 }
@@ -588,8 +668,20 @@ extern "C" int xg_sdpa_backward(const void* q, const void* k, const void* v, con
                                 const int64_t v_strides[3], const int64_t o_strides[3], const int64_t do_strides[3],
                                 const int64_t dq_strides[3], const int64_t dk_strides[3], const int64_t dv_strides[3], float scale,
                                 int causal, int dtype, xg_stream_t stream) {
-  return backward_entry(q, k, v, out, d_out, lse, dq, dk, dv, delta_ws, B, H, Hkv, Sq, Skv, D, q_strides, k_strides, v_strides, o_strides,
-                        do_strides, dq_strides, dk_strides, dv_strides, scale, causal, dtype, stream);
+  return backward_entry(q, k, v, out, d_out, lse, nullptr, nullptr, dtype, nullptr, dq, dk, dv, delta_ws, B, H, Hkv, Sq, Skv, D, q_strides,
+                        k_strides, v_strides, o_strides, do_strides, dq_strides, dk_strides, dv_strides, scale, causal, dtype, stream);
+}
+
+extern "C" int xg_sdpa_backward_masked(const void* q, const void* k, const void* v, const void* out, const void* d_out, const float* lse,
+                                       const void* mask, const int64_t mask_strides[3], int mask_dtype, const float* scale_dev, void* dq,
+                                       void* dk, void* dv, float* delta_ws, int64_t B, int64_t H, int64_t Hkv, int64_t Sq, int64_t Skv,
+                                       int64_t D, const int64_t q_strides[3], const int64_t k_strides[3], const int64_t v_strides[3],
+                                       const int64_t o_strides[3], const int64_t do_strides[3], const int64_t dq_strides[3],
+                                       const int64_t dk_strides[3], const int64_t dv_strides[3], float scale, int causal, int dtype,
+                                       xg_stream_t stream) {
+  return backward_entry(q, k, v, out, d_out, lse, mask, mask_strides, mask_dtype, scale_dev, dq, dk, dv, delta_ws, B, H, Hkv, Sq, Skv, D,
+                        q_strides, k_strides, v_strides, o_strides, do_strides, dq_strides, dk_strides, dv_strides, scale, causal, dtype,
+                        stream);
 }
 
 extern "C" int xg_sdpa_backward_static(const void* q, const void* k, const void* v, const void* out, const void* d_out,
@@ -604,6 +696,6 @@ extern "C" int xg_sdpa_backward_static(const void* q, const void* k, const void*
   if (B == 0 || H == 0) return XG_OK;
   float* ws = nullptr;
   if (int st = scratch_address(&ws)) return st;
-  return backward_entry(q, k, v, out, d_out, lse, dq, dk, dv, ws, B, H, Hkv, Sq, Skv, D, q_strides, k_strides, v_strides, o_strides,
-                        do_strides, dq_strides, dk_strides, dv_strides, scale, causal, dtype, stream);
+  return backward_entry(q, k, v, out, d_out, lse, nullptr, nullptr, dtype, nullptr, dq, dk, dv, ws, B, H, Hkv, Sq, Skv, D, q_strides, k_strides,
+                        v_strides, o_strides, do_strides, dq_strides, dk_strides, dv_strides, scale, causal, dtype, stream);
 }

@@ -614,6 +614,11 @@ _library.define(
     "sdpa_bwd(Tensor q, Tensor k, Tensor v, Tensor out, Tensor d_out, Tensor lse, bool is_causal, float scale) -> (Tensor, Tensor, Tensor)"
 )
 _library.define("sdpa_masked(Tensor q, Tensor k, Tensor v, Tensor? mask, Tensor? scale_t, bool is_causal, float scale) -> Tensor")
+_library.define("sdpa_masked_lse(Tensor q, Tensor k, Tensor v, Tensor? mask, Tensor? scale_t, bool is_causal, float scale) -> (Tensor, Tensor)")
+_library.define(
+    "sdpa_masked_bwd(Tensor q, Tensor k, Tensor v, Tensor out, Tensor d_out, Tensor lse, Tensor? mask, Tensor? scale_t, bool is_causal, "
+    "float scale) -> (Tensor, Tensor, Tensor)"
+)
 _library.define("rope(Tensor x, Tensor cos, Tensor sin) -> Tensor")
 
 
@@ -945,9 +950,34 @@ def sdpa_mask_fits(mask_shape, q_shape, skv):
     return full[2] == Sq and full[3] == skv and full[0] in (1, B) and full[1] in (1, H)
 
 
-def _sdpa_masked(q, k, v, mask, scale_t, is_causal, scale):
-    """Attention with an additive mask and / or a scale held in a one-element device tensor (read by the kernel:
-    no .item(), no synchronisation)."""
+def _mask_operand(mask, q, Skv):
+    """The additive mask as the kernels index it: (tensor kept alive, three element strides, dtype code)."""
+    S3 = ctypes.c_int64 * 3
+    if mask is None:
+        return None, None, _code(q.dtype)
+    if not sdpa_mask_fits(tuple(mask.shape), tuple(q.shape), Skv):
+        raise ValueError("sdpa_masked: the mask must be [Sq, Skv] with up to two leading dims of size 1, B or H")
+    if mask.dtype not in (q.dtype, torch.float32):
+        if not mask.dtype.is_floating_point:
+            raise TypeError("sdpa_masked: the mask must be a floating-point additive mask")
+        mask = mask.float()
+    while mask.dim() < 4:
+        mask = mask.unsqueeze(0)
+    if mask.stride(-1) != 1:
+        mask = mask.contiguous()
+    strides = S3(*[0 if mask.shape[i] == 1 else mask.stride(i) for i in range(2)], mask.stride(2) if q.shape[2] > 1 else 0)
+    return mask, strides, _code(mask.dtype)
+
+
+def _scale_operand(scale_t):
+    if scale_t is None:
+        return None
+    if scale_t.numel() != 1:
+        raise ValueError("sdpa_masked: the scale tensor must have one element")
+    return scale_t.reshape(1).to(torch.float32)  # a device op, not a read
+
+
+def _sdpa_masked_run(q, k, v, mask, scale_t, is_causal, scale, want_lse):
     _sdpa_check(q, k, v)
     if k.dtype != q.dtype or v.dtype != q.dtype:
         raise TypeError("sdpa: q, k, v must share a dtype")
@@ -955,39 +985,74 @@ def _sdpa_masked(q, k, v, mask, scale_t, is_causal, scale):
     B, H, Sq, D = q.shape
     Skv = k.shape[2]
     out = _empty_like_layout(q)
+    lse = torch.empty((B, H, Sq), dtype=torch.float32, device=q.device) if want_lse else None
     if out.numel() == 0:
-        return out
+        return out, lse
     S3 = ctypes.c_int64 * 3
-    mask_strides, mask_dt = None, _code(q.dtype)
-    if mask is not None:
-        if not sdpa_mask_fits(tuple(mask.shape), tuple(q.shape), Skv):
-            raise ValueError("sdpa_masked: the mask must be [Sq, Skv] with up to two leading dims of size 1, B or H")
-        if mask.dtype not in (q.dtype, torch.float32):
-            mask = mask.float() if mask.dtype.is_floating_point else None
-            if mask is None:
-                raise TypeError("sdpa_masked: the mask must be a floating-point additive mask")
-        while mask.dim() < 4:
-            mask = mask.unsqueeze(0)
-        if mask.stride(-1) != 1:
-            mask = mask.contiguous()
-        mask_strides = S3(*[0 if mask.shape[i] == 1 else mask.stride(i) for i in range(2)], mask.stride(2) if Sq > 1 else 0)
-        mask_dt = _code(mask.dtype)
-    if scale_t is not None:
-        if scale_t.numel() != 1:
-            raise ValueError("sdpa_masked: the scale tensor must have one element")
-        scale_t = scale_t.reshape(1).to(torch.float32)  # a device op, not a read
-    st = _lib.lib().xg_sdpa_masked(
-        _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(mask), mask_strides, mask_dt, _ptr(scale_t), B, H, k.shape[1], Sq, Skv, D,
-        S3(*q.stride()[:3]), S3(*k.stride()[:3]), S3(*v.stride()[:3]), S3(*out.stride()[:3]), scale, 1 if is_causal else 0,
+    mask, mask_strides, mask_dt = _mask_operand(mask, q, Skv)
+    scale_t = _scale_operand(scale_t)
+    tail = (mask_strides, mask_dt, _ptr(scale_t), B, H, k.shape[1], Sq, Skv, D, S3(*q.stride()[:3]), S3(*k.stride()[:3]), S3(*v.stride()[:3]),
+            S3(*out.stride()[:3]), scale, 1 if is_causal else 0, _code(q.dtype), _stream())
+    if want_lse:
+        _lib.check(_lib.lib().xg_sdpa_masked_lse(_ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), _ptr(mask), *tail), "xg_sdpa_masked_lse")
+    else:
+        _lib.check(_lib.lib().xg_sdpa_masked(_ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(mask), *tail), "xg_sdpa_masked")
+    return out, lse
+
+
+def _sdpa_masked(q, k, v, mask, scale_t, is_causal, scale):
+    """Attention with an additive mask and / or a scale held in a one-element device tensor (read by the kernel:
+    no .item(), no synchronisation)."""
+    return _sdpa_masked_run(q, k, v, mask, scale_t, is_causal, scale, False)[0]
+
+
+def _sdpa_masked_lse(q, k, v, mask, scale_t, is_causal, scale):
+    """The same, also returning the log-sum-exp of every query row for the backward kernels."""
+    return _sdpa_masked_run(q, k, v, mask, scale_t, is_causal, scale, True)
+
+
+def _sdpa_masked_bwd(q, k, v, out, d_out, lse, mask, scale_t, is_causal, scale):
+    """Gradients of masked / tensor-scaled attention with respect to q, k, v (the mask and the scale tensor get
+    none): the backward kernels add the mask to the recomputed scores as the forward did."""
+    _sdpa_check(q, k, v)
+    if out.shape != q.shape or d_out.shape != q.shape or tuple(lse.shape) != tuple(q.shape[:3]):
+        raise ValueError("sdpa_masked_bwd: out and d_out must have the shape of q, lse its first three dims")
+    if any(t.dtype != q.dtype for t in (k, v, out, d_out)) or lse.dtype != torch.float32:
+        raise TypeError("sdpa_masked_bwd: q, k, v, out, d_out must share a dtype; lse is float32")
+    q, k, v, out, d_out = (_unit_last(t) for t in (q, k, v, out, d_out))
+    lse = lse.contiguous()
+    B, H, Sq, D = q.shape
+    Hkv, Skv = k.shape[1], k.shape[2]
+    dq, dk, dv = _empty_like_layout(q), _empty_like_layout(k), _empty_like_layout(v)
+    if dq.numel() == 0 or dk.numel() == 0:
+        return dq.zero_(), dk.zero_(), dv.zero_()
+    mask, mask_strides, mask_dt = _mask_operand(mask, q, Skv)
+    scale_t = _scale_operand(scale_t)
+    delta = torch.empty((B, H, Sq), dtype=torch.float32, device=q.device)
+    S3 = ctypes.c_int64 * 3
+    st = _lib.lib().xg_sdpa_backward_masked(
+        _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(d_out), _ptr(lse), _ptr(mask), mask_strides, mask_dt, _ptr(scale_t), _ptr(dq), _ptr(dk),
+        _ptr(dv), _ptr(delta), B, H, Hkv, Sq, Skv, D, S3(*q.stride()[:3]), S3(*k.stride()[:3]), S3(*v.stride()[:3]), S3(*out.stride()[:3]),
+        S3(*d_out.stride()[:3]), S3(*dq.stride()[:3]), S3(*dk.stride()[:3]), S3(*dv.stride()[:3]), scale, 1 if is_causal else 0,
         _code(q.dtype), _stream(),
     )
-    _lib.check(st, "xg_sdpa_masked")
-    return out
+    _lib.check(st, "xg_sdpa_backward_masked")
+    return dq, dk, dv
 
 
 def _sdpa_masked_meta(q, k, v, mask, scale_t, is_causal, scale):
     _sdpa_check(q, k, v)
     return _empty_like_layout(_unit_last(q))
+
+
+def _sdpa_masked_lse_meta(q, k, v, mask, scale_t, is_causal, scale):
+    _sdpa_check(q, k, v)
+    return _empty_like_layout(_unit_last(q)), torch.empty(tuple(q.shape[:3]), dtype=torch.float32, device=q.device)
+
+
+def _sdpa_masked_bwd_meta(q, k, v, out, d_out, lse, mask, scale_t, is_causal, scale):
+    _sdpa_check(q, k, v)
+    return tuple(_empty_like_layout(_unit_last(t)) for t in (q, k, v))
 
 
 def _sdpa_meta(q, k, v, is_causal, scale):
@@ -1122,6 +1187,10 @@ _library.impl("sdpa_bwd", _sdpa_bwd, "CUDA")
 _library.impl("sdpa_bwd", _sdpa_bwd_meta, "Meta")
 _library.impl("sdpa_masked", _sdpa_masked, "CUDA")
 _library.impl("sdpa_masked", _sdpa_masked_meta, "Meta")
+_library.impl("sdpa_masked_lse", _sdpa_masked_lse, "CUDA")
+_library.impl("sdpa_masked_lse", _sdpa_masked_lse_meta, "Meta")
+_library.impl("sdpa_masked_bwd", _sdpa_masked_bwd, "CUDA")
+_library.impl("sdpa_masked_bwd", _sdpa_masked_bwd_meta, "Meta")
 _library.impl("rope", _rope, "CUDA")
 _library.impl("rope", _rope_meta, "Meta")
 

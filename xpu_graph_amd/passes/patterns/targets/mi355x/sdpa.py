@@ -11,8 +11,9 @@ Any other floating-point additive mask ([Sq, Skv] with broadcast batch / head
 dims) goes to the kernel as an operand, and so does the one-element scale
 tensor of the reference's `xpu_graph::sdpa_wrapped_scale` form
 (utils/default_replacements.py:39-55), which the kernel reads on the device
-instead of the host reading it with .item() (inference graphs only: these two
-forms carry no backward formula).
+instead of the host reading it with .item().  In training graphs these two
+forms are taken when the mask and the scale tensor need no gradient (the
+backward kernels produce dq, dk, dv only); otherwise the Aten subgraph stays.
 
 The rewrite also looks through the contiguous clones and 3-D reshapes FusedSDPA
 puts in front of q, k, v: the kernel takes strides, so the [B, H, S, D] views
@@ -46,7 +47,35 @@ class SDPAModule(nn.Module):
 
 class SDPAMaskedModule(nn.Module):
     def forward(self, q, k, v, mask, scale_t, is_causal, scale):
+        if torch.is_grad_enabled() and (q.requires_grad or k.requires_grad or v.requires_grad):
+            return torch.ops.xpu_ops.sdpa_masked_lse(q, k, v, mask, scale_t, is_causal, scale)[0]
         return torch.ops.xpu_ops.sdpa_masked(q, k, v, mask, scale_t, is_causal, scale)
+
+
+def _needs_no_grad(node):
+    """In a graph that will be differentiated: the operand is known not to require a gradient, i.e. every graph input
+    it is computed from is marked as not requiring one (the pregrad stage marks the placeholders; an unmarked input
+    counts as requiring a gradient)."""
+    if not isinstance(node, fx.Node):
+        return False
+    seen, todo = set(), [node]
+    while todo:
+        n = todo.pop()
+        if n in seen:
+            continue
+        seen.add(n)
+        if n.op == "placeholder":
+            if n.meta.get("xg_requires_grad", True):
+                return False
+        elif n.op == "get_attr":
+            obj = n.graph.owning_module
+            for part in n.target.split("."):
+                obj = getattr(obj, part, None)
+            if not isinstance(obj, torch.Tensor) or obj.requires_grad:
+                return False
+        else:
+            todo.extend(n.all_input_nodes)
+    return True
 
 
 def _mask_operand_ok(mask, q, k):
@@ -252,7 +281,8 @@ class FusedCausalSDPA(Pattern):
                 if mask is not None:
                     if not causal and is_causal_constant(mask, sq, skv):
                         causal = True
-                    elif self._current_stage == FxStage.inference and isinstance(mask, fx.Node) and _supported(q, k, v) and _mask_operand_ok(mask, q, k):
+                    elif (isinstance(mask, fx.Node) and (self._current_stage == FxStage.inference or _needs_no_grad(mask))
+                          and _supported(q, k, v) and _mask_operand_ok(mask, q, k)):
                         mask_operand = mask  # the kernel adds it; q, k, v go as they are (no peeling: the mask is indexed by [B, H])
                     else:
                         continue
@@ -305,19 +335,20 @@ class FusedCausalSDPA(Pattern):
                         u.replace_all_uses_with(new)
 
                 changed |= self._emit(gm, node, q, k, v, causal, node.kwargs.get("scale"), replace)
-        if self._current_stage == FxStage.inference:
-            for node in self._wrapped_scale_calls(gm):
-                q, k, v, mask, scale_t = node.args
-                if not all(isinstance(n, fx.Node) and isinstance(n.meta.get("val"), torch.Tensor) for n in (q, k, v, scale_t)):
+        for node in self._wrapped_scale_calls(gm):
+            q, k, v, mask, scale_t = node.args
+            if not all(isinstance(n, fx.Node) and isinstance(n.meta.get("val"), torch.Tensor) for n in (q, k, v, scale_t)):
+                continue
+            if self._current_stage != FxStage.inference and not (_needs_no_grad(scale_t) and (mask is None or _needs_no_grad(mask))):
+                continue
+            if not _supported(q, k, v) or scale_t.meta["val"].numel() != 1:
+                continue
+            causal = False
+            if mask is not None:
+                sq, skv = q.meta["val"].shape[2], k.meta["val"].shape[2]
+                if isinstance(mask, fx.Node) and is_causal_constant(mask, sq, skv):
+                    mask, causal = None, True
+                elif not (isinstance(mask, fx.Node) and _mask_operand_ok(mask, q, k)):
                     continue
-                if not _supported(q, k, v) or scale_t.meta["val"].numel() != 1:
-                    continue
-                causal = False
-                if mask is not None:
-                    sq, skv = q.meta["val"].shape[2], k.meta["val"].shape[2]
-                    if isinstance(mask, fx.Node) and is_causal_constant(mask, sq, skv):
-                        mask, causal = None, True
-                    elif not (isinstance(mask, fx.Node) and _mask_operand_ok(mask, q, k)):
-                        continue
-                changed |= self._emit(gm, node, q, k, v, causal, 1.0, node.replace_all_uses_with, mask=mask, scale_t=scale_t)
+            changed |= self._emit(gm, node, q, k, v, causal, 1.0, node.replace_all_uses_with, mask=mask, scale_t=scale_t)
         return changed
