@@ -380,6 +380,27 @@ int xg_sdpa_backward_masked(const void* q, const void* k, const void* v, const v
                             const int64_t dv_strides[3], float scale, int causal, int dtype, xg_stream_t stream);
 
 /* ---------------------------------------------------------------------------
+ * xg_sdpa (no causal flag, no mask) for a decode step: Sq <= 32 query rows per
+ * head against long K / V.  The keys are split over workgroups (and the query
+ * heads of one key/value head share a workgroup when H / Hkv * Sq <= 32), so
+ * K and V stream at memory speed instead of through B * H compute units.
+ *   lse: NULL or [B,H,Sq] fp32 as in xg_sdpa_lse.
+ *   workspace: NULL or `workspace_floats` fp32 of device memory for the partial
+ *     results of the key ranges; xg_sdpa_decode_workspace_floats gives the size
+ *     that allows the preferred split (0: none needed).  With less, the keys
+ *     are split into as many ranges as fit, down to one.
+ *   Sq > 32: XG_ERR_BAD_SHAPE (use xg_sdpa).
+ * replaces aten.scaled_dot_product_attention as emitted by FusedSDPA
+ *   (passes/patterns/common/fuse_scaled_dot_product_attention.py:184-234) for
+ *   the shapes of incremental decoding.
+ * ------------------------------------------------------------------------- */
+int64_t xg_sdpa_decode_workspace_floats(int64_t B, int64_t H, int64_t Hkv, int64_t Sq, int64_t Skv, int64_t D);
+int xg_sdpa_decode(const void* q, const void* k, const void* v, void* out, float* lse, float* workspace,
+                   int64_t workspace_floats, int64_t B, int64_t H, int64_t Hkv, int64_t Sq, int64_t Skv, int64_t D,
+                   const int64_t q_strides[3], const int64_t k_strides[3], const int64_t v_strides[3],
+                   const int64_t o_strides[3], float scale, int dtype, xg_stream_t stream);
+
+/* ---------------------------------------------------------------------------
  * xg_sdpa_backward without the workspace argument, for callers that cannot
  * allocate device memory (code under HIP graph capture, serving loops and
  * harnesses that forbid hipMalloc).  No counterpart in the reference.  The

@@ -19,7 +19,7 @@ def declared_symbols():
 def test_header_declares_the_expected_entry_points():
     syms = declared_symbols()
     for s in ("xg_rms_norm", "xg_layer_norm", "xg_add_rms_norm", "xg_add_layer_norm", "xg_rms_norm_bwd", "xg_layer_norm_bwd", "xg_slice_cat", "xg_addn",
-              "xg_combo_sum", "xg_slice_sum_cat", "xg_silu_mul", "xg_silu_mul2", "xg_silu_mul2_bwd", "xg_activation", "xg_activation_bwd", "xg_dense", "xg_dense_batched", "xg_dense_at", "xg_dense_glu", "xg_dense_glu_save", "xg_dense_fp8", "xg_slice_cat_check_table", "xg_sdpa", "xg_sdpa_masked", "xg_sdpa_lse", "xg_sdpa_backward", "xg_sdpa_masked_lse", "xg_sdpa_backward_masked", "xg_sdpa_backward_static", "xg_rope", "xg_copy_bytes", "xg_clock_probe", "xg_wall_clock_khz",
+              "xg_combo_sum", "xg_slice_sum_cat", "xg_silu_mul", "xg_silu_mul2", "xg_silu_mul2_bwd", "xg_activation", "xg_activation_bwd", "xg_dense", "xg_dense_batched", "xg_dense_at", "xg_dense_glu", "xg_dense_glu_save", "xg_dense_fp8", "xg_slice_cat_check_table", "xg_sdpa", "xg_sdpa_masked", "xg_sdpa_lse", "xg_sdpa_backward", "xg_sdpa_masked_lse", "xg_sdpa_backward_masked", "xg_sdpa_decode", "xg_sdpa_decode_workspace_floats", "xg_sdpa_backward_static", "xg_rope", "xg_copy_bytes", "xg_clock_probe", "xg_wall_clock_khz",
               "xg_version", "xg_status_string"):
         assert s in syms
 
@@ -185,6 +185,27 @@ def test_masked_backward_validation_needs_no_gpu():
     assert call(ctypes.c_void_p(257), S3(0, 0, 64), 2, None) == -3
     assert call(None, None, 2, ctypes.c_void_p(258)) == -3
     assert lib.xg_sdpa_masked_lse(p, p, p, p, None, None, None, 2, None, 1, 4, 4, 64, 64, 64, st, st, st, st, 0.125, 0, 2, None) == -4
+
+
+def test_decode_attention_validation_and_workspace_size_need_no_gpu():
+    from xpu_graph_amd import _lib
+
+    lib = _lib.lib()
+    S3 = ctypes.c_int64 * 3
+    p = ctypes.c_void_p(256)
+    st = S3(32 * 4096 * 128, 4096 * 128, 128)
+    tail = (st, st, st, st, 0.1, 2, None)
+    assert lib.xg_sdpa_decode(p, p, p, p, None, None, 0, 1, 32, 32, 33, 4096, 128, *tail) == -2   # more rows than a workgroup holds
+    assert lib.xg_sdpa_decode(p, p, p, p, None, None, 0, 1, 32, 32, 1, 4096, 96, *tail) == -2    # head size
+    assert lib.xg_sdpa_decode(p, p, p, p, None, None, 0, 1, 32, 5, 1, 4096, 128, *tail) == -2    # heads do not divide
+    assert lib.xg_sdpa_decode(p, p, None, p, None, None, 0, 1, 32, 32, 1, 4096, 128, *tail) == -4
+    assert lib.xg_sdpa_decode(p, p, p, p, None, None, 0, 1, 32, 32, 1, 4096, 128, st, st, st, st, 0.1, 0, None) == -1  # fp32 tensors
+    assert lib.xg_sdpa_decode(p, p, p, p, None, ctypes.c_void_p(260), 1 << 20, 1, 32, 32, 1, 4096, 128, *tail) == -3
+    assert lib.xg_sdpa_decode(p, p, p, p, None, None, 0, 0, 32, 32, 1, 4096, 128, *tail) == 0    # nothing to do
+    # 32 problems of 32 tiles: 16 key ranges of two tiles each, 32 x 128 + 64 floats per range
+    assert lib.xg_sdpa_decode_workspace_floats(1, 32, 32, 1, 4096, 128) == 32 * 16 * (32 * 128 + 64)
+    assert lib.xg_sdpa_decode_workspace_floats(64, 32, 32, 1, 4096, 128) == 0                     # 2048 problems fill the chip as they are
+    assert lib.xg_sdpa_decode_workspace_floats(1, 32, 32, 33, 4096, 128) == 0
 
 
 def test_a_missing_library_is_an_error_not_a_fallback(monkeypatch, tmp_path):

@@ -133,6 +133,55 @@ def test_sdpa_scale_from_a_device_tensor(device):
         _ops().sdpa_masked(q, k, v, torch.zeros(3, 192, 160, device=device), None, False, 0.1)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("B,H,Hkv,Sq,Skv,D", [
+    (1, 32, 32, 1, 2048, 128),   # one query row per head
+    (2, 8, 2, 1, 1000, 128),     # four query heads share a key/value head and a workgroup; ragged last tile
+    (2, 8, 2, 4, 513, 64),       # 16 packed rows, one key in the last tile
+    (1, 8, 1, 5, 4100, 128),     # 40 rows do not fit one tile: one query head per workgroup
+    (3, 4, 4, 32, 777, 64),      # the most rows a workgroup holds
+    (1, 2, 1, 16, 640, 128),     # 32 packed rows exactly
+    (1, 4, 4, 3, 8192, 128),     # long context: many key ranges per head
+])
+def test_sdpa_decode_sizes_split_the_keys(device, dtype, B, H, Hkv, Sq, Skv, D):
+    """A decode step (at most 32 query rows per head, no causal flag) runs on the key-split kernel: against the fp32
+    anchor, with the log-sum-exp of every row, on K / V held as [B, S, H, D] (a cache layout) as well, and through the
+    C ABI with no workspace (one key range) and with the preferred one."""
+    import ctypes
+
+    from xpu_graph_amd import _lib
+
+    q, k, v = make(B, H, Hkv, Sq, Skv, D, dtype, device, seed=Sq + Skv + D + H)
+    scale = 1.0 / math.sqrt(D)
+    want = ref32(q, k, v, False, scale)
+    got = _ops().sdpa(q, k, v, False, scale)
+    assert got.shape == q.shape and got.dtype == dtype
+    close(got, want)
+    out, lse = _ops().sdpa_lse(q, k, v, False, scale)
+    assert torch.equal(out, got)
+    rep = H // Hkv
+    s = torch.matmul(q.float(), k.float().repeat_interleave(rep, dim=1).transpose(-1, -2)) * scale
+    torch.testing.assert_close(lse, torch.logsumexp(s, dim=-1), rtol=1e-4, atol=1e-4)
+    kc, vc = (t.transpose(1, 2).contiguous().transpose(1, 2) for t in (k, v))  # [B, S, Hkv, D] storage
+    assert torch.equal(_ops().sdpa(q, kc, vc, False, scale), got)
+    S3 = ctypes.c_int64 * 3
+    P = lambda t: ctypes.c_void_p(t.data_ptr())  # noqa: E731
+    st = lambda t: S3(*t.stride()[:3])  # noqa: E731
+    lib = _lib.lib()
+    n_ws = lib.xg_sdpa_decode_workspace_floats(B, H, Hkv, Sq, Skv, D)
+    code = 2 if dtype == torch.bfloat16 else 1
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    for ws_floats in sorted({0, n_ws}):
+        ws = torch.empty(max(ws_floats, 1), device=device)
+        o = torch.full_like(q, float("nan"))
+        rc = lib.xg_sdpa_decode(P(q), P(k), P(v), P(o), None, P(ws) if ws_floats else None, ws_floats, B, H, Hkv, Sq, Skv, D, st(q), st(k), st(v),
+                                st(o), scale, code, stream)
+        assert rc == 0
+        close(o, want)
+        if ws_floats == n_ws:
+            assert torch.equal(o, got)
+
+
 def test_sdpa_matches_oracle_causal(device):
     q, k, v = make(1, 4, 4, 512, 512, 128, torch.bfloat16, device, seed=5)
     got = _ops().sdpa(q, k, v, True, 1.0 / math.sqrt(128))

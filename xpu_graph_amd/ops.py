@@ -883,6 +883,12 @@ def _empty_like_layout(t):
     return torch.empty(t.shape, dtype=t.dtype, device=t.device)
 
 
+# Up to this many query rows per head, against at least this many keys, attention runs on the key-split decode kernel
+# (with fewer keys the general kernel's single tile walk is as fast).
+_DECODE_ROWS = 32
+_DECODE_MIN_KEYS = 512
+
+
 def _sdpa_run(q, k, v, is_causal, scale, want_lse):
     _sdpa_check(q, k, v)
     if k.dtype != q.dtype or v.dtype != q.dtype:
@@ -895,6 +901,13 @@ def _sdpa_run(q, k, v, is_causal, scale, want_lse):
         return out, lse
     S3 = ctypes.c_int64 * 3
     shape = (B, H, k.shape[1], Sq, k.shape[2], D, S3(*q.stride()[:3]), S3(*k.stride()[:3]), S3(*v.stride()[:3]), S3(*out.stride()[:3]))
+    if not is_causal and Sq <= _DECODE_ROWS and k.shape[2] >= _DECODE_MIN_KEYS:
+        # a decode step: the keys are split over workgroups; the partial results go through a small workspace
+        n_ws = _lib.lib().xg_sdpa_decode_workspace_floats(B, H, k.shape[1], Sq, k.shape[2], D)
+        ws = torch.empty((n_ws,), dtype=torch.float32, device=q.device) if n_ws > 0 else None
+        st = _lib.lib().xg_sdpa_decode(_ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), _ptr(ws), n_ws, *shape, scale, _code(q.dtype), _stream())
+        _lib.check(st, "xg_sdpa_decode")
+        return out, lse
     tail = (scale, 1 if is_causal else 0, _code(q.dtype), _stream())
     if want_lse:
         _lib.check(_lib.lib().xg_sdpa_lse(_ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), *shape, *tail), "xg_sdpa_lse")
