@@ -380,11 +380,12 @@ int xg_sdpa_backward_masked(const void* q, const void* k, const void* v, const v
                             const int64_t dv_strides[3], float scale, int causal, int dtype, xg_stream_t stream);
 
 /* ---------------------------------------------------------------------------
- * xg_sdpa (no causal flag, no mask) for a decode step: Sq <= 32 query rows per
- * head against long K / V.  The keys are split over workgroups (and the query
+ * xg_sdpa / xg_sdpa_masked (no causal flag) for a decode step: Sq <= 32 query
+ * rows per head against long K / V.  The keys are split over workgroups (and the query
  * heads of one key/value head share a workgroup when H / Hkv * Sq <= 32), so
  * K and V stream at memory speed instead of through B * H compute units.
  *   lse: NULL or [B,H,Sq] fp32 as in xg_sdpa_lse.
+ *   mask, mask_strides, mask_dtype, scale_dev: as in xg_sdpa_masked (NULL: none).
  *   workspace: NULL or `workspace_floats` fp32 of device memory for the partial
  *     results of the key ranges; xg_sdpa_decode_workspace_floats gives the size
  *     that allows the preferred split (0: none needed).  With less, the keys
@@ -395,7 +396,8 @@ int xg_sdpa_backward_masked(const void* q, const void* k, const void* v, const v
  *   the shapes of incremental decoding.
  * ------------------------------------------------------------------------- */
 int64_t xg_sdpa_decode_workspace_floats(int64_t B, int64_t H, int64_t Hkv, int64_t Sq, int64_t Skv, int64_t D);
-int xg_sdpa_decode(const void* q, const void* k, const void* v, void* out, float* lse, float* workspace,
+int xg_sdpa_decode(const void* q, const void* k, const void* v, void* out, float* lse, const void* mask,
+                   const int64_t mask_strides[3], int mask_dtype, const float* scale_dev, float* workspace,
                    int64_t workspace_floats, int64_t B, int64_t H, int64_t Hkv, int64_t Sq, int64_t Skv, int64_t D,
                    const int64_t q_strides[3], const int64_t k_strides[3], const int64_t v_strides[3],
                    const int64_t o_strides[3], float scale, int dtype, xg_stream_t stream);

@@ -195,13 +195,21 @@ def test_decode_attention_validation_and_workspace_size_need_no_gpu():
     p = ctypes.c_void_p(256)
     st = S3(32 * 4096 * 128, 4096 * 128, 128)
     tail = (st, st, st, st, 0.1, 2, None)
-    assert lib.xg_sdpa_decode(p, p, p, p, None, None, 0, 1, 32, 32, 33, 4096, 128, *tail) == -2   # more rows than a workgroup holds
-    assert lib.xg_sdpa_decode(p, p, p, p, None, None, 0, 1, 32, 32, 1, 4096, 96, *tail) == -2    # head size
-    assert lib.xg_sdpa_decode(p, p, p, p, None, None, 0, 1, 32, 5, 1, 4096, 128, *tail) == -2    # heads do not divide
-    assert lib.xg_sdpa_decode(p, p, None, p, None, None, 0, 1, 32, 32, 1, 4096, 128, *tail) == -4
-    assert lib.xg_sdpa_decode(p, p, p, p, None, None, 0, 1, 32, 32, 1, 4096, 128, st, st, st, st, 0.1, 0, None) == -1  # fp32 tensors
-    assert lib.xg_sdpa_decode(p, p, p, p, None, ctypes.c_void_p(260), 1 << 20, 1, 32, 32, 1, 4096, 128, *tail) == -3
-    assert lib.xg_sdpa_decode(p, p, p, p, None, None, 0, 0, 32, 32, 1, 4096, 128, *tail) == 0    # nothing to do
+
+    def call(B, H, Hkv, Sq, Skv, D, v=p, mask=None, mask_strides=None, mask_dtype=2, scale_dev=None, ws=None, ws_floats=0, tail=tail):
+        return lib.xg_sdpa_decode(p, p, v, p, None, mask, mask_strides, mask_dtype, scale_dev, ws, ws_floats, B, H, Hkv, Sq, Skv, D, *tail)
+
+    assert call(1, 32, 32, 33, 4096, 128) == -2   # more rows than a workgroup holds
+    assert call(1, 32, 32, 1, 4096, 96) == -2     # head size
+    assert call(1, 32, 5, 1, 4096, 128) == -2     # heads do not divide
+    assert call(1, 32, 32, 1, 4096, 128, v=None) == -4
+    assert call(1, 32, 32, 1, 4096, 128, tail=(st, st, st, st, 0.1, 0, None)) == -1  # fp32 tensors
+    assert call(1, 32, 32, 1, 4096, 128, ws=ctypes.c_void_p(260), ws_floats=1 << 20) == -3
+    assert call(1, 32, 32, 1, 4096, 128, mask=p) == -4                                 # a mask without strides
+    assert call(1, 32, 32, 1, 4096, 128, mask=p, mask_strides=S3(0, 0, 0), mask_dtype=1) == -1
+    assert call(1, 32, 32, 2, 4096, 128, mask=p, mask_strides=S3(0, 0, 100)) == -2     # mask rows overlap
+    assert call(1, 32, 32, 1, 4096, 128, scale_dev=ctypes.c_void_p(258)) == -3
+    assert call(0, 32, 32, 1, 4096, 128) == 0     # nothing to do
     # 32 problems of 32 tiles: 16 key ranges of two tiles each, 32 x 128 + 64 floats per range
     assert lib.xg_sdpa_decode_workspace_floats(1, 32, 32, 1, 4096, 128) == 32 * 16 * (32 * 128 + 64)
     assert lib.xg_sdpa_decode_workspace_floats(64, 32, 32, 1, 4096, 128) == 0                     # 2048 problems fill the chip as they are

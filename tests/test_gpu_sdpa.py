@@ -174,12 +174,46 @@ def test_sdpa_decode_sizes_split_the_keys(device, dtype, B, H, Hkv, Sq, Skv, D):
     for ws_floats in sorted({0, n_ws}):
         ws = torch.empty(max(ws_floats, 1), device=device)
         o = torch.full_like(q, float("nan"))
-        rc = lib.xg_sdpa_decode(P(q), P(k), P(v), P(o), None, P(ws) if ws_floats else None, ws_floats, B, H, Hkv, Sq, Skv, D, st(q), st(k), st(v),
-                                st(o), scale, code, stream)
+        rc = lib.xg_sdpa_decode(P(q), P(k), P(v), P(o), None, None, None, code, None, P(ws) if ws_floats else None, ws_floats, B, H, Hkv, Sq, Skv,
+                                D, st(q), st(k), st(v), st(o), scale, code, stream)
         assert rc == 0
         close(o, want)
         if ws_floats == n_ws:
             assert torch.equal(o, got)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("mask_shape,mask_dtype", [("full", "same"), ("rows", "f32"), ("per_batch", "same"), ("per_head", "f32")])
+@pytest.mark.parametrize("H,Hkv,Sq,Skv,D", [(8, 8, 1, 1024, 128), (8, 2, 3, 777, 64), (4, 4, 32, 2050, 128)])
+def test_sdpa_decode_sizes_with_a_mask_and_a_tensor_scale(device, dtype, mask_shape, mask_dtype, H, Hkv, Sq, Skv, D):
+    """The attn_mask form at decode shapes (padding masks of batched decoding: [B, 1, 1 | Sq, Skv]) and the scale in a
+    device tensor run on the key-split kernel as well; keys hidden with -inf, whole 32-key blocks of them included; a
+    row hidden completely is NaN, as in eager."""
+    B = 2
+    q, k, v = make(B, H, Hkv, Sq, Skv, D, dtype, device, seed=Sq * 7 + Skv + D)
+    g = torch.Generator().manual_seed(Sq + Skv)
+    shape = {"full": (B, H, Sq, Skv), "rows": (Sq, Skv), "per_batch": (B, 1, Sq, Skv), "per_head": (1, H, Sq, Skv)}[mask_shape]
+    mask = torch.randn(shape, generator=g)
+    pad = torch.rand(shape[:-2] + (1, Skv), generator=g) < 0.2
+    pad[..., 0] = False
+    pad[..., 200:300] = True  # whole blocks of hidden keys
+    mask = mask.masked_fill(pad.expand(shape), float("-inf")).to(dtype if mask_dtype == "same" else torch.float32).to(device)
+    scale = 1.0 / math.sqrt(D)
+    got = _ops().sdpa_masked(q, k, v, mask, None, False, scale)
+    close(got, ref32_masked(q, k, v, mask, False, scale))
+    t = torch.tensor([0.05], device=device)
+    close(_ops().sdpa_masked(q, k, v, mask, t, False, 123.0), ref32_masked(q, k, v, mask, False, 0.05))
+    assert torch.equal(_ops().sdpa_masked(q, k, v, None, t, False, 123.0), _ops().sdpa(q, k, v, False, t.item()))
+    out, lse = _ops().sdpa_masked_lse(q, k, v, mask, None, False, scale)
+    assert torch.equal(out, got)
+    rep = H // Hkv
+    s = torch.matmul(q.float(), k.float().repeat_interleave(rep, dim=1).transpose(-1, -2)) * scale + mask.float()
+    torch.testing.assert_close(lse, torch.logsumexp(s, dim=-1), rtol=1e-4, atol=1e-4)
+    if mask_shape == "rows":
+        hidden = mask.clone()
+        hidden[0] = float("-inf")
+        out = _ops().sdpa_masked(q, k, v, hidden, None, False, scale)
+        assert torch.isnan(out[:, :, 0]).all() and (Sq == 1 or not torch.isnan(out[:, :, 1:]).any())
 
 
 def test_sdpa_matches_oracle_causal(device):

@@ -59,7 +59,7 @@ def run_backward(q, k, v, g, causal, scale):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("D", [128, 64])
 @pytest.mark.parametrize("causal", [True, False])
-@pytest.mark.parametrize("Sq,Skv", [(256, 256), (128, 64), (1, 1), (1, 300), (129, 65), (200, 333), (333, 200), (64, 1000), (640, 512)])
+@pytest.mark.parametrize("Sq,Skv", [(256, 256), (128, 64), (1, 1), (1, 300), (129, 65), (200, 333), (333, 200), (64, 1000), (640, 512), (16, 640)])
 def test_backward_shapes(device, dtype, D, causal, Sq, Skv):
     q, k, v = make(2, 3, 3, Sq, Skv, D, dtype, device, seed=Sq + Skv + D)
     g = torch.randn(q.shape, generator=torch.Generator().manual_seed(7)).to(dtype).to(device)

@@ -133,7 +133,8 @@ _SIGNATURES = {
     "xg_sdpa_decode_workspace_floats": (c_int64, [c_int64] * 6),
     "xg_sdpa_decode": (
         c_int,
-        [c_void_p] * 6 + [c_int64] * 7 + [ctypes.POINTER(c_int64)] * 4 + [c_float, c_int, c_void_p],
+        [c_void_p] * 6 + [ctypes.POINTER(c_int64), c_int, c_void_p, c_void_p] + [c_int64] * 7 + [ctypes.POINTER(c_int64)] * 4
+        + [c_float, c_int, c_void_p],
     ),
     "xg_sdpa_masked_lse": (
         c_int,

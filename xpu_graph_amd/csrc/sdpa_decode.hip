@@ -1,4 +1,4 @@
-// Attention for a decode step on gfx950: at most 32 query rows per key/value head, no mask.
+// Attention for a decode step on gfx950: at most 32 query rows per head, optional additive mask, no causal flag.
 //
 // The general forward kernel gives every workgroup 128 query rows and lets it walk all keys: with one query row per
 // head that is B x H workgroups, each streaming a whole K and V through one compute unit.  Here the KEYS are split
@@ -29,6 +29,11 @@ struct DecodeParams {
   int B, H, Hkv, Sq, Skv;
   int64_t qs[3], ks[3], vs[3], os[3];
   float c;         // scale * log2(e)
+  const float* scale_dev;  // when set: the scale is read from this one-element device tensor instead
+  const void* mask;        // additive mask (MASK kernels only), element [b, h, i, j] at ms[0] b + ms[1] h + ms[2] i + j
+  int64_t ms[3];           // element strides of batch, head, query row (0: broadcast)
+  int mask_f32;            // mask elements are fp32 (else the dtype of q)
+  int mask_vec;            // rows of the mask can be read four elements at a time
   int pack;        // query heads per workgroup (H / Hkv, or 1)
   int n_split;     // key ranges per problem
   int tiles_per_split;
@@ -45,7 +50,8 @@ constexpr int decode_ws_floats() {
 }
 
 // Merge n partial results of one query row: out = sum_i 2^(m_i - M) o_i, L = sum_i 2^(m_i - M) l_i, M = max m_i.
-// A partial without any visible key has m = -inf and weight 0; at least one partial has a finite maximum.
+// A partial without any visible key has m = -inf and weight 0; a row that a mask hides completely has sum 0 and comes
+// out as NaN (0 / 0), as in eager.
 template <typename T, int D>
 __device__ __forceinline__ void store_row_part(const DecodeParams& p, int b, int head0, int r, int d0, const float (&acc)[D / 8], float M, float L) {
   const int rows = p.pack * p.Sq;
@@ -66,7 +72,9 @@ __device__ __forceinline__ void store_row_part(const DecodeParams& p, int b, int
   if (p.lse && d0 == 0) p.lse[((int64_t)b * p.H + head) * p.Sq + sq] = (M + log2f(L)) * 0.69314718055994530942f;
 }
 
-template <typename T, int D>
+// MASK: an additive mask is added to the scaled scores, as in the general kernel; a row whose every key is masked with
+// -inf comes out as NaN, as it does in eager.
+template <typename T, int D, bool MASK = false>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 2))) void sdpa_decode_kernel(DecodeParams p) {
   typedef typename Vec8<T>::type V8;
   constexpr int RB = D * 2, TILE = DKV * RB, STAGE = 2 * TILE, KK = D / 16, DT = D / 32;
@@ -84,11 +92,15 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 2))
   const int head0 = hg * p.pack, hkv = head0 / (p.H / p.Hkv);
   const int rows = p.pack * p.Sq;
 
+  const float c_eff = p.scale_dev ? *p.scale_dev * 1.44269504088896340736f : p.c;
+
   // ---- this lane's query row (rows past the end repeat the last one; they are not stored)
   V8 qf[KK];
+  int64_t mbase = 0;
   {
     const int r = l32 < rows ? l32 : rows - 1;
     const int head = head0 + r / p.Sq, sq = r % p.Sq;
+    if constexpr (MASK) mbase = (int64_t)b * p.ms[0] + (int64_t)head * p.ms[1] + (int64_t)sq * p.ms[2];
     const T* qg = reinterpret_cast<const T*>(p.q) + (int64_t)b * p.qs[0] + (int64_t)head * p.qs[1] + (int64_t)sq * p.qs[2];
     static_for<KK>([&](auto KI) {
       constexpr int kk = decltype(KI)::value;
@@ -155,20 +167,50 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 2))
     });
     // s[v] = <key key0 + 8 (v / 4) + 4 h + v % 4, query row l32>, scaled to the exponent's base 2; keys past the end -> -inf
     const int rel = p.Skv - 1 - key0 - 4 * h;
+    if constexpr (MASK) {
+      // key indices are clamped for the loads; what lies past the end is masked by index below
+      constexpr float kLog2e = 1.44269504088896340736f;
+      static_for<4>([&](auto GI) {
+        constexpr int g = decltype(GI)::value;
+        const int kfirst = key0 + 8 * g + 4 * h;
+        float m4[4];
+        if (p.mask_vec && kfirst + 3 < p.Skv) {
+          if (p.mask_f32) {
+            const f32x4 mv = *reinterpret_cast<const f32x4*>(reinterpret_cast<const float*>(p.mask) + mbase + kfirst);
+            m4[0] = mv[0], m4[1] = mv[1], m4[2] = mv[2], m4[3] = mv[3];
+          } else {
+            typedef T t4 __attribute__((ext_vector_type(4)));
+            const t4 mv = *reinterpret_cast<const t4*>(reinterpret_cast<const T*>(p.mask) + mbase + kfirst);
+            m4[0] = (float)mv[0], m4[1] = (float)mv[1], m4[2] = (float)mv[2], m4[3] = (float)mv[3];
+          }
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const int key = kfirst + e < p.Skv ? kfirst + e : p.Skv - 1;
+            m4[e] = p.mask_f32 ? reinterpret_cast<const float*>(p.mask)[mbase + key] : (float)reinterpret_cast<const T*>(p.mask)[mbase + key];
+          }
+        }
+        static_for<4>([&](auto EI) {
+          constexpr int e = decltype(EI)::value;
+          s[4 * g + e] = __builtin_fmaf(s[4 * g + e], c_eff, m4[e] * kLog2e);
+        });
+      });
+    }
     float mx = -INFINITY;
     static_for<16>([&](auto VI) {
       constexpr int v = decltype(VI)::value;
       constexpr int key = 8 * (v / 4) + (v % 4);
-      s[v] = key > rel ? -INFINITY : s[v] * p.c;
+      s[v] = key > rel ? -INFINITY : (MASK ? s[v] : s[v] * c_eff);
       mx = fmaxf(mx, s[v]);
     });
     mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));  // lanes l and l ^ 32 share a query row
-    const float m_new = fmaxf(m_run, mx);       // finite: key key0 itself is visible
-    const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+    const float m_new = fmaxf(m_run, mx);
+    const float m_use = m_new == -INFINITY ? 0.f : m_new;  // a row that a mask has hidden completely so far
+    const float alpha = __builtin_amdgcn_exp2f(m_run - m_use);
     float psum = 0.f;
     static_for<16>([&](auto VI) {
       constexpr int v = decltype(VI)::value;
-      const float e = __builtin_amdgcn_exp2f(s[v] - m_new);
+      const float e = __builtin_amdgcn_exp2f(s[v] - m_use);
       s[v] = e;
       psum += e;
     });
@@ -225,7 +267,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 2))
   for (int e = 0; e < PER; ++e) acc[e] = 0.f;
 #pragma unroll
   for (int w = 0; w < 4; ++w) {
-    const float f = __builtin_amdgcn_exp2f(stat[w * 64 + r] - M);  // 0 for a wave that saw no key
+    const float mw = stat[w * 64 + r];
+    const float f = mw == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mw - M);  // a wave that saw no visible key adds nothing
     L = __builtin_fmaf(stat[w * 64 + 32 + r], f, L);
 #pragma unroll
     for (int e = 0; e < PER; e += 4) {
@@ -284,7 +327,7 @@ __global__ __launch_bounds__(kThreads) void sdpa_decode_merge_kernel(DecodeParam
     }
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
-      const float w = s0 + u < p.n_split ? __builtin_amdgcn_exp2f(f[u] - M) : 0.f;
+      const float w = (s0 + u < p.n_split && f[u] != -INFINITY) ? __builtin_amdgcn_exp2f(f[u] - M) : 0.f;  // a range without a visible key adds nothing
       L = __builtin_fmaf(l4[u], w, L);
 #pragma unroll
       for (int e = 0; e < PER / 4; ++e) {
@@ -308,12 +351,12 @@ inline void decode_split(int64_t problems, int64_t Skv, int& n_split, int& tiles
   n_split = (int)((n_tiles + tps - 1) / tps);
 }
 
-template <typename T, int D>
+template <typename T, int D, bool MASK = false>
 int launch_decode(const DecodeParams& p, hipStream_t stream) {
   constexpr int STAGES = 2 * 2 * DKV * D * 2;
   constexpr int PARK = (4 * DROWS * (D + 4) + 4 * 64) * 4;
   constexpr int SMEM = STAGES > PARK ? STAGES : PARK;
-  auto kernel = sdpa_decode_kernel<T, D>;
+  auto kernel = sdpa_decode_kernel<T, D, MASK>;
   if (int st = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), SMEM)) return st;
   const int64_t problems = (int64_t)p.B * (p.H / p.pack);
   hipLaunchKernelGGL(kernel, dim3((unsigned)(problems * p.n_split)), dim3(kThreads), SMEM, stream, p);
@@ -345,7 +388,8 @@ extern "C" int64_t xg_sdpa_decode_workspace_floats(int64_t B, int64_t H, int64_t
   return problems * n_split * (D == 128 ? sdpa::decode_ws_floats<128>() : sdpa::decode_ws_floats<64>());
 }
 
-extern "C" int xg_sdpa_decode(const void* q, const void* k, const void* v, void* out, float* lse, float* workspace, int64_t workspace_floats,
+extern "C" int xg_sdpa_decode(const void* q, const void* k, const void* v, void* out, float* lse, const void* mask,
+                              const int64_t mask_strides[3], int mask_dtype, const float* scale_dev, float* workspace, int64_t workspace_floats,
                               int64_t B, int64_t H, int64_t Hkv, int64_t Sq, int64_t Skv, int64_t D, const int64_t q_strides[3],
                               const int64_t k_strides[3], const int64_t v_strides[3], const int64_t o_strides[3], float scale, int dtype,
                               xg_stream_t stream) {
@@ -385,6 +429,27 @@ extern "C" int xg_sdpa_decode(const void* q, const void* k, const void* v, void*
   p.Sq = (int)Sq;
   p.Skv = (int)Skv;
   p.c = scale * 1.44269504088896340736f;
+  if (scale_dev && !aligned_to(scale_dev, 4)) return XG_ERR_BAD_ALIGN;
+  p.scale_dev = scale_dev;
+  p.mask = mask;
+  p.mask_f32 = 0;
+  p.mask_vec = 0;
+  p.ms[0] = p.ms[1] = p.ms[2] = 0;
+  if (mask) {  // the same conditions as xg_sdpa_masked
+    if (!mask_strides) return XG_ERR_NULL_PTR;
+    if (mask_dtype != dtype && mask_dtype != XG_F32) return XG_ERR_BAD_DTYPE;
+    const size_t esz = mask_dtype == XG_F32 ? 4 : 2;
+    if (!aligned_to(mask, esz)) return XG_ERR_BAD_ALIGN;
+    bool vec = aligned_to(mask, 4 * esz);
+    for (int i = 0; i < 3; ++i) {
+      if (mask_strides[i] < 0) return XG_ERR_BAD_SHAPE;
+      p.ms[i] = mask_strides[i];
+      vec = vec && mask_strides[i] % 4 == 0;
+    }
+    if (Sq > 1 && mask_strides[2] != 0 && mask_strides[2] < Skv) return XG_ERR_BAD_SHAPE;  // rows would overlap
+    p.mask_f32 = mask_dtype == XG_F32 ? 1 : 0;
+    p.mask_vec = vec ? 1 : 0;
+  }
   p.pack = decode_pack(H, Hkv, Sq);
   const int64_t problems = B * (H / p.pack);
   sdpa::decode_split(problems, Skv, p.n_split, p.tiles_per_split);
@@ -399,6 +464,10 @@ extern "C" int xg_sdpa_decode(const void* q, const void* k, const void* v, void*
   }
   if (problems * p.n_split > 0x7fffffffLL) return XG_ERR_TOO_LARGE;
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  if (mask) {
+    if (dtype == XG_BF16) return D == 128 ? sdpa::launch_decode<bf16_t, 128, true>(p, st) : sdpa::launch_decode<bf16_t, 64, true>(p, st);
+    return D == 128 ? sdpa::launch_decode<f16_t, 128, true>(p, st) : sdpa::launch_decode<f16_t, 64, true>(p, st);
+  }
   if (dtype == XG_BF16) return D == 128 ? sdpa::launch_decode<bf16_t, 128>(p, st) : sdpa::launch_decode<bf16_t, 64>(p, st);
   return D == 128 ? sdpa::launch_decode<f16_t, 128>(p, st) : sdpa::launch_decode<f16_t, 64>(p, st);
 }

@@ -905,7 +905,8 @@ def _sdpa_run(q, k, v, is_causal, scale, want_lse):
         # a decode step: the keys are split over workgroups; the partial results go through a small workspace
         n_ws = _lib.lib().xg_sdpa_decode_workspace_floats(B, H, k.shape[1], Sq, k.shape[2], D)
         ws = torch.empty((n_ws,), dtype=torch.float32, device=q.device) if n_ws > 0 else None
-        st = _lib.lib().xg_sdpa_decode(_ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), _ptr(ws), n_ws, *shape, scale, _code(q.dtype), _stream())
+        st = _lib.lib().xg_sdpa_decode(_ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), None, None, _code(q.dtype), None, _ptr(ws), n_ws, *shape,
+                                       scale, _code(q.dtype), _stream())
         _lib.check(st, "xg_sdpa_decode")
         return out, lse
     tail = (scale, 1 if is_causal else 0, _code(q.dtype), _stream())
@@ -1004,6 +1005,15 @@ def _sdpa_masked_run(q, k, v, mask, scale_t, is_causal, scale, want_lse):
     S3 = ctypes.c_int64 * 3
     mask, mask_strides, mask_dt = _mask_operand(mask, q, Skv)
     scale_t = _scale_operand(scale_t)
+    if not is_causal and Sq <= _DECODE_ROWS and Skv >= _DECODE_MIN_KEYS:
+        n_ws = _lib.lib().xg_sdpa_decode_workspace_floats(B, H, k.shape[1], Sq, Skv, D)
+        ws = torch.empty((n_ws,), dtype=torch.float32, device=q.device) if n_ws > 0 else None
+        st = _lib.lib().xg_sdpa_decode(
+            _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), _ptr(mask), mask_strides, mask_dt, _ptr(scale_t), _ptr(ws), n_ws, B, H, k.shape[1],
+            Sq, Skv, D, S3(*q.stride()[:3]), S3(*k.stride()[:3]), S3(*v.stride()[:3]), S3(*out.stride()[:3]), scale, _code(q.dtype), _stream(),
+        )
+        _lib.check(st, "xg_sdpa_decode")
+        return out, lse
     tail = (mask_strides, mask_dt, _ptr(scale_t), B, H, k.shape[1], Sq, Skv, D, S3(*q.stride()[:3]), S3(*k.stride()[:3]), S3(*v.stride()[:3]),
             S3(*out.stride()[:3]), scale, 1 if is_causal else 0, _code(q.dtype), _stream())
     if want_lse:
