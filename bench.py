@@ -638,6 +638,100 @@ class SdpaBackwardC5(Workload):
         return run, "eager autograd on one batch entry (B1 H32 S2048 D128; forward and backward, the forward's flops not counted)"
 
 
+class DenseDecode(Workload):
+    name = "decode dense + bias bf16 M1 K4096 N11008, [N,K] weights"
+    dtype = "bf16"
+    kernel = "gemm_skinny_kernel<bf16,1>"
+    work = 11008 * 4096 * 2 + (4096 + 2 * 11008) * 2  # the weights once, x, bias and the output row
+    n_sets = 3  # 270 MB of weights in rotation: more than the last-level cache holds
+
+    def setup(self, torch, dev):
+        from xpu_graph_amd import _lib
+
+        self.torch = torch
+        g = torch.Generator().manual_seed(0)
+        self.sets = [
+            (torch.randn(1, 4096, generator=g).bfloat16().to(dev), (torch.randn(11008, 4096, generator=g) * 0.02).bfloat16().to(dev),
+             (torch.randn(11008, generator=g) * 0.02).bfloat16().to(dev))
+            for _ in range(self.n_sets)
+        ]
+        self.outs = [torch.empty(1, 11008, device=dev, dtype=torch.bfloat16) for _ in range(self.n_sets)]
+        self.lib = _lib.lib()
+        self.st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def op_call(self, i):
+        x, W, b = self.sets[i]
+        return self.torch.ops.xpu_ops.dense(x, W, True, b, None, "none")
+
+    def abi_call(self, i):
+        x, W, b = self.sets[i]
+        self.lib.xg_dense(_p(x), _p(W), _p(b), None, _p(self.outs[i]), 1, 11008, 4096, 4096, 4096, 0, 1, 0, 2, 2, self.st)
+
+    def check(self, torch):
+        from oracle import eager
+
+        x, W, b = self.sets[0]
+        want = eager.dense_eager(x.float(), W.float(), True, b.float(), "none")
+        torch.testing.assert_close(self.op_call(0).float(), want, rtol=1.6e-2, atol=2e-2)
+
+    def cpu_fn(self, torch):
+        from oracle import eager
+
+        x, W, b = (t.cpu() for t in self.sets[0])
+        fn, how = _default_path_compile(lambda x, W, b: eager.dense_eager(x, W, True, b, "none"))
+        return (lambda: fn(x, W, b)), how
+
+
+class SdpaDecode(Workload):
+    name = "decode attention bf16 B8 H32 Hkv8 Sq1 Skv8192 D128"
+    dtype = "bf16"
+    kernel = "sdpa_decode_kernel<bf16,128> + sdpa_decode_merge_kernel (kernel_us covers both launches)"
+    work = 2 * 8 * 8 * 8192 * 128 * 2 + 2 * 8 * 32 * 128 * 2  # K and V once, q and the output
+    n_sets = 3
+
+    def setup(self, torch, dev):
+        from xpu_graph_amd import _lib
+
+        self.torch = torch
+        g = torch.Generator().manual_seed(0)
+        self.sets = [
+            (torch.randn(8, 32, 1, 128, generator=g).bfloat16().to(dev), torch.randn(8, 8, 8192, 128, generator=g).bfloat16().to(dev),
+             torch.randn(8, 8, 8192, 128, generator=g).bfloat16().to(dev))
+            for _ in range(self.n_sets)
+        ]
+        self.outs = [torch.empty_like(s[0]) for s in self.sets]
+        self.lib = _lib.lib()
+        self.st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        S3 = ctypes.c_int64 * 3
+        self.qs, self.ks = S3(32 * 128, 128, 128), S3(8 * 8192 * 128, 8192 * 128, 128)
+        self.n_ws = self.lib.xg_sdpa_decode_workspace_floats(8, 32, 8, 1, 8192, 128)
+        self.ws = torch.empty(max(self.n_ws, 1), device=dev)
+        self.scale = ctypes.c_float(128**-0.5)
+
+    def op_call(self, i):
+        q, k, v = self.sets[i]
+        return self.torch.ops.xpu_ops.sdpa(q, k, v, False, 128**-0.5)
+
+    def abi_call(self, i):
+        q, k, v = self.sets[i]
+        self.lib.xg_sdpa_decode(_p(q), _p(k), _p(v), _p(self.outs[i]), None, None, None, 2, None, _p(self.ws), self.n_ws, 8, 32, 8, 1, 8192, 128,
+                                self.qs, self.ks, self.ks, self.qs, self.scale, 2, self.st)
+
+    def check(self, torch):
+        from oracle import eager
+
+        q, k, v = (t[:1] for t in self.sets[0])
+        want = eager.sdpa_eager(q.float(), k.float(), v.float())
+        torch.testing.assert_close(self.op_call(0)[:1].float(), want, rtol=1.6e-2, atol=2e-3)
+
+    def cpu_fn(self, torch):
+        from oracle import eager
+
+        q, k, v = (t.cpu() for t in self.sets[0])
+        fn, how = _default_path_compile(eager.sdpa_eager)
+        return (lambda: fn(q, k, v)), how
+
+
 class DenseWeightGradC4(Workload):
     zero_operands = True
     name = "C4 dense weight gradient bf16 x[8192,4096]^T g[8192,11008]"
@@ -868,7 +962,8 @@ def traffic_from(fetch_dir, write_dir, out_path=TRAFFIC_FILE):
 
 
 HEADLINE = AddLayerNormC2
-OTHERS = [RmsNormC1, SliceCatC3a, AddNC3b, DenseC4, DenseFp32, DenseFp8C4, DenseGluC5, SdpaC5, SdpaBackwardC5, DenseWeightGradC4, LlamaBlockC5, LlamaBlockTrainC5]
+OTHERS = [RmsNormC1, SliceCatC3a, AddNC3b, DenseC4, DenseFp32, DenseFp8C4, DenseGluC5, SdpaC5, SdpaBackwardC5, DenseWeightGradC4, DenseDecode, SdpaDecode,
+          LlamaBlockC5, LlamaBlockTrainC5]
 
 
 def run_workload(torch, dev, wl, steps, warmup, with_cpu=True):

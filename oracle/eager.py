@@ -180,6 +180,21 @@ def causal_sdpa_eager(q, k, v, scale=None):
     return torch.matmul(p, v)
 
 
+def sdpa_eager(q, k, v, mask=None, scale=None):
+    """softmax(q k^T * scale + mask) v with fp32 softmax and no causal mask: the same attention form
+    (passes/patterns/common/fuse_scaled_dot_product_attention.py:63-242) as a decode step meets it -- few query rows,
+    an optional additive mask, key/value heads shared by groups of query heads (repeated here)."""
+    D = q.shape[-1]
+    scale = (1.0 / math.sqrt(D)) if scale is None else scale
+    rep = q.shape[1] // k.shape[1]
+    if rep > 1:
+        k, v = k.repeat_interleave(rep, dim=1), v.repeat_interleave(rep, dim=1)
+    s = torch.matmul(q, k.transpose(-1, -2)).float() * scale
+    if mask is not None:
+        s = s + mask.float()
+    return torch.matmul(torch.softmax(s, dim=-1).to(q.dtype), v)
+
+
 def silu_mul_eager(x):
     """SwiGLU gate as tests/npu/test_silu_mul.py:8-16 writes it."""
     d = x.shape[-1] // 2

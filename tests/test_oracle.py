@@ -160,6 +160,29 @@ def test_causal_sdpa_against_library_and_invariants():
     np.testing.assert_allclose(np64(got[0, 0]), out, rtol=1e-5, atol=1e-6)
 
 
+def test_sdpa_against_library_brute_force_and_special_cases():
+    g = torch.Generator().manual_seed(1)
+    q = torch.randn(2, 4, 3, 8, generator=g)
+    k, v = (torch.randn(2, 2, 20, 8, generator=g) for _ in range(2))  # two query heads per key/value head
+    mask = torch.randn(2, 1, 3, 20, generator=g)
+    mask[0, 0, :, 5:9] = float("-inf")
+    got = eager.sdpa_eager(q, k, v, mask, 0.3)
+    kr, vr = k.repeat_interleave(2, dim=1), v.repeat_interleave(2, dim=1)
+    torch.testing.assert_close(got, F.scaled_dot_product_attention(q, kr, vr, attn_mask=mask, scale=0.3), rtol=1e-5, atol=1e-6)
+    # brute force, float64: query head 3 of batch 0 reads key/value head 1
+    Q, K, V, M = np64(q[0, 3]), np64(k[0, 1]), np64(v[0, 1]), np64(mask[0, 0])
+    out = np.zeros_like(Q)
+    for i in range(3):
+        sc = Q[i] @ K.T * 0.3 + M[i]
+        pr = np.exp(sc - sc.max())
+        out[i] = (pr / pr.sum()) @ V
+    np.testing.assert_allclose(np64(got[0, 3]), out, rtol=1e-5, atol=1e-6)
+    # one key: the output is that key's value row; a zero query: the mean of the values; default scale 1 / sqrt(D)
+    torch.testing.assert_close(eager.sdpa_eager(q, k[:, :, :1], v[:, :, :1]), vr[:, :, :1].expand(2, 4, 3, 8))
+    torch.testing.assert_close(eager.sdpa_eager(torch.zeros_like(q), k, v), vr.mean(dim=2, keepdim=True).expand(2, 4, 3, 8), rtol=1e-5, atol=1e-6)
+    torch.testing.assert_close(eager.sdpa_eager(q, k, v), eager.sdpa_eager(q, k, v, None, 1 / math.sqrt(8)))
+
+
 def test_silu_mul_and_rope_closed_forms():
     x = torch.randn(4, 32)
     a, b = np64(x[:, :16]), np64(x[:, 16:])
