@@ -292,53 +292,52 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 2))
   }
 }
 
-// Merge the key ranges of one problem: same thread-to-element map as the end of the kernel above.  The ranges are
-// taken four at a time so that their loads are in flight together (the loop is a chain of memory round trips).
+// Merge the key ranges of one problem.  A thread owns four output columns of one query row (the rows that exist are
+// dealt over the 256 threads) and walks the ranges with a running maximum, sixteen at a time so that their loads are in
+// flight together: the kernel is a chain of memory round trips and nothing else.
 template <typename T, int D>
 __global__ __launch_bounds__(kThreads) void sdpa_decode_merge_kernel(DecodeParams p) {
-  constexpr int PER = D / 8, WS = decode_ws_floats<D>();
-  const int tid = threadIdx.x;
+  constexpr int WS = decode_ws_floats<D>(), G = 16, CPR = D / 4;  // four-column chunks per row
   const int prob = blockIdx.x, n_hg = p.H / p.pack;
   const int b = prob / n_hg, head0 = (prob % n_hg) * p.pack;
-  const int r = tid >> 3, d0 = (tid & 7) * PER;
-  if (r >= p.pack * p.Sq) return;  // rows the workgroups neither wrote nor own
+  const int rows = p.pack * p.Sq;
   const float* src = p.ws + (int64_t)prob * p.n_split * WS;
-  float M = -INFINITY;
-  for (int s0 = 0; s0 < p.n_split; s0 += 4) {
-    float m4[4];
+  for (int item = threadIdx.x; item < rows * CPR; item += kThreads) {
+    const int r = item / CPR, d0 = (item % CPR) * 4;
+    float M = -INFINITY, L = 0.f;
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    for (int s0 = 0; s0 < p.n_split; s0 += G) {
+      float m[G], l[G];
+      f32x4 o4[G];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) m4[u] = s0 + u < p.n_split ? src[(int64_t)(s0 + u) * WS + DROWS * D + r] : -INFINITY;
-    M = fmaxf(fmaxf(M, fmaxf(m4[0], m4[1])), fmaxf(m4[2], m4[3]));
-  }
-  float L = 0.f, acc[PER];
-#pragma unroll
-  for (int e = 0; e < PER; ++e) acc[e] = 0.f;
-  for (int s0 = 0; s0 < p.n_split; s0 += 4) {
-    float f[4], l4[4];
-    f32x4 o4[4][PER / 4];
-#pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      const int s = s0 + u < p.n_split ? s0 + u : p.n_split - 1;  // a repeated range gets weight 0 below
-      const float* part = src + (int64_t)s * WS;
-      f[u] = part[DROWS * D + r];
-      l4[u] = part[DROWS * D + DROWS + r];
-#pragma unroll
-      for (int e = 0; e < PER / 4; ++e) o4[u][e] = *reinterpret_cast<const f32x4*>(part + r * D + d0 + 4 * e);
-    }
-#pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      const float w = (s0 + u < p.n_split && f[u] != -INFINITY) ? __builtin_amdgcn_exp2f(f[u] - M) : 0.f;  // a range without a visible key adds nothing
-      L = __builtin_fmaf(l4[u], w, L);
-#pragma unroll
-      for (int e = 0; e < PER / 4; ++e) {
-        acc[4 * e] = __builtin_fmaf(o4[u][e][0], w, acc[4 * e]);
-        acc[4 * e + 1] = __builtin_fmaf(o4[u][e][1], w, acc[4 * e + 1]);
-        acc[4 * e + 2] = __builtin_fmaf(o4[u][e][2], w, acc[4 * e + 2]);
-        acc[4 * e + 3] = __builtin_fmaf(o4[u][e][3], w, acc[4 * e + 3]);
+      for (int u = 0; u < G; ++u) {
+        const int s = s0 + u < p.n_split ? s0 + u : p.n_split - 1;  // a repeated range gets weight 0 below
+        const float* part = src + (int64_t)s * WS;
+        m[u] = part[DROWS * D + r];
+        l[u] = part[DROWS * D + DROWS + r];
+        o4[u] = *reinterpret_cast<const f32x4*>(part + r * D + d0);
       }
+      float Mg = M;
+#pragma unroll
+      for (int u = 0; u < G; ++u) Mg = fmaxf(Mg, s0 + u < p.n_split ? m[u] : -INFINITY);
+      const float keep = M == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(M - Mg);  // what was summed so far, at the new reference
+      L *= keep;
+      acc *= keep;
+#pragma unroll
+      for (int u = 0; u < G; ++u) {
+        const float w = (s0 + u < p.n_split && m[u] != -INFINITY) ? __builtin_amdgcn_exp2f(m[u] - Mg) : 0.f;  // a range without a visible key adds nothing
+        L = __builtin_fmaf(l[u], w, L);
+        acc += o4[u] * w;
+      }
+      M = Mg;
     }
+    const int head = head0 + r / p.Sq, sq = r % p.Sq;
+    const float inv = 1.f / L;
+    typedef T t4 __attribute__((ext_vector_type(4)));
+    const t4 w4 = {(T)(acc[0] * inv), (T)(acc[1] * inv), (T)(acc[2] * inv), (T)(acc[3] * inv)};
+    *reinterpret_cast<t4*>(reinterpret_cast<T*>(p.o) + (int64_t)b * p.os[0] + (int64_t)head * p.os[1] + (int64_t)sq * p.os[2] + d0) = w4;
+    if (p.lse && d0 == 0) p.lse[((int64_t)b * p.H + head) * p.Sq + sq] = (M + log2f(L)) * 0.69314718055994530942f;
   }
-  store_row_part<T, D>(p, b, head0, r, d0, acc, M, L);
 }
 
 // How the keys of one problem are split: enough workgroups to fill the chip about three times over, whole tiles per range.
