@@ -210,8 +210,8 @@ def test_decode_attention_validation_and_workspace_size_need_no_gpu():
     assert call(1, 32, 32, 2, 4096, 128, mask=p, mask_strides=S3(0, 0, 100)) == -2     # mask rows overlap
     assert call(1, 32, 32, 1, 4096, 128, scale_dev=ctypes.c_void_p(258)) == -3
     assert call(0, 32, 32, 1, 4096, 128) == 0     # nothing to do
-    # 32 problems of 32 tiles: 16 key ranges of two tiles each, 32 x 128 + 64 floats per range
-    assert lib.xg_sdpa_decode_workspace_floats(1, 32, 32, 1, 4096, 128) == 32 * 16 * (32 * 128 + 64)
+    # 32 problems of 32 tiles on 256 compute units: 8 key ranges of four tiles each, 32 x 128 + 64 floats per range
+    assert lib.xg_sdpa_decode_workspace_floats(1, 32, 32, 1, 4096, 128) == 32 * 8 * (32 * 128 + 64)
     assert lib.xg_sdpa_decode_workspace_floats(64, 32, 32, 1, 4096, 128) == 0                     # 2048 problems fill the chip as they are
     assert lib.xg_sdpa_decode_workspace_floats(1, 32, 32, 33, 4096, 128) == 0
 

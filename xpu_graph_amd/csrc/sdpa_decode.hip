@@ -340,10 +340,22 @@ __global__ __launch_bounds__(kThreads) void sdpa_decode_merge_kernel(DecodeParam
   }
 }
 
-// How the keys of one problem are split: enough workgroups to fill the chip about three times over, whole tiles per range.
+// How the keys of one problem are split: one workgroup per compute unit, whole tiles per range.  A workgroup pays
+// ~5 us before its first tile and after its last that nothing hides (it has the CU's LDS to itself), so more, shorter
+// workgroups lose: B8 H32 Hkv8 Skv8192 53.8 us at 256 workgroups, 57.2 at 512, 60.4 at 768, 68.4 at 128.  Without a GPU
+// (argument checks on a host) the published 256 compute units stand in.
+inline int decode_cu_count() {
+  static const int n = [] {
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+      cus = 256;
+    return cus;
+  }();
+  return n;
+}
 inline void decode_split(int64_t problems, int64_t Skv, int& n_split, int& tiles_per_split) {
   const int64_t n_tiles = (Skv + DKV - 1) / DKV;
-  int64_t want = (768 + problems - 1) / problems;
+  int64_t want = (decode_cu_count() + problems - 1) / problems;
   want = want < 1 ? 1 : (want > n_tiles ? n_tiles : want);
   const int64_t tps = (n_tiles + want - 1) / want;
   tiles_per_split = (int)tps;
