@@ -456,6 +456,35 @@ def test_sdpa_with_an_additive_mask_runs_the_kernel(device, mask_kind):
     assert_close_16bit(out.to(torch.bfloat16) if out.dtype != torch.bfloat16 else out, want, attention_floor(want, torch.bfloat16), f"sdpa masked compiled {mask_kind}")
 
 
+@pytest.mark.parametrize("mask_kind", ["additive", "boolean"])
+@pytest.mark.parametrize("Sq,Skv", [(192, 192), (1, 1536), (8, 1024)])
+def test_library_attention_with_a_mask_runs_the_kernel(device, mask_kind, Sq, Skv):
+    """F.scaled_dot_product_attention(attn_mask=...) itself -- a float mask, or a boolean one that torch turns into
+    0 / -inf -- at a prefill shape and at decode shapes (the key-split kernel): the graph calls the masked attention
+    module and the result follows fp32 attention."""
+    import torch.nn.functional as F
+
+    from tests.test_gpu_sdpa import ref32_masked
+    from tests.tolerance import assert_close_16bit, attention_floor
+
+    g = torch.Generator().manual_seed(Sq + Skv)
+    B, H, D = 2, 8, 128
+    q = torch.randn(B, H, Sq, D, generator=g).bfloat16().to(device)
+    k, v = (torch.randn(B, H, Skv, D, generator=g).bfloat16().to(device) for _ in range(2))
+    if mask_kind == "additive":
+        m = torch.randn(B, 1, Sq, Skv, generator=g).bfloat16().to(device)
+        add = m
+    else:
+        m = torch.rand(B, 1, Sq, Skv, generator=g) < 0.8
+        m[..., 0] = True  # every row sees key 0
+        m = m.to(device)
+        add = torch.zeros(B, 1, Sq, Skv, device=device).masked_fill(~m, float("-inf"))
+    out, mods, rest = run(lambda q, k, v, m: F.scaled_dot_product_attention(q, k, v, attn_mask=m), q, k, v, m)
+    assert "mi355x_sdpa_masked" in mods, (mods, rest)
+    want = ref32_masked(q, k, v, add, False, 1.0 / D**0.5)
+    assert_close_16bit(out, want, attention_floor(want, torch.bfloat16), f"sdpa library mask {mask_kind} {Sq}x{Skv}")
+
+
 @pytest.mark.parametrize("form", ["permuted_fp32_softmax", "permuted_prescaled_query", "permuted_divide", "decoder_output_transposed"])
 def test_permuted_input_sdpa_forms_reach_the_kernel(device, form):
     """The reference's attention forms whose operands arrive as [B, S, H, E] and are permuted inside the function

@@ -129,3 +129,41 @@ def test_backend_with_device_graph_vendor_config(device):
     assert region.recorded == 1
     mods = [n.target for n in region.region.graph.nodes if n.op == "call_module"]
     assert len(mods) >= 3, mods  # add+norm, dense+silu, dense
+
+
+def test_a_decode_step_replays_from_a_hip_graph(device):
+    """One token against a cache of keys and values: the projections run on the row-streaming dense kernel, the
+    attention on the key-split kernel (two launches and a workspace from the allocator, all inside the capture);
+    every replay with new values matches eager."""
+
+    def step(x, wq, wo, k_cache, v_cache, pad):
+        B = x.shape[0]
+        q = F.linear(x, wq).view(B, 1, 8, 128).transpose(1, 2)
+        a = F.scaled_dot_product_attention(q, k_cache, v_cache, attn_mask=pad)
+        return F.linear(a.transpose(1, 2).reshape(B, 1024), wo)
+
+    g = torch.Generator().manual_seed(3)
+    bf = torch.bfloat16
+    B, S = 4, 1536
+    mk = lambda *s, k=1.0: (torch.randn(*s, generator=g) * k).to(bf).to(device)  # noqa: E731
+    x, wq, wo = mk(B, 1024), mk(1024, 1024, k=0.03), mk(1024, 1024, k=0.03)
+    kc, vc = mk(B, 8, S, 128), mk(B, 8, S, 128)
+    pad = torch.zeros(B, 1, 1, S, device=device, dtype=bf)
+    pad[1, :, :, 1000:] = float("-inf")
+    backend = mi355x_compiler()
+    compiled = torch.compile(step, backend=backend, dynamic=False)
+    with torch.no_grad():
+        compiled(x, wq, wo, kc, vc, pad)
+    mods = [n.target for n in backend.compiled_graphs[-1].graph.nodes if n.op == "call_module"]
+    assert "mi355x_sdpa_masked" in mods, mods
+    runner = HIPGraphRunner(compiled)
+    runner.capture(x, wq, wo, kc, vc, pad, clone_args=True)
+    for it in range(3):
+        xs, ks, vs = mk(B, 1024), mk(B, 8, S, 128), mk(B, 8, S, 128)
+        (torch.randn(512, 512, device=device) @ torch.randn(512, 512, device=device)).sum().item()
+        y = runner(xs, wq, wo, ks, vs, pad).clone()
+        with torch.no_grad():
+            kr, vr = ks, vs
+            q = F.linear(xs, wq).view(B, 1, 8, 128).transpose(1, 2)
+            want = F.linear(F.scaled_dot_product_attention(q, kr, vr, attn_mask=pad).transpose(1, 2).reshape(B, 1024), wo)
+        torch.testing.assert_close(y.float(), want.float(), rtol=1.6e-2, atol=2e-2)

@@ -624,3 +624,32 @@ def test_masked_and_tensor_scale_attention_become_the_masked_kernel_call(caplog,
     torch._dynamo.reset()
     gm = rewrite(backend, att_tscale, q, k, v, torch.tensor([math.sqrt(D)]))
     assert "mi355x_sdpa_masked" in modules_called(gm) and "fused_sdpa" not in modules_called(gm), (modules_called(gm), aten_ops(gm))
+
+
+def test_library_attention_with_a_mask_or_grouped_heads_reaches_the_kernels(caplog, backend):
+    """F.scaled_dot_product_attention with attn_mask arrives as a backend-specific op that carries the mask as its
+    bias (a boolean mask already turned into 0 / -inf): it becomes the masked kernel call.  The pre-dispatch composite op with
+    enable_gqa=True (fewer key/value heads, query head h reading key/value head h // (H / Hkv)) is what the kernels
+    compute, so the pregrad stage takes it as it is."""
+    import torch.nn.functional as F
+
+    from xpu_graph_amd import OptLevel, Target, XpuGraph, XpuGraphConfig
+
+    B, H, S, D = 2, 4, 64, 128
+    q, k, v = (torch.randn(B, H, S, D).to(bf16) for _ in range(3))
+    gm = rewrite(backend, lambda q, k, v, m: F.scaled_dot_product_attention(q, k, v, attn_mask=m) * 2.0, q, k, v, torch.randn(B, 1, S, S).to(bf16))
+    assert modules_called(gm) == ["mi355x_sdpa_masked"], (modules_called(gm), aten_ops(gm))
+    torch._dynamo.reset()
+    # a boolean mask reaches the backend op as where(mask, 0, -inf): an additive mask like any other
+    gm = rewrite(backend, lambda q, k, v, m: F.scaled_dot_product_attention(q, k, v, attn_mask=m) * 2.0, q, k, v, torch.rand(B, 1, S, S) > 0.5)
+    assert modules_called(gm) == ["mi355x_sdpa_masked"] and any("where" in t for t in aten_ops(gm)), (modules_called(gm), aten_ops(gm))
+    torch._dynamo.reset()
+    train = XpuGraph(XpuGraphConfig(is_training=True, target=Target.mi355x, opt_level=OptLevel.level2, enable_cache=False))
+    args = [t.clone().requires_grad_(True) for t in (q, k[:, :2], v[:, :2])]
+    with need_xpu_graph_logs(), pytest.raises(NotImplementedError):
+        torch.compile(lambda q, k, v: F.scaled_dot_product_attention(q, k, v, is_causal=True, enable_gqa=True) * 2.0, backend=train)(*args)
+    pregrad = train.compiled_graphs[-2]
+    calls = [n for n in pregrad.graph.nodes if n.op == "call_module"]
+    assert [n.target for n in calls] == ["mi355x_sdpa"] and calls[0].args[3] is True
+    assert tuple(calls[0].args[1].meta["val"].shape) == (B, 2, S, D)  # the key/value heads go to the kernel unrepeated
+    torch._dynamo.reset()

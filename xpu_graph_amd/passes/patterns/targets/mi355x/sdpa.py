@@ -272,8 +272,15 @@ class FusedCausalSDPA(Pattern):
                 dropout = node.args[4] if len(node.args) > 4 else node.kwargs.get("dropout_p", 0.0)
                 causal = node.args[5] if len(node.args) > 5 else node.kwargs.get("is_causal", False)
                 scale = node.kwargs.get("scale")
-                if node.kwargs.get("enable_gqa", False) or dropout != 0.0:
+                if dropout != 0.0:
                     continue
+                # enable_gqa=True (query head h reads key/value head h // (H / Hkv)) is what the kernels do with fewer
+                # key/value heads; _supported checks that the head counts divide
+                gqa = bool(node.kwargs.get("enable_gqa", False))
+                if not gqa and isinstance(q, fx.Node) and isinstance(k, fx.Node):
+                    vq, vk = q.meta.get("val"), k.meta.get("val")
+                    if isinstance(vq, torch.Tensor) and isinstance(vk, torch.Tensor) and vq.dim() == 4 and vk.dim() == 4 and vq.shape[1] != vk.shape[1]:
+                        continue  # eager broadcasts (or refuses) differing head counts without the flag: not this kernel's rule
                 if not all(isinstance(n, fx.Node) and isinstance(n.meta.get("val"), torch.Tensor) and n.meta["val"].dim() == 4 for n in (q, k, v)):
                     continue
                 sq, skv = q.meta["val"].shape[2], k.meta["val"].shape[2]
@@ -327,14 +334,24 @@ class FusedCausalSDPA(Pattern):
                 dropout = args[drop_idx] if len(args) > drop_idx else node.kwargs.get("dropout_p", 0.0)
                 causal = args[causal_idx] if len(args) > causal_idx else node.kwargs.get("is_causal", False)
                 bias = (args[bias_idx] if len(args) > bias_idx else None) if bias_idx is not None else node.kwargs.get("attn_mask")
-                if dropout != 0.0 or bias is not None or not _supported(q, k, v):
+                if dropout != 0.0 or not _supported(q, k, v):
                     continue
+                mask_operand = None
+                if bias is not None:
+                    # the additive bias of the memory-efficient backend op is the attn_mask of the call it came from
+                    sq, skv = q.meta["val"].shape[2], k.meta["val"].shape[2]
+                    if not causal and is_causal_constant(bias, sq, skv):
+                        causal = True
+                    elif self._current_stage == FxStage.inference and isinstance(bias, fx.Node) and _mask_operand_ok(bias, q, k):
+                        mask_operand = bias
+                    else:
+                        continue
 
                 def replace(new, users=users):
                     for u in users:
                         u.replace_all_uses_with(new)
 
-                changed |= self._emit(gm, node, q, k, v, causal, node.kwargs.get("scale"), replace)
+                changed |= self._emit(gm, node, q, k, v, causal, node.kwargs.get("scale"), replace, mask=mask_operand)
         for node in self._wrapped_scale_calls(gm):
             q, k, v, mask, scale_t = node.args
             if not all(isinstance(n, fx.Node) and isinstance(n.meta.get("val"), torch.Tensor) for n in (q, k, v, scale_t)):
