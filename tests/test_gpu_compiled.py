@@ -485,6 +485,31 @@ def test_library_attention_with_a_mask_runs_the_kernel(device, mask_kind, Sq, Sk
     assert_close_16bit(out, want, attention_floor(want, torch.bfloat16), f"sdpa library mask {mask_kind} {Sq}x{Skv}")
 
 
+@pytest.mark.parametrize("Sq,Skv,causal", [(256, 256, True), (1, 2048, False)])
+def test_grouped_query_attention_of_a_decoder_runs_unrepeated(device, Sq, Skv, causal):
+    """`repeat_kv` in front of the attention (the HF decoders' grouped-query form), prefill and decode: the kernel gets the
+    [B, Hkv, S, D] keys and values, no repeated copy is made, and the result follows fp32 attention over the repeated heads."""
+    import torch.nn.functional as F
+
+    from tests.test_gpu_sdpa import ref32
+    from tests.tolerance import assert_close_16bit, attention_floor
+
+    def repeat_kv(h, n):
+        b, hk, s, d = h.shape
+        return h[:, :, None, :, :].expand(b, hk, n, s, d).reshape(b, hk * n, s, d)
+
+    def att(q, k, v):
+        return F.scaled_dot_product_attention(q, repeat_kv(k, 4), repeat_kv(v, 4), is_causal=causal)
+
+    g = torch.Generator().manual_seed(Sq + Skv)
+    q = torch.randn(2, 8, Sq, 128, generator=g).bfloat16().to(device)
+    k, v = (torch.randn(2, 2, Skv, 128, generator=g).bfloat16().to(device) for _ in range(2))
+    out, mods, rest = run(att, q, k, v)
+    assert mods == ["mi355x_sdpa"] and not any("expand" in t or "clone" in t for t in rest), (mods, rest)
+    want = ref32(q, k, v, causal, 128**-0.5)
+    assert_close_16bit(out, want, attention_floor(want, torch.bfloat16), f"sdpa grouped compiled {Sq}x{Skv}")
+
+
 @pytest.mark.parametrize("form", ["permuted_fp32_softmax", "permuted_prescaled_query", "permuted_divide", "decoder_output_transposed"])
 def test_permuted_input_sdpa_forms_reach_the_kernel(device, form):
     """The reference's attention forms whose operands arrive as [B, S, H, E] and are permuted inside the function

@@ -502,6 +502,37 @@ def test_attention_with_a_padding_mask_trains_on_the_kernels(device):
     assert (gb.float() - want).abs().mean().item() <= 0.1 * want.abs().mean().item() + 1e-6
 
 
+def test_grouped_query_attention_trains_unrepeated(device):
+    """`repeat_kv` + causal attention compiled for training: the pregrad stage hands the kernels the unrepeated keys and
+    values, the backward kernels sum the gradients of a group's query heads, and dq, dk, dv follow fp32 autograd of the
+    written-out form."""
+
+    def repeat_kv(h, n):
+        b, hk, s, d = h.shape
+        return h[:, :, None, :, :].expand(b, hk, n, s, d).reshape(b, hk * n, s, d)
+
+    def att(q, k, v):
+        return F.scaled_dot_product_attention(q, repeat_kv(k, 4), repeat_kv(v, 4), is_causal=True)
+
+    torch.manual_seed(5)
+    bf = torch.bfloat16
+    q = torch.randn(2, 8, 192, 64, device=device).to(bf).requires_grad_(True)
+    k, v = (torch.randn(2, 2, 192, 64, device=device).to(bf).requires_grad_(True) for _ in range(2))
+    be = backend()
+    y = torch.compile(att, backend=be, dynamic=False)(q, k, v)
+    g0 = torch.autograd.grad(y.float().pow(2).mean(), (q, k, v))
+    fwd_ops = [str(n.target) for n in be.compiled_graphs[1].graph.nodes if n.op == "call_function"]
+    assert fwd_ops.count("xpu_ops.sdpa_lse.default") == 1 and not any("expand" in o or "clone" in o for o in fwd_ops), fwd_ops
+    ref = [t.detach().float().requires_grad_(True) for t in (q, k, v)]
+    g1 = torch.autograd.grad(att(*ref).pow(2).mean(), ref)
+    eag = [t.detach().clone().requires_grad_(True) for t in (q, k, v)]
+    g2 = torch.autograd.grad(att(*eag).float().pow(2).mean(), eag)
+    err = lambda a, c: (a.float() - c).abs().mean().item()  # noqa: E731
+    for a, c, e in zip(g0, g1, g2):
+        assert a.shape == c.shape
+        assert err(a, c) <= 2 * err(e, c) + 1e-2 * c.abs().mean().item(), (err(a, c), err(e, c), c.abs().mean().item())
+
+
 def test_llama_block_training_step(device):
     """The whole decoder block of benchmark config 5 (small batch and sequence), compiled for training on the mi355x
     target: the forward graph runs on the HIP kernels, and the gradients of every weight follow fp32 autograd as

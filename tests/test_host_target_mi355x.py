@@ -653,3 +653,31 @@ def test_library_attention_with_a_mask_or_grouped_heads_reaches_the_kernels(capl
     assert [n.target for n in calls] == ["mi355x_sdpa"] and calls[0].args[3] is True
     assert tuple(calls[0].args[1].meta["val"].shape) == (B, 2, S, D)  # the key/value heads go to the kernel unrepeated
     torch._dynamo.reset()
+
+
+def test_repeated_key_value_heads_go_to_the_kernel_unrepeated(caplog, backend):
+    """Grouped-query attention as decoders write it -- `repeat_kv` (index with None, expand, reshape) or
+    repeat_interleave(n, dim=1) in front of the attention: the copies that repeat the heads disappear and the kernel
+    call gets the [B, Hkv, S, D] tensors (query head h reads key/value head h // n).  Heads repeated in another order
+    (`repeat`) stay as they are."""
+    import torch.nn.functional as F
+
+    B, H, Hkv, S, D = 2, 8, 2, 64, 128
+
+    def repeat_kv(h, n):
+        b, hk, s, d = h.shape
+        return h[:, :, None, :, :].expand(b, hk, n, s, d).reshape(b, hk * n, s, d)
+
+    q = torch.randn(B, H, S, D).to(bf16)
+    k, v = (torch.randn(B, Hkv, S, D).to(bf16) for _ in range(2))
+    for fn in (lambda q, k, v: F.scaled_dot_product_attention(q, repeat_kv(k, 4), repeat_kv(v, 4), is_causal=True) * 2.0,
+               lambda q, k, v: F.scaled_dot_product_attention(q, k.repeat_interleave(4, dim=1), v.repeat_interleave(4, dim=1)) * 2.0):
+        gm = rewrite(backend, fn, q, k, v)
+        call = next(n for n in gm.graph.nodes if n.target == "mi355x_sdpa")
+        assert tuple(call.args[1].meta["val"].shape) == (B, Hkv, S, D) and tuple(call.args[2].meta["val"].shape) == (B, Hkv, S, D)
+        assert not any("expand" in t or "clone" in t for t in aten_ops(gm)), aten_ops(gm)
+        torch._dynamo.reset()
+    gm = rewrite(backend, lambda q, k, v: F.scaled_dot_product_attention(q, k.repeat(1, 4, 1, 1), v.repeat(1, 4, 1, 1)) * 2.0, q, k, v)
+    call = next(n for n in gm.graph.nodes if n.target == "mi355x_sdpa")
+    assert tuple(call.args[1].meta["val"].shape) == (B, H, S, D)  # head h reads key/value head h % Hkv there: not the kernels' rule
+    torch._dynamo.reset()

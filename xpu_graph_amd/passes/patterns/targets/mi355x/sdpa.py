@@ -201,6 +201,30 @@ def _peel_k(node, dims):
     return src if _same_attention_problem(src, dims) else node
 
 
+def _peel_repeat(node):
+    """reshape(clone(expand(unsqueeze(x, 2), [B, Hkv, n, S, D])), [B, Hkv * n, S, D]) -> x: key/value heads repeated for
+    grouped-query attention (`repeat_kv` of the HF decoders, `repeat_interleave(n, dim=1)`).  Query head h of the
+    repeated tensor is key/value head h // n of x, which is how the kernels index fewer key/value heads."""
+    if not is_call(node, *VIEW_OPS):
+        return node
+    inner = _through_clone(node.args[0])
+    if not is_call(inner, aten.expand.default):
+        return node
+    src = inner.args[0]
+    if not is_call(src, aten.unsqueeze.default) or src.args[1] != 2:
+        return node
+    x = src.args[0]
+    vals = [n.meta.get("val") if isinstance(n, fx.Node) else None for n in (x, inner, node)]
+    if not all(isinstance(t, torch.Tensor) for t in vals):
+        return node
+    xs, es, ns = (list(t.shape) for t in vals)
+    if len(xs) != 4 or len(es) != 5 or len(ns) != 4 or not _static(*xs[1:], *es[1:], *ns[1:]):
+        return node
+    ok = es[1] == xs[1] and es[3:] == xs[2:] and ns[1] == xs[1] * es[2] and ns[2:] == xs[2:]
+    ok = ok and same_shape([es[0]], [xs[0]]) and same_shape([ns[0]], [xs[0]])
+    return x if ok else node
+
+
 def _supported(q, k, v):
     """bf16 / f16 4-D operands, head dim 64 or 128, static head counts and sequence lengths (the batch may be
     symbolic), kv heads dividing the query heads."""
@@ -227,6 +251,9 @@ class FusedCausalSDPA(Pattern):
     _support_stages = [FxStage.inference, FxStage.pregrad]  # sdpa carries a backward formula
 
     def _emit(self, gm, node, q, k, v, causal, scale, replace, mask=None, scale_t=None):
+        k0, v0 = _peel_repeat(k), _peel_repeat(v)
+        if k0 is not k and v0 is not v and _supported(q, k0, v0):
+            k, v = k0, v0  # grouped heads go to the kernel unrepeated (the copies that repeated them die with their last user)
         if scale is None:
             scale = 1.0 / math.sqrt(q.meta["val"].shape[-1])
         if not isinstance(scale, (int, float)):
