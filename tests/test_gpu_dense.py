@@ -446,6 +446,12 @@ def test_batch_dense_compiled(device, form):
         (1000, 200, 128),    # ragged rows and a last tile with 72 of 128 columns
         (130, 8, 4096),      # a sliver of columns, deep K
         (4096, 11008, 512),  # the Llama gate / up width
+        (1, 11008, 4096),    # a decode step: both weights streamed row by row
+        (4, 4096, 1024),
+        (32, 4096, 512),     # two 16-row tiles of activations
+        (13, 1032, 640),     # ragged rows and columns
+        (16, 11008, 4096),   # where the plain layer takes the 64 x 64 kernel, so does the gated one
+        (64, 11008, 512),
     ],
 )
 def test_dense_glu_bit_identical_to_the_unfused_ops(device, dtype, M, N, K):
@@ -457,9 +463,13 @@ def test_dense_glu_bit_identical_to_the_unfused_ops(device, dtype, M, N, K):
     wu = (torch.randn(N, K, generator=g) / K**0.5).to(dtype).to(device)
     ops = torch.ops.xpu_ops
     got = ops.dense_glu(x, wg, wu)
-    two = ops.silu_mul2(ops.dense(x, wg, True, None, None, "none"), ops.dense(x, wu, True, None, None, "none"))
+    gate, up = ops.dense(x, wg, True, None, None, "none"), ops.dense(x, wu, True, None, None, "none")
+    two = ops.silu_mul2(gate, up)
     assert torch.equal(got, two)
     close_glu(got, x, wg, wu)
+    if M <= 64:  # the variant that also hands back the two projections, at the decode sizes
+        y, g_out, u_out = ops.dense_glu_save(x, wg, wu)
+        assert torch.equal(y, got) and torch.equal(g_out, gate) and torch.equal(u_out, up)
 
 
 @pytest.mark.parametrize("M,N,K", [(1024, 4096, 256), (900, 2056, 128)])
