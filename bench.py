@@ -829,6 +829,72 @@ class LlamaBlockC5(Workload):
         return run, how
 
 
+class LlamaBlockDecode(Workload):
+    name = "Llama block decode step bf16 B8, one token against 4096 cached positions, compiled + HIP graph"
+    dtype = "bf16"
+    kernel = "compiled decode step (norms, rotary, 7 row-streaming dense launches incl. the gated one, key-split attention)"
+    traffic_key = None
+    # what one step must read: the seven weight matrices and the two caches (activations are a few KB)
+    work = 2 * (4 * 4096 * 4096 + 3 * 4096 * 11008) + 2 * 8 * 32 * 4096 * 128 * 2
+    n_sets = 1
+    cpu_warmups = 1
+    B, S = 8, 4096
+
+    def _inputs(self, torch, dev):
+        from oracle import eager, inputs
+
+        _, p = inputs.c5_llama_block(B=1, S=1, device=dev)
+        g = torch.Generator().manual_seed(1)
+        x = torch.randn(self.B, 1, 4096, generator=g).bfloat16().to(dev)
+        kc, vc = (torch.randn(self.B, 32, self.S, 128, generator=g).bfloat16().to(dev) for _ in range(2))
+        cos, sin = eager.rope_tables(self.S, 128, device=dev, dtype=torch.bfloat16)
+        return x, p, kc, vc, cos[-1].contiguous(), sin[-1].contiguous()
+
+    def setup(self, torch, dev):
+        from oracle import eager
+        from xpu_graph_amd import HIPGraphRunner, mi355x_compiler
+
+        self.torch = torch
+        x, p, kc, vc, cos, sin = self._inputs(torch, dev)
+        names = sorted(p)
+
+        def step(x, kc, vc, cos, sin, *ws):
+            return eager.llama_block_decode_eager(x, dict(zip(names, ws)), kc, vc, cos, sin, n_heads=32)
+
+        self.eager_fn = step
+        self.args = (x, kc, vc, cos, sin, *[p[n] for n in names])
+        compiled = torch.compile(step, backend=mi355x_compiler(), dynamic=False)
+        with torch.no_grad():
+            compiled(*self.args)  # compile outside the capture
+        self.runner = HIPGraphRunner(compiled)
+        self.runner.capture(*self.args, clone_args=False)
+
+    def op_call(self, i):
+        return self.runner(*self.args)
+
+    abi_call = op_call
+
+    def check(self, torch):
+        got = [t.clone() for t in self.op_call(0)]
+        with torch.no_grad():
+            want = self.eager_fn(*self.args)
+            self.eager_ms = _events_time(torch, lambda i: self.eager_fn(*self.args), 1, 20, 5) * 1e3
+        for a, b in zip(got, want):
+            assert (a.float() - b.float()).abs().mean().item() < 2e-2
+
+    def cpu_fn(self, torch):
+        from oracle import eager
+
+        x, p, kc, vc, cos, sin = self._inputs(torch, "cpu")
+        fn, how = _default_path_compile(lambda x, kc, vc: eager.llama_block_decode_eager(x, p, kc, vc, cos, sin, n_heads=32))
+
+        def run():
+            with torch.no_grad():
+                return fn(x, kc, vc)
+
+        return run, how
+
+
 class LlamaBlockTrainC5(LlamaBlockC5):
     name = "C5 Llama decoder block bf16 B4 S2048 compiled training step"
     kernel = "compiled training step"
@@ -963,7 +1029,7 @@ def traffic_from(fetch_dir, write_dir, out_path=TRAFFIC_FILE):
 
 HEADLINE = AddLayerNormC2
 OTHERS = [RmsNormC1, SliceCatC3a, AddNC3b, DenseC4, DenseFp32, DenseFp8C4, DenseGluC5, SdpaC5, SdpaBackwardC5, DenseWeightGradC4, DenseDecode, SdpaDecode,
-          LlamaBlockC5, LlamaBlockTrainC5]
+          LlamaBlockDecode, LlamaBlockC5, LlamaBlockTrainC5]
 
 
 def run_workload(torch, dev, wl, steps, warmup, with_cpu=True):

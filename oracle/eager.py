@@ -242,3 +242,31 @@ def llama_block_eager(x, p, n_heads=32, eps=1e-6, rope_base=10000.0):
     h = rms(x, p["ln2"])
     mlp = F.linear(F.silu(F.linear(h, p["wg"])) * F.linear(h, p["wu"]), p["wd"])
     return x + mlp
+
+
+def llama_block_decode_eager(x, p, k_cache, v_cache, cos_row, sin_row, n_heads=32, eps=1e-6):
+    """llama_block_eager for ONE new token per sequence against cached keys and values (incremental decoding of the same
+    block).  x [B, 1, hidden]; k_cache / v_cache [B, H, S, D] hold the rotated keys and the values of every position the
+    token attends to, its own included (the caller stores the k_new, v_new of an earlier call there: they do not depend on
+    the caches); cos_row / sin_row [D] are the rotary table's row of the token's position.  No mask: every cached position
+    is visible.  Returns (out [B, 1, hidden], k_new [B, H, 1, D], v_new [B, H, 1, D])."""
+    B, _, Hd = x.shape
+    D = Hd // n_heads
+
+    def rms(t, w):
+        tf = t.float()
+        return (w * (tf * torch.rsqrt(tf.pow(2).mean(-1, keepdim=True) + eps)).to(t.dtype))
+
+    h = rms(x, p["ln1"])
+    q = F.linear(h, p["wq"]).view(B, 1, n_heads, D).transpose(1, 2)
+    k_new = F.linear(h, p["wk"]).view(B, 1, n_heads, D).transpose(1, 2)
+    v_new = F.linear(h, p["wv"]).view(B, 1, n_heads, D).transpose(1, 2)
+    q = q * cos_row + _rotate_half(q) * sin_row
+    k_new = k_new * cos_row + _rotate_half(k_new) * sin_row
+    att = torch.matmul(q, k_cache.transpose(2, 3)) / math.sqrt(D)
+    att = torch.softmax(att, dim=-1, dtype=torch.float32).to(q.dtype)
+    o = torch.matmul(att, v_cache).transpose(1, 2).reshape(B, 1, Hd)
+    x = x + F.linear(o, p["wo"])
+    h = rms(x, p["ln2"])
+    mlp = F.linear(F.silu(F.linear(h, p["wg"])) * F.linear(h, p["wu"]), p["wd"])
+    return x + mlp, k_new, v_new

@@ -38,6 +38,23 @@ def test_rope_shapes_and_layouts(device, dtype, B, H, S, D, layout):
     torch.testing.assert_close(got.float(), ref32(x, cos.float(), sin.float()), rtol=1.6e-2, atol=1e-2)
 
 
+@pytest.mark.parametrize("S", [1, 5])
+@pytest.mark.parametrize("table_shape", ["row", "one_by_d", "leading_ones"])
+def test_rope_with_one_table_row_for_every_position(device, S, table_shape):
+    """A decode step rotates its one new position with that position's row of the tables: cos / sin [D] (or [1, D],
+    [1, 1, 1, D]) are shared by every position of x, as broadcasting in the eager form says."""
+    g = torch.Generator().manual_seed(S)
+    x = torch.randn(3, 4, S, 128, generator=g).bfloat16().to(device)
+    cos, sin = (t[37] for t in eager.rope_tables(64, 128, device=device, dtype=torch.bfloat16))
+    if table_shape == "one_by_d":
+        cos, sin = cos[None], sin[None]
+    elif table_shape == "leading_ones":
+        cos, sin = cos[None, None, None], sin[None, None, None]
+    got = _ops().rope(x, cos, sin)
+    assert got.shape == x.shape and got.dtype == x.dtype
+    torch.testing.assert_close(got.float(), ref32(x, cos, sin), rtol=1.6e-2, atol=1e-2)
+
+
 def test_rope_invariants(device):
     """cos = 1, sin = 0 is the identity; cos = 0, sin = 1 is rotate-half exactly; position 0 of the real tables
     leaves x unchanged; the rotation preserves the norm of every (c, c + D/2) pair."""

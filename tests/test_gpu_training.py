@@ -362,8 +362,9 @@ def test_gated_mlp_training_step(device):
         assert err(a, c) <= 2 * err(e, c) + 1e-2 * c.abs().mean().item(), (err(a, c), err(e, c), c.abs().mean().item())
 
 
+@pytest.mark.parametrize("one_row", [False, True])
 @pytest.mark.parametrize("table_grads", [False, True])
-def test_rotary_backward_formula(device, table_grads):
+def test_rotary_backward_formula(device, table_grads, one_row):
     """The input gradient of xpu_ops.rope is the rotary kernel on a rewritten sine table (halves swapped, negated);
     the table gradients are Aten sums.  Against autograd of the written-out formula in fp32; the sine table has
     different halves so that the swap matters."""
@@ -374,8 +375,9 @@ def test_rotary_backward_formula(device, table_grads):
     B, H, S, D = 2, 4, 96, 64
     bf = torch.bfloat16
     x = torch.randn(B, S, H, D, device=device).to(bf).transpose(1, 2).requires_grad_(True)  # [B, H, S, D] view
-    cos = torch.randn(S, D, device=device).to(bf).requires_grad_(table_grads)
-    sin = torch.randn(S, D, device=device).to(bf).requires_grad_(table_grads)
+    tshape = (D,) if one_row else (S, D)  # one row: shared by every position, so its gradient sums over them too
+    cos = torch.randn(*tshape, device=device).to(bf).requires_grad_(table_grads)
+    sin = torch.randn(*tshape, device=device).to(bf).requires_grad_(table_grads)
     dy = torch.randn(B, H, S, D, device=device).to(bf)
     wrt = (x, cos, sin) if table_grads else (x,)
     g = torch.autograd.grad((torch.ops.xpu_ops.rope(x, cos, sin),), wrt, (dy,))

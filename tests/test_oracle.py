@@ -214,3 +214,25 @@ def test_llama_block_against_module_composition():
     h2 = F.rms_norm(x1, (64,), p["ln2"], 1e-6)
     want = x1 + F.linear(F.silu(F.linear(h2, p["wg"])) * F.linear(h2, p["wu"]), p["wd"])
     torch.testing.assert_close(got, want, rtol=1e-4, atol=1e-5)
+
+
+def test_llama_block_decode_step_equals_the_last_position_of_the_whole_block():
+    """Incremental decoding of the block: keys and values of earlier calls stored in the caches, then the step for the
+    last token gives what the whole block gives at that position (the causal mask hides nothing from the last row)."""
+    S, H, hidden = 9, 4, 64
+    x, p = inputs.c5_llama_block(B=2, S=S, hidden=hidden, inter=96, dtype=torch.float32)
+    D = hidden // H
+    want = eager.llama_block_eager(x, p, n_heads=H)[:, S - 1 :]
+    cos, sin = eager.rope_tables(S, D)
+    k_cache, v_cache = torch.zeros(2, H, S, D), torch.zeros(2, H, S, D)
+    empty = torch.zeros(2, H, 1, D)
+    for t in range(S):
+        _, k_new, v_new = eager.llama_block_decode_eager(x[:, t : t + 1], p, empty, empty, cos[t], sin[t], n_heads=H)
+        k_cache[:, :, t : t + 1], v_cache[:, :, t : t + 1] = k_new, v_new
+    got, _, _ = eager.llama_block_decode_eager(x[:, S - 1 :], p, k_cache, v_cache, cos[S - 1], sin[S - 1], n_heads=H)
+    torch.testing.assert_close(got, want, rtol=1e-5, atol=1e-5)
+    # and a middle position, against the block run on the prefix that ends there
+    t = 4
+    want_t = eager.llama_block_eager(x[:, : t + 1], p, n_heads=H)[:, t:]
+    got_t, _, _ = eager.llama_block_decode_eager(x[:, t : t + 1], p, k_cache[:, :, : t + 1], v_cache[:, :, : t + 1], cos[t], sin[t], n_heads=H)
+    torch.testing.assert_close(got_t, want_t, rtol=1e-5, atol=1e-5)

@@ -271,10 +271,10 @@ def _rope_backward(ctx, gy):
     gcos = gsin = None
     if need[1] or need[2]:
         gf, xf = gy.float(), x.float()
-        if need[1]:
-            gcos = (gf * xf).sum(dim=(0, 1)).reshape(cos.shape).to(cos.dtype)
+        if need[1]:  # summed over everything the table was broadcast along (batch and heads; positions too for one row)
+            gcos = (gf * xf).sum_to_size(*([1] * (4 - cos.dim()) + list(cos.shape))).reshape(cos.shape).to(cos.dtype)
         if need[2]:
-            gsin = (gf * _rotate_half(xf)).sum(dim=(0, 1)).reshape(sin.shape).to(sin.dtype)
+            gsin = (gf * _rotate_half(xf)).sum_to_size(*([1] * (4 - sin.dim()) + list(sin.shape))).reshape(sin.shape).to(sin.dtype)
     return gx, gcos, gsin
 
 

@@ -1100,8 +1100,11 @@ def _rope_check(x, cos, sin):
     if D % 16 != 0:
         raise ValueError("rope: head dim must be a multiple of 16")
     for t in (cos, sin):
-        if t.dim() < 2 or tuple(t.shape[-2:]) != (S, D) or any(d != 1 for d in t.shape[:-2]):
-            raise ValueError("rope: cos / sin must be [S, D] tables (leading dims of size 1 allowed)")
+        rows_ok = t.dim() == 1 or (t.dim() >= 2 and t.shape[-2] in (1, S))
+        if t.dim() < 1 or t.shape[-1] != D or not rows_ok or any(d != 1 for d in t.shape[:-2]):
+            raise ValueError("rope: cos / sin must be [S, D] tables or one row [D] (leading dims of size 1 allowed)")
+    if cos.shape != sin.shape:
+        raise ValueError("rope: cos and sin must have the same shape")
     if cos.dtype != sin.dtype or cos.dtype not in (x.dtype, torch.float32):
         raise TypeError("rope: cos / sin must share a dtype, that of x or float32")
 
@@ -1113,12 +1116,14 @@ def _rope(x, cos, sin):
     out = _empty_like_layout(x)
     if out.numel() == 0:
         return out
-    cos2, sin2 = cos.reshape(S, D), sin.reshape(S, D)
-    if cos2.stride(1) != 1 or sin2.stride() != cos2.stride():
+    cos2, sin2 = cos.reshape(-1, D), sin.reshape(-1, D)
+    if cos2.shape[0] != S:  # one row for every position: a table of S equal rows (S is 1 in a decode step: a view)
+        cos2, sin2 = cos2.expand(S, D), sin2.expand(S, D)
+    if cos2.stride(1) != 1 or sin2.stride() != cos2.stride() or (S > 1 and cos2.stride(0) < D):
         cos2, sin2 = cos2.contiguous(), sin2.contiguous()
     S3 = ctypes.c_int64 * 3
     st = _lib.lib().xg_rope(
-        _ptr(x), _ptr(cos2), _ptr(sin2), _ptr(out), B, H, S, D, S3(*x.stride()[:3]), S3(*out.stride()[:3]), cos2.stride(0),
+        _ptr(x), _ptr(cos2), _ptr(sin2), _ptr(out), B, H, S, D, S3(*x.stride()[:3]), S3(*out.stride()[:3]), max(cos2.stride(0), D),
         _code(x.dtype), _code(cos2.dtype), _stream(),
     )
     _lib.check(st, "xg_rope")

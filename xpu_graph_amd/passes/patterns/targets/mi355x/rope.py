@@ -5,7 +5,8 @@
 x is a [B, H, S, D] tensor (usually the transposed view of a projection's
 [B, S, H, D] output: the kernel takes strides and writes in the same layout,
 so no copy is made), cos / sin are [S, D] tables in x's dtype, possibly with
-leading dimensions of size 1.  The reference has no rotary pattern; unfused,
+leading dimensions of size 1, or one row [D] shared by every position (a
+decode step's).  The reference has no rotary pattern; unfused,
 the subgraph is seven elementwise / copy kernels per tensor in the Llama block
 of benchmark config 5.
 """
@@ -33,13 +34,16 @@ def _val(node):
 
 
 def _is_table(node, x_val):
+    """[S, D] in x's dtype, possibly with leading dimensions of size 1 -- or a single row ([D], [1, D]) that every
+    position shares, which is what a decode step passes for its one position."""
     v = _val(node)
-    if v is None or v.dtype != x_val.dtype or v.dim() < 2:
+    if v is None or v.dtype != x_val.dtype or v.dim() < 1:
         return False
     shape = list(v.shape)
-    if not all(isinstance(d, int) for d in shape):
+    if not all(isinstance(d, int) for d in shape) or shape[-1] != x_val.shape[-1]:
         return False
-    return shape[-2:] == list(x_val.shape[-2:]) and all(d == 1 for d in shape[:-2])
+    rows_ok = v.dim() == 1 or shape[-2] in (1, x_val.shape[-2])
+    return rows_ok and all(d == 1 for d in shape[:-2])
 
 
 def _rotate_half_source(node):
