@@ -1770,11 +1770,15 @@ int launch_gemm_at(const GemmParams& p, hipStream_t stream) {
 template <typename T, typename OT>
 int launch_glu(const GemmParams& p, hipStream_t stream) {
   constexpr int EB = Elem<T>::BYTES;
-  // The row-streaming and the 64 x 64 kernel are taken exactly where the plain layer takes them for the same M, N, K (its
-  // tiles are 256 columns wide, the gated layer's 128), so that the gated layer stays two plain layers and the gate kernel bit
-  // for bit.  A decode step (M = 1, K = 4096, N = 11008) took 74 us on the large tiles, 86 of them for 256 compute units.
+  // Up to 128 rows the row-streaming and the 64 x 64 kernel are taken exactly where the plain layer takes them for the same
+  // M, N, K (its tiles are 256 columns wide, the gated layer's 128), so that the gated layer stays two plain layers and the
+  // gate kernel bit for bit there.  A decode step (M = 1, K = 4096, N = 11008) took 74 us on the large tiles, 86 of them for
+  // 256 compute units; 33 us row by row.  Measured at N = 11008, K = 4096 (us, 64 x 64 kernel / large tiles): M = 64 47 / 76,
+  // M = 128 61 / 76, M = 256 101 / 80: beyond 128 rows the tile count of the gated layer's own tiles decides, as before.
   if (skinny_fits(p)) return launch_skinny<T, OT, true>(p, stream);
-  if ((int64_t)p.tiles_m * ((p.N + BN - 1) / BN) <= small_tile_limit()) return launch_small<T, OT, BLayout::KMajor, true>(p, stream);
+  const int64_t plain_tiles = (int64_t)p.tiles_m * ((p.N + BN - 1) / BN);
+  if ((p.M <= 128 && plain_tiles <= small_tile_limit()) || (int64_t)p.tiles_m * p.tiles_n <= small_tile_limit())
+    return launch_small<T, OT, BLayout::KMajor, true>(p, stream);
   const int keep = full_tile_columns(p.tiles_m, p.tiles_n);
   if (keep == p.tiles_n) {
     if (half_height_wins(p.M, p.tiles_n)) {
