@@ -452,6 +452,7 @@ def test_batch_dense_compiled(device, form):
         (13, 1032, 640),     # ragged rows and columns
         (16, 11008, 4096),   # where the plain layer takes the 64 x 64 kernel, so does the gated one
         (64, 11008, 512),
+        (128, 11008, 512),   # the last row count at which the gated layer follows the plain layer's small-size choices
     ],
 )
 def test_dense_glu_bit_identical_to_the_unfused_ops(device, dtype, M, N, K):
