@@ -462,7 +462,7 @@ def test_dense_glu_bit_identical_to_the_unfused_ops(device, dtype, M, N, K):
     x = torch.randn(M, K, generator=g).to(dtype).to(device)
     wg = (torch.randn(N, K, generator=g) / K**0.5).to(dtype).to(device)
     wu = (torch.randn(N, K, generator=g) / K**0.5).to(dtype).to(device)
-    ops = torch.ops.xpu_ops
+    ops = _ops()
     got = ops.dense_glu(x, wg, wu)
     gate, up = ops.dense(x, wg, True, None, None, "none"), ops.dense(x, wu, True, None, None, "none")
     two = ops.silu_mul2(gate, up)
@@ -490,7 +490,7 @@ def test_dense_glu_half_height_grid(device, M, N, K):
 
 
 def test_dense_glu_strided_operands_and_rejects(device):
-    ops = torch.ops.xpu_ops
+    ops = _ops()
     big = torch.randn(64, 512, device=device).bfloat16()
     x = big[:, 128:384]  # row stride 512, K = 256
     wbig = (torch.randn(2, 40, 256, device=device) / 16).bfloat16()
