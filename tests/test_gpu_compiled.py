@@ -156,6 +156,42 @@ def test_c5_llama_block(device, B, S):
     torch.testing.assert_close(out.float(), want_f32, rtol=1.6e-2, atol=err_eager.max().item())
 
 
+@pytest.mark.parametrize("B,S", [(1, 700), (8, 2048)])
+def test_c5_llama_block_decode_step(device, B, S):
+    # One new token per sequence against S cached positions: every projection is a few rows against a whole weight
+    # matrix, the rotary table is one row, and attention has one query row per head.
+    H, D = 32, 128
+    x, p = inputs.c5_llama_block(B=B, S=1, device=device)
+    names = sorted(p)
+    g = torch.Generator().manual_seed(11)
+    kc = torch.randn(B, H, S, D, generator=g).to(torch.bfloat16).to(device)
+    vc = torch.randn(B, H, S, D, generator=g).to(torch.bfloat16).to(device)
+    ang = torch.rand(D // 2, generator=g) * 6.283
+    cos = torch.cat([ang.cos(), ang.cos()]).to(torch.bfloat16).to(device)
+    sin = torch.cat([ang.sin(), ang.sin()]).to(torch.bfloat16).to(device)
+
+    def fn(x, kc, vc, cos, sin, *ws):
+        return eager.llama_block_decode_eager(x, dict(zip(names, ws)), kc, vc, cos, sin, n_heads=H)
+
+    (out, k_new, v_new), mods, rest = run(fn, x, kc, vc, cos, sin, *[p[n] for n in names])
+    print("decode step modules:", mods)
+    print("decode step remaining aten:", rest)
+    assert "mi355x_sdpa" in mods and mods.count("mi355x_rope") == 2 and "mi355x_dense_glu" in mods
+    heavy = [t for t in rest if any(k in t for k in ("aten.mm", "aten.bmm", "aten.addmm", "softmax", "aten.matmul"))]
+    assert heavy == [], heavy
+    with torch.no_grad():
+        want_bf16 = fn(x, kc, vc, cos, sin, *[p[n] for n in names])
+        want_f32 = eager.llama_block_decode_eager(
+            x.float(), {n: w.float() for n, w in p.items()}, kc.float(), vc.float(), cos.float(), sin.float(), n_heads=H
+        )
+    for got, eb, ef, what in zip((out, k_new, v_new), want_bf16, want_f32, ("out", "k_new", "v_new")):
+        err_eager = (eb.float() - ef).abs()
+        err_fused = (got.float() - ef).abs()
+        print(f"decode step B{B} S{S} {what}: mean |err| fused {err_fused.mean().item():.4g} eager {err_eager.mean().item():.4g}")
+        assert err_fused.mean().item() <= 1.05 * err_eager.mean().item() + 1e-6
+        torch.testing.assert_close(got.float(), ef, rtol=1.6e-2, atol=max(err_eager.max().item(), 1e-3))
+
+
 @pytest.mark.parametrize("rank", [2, 3])
 def test_fused_slice_compiled(device, rank):
     """Equally wide slices of one tensor, each with a consumer (reference tests/mlu/test_fuse_slice.py:43-60, 128-147):
