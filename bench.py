@@ -682,6 +682,47 @@ class DenseDecode(Workload):
         return (lambda: fn(x, W, b)), how
 
 
+class DenseDecodeFp8(DenseDecode):
+    name = "decode dense + bias fp8 e4m3 M1 K4096 N11008, [N,K] weights"
+    dtype = "fp8"
+    kernel = "gemm_skinny_fp8_kernel<bf16,1>"
+    work = 11008 * 4096 + 4096 + 11008 * 4 + 2 * 11008 * 2  # the weights once, x, the weight scales, bias and the output row
+    n_sets = 6  # 270 MB of weights in rotation
+
+    def setup(self, torch, dev):
+        from oracle import eager
+        from xpu_graph_amd import _lib
+
+        self.torch = torch
+        g = torch.Generator().manual_seed(0)
+        self.sets = []
+        for _ in range(self.n_sets):
+            x_q, s_x = eager.quantize_fp8_per_tensor(torch.randn(1, 4096, generator=g))
+            W_q, s_w = eager.quantize_fp8_per_out_channel(torch.randn(4096, 11008, generator=g) * 0.02)
+            b = (torch.randn(11008, generator=g) * 0.02).bfloat16()
+            self.sets.append((x_q.to(dev), W_q.t().contiguous().to(dev), s_x.to(dev), s_w.contiguous().to(dev), b.to(dev)))
+        self.outs = [torch.empty(1, 11008, device=dev, dtype=torch.bfloat16) for _ in range(self.n_sets)]
+        self.lib = _lib.lib()
+        self.st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def op_call(self, i):
+        x_q, w_nk, s_x, s_w, b = self.sets[i]
+        return self.torch.ops.xpu_ops.dense_fp8(x_q, w_nk, True, s_x, s_w, b, "none", self.torch.bfloat16)
+
+    def abi_call(self, i):
+        x_q, w_nk, s_x, s_w, b = self.sets[i]
+        self.lib.xg_dense_fp8(_p(x_q), _p(w_nk), _p(s_x), _p(s_w), _p(b), _p(self.outs[i]), 1, 11008, 4096, 4096, 4096, 1, 0, 2, 2, self.st)
+
+    def check(self, torch):
+        x_q, w_nk, s_x, s_w, b = self.sets[0]
+        want = (x_q.float() @ w_nk.float().t()) * s_x * s_w + b.float()
+        torch.testing.assert_close(self.op_call(0).float(), want, rtol=1.6e-2, atol=2e-3)
+
+    def cpu_fn(self, torch):
+        x_q, w_nk, s_x, s_w, b = (t.cpu() for t in self.sets[0])
+        return (lambda: (x_q.float() @ w_nk.float().t()) * s_x * s_w + b.float()), "eager dequantise + fp32 matmul"
+
+
 class SdpaDecode(Workload):
     name = "decode attention bf16 B8 H32 Hkv8 Sq1 Skv8192 D128"
     dtype = "bf16"
@@ -1028,7 +1069,7 @@ def traffic_from(fetch_dir, write_dir, out_path=TRAFFIC_FILE):
 
 
 HEADLINE = AddLayerNormC2
-OTHERS = [RmsNormC1, SliceCatC3a, AddNC3b, DenseC4, DenseFp32, DenseFp8C4, DenseGluC5, SdpaC5, SdpaBackwardC5, DenseWeightGradC4, DenseDecode, SdpaDecode,
+OTHERS = [RmsNormC1, SliceCatC3a, AddNC3b, DenseC4, DenseFp32, DenseFp8C4, DenseGluC5, SdpaC5, SdpaBackwardC5, DenseWeightGradC4, DenseDecode, DenseDecodeFp8, SdpaDecode,
           LlamaBlockDecode, LlamaBlockC5, LlamaBlockTrainC5]
 
 

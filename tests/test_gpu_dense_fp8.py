@@ -86,6 +86,50 @@ def test_dense_fp8_decodes_every_code(device):
         assert got[code, 5].item() == val
 
 
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize(
+    "M,N,K",
+    [(1, 4096, 4096), (16, 4096, 4096), (17, 4096, 4096), (32, 4096, 11008), (5, 11008, 4096), (3, 520, 1024), (32, 1000, 1280), (9, 512, 2304)],
+)
+def test_dense_fp8_decode_sizes(device, out_dtype, M, N, K):
+    """At most 32 rows against a whole weight matrix: the row-streaming e4m3 kernel (a workgroup per 16 weight rows, K
+    split over its four wavefronts).  Ragged N (not a multiple of 16), K quarters that leave a tail after the unrolled
+    groups (1280, 2304), both row-tile counts."""
+    x_q, W_q, s_x, s_w, b = quantised(M, N, K, device, seed=M + N + K)
+    w_nk = W_q.t().contiguous()
+    for bias, act in ((b, "silu"), (None, "none"), (b.to(out_dtype), "gelu")):
+        got = _ops().dense_fp8(x_q, w_nk, True, s_x, s_w, bias, act, out_dtype)
+        assert got.shape == (M, N) and got.dtype == out_dtype
+        z = (x_q.float() @ W_q.float()) * s_x * s_w
+        if bias is not None:
+            z = z + bias.float()
+        want = {"silu": torch.nn.functional.silu, "gelu": torch.nn.functional.gelu, "none": lambda t: t}[act](z)
+        close(got, want)
+    # a row of the batch equals the same row computed alone: the kernels of 1..16 and of 17..32 rows add in one order
+    alone = _ops().dense_fp8(x_q[M - 1 :], w_nk, True, s_x, s_w, b, "silu", out_dtype)
+    batch = _ops().dense_fp8(x_q, w_nk, True, s_x, s_w, b, "silu", out_dtype)
+    assert torch.equal(alone[0], batch[M - 1])
+
+
+def test_dense_fp8_decode_kernel_pairs_every_k(device):
+    """One non-zero activation at position k and one-hot weight rows: the output is the product exactly when the
+    kernel pairs activation byte k with weight byte k, for every k of a wavefront's quarter and every quarter."""
+    K, N = 1024, 512
+    one = torch.ones(1, device=device)
+    for k in list(range(0, 80)) + [255, 256, 511, 777, 1023]:
+        x = torch.zeros(2, K, dtype=torch.uint8)
+        x[1, k] = 0x40  # 2.0
+        w = torch.zeros(N, K, dtype=torch.uint8)
+        w[:, k] = 0x38  # 1.0
+        w[7, k] = 0x34  # 0.75
+        w[7, (k + 8) % K] = 0x48  # 4.0 at a position the activation does not have
+        got = _ops().dense_fp8(x.view(torch.float8_e4m3fn).to(device), w.view(torch.float8_e4m3fn).to(device), True, one, one.expand(N).contiguous(), None, "none", torch.float32)
+        want = torch.full((N,), 2.0)
+        want[7] = 1.5
+        assert torch.equal(got[1].cpu(), want), k
+        assert torch.count_nonzero(got[0]) == 0
+
+
 def test_dense_fp8_c4_full_size(device):
     x, W, b = inputs.c4_dense(device=device)
     x_q, s_x = eager.quantize_fp8_per_tensor(x)

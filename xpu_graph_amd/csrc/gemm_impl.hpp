@@ -1297,6 +1297,94 @@ __global__ __launch_bounds__(kThreads) void gemm_skinny_kernel(GemmParams p_all)
   }
 }
 
+// The same walk for e4m3 operands (the quantised weight is always K-contiguous): a lane's 16 bytes are 16 values of k, the
+// low and the high eight feed one 16 x 16 x 32 MFMA each -- which 32 values of k meet in one instruction does not matter,
+// as long as the weight and the activation fragment pair the same ones -- so a wavefront advances 64 values of k per step.
+// Scales, bias and activation as in the other fp8 kernels: act(sum * a_scale * b_scale[n] + bias[n]).
+template <typename OT, int MT>
+__global__ __launch_bounds__(kThreads) void gemm_skinny_fp8_kernel(GemmParams p) {
+  constexpr int U = MT == 1 ? 8 : 4;
+  __shared__ float part[4][MT][16][16];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l16 = lane & 15, q = lane >> 4;
+  const int n0 = blockIdx.x * 16;
+  int n = n0 + l16;
+  n = n < p.N ? n : p.N - 1;  // columns past the edge re-read the last row of W; their results are never stored
+  const int kq = p.K / 4;     // K % 256 == 0 is checked on the host: every quarter is a whole number of 64-byte steps
+  const uint8_t* w_at = reinterpret_cast<const uint8_t*>(p.B) + (int64_t)n * p.ldb + wave * kq + 16 * q;
+  const uint8_t* x_at[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    int m = 16 * t + l16;
+    m = m < p.M ? m : p.M - 1;
+    x_at[t] = reinterpret_cast<const uint8_t*>(p.A) + (int64_t)m * p.lda + wave * kq + 16 * q;
+  }
+  f32x4 acc[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+  typedef long l64x2 __attribute__((ext_vector_type(2)));
+  auto two = [](const l64x2 a, const l64x2 b, f32x4 c) {
+    c = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a[0], b[0], c, 0, 0, 0);
+    return __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a[1], b[1], c, 0, 0, 0);
+  };
+
+  l64x2 fw[2][U], fx[2][MT][U];
+  auto load = [&](int buf, int k) {  // steps k .. k + U - 1 of this wavefront's quarter
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      fw[buf][u] = *reinterpret_cast<const l64x2*>(w_at + (k + u) * 64);
+#pragma unroll
+      for (int t = 0; t < MT; ++t) fx[buf][t][u] = *reinterpret_cast<const l64x2*>(x_at[t] + (k + u) * 64);
+    }
+  };
+  auto math = [&](int buf) {
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int t = 0; t < MT; ++t) acc[t] = two(fw[buf][u], fx[buf][t][u], acc[t]);
+  };
+  const int steps = kq / 64, groups = steps / U;
+  if (groups > 0) load(0, 0);
+  for (int g = 0; g + 1 < groups; g += 2) {  // two groups per trip: the buffer indices stay compile-time
+    load(1, (g + 1) * U);
+    math(0);
+    if (g + 2 < groups) load(0, (g + 2) * U);
+    math(1);
+  }
+  if (groups & 1) math(0);
+  for (int k = groups * U; k < steps; ++k) {  // what does not fill a group
+    const l64x2 a = *reinterpret_cast<const l64x2*>(w_at + k * 64);
+#pragma unroll
+    for (int t = 0; t < MT; ++t) acc[t] = two(a, *reinterpret_cast<const l64x2*>(x_at[t] + k * 64), acc[t]);
+  }
+
+  // accumulator t of a lane: output rows 16 t + l16 (A rows), columns n0 + 4 q .. + 3
+#pragma unroll
+  for (int t = 0; t < MT; ++t)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) part[wave][t][4 * q + e][l16] = acc[t][e];
+  __syncthreads();
+  const float a_sc = p.a_scale ? *p.a_scale : 1.f;
+  for (int idx = tid; idx < MT * 256; idx += kThreads) {
+    const int nl = idx & 15, ml = (idx >> 4) & 15, t = idx >> 8;
+    const int m = 16 * t + ml, nn = n0 + nl;
+    if (m >= p.M || nn >= p.N) continue;
+    float v = (part[0][t][nl][ml] + part[1][t][nl][ml]) + (part[2][t][nl][ml] + part[3][t][nl][ml]);
+    const float sc = p.b_scale ? a_sc * p.b_scale[nn] : a_sc;
+    const float bias = !p.bias ? 0.f : p.bias_f32 ? reinterpret_cast<const float*>(p.bias)[nn] : to_f32(reinterpret_cast<const OT*>(p.bias)[nn]);
+    v = v * sc + bias;
+    switch (p.act) {
+      case XG_ACT_RELU: v = fmaxf(v, 0.f); break;
+      case XG_ACT_GELU: v = 0.5f * v * (1.f + erff(v * 0.70710678118654752f)); break;
+      case XG_ACT_SILU: v = silu_f32(v); break;
+      case XG_ACT_SIGMOID: v = sigmoid_f32(v); break;
+      default: break;
+    }
+    reinterpret_cast<OT*>(p.out)[(int64_t)m * p.ldc + nn] = from_f32<OT>(v);
+  }
+}
+
 // ---- 128 x 128 tiles: between the 64 x 64 kernel and the large tiles -------------------------------------------
 // A problem whose 256 x 256 grid fills a fraction of the compute units, or just over a whole number of rounds, has four
 // times as many 128 x 128 tiles: each of the four wavefronts owns a 64 x 64 quadrant (2 x 2 MFMA tiles) over the whole
@@ -1586,6 +1674,24 @@ inline bool skinny_fits(const GemmParams& p) {
   return p.M <= 4 || (p.M <= 16 && p.N <= 4608) || (p.M <= 32 && p.N <= 4096);
 }
 
+// Where the e4m3 walk beats the 64 x 64 kernel.  Measured (us, this kernel at M = 1 / 8 / 16 / 32, then the 64 x 64 kernel,
+// which is flat in M here): N = K = 4096 5.6 / 6.2 / 6.8 / 9.0, 9.6; N = 11008, K = 4096 10.2 / 12.0 / 13.9 / 19.5, 13.1;
+// N = 4096, K = 11008 10.6 / 12.0 / 13.6 / 18.8, 23.8; N = K = 8192 13.6 / 14.9 / 18.0 / 24.5, 21.2; N = 1024, K = 4096
+// 4.8 / 5.6 / 6.3 / 8.4, 9.5.  Every workgroup re-reads the M activation rows (M / 16 of its weight bytes), which is
+// what the limits on M follow.
+inline bool skinny_fp8_fits(const GemmParams& p) {
+  if (p.N < 512 || p.K < 1024 || p.K % 256 != 0 || p.batch != 1 || p.res != nullptr) return false;
+  return p.M <= 8 || (p.M <= 16 && p.N <= 8192) || (p.M <= 32 && p.N <= 4096);
+}
+template <typename OT>
+int launch_skinny_fp8(const GemmParams& p, hipStream_t stream) {
+  const int64_t blocks = (p.N + 15) / 16;
+  if (blocks > 0x7fffffffLL) return XG_ERR_TOO_LARGE;
+  if (p.M <= 16) hipLaunchKernelGGL((gemm_skinny_fp8_kernel<OT, 1>), dim3((unsigned)blocks), dim3(kThreads), 0, stream, p);
+  else hipLaunchKernelGGL((gemm_skinny_fp8_kernel<OT, 2>), dim3((unsigned)blocks), dim3(kThreads), 0, stream, p);
+  return status_from_hip(hipGetLastError());
+}
+
 template <typename T, typename OT, bool GLU = false>
 int launch_skinny(const GemmParams& p, hipStream_t stream) {
   const int64_t blocks = (p.N + 15) / 16;
@@ -1692,6 +1798,9 @@ int launch_gemm(const GemmParams& p, hipStream_t stream) {
   if (!dma_ok<T>(p, BL)) return launch_kernel(gemm_staged_kernel<T, OT, BL>, p, stream);
   if constexpr (Elem<T>::BYTES == 2 && BL == BLayout::KMajor) {
     if (skinny_fits(p)) return launch_skinny<T, OT>(p, stream);
+  }
+  if constexpr (Elem<T>::BYTES == 1 && BL == BLayout::KMajor) {
+    if (skinny_fp8_fits(p)) return launch_skinny_fp8<OT>(p, stream);
   }
   if constexpr (Elem<T>::BYTES == 2) {
     if (mid_tiles_win(p)) return launch_mid<T, OT, BL>(p, stream);
